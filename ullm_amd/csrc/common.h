@@ -1,0 +1,69 @@
+// Shared helpers of the gfx950 kernels: storage types, 32-bit conversion, wave and block
+// reductions with a fixed order (so a row's result never depends on what else is in the batch).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+typedef uint16_t bf16_t;  // bfloat16 as raw bits; all arithmetic is done in float
+
+enum { ULLM_F32 = 0, ULLM_BF16 = 1 };
+
+// error codes of the extern "C" launchers (0 = ok, >0 = hipError_t of the launch)
+enum { ULLM_ERR_DTYPE = -1, ULLM_ERR_SHAPE = -2, ULLM_ERR_UNSUPPORTED = -3 };
+
+#define WAVE 64
+
+__device__ __forceinline__ float bf16_bits_to_f32(bf16_t v) {
+  return __uint_as_float(((uint32_t)v) << 16);
+}
+
+// round to nearest even; NaN stays NaN
+__device__ __forceinline__ bf16_t f32_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x0040u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (bf16_t)(u >> 16);
+}
+
+__device__ __forceinline__ float ld_f32(const float* p) { return *p; }
+__device__ __forceinline__ float ld_f32(const bf16_t* p) { return bf16_bits_to_f32(*p); }
+__device__ __forceinline__ void st_f32(float* p, float v) { *p = v; }
+__device__ __forceinline__ void st_f32(bf16_t* p, float v) { *p = f32_to_bf16_bits(v); }
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int m = WAVE / 2; m > 0; m >>= 1) v += __shfl_xor(v, m, WAVE);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int m = WAVE / 2; m > 0; m >>= 1) v = fmaxf(v, __shfl_xor(v, m, WAVE));
+  return v;
+}
+
+// Block reductions over up to 1024 threads (16 waves); every thread gets the result.
+// `scratch` must hold 16 floats of shared memory; the caller may reuse it after the call.
+__device__ __forceinline__ float block_sum(float v, float* scratch) {
+  const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
+  const int nwaves = (blockDim.x + WAVE - 1) / WAVE;
+  v = wave_sum(v);
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  float r = 0.f;
+  for (int w = 0; w < nwaves; ++w) r += scratch[w];
+  return r;
+}
+__device__ __forceinline__ float block_max(float v, float* scratch) {
+  const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
+  const int nwaves = (blockDim.x + WAVE - 1) / WAVE;
+  v = wave_max(v);
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  float r = scratch[0];
+  for (int w = 1; w < nwaves; ++w) r = fmaxf(r, scratch[w]);
+  return r;
+}
+
+#define ULLM_LAUNCH_CHECK() return (int)hipGetLastError()

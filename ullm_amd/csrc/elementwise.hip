@@ -1,0 +1,206 @@
+// Row-wise kernels of the layer: embedding gather into the 32-bit residual stream, fused
+// residual add + RMS norm, per-head q/k norm + rotary position encoding + paged cache write,
+// and SiLU(gate)*up.  All arithmetic is 32-bit; T selects the storage type only.
+//
+// Formulas follow the reference's layers: RMS norm (ullm/layers/layernorm.py:20-34),
+// half-split rotary pairs (ullm/layers/rotary_embedding.py:5-24), SiLU-and-mul
+// (ullm/layers/activation.py:16-18), cache write of k after norm+rotation and raw v
+// (ullm/layers/attention.py:288-296).
+#include "common.h"
+
+// ------------------------------------------------------------------ embedding
+// residual[t, :] = float(table[ids[t], :]); ids outside [0, V) give a zero row.
+template <typename T>
+__global__ void embedding_kernel(const int* __restrict__ ids, const T* __restrict__ table,
+                                 float* __restrict__ residual, int H, int V) {
+  const int t = blockIdx.x;
+  const int id = ids[t];
+  float* out = residual + (size_t)t * H;
+  if (id < 0 || id >= V) {
+    for (int i = threadIdx.x; i < H; i += blockDim.x) out[i] = 0.f;
+    return;
+  }
+  const T* row = table + (size_t)id * H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) out[i] = ld_f32(row + i);
+}
+
+extern "C" int ullm_embedding(const int* ids, const void* table, float* residual, int T_, int H,
+                              int V, int dtype, hipStream_t stream) {
+  if (T_ <= 0) return 0;
+  if (H <= 0 || V <= 0) return ULLM_ERR_SHAPE;
+  dim3 grid(T_), block(256);
+  if (dtype == ULLM_F32)
+    hipLaunchKernelGGL(embedding_kernel<float>, grid, block, 0, stream, ids, (const float*)table, residual, H, V);
+  else if (dtype == ULLM_BF16)
+    hipLaunchKernelGGL(embedding_kernel<bf16_t>, grid, block, 0, stream, ids, (const bf16_t*)table, residual, H, V);
+  else
+    return ULLM_ERR_DTYPE;
+  ULLM_LAUNCH_CHECK();
+}
+
+// ------------------------------------------------------------------ add + RMS norm
+// For output row r (input row i = rows ? rows[r] : r):
+//   s = residual[i] + float(branch[i])      (branch may be null: s = residual[i])
+//   if write_res: residual[i] = s           (the stream stays 32-bit, never rounded)
+//   y[r] = s * rsqrt(mean(s^2) + eps) * gain
+template <typename TB, typename TY>
+__global__ void add_rmsnorm_kernel(const TB* __restrict__ branch, float* __restrict__ residual,
+                                   const float* __restrict__ gain, float eps, TY* __restrict__ y,
+                                   const int* __restrict__ rows, int H, int write_res) {
+  __shared__ float scratch[16];
+  const int r = blockIdx.x;
+  const int i = rows ? rows[r] : r;
+  float* res = residual + (size_t)i * H;
+  const TB* br = branch ? branch + (size_t)i * H : nullptr;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < H; c += blockDim.x) {
+    float s = res[c];
+    if (br) s += ld_f32(br + c);
+    if (write_res && br) res[c] = s;
+    ss += s * s;
+  }
+  const float total = block_sum(ss, scratch);
+  const float rs = rsqrtf(total / (float)H + eps);
+  TY* out = y + (size_t)r * H;
+  for (int c = threadIdx.x; c < H; c += blockDim.x) {
+    float s = res[c];
+    if (br && !write_res) s += ld_f32(br + c);
+    st_f32(out + c, (s * rs) * gain[c]);
+  }
+}
+
+extern "C" int ullm_add_rmsnorm(const void* branch, float* residual, const float* gain, float eps,
+                                void* y, const int* rows, int n_rows, int H, int branch_dtype,
+                                int y_dtype, int write_res, hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  if (H <= 0) return ULLM_ERR_SHAPE;
+  if (rows && write_res) return ULLM_ERR_UNSUPPORTED;  // a gathered row could be updated twice
+  dim3 grid(n_rows), block(H >= 2048 ? 512 : 256);
+#define GO(TB, TY) hipLaunchKernelGGL((add_rmsnorm_kernel<TB, TY>), grid, block, 0, stream, \
+    (const TB*)branch, residual, gain, eps, (TY*)y, rows, H, write_res)
+  if (branch_dtype == ULLM_F32 && y_dtype == ULLM_F32) GO(float, float);
+  else if (branch_dtype == ULLM_BF16 && y_dtype == ULLM_BF16) GO(bf16_t, bf16_t);
+  else if (branch_dtype == ULLM_BF16 && y_dtype == ULLM_F32) GO(bf16_t, float);
+  else if (branch_dtype == ULLM_F32 && y_dtype == ULLM_BF16) GO(float, bf16_t);
+  else return ULLM_ERR_DTYPE;
+#undef GO
+  ULLM_LAUNCH_CHECK();
+}
+
+// ------------------------------------------------------------------ SiLU(gate) * up
+template <typename T>
+__global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int I, size_t total) {
+  size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const size_t t = idx / I;
+  const int i = (int)(idx - t * I);
+  const T* row = gu + t * (size_t)(2 * I);
+  const float g = ld_f32(row + i), u = ld_f32(row + I + i);
+  const float s = g / (1.f + expf(-g));
+  st_f32(out + idx, s * u);
+}
+
+extern "C" int ullm_silu_mul(const void* gu, void* out, int T_, int I, int dtype, hipStream_t stream) {
+  if (T_ <= 0) return 0;
+  if (I <= 0) return ULLM_ERR_SHAPE;
+  const size_t total = (size_t)T_ * I;
+  dim3 block(256), grid((unsigned)((total + 255) / 256));
+  if (dtype == ULLM_F32)
+    hipLaunchKernelGGL(silu_mul_kernel<float>, grid, block, 0, stream, (const float*)gu, (float*)out, I, total);
+  else if (dtype == ULLM_BF16)
+    hipLaunchKernelGGL(silu_mul_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)gu, (bf16_t*)out, I, total);
+  else
+    return ULLM_ERR_DTYPE;
+  ULLM_LAUNCH_CHECK();
+}
+
+// ------------------------------------------------------------------ q/k norm + rotary + cache write
+// One wave per (token, head) of the fused projection row  [q heads | k heads | v heads].
+//   q heads: per-head RMS norm (gain shared by all heads, may be null), rotation, written to q_out
+//   k heads: the same with the k gain, written into the token's cache page
+//   v heads: copied into the cache page
+// Rotation: pair (i, i + rot/2) for style 1 (half split), (2i, 2i+1) for style 2, i < rot/2;
+//   o_a = a cos - b sin, o_b = b cos + a sin with cos/sin = table[pos, i], table[pos, rot/2 + i];
+//   dims >= rot pass through.  style 0: no rotation.
+// Cache page of token t: block_table[entry[t], pos / page_size], row pos % page_size;
+// pool layout [page, kv_head, row, head_dim].  Tokens whose page id is negative are not written.
+#define MAX_HEAD_DIM 512
+template <typename T>
+__global__ void qk_norm_rope_write_kernel(
+    const T* __restrict__ qkv, int qkv_stride, T* __restrict__ q_out, int q_out_stride,
+    const float* __restrict__ q_gain, const float* __restrict__ k_gain, float eps,
+    const float* __restrict__ cos_sin, int table_rows, int rot, int style,
+    const int* __restrict__ positions, const int* __restrict__ token_entry,
+    const int* __restrict__ block_table, int bt_stride, T* __restrict__ k_pool, T* __restrict__ v_pool,
+    int page_size, int nq, int nkv, int hd, int write_kv) {
+  __shared__ float vals[MAX_HEAD_DIM];
+  const int t = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+  const int pos = positions[t];
+  const T* src = qkv + (size_t)t * qkv_stride + (size_t)head * hd;
+  const bool is_q = head < nq, is_k = !is_q && head < nq + nkv;
+  T* dst;
+  if (is_q) {
+    dst = q_out + (size_t)t * q_out_stride + (size_t)head * hd;
+  } else {
+    if (!write_kv) return;
+    const int kvh = is_k ? head - nq : head - nq - nkv;
+    const int page = block_table[(size_t)token_entry[t] * bt_stride + pos / page_size];
+    if (page < 0) return;
+    T* pool = is_k ? k_pool : v_pool;
+    dst = pool + (((size_t)page * nkv + kvh) * page_size + (pos % page_size)) * hd;
+  }
+  if (!is_q && !is_k) {  // v: plain copy
+    for (int i = lane; i < hd; i += WAVE) dst[i] = src[i];
+    return;
+  }
+  const float* gain = is_q ? q_gain : k_gain;
+  float ss = 0.f;
+  for (int i = lane; i < hd; i += WAVE) {
+    const float x = ld_f32(src + i);
+    vals[i] = x;
+    ss += x * x;
+  }
+  if (gain) {
+    ss = wave_sum(ss);
+    const float rs = rsqrtf(ss / (float)hd + eps);
+    for (int i = lane; i < hd; i += WAVE) vals[i] = (vals[i] * rs) * gain[i];
+  }
+  __syncthreads();
+  if (style == 0 || rot <= 0) {
+    for (int i = lane; i < hd; i += WAVE) st_f32(dst + i, vals[i]);
+    return;
+  }
+  const int half = rot / 2;
+  const int p = pos < table_rows ? pos : table_rows - 1;  // host rejects positions past the table
+  const float* cs = cos_sin + (size_t)p * rot;
+  for (int i = lane; i < half; i += WAVE) {
+    const int ia = style == 1 ? i : 2 * i, ib = style == 1 ? i + half : 2 * i + 1;
+    const float c = cs[i], s = cs[half + i];
+    const float a = vals[ia], b = vals[ib];
+    st_f32(dst + ia, a * c - b * s);
+    st_f32(dst + ib, b * c + a * s);
+  }
+  for (int i = rot + lane; i < hd; i += WAVE) st_f32(dst + i, vals[i]);
+}
+
+extern "C" int ullm_qk_norm_rope_write(
+    const void* qkv, int qkv_stride, void* q_out, int q_out_stride, const float* q_gain,
+    const float* k_gain, float eps, const float* cos_sin, int table_rows, int rot, int style,
+    const int* positions, const int* token_entry, const int* block_table, int bt_stride,
+    void* k_pool, void* v_pool, int page_size, int T_, int nq, int nkv, int hd, int write_kv,
+    int dtype, hipStream_t stream) {
+  if (T_ <= 0) return 0;
+  if (hd <= 0 || hd > MAX_HEAD_DIM || nq <= 0 || nkv <= 0 || page_size <= 0) return ULLM_ERR_SHAPE;
+  if (rot < 0 || rot > hd || (rot & 1) || (style != 0 && style != 1 && style != 2)) return ULLM_ERR_SHAPE;
+  if (style != 0 && rot > 0 && (!cos_sin || table_rows <= 0)) return ULLM_ERR_SHAPE;
+  dim3 grid(T_, nq + 2 * nkv), block(WAVE);
+#define GO(TT) hipLaunchKernelGGL(qk_norm_rope_write_kernel<TT>, grid, block, 0, stream, \
+    (const TT*)qkv, qkv_stride, (TT*)q_out, q_out_stride, q_gain, k_gain, eps, cos_sin, table_rows, \
+    rot, style, positions, token_entry, block_table, bt_stride, (TT*)k_pool, (TT*)v_pool, page_size, \
+    nq, nkv, hd, write_kv)
+  if (dtype == ULLM_F32) GO(float);
+  else if (dtype == ULLM_BF16) GO(bf16_t);
+  else return ULLM_ERR_DTYPE;
+#undef GO
+  ULLM_LAUNCH_CHECK();
+}

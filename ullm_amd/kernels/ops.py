@@ -1,0 +1,226 @@
+"""Python faces of the HIP kernels: each checks operand shapes, dtypes and contiguity on the host,
+then launches on torch's current stream through the family's ``extern "C"`` entry point.
+A non-zero return of a launcher raises ``KernelError``; nothing falls back to another path.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from . import build
+
+F32, BF16 = 0, 1
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+_ERR_NAMES = {-1: "unsupported dtype combination", -2: "operand shape outside what the kernel takes",
+              -3: "unsupported argument combination"}
+
+
+def _check(rc: int, what: str) -> None:
+    if rc != 0:
+        reason = _ERR_NAMES.get(rc, f"HIP error {rc}")
+        raise KernelError(f"{what}: {reason}")
+
+
+def _dt(t: torch.Tensor) -> int:
+    if t.dtype == torch.float32:
+        return F32
+    if t.dtype == torch.bfloat16:
+        return BF16
+    raise KernelError(f"dtype {t.dtype} is not float32 or bfloat16")
+
+
+def _stream() -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _p(t: Optional[torch.Tensor]) -> ctypes.c_void_p:
+    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+def _need(cond: bool, msg: str) -> None:
+    if not cond:
+        raise KernelError(msg)
+
+
+def _i32(t: torch.Tensor, name: str, n: Optional[int] = None) -> None:
+    _need(t.dtype == torch.int32 and t.is_contiguous(), f"{name} must be contiguous int32")
+    if n is not None:
+        _need(t.numel() >= n, f"{name} holds {t.numel()} entries, {n} needed")
+
+
+_c_int, _c_float = ctypes.c_int, ctypes.c_float
+
+
+# ---------------------------------------------------------------------------------- elementwise
+
+def embedding(ids: torch.Tensor, table: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """float32 [T, H] rows of ``table`` [V, H] at ``ids`` [T] (int32)."""
+    T = ids.numel()
+    V, H = table.shape
+    _i32(ids, "ids")
+    _need(table.is_contiguous(), "embedding table must be contiguous")
+    if out is None:
+        out = torch.empty((T, H), dtype=torch.float32, device=table.device)
+    _need(out.dtype == torch.float32 and out.is_contiguous() and out.shape == (T, H), "bad embedding output")
+    lib = build.load("elementwise")
+    _check(lib.ullm_embedding(_p(ids), _p(table), _p(out), _c_int(T), _c_int(H), _c_int(V),
+                              _c_int(_dt(table)), _stream()), "embedding")
+    return out
+
+
+def add_rmsnorm(branch: Optional[torch.Tensor], residual: torch.Tensor, gain: torch.Tensor, eps: float,
+                out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None,
+                out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """residual (float32 [T, H], updated in place unless ``rows``) += branch; returns the RMS-normed
+    sum times ``gain`` (float32 [H]) in ``out_dtype``.  With ``rows`` (int32 [n]) only those rows are
+    produced and the residual stays untouched."""
+    T, H = residual.shape
+    _need(residual.dtype == torch.float32 and residual.is_contiguous(), "residual must be contiguous float32")
+    _need(gain.dtype == torch.float32 and gain.numel() == H and gain.is_contiguous(), "gain must be float32 [H]")
+    if branch is not None:
+        _need(branch.shape == (T, H) and branch.is_contiguous(), "branch must be contiguous [T, H]")
+    n = T
+    if rows is not None:
+        _i32(rows, "rows")
+        n = rows.numel()
+    if out is None:
+        out = torch.empty((n, H), dtype=out_dtype, device=residual.device)
+    _need(out.shape == (n, H) and out.is_contiguous() and out.dtype == out_dtype, "bad norm output")
+    lib = build.load("elementwise")
+    bdt = _dt(branch) if branch is not None else _dt(out)
+    _check(lib.ullm_add_rmsnorm(_p(branch), _p(residual), _p(gain), _c_float(eps), _p(out), _p(rows),
+                                _c_int(n), _c_int(H), _c_int(bdt), _c_int(_dt(out)),
+                                _c_int(0 if rows is not None else 1), _stream()), "add_rmsnorm")
+    return out
+
+
+def silu_mul(gate_up: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """silu(gate_up[:, :I]) * gate_up[:, I:] for a contiguous [T, 2I] input."""
+    T, two_i = gate_up.shape
+    _need(two_i % 2 == 0 and gate_up.is_contiguous(), "gate_up must be contiguous [T, 2I]")
+    inter = two_i // 2
+    if out is None:
+        out = torch.empty((T, inter), dtype=gate_up.dtype, device=gate_up.device)
+    _need(out.shape == (T, inter) and out.is_contiguous() and out.dtype == gate_up.dtype, "bad silu_mul output")
+    lib = build.load("elementwise")
+    _check(lib.ullm_silu_mul(_p(gate_up), _p(out), _c_int(T), _c_int(inter), _c_int(_dt(gate_up)), _stream()),
+           "silu_mul")
+    return out
+
+
+def qk_norm_rope_write(qkv: torch.Tensor, q_out: torch.Tensor, q_gain: Optional[torch.Tensor],
+                       k_gain: Optional[torch.Tensor], eps: float, cos_sin: Optional[torch.Tensor],
+                       rotary_dim: int, style: int, positions: torch.Tensor, token_entry: torch.Tensor,
+                       block_table: torch.Tensor, k_pool: Optional[torch.Tensor], v_pool: Optional[torch.Tensor],
+                       page_size: int, nq: int, nkv: int, hd: int, write_kv: bool) -> None:
+    """Per-head norm and rotation of q (to ``q_out`` [T, nq*hd]) and k, and the cache write of k and v.
+    ``qkv`` is [T, (nq + 2 nkv) * hd]; pools are [pages, nkv, page_size, hd]; ``block_table`` is
+    int32 [B, stride] with one row per batch entry."""
+    T = qkv.shape[0]
+    _need(qkv.dim() == 2 and qkv.shape[1] == (nq + 2 * nkv) * hd and qkv.stride(1) == 1, "bad qkv shape")
+    _need(q_out.shape == (T, nq * hd) and q_out.is_contiguous() and q_out.dtype == qkv.dtype, "bad q_out")
+    _need(hd <= 512, f"head_dim {hd} exceeds 512")
+    _i32(positions, "positions", T)
+    _i32(token_entry, "token_entry", T)
+    _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.stride(1) == 1,
+          "block_table must be int32 [B, stride]")
+    for g, nm in ((q_gain, "q_gain"), (k_gain, "k_gain")):
+        if g is not None:
+            _need(g.dtype == torch.float32 and g.numel() == hd and g.is_contiguous(), f"{nm} must be float32 [hd]")
+    table_rows = 0
+    if style != 0 and rotary_dim > 0:
+        _need(cos_sin is not None and cos_sin.dtype == torch.float32 and cos_sin.dim() == 2
+              and cos_sin.shape[1] == rotary_dim and cos_sin.is_contiguous(),
+              "cos_sin must be float32 [positions, rotary_dim]")
+        table_rows = cos_sin.shape[0]
+    if write_kv:
+        for pool, nm in ((k_pool, "k_pool"), (v_pool, "v_pool")):
+            _need(pool is not None and pool.dim() == 4 and tuple(pool.shape[1:]) == (nkv, page_size, hd)
+                  and pool.is_contiguous() and pool.dtype == qkv.dtype,
+                  f"{nm} must be contiguous [pages, {nkv}, {page_size}, {hd}] of {qkv.dtype}")
+    lib = build.load("elementwise")
+    _check(lib.ullm_qk_norm_rope_write(
+        _p(qkv), _c_int(qkv.stride(0)), _p(q_out), _c_int(q_out.stride(0)), _p(q_gain), _p(k_gain),
+        _c_float(eps), _p(cos_sin), _c_int(table_rows), _c_int(rotary_dim), _c_int(style), _p(positions),
+        _p(token_entry), _p(block_table), _c_int(block_table.stride(0)), _p(k_pool), _p(v_pool),
+        _c_int(page_size), _c_int(T), _c_int(nq), _c_int(nkv), _c_int(hd), _c_int(1 if write_kv else 0),
+        _c_int(_dt(qkv)), _stream()), "qk_norm_rope_write")
+
+
+# ---------------------------------------------------------------------------------- attention
+
+def paged_attention_generic(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
+                            positions: torch.Tensor, token_entry: torch.Tensor, block_table: torch.Tensor,
+                            page_size: int, nq: int, nkv: int, hd: int, scale: float, window: int,
+                            out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    T = q.shape[0]
+    _need(q.shape == (T, nq * hd) and q.stride(1) == 1, "q must be [T, nq*hd]")
+    _need(hd <= 512 and nq % nkv == 0, "head_dim > 512 or heads not a multiple of kv heads")
+    for pool, nm in ((k_pool, "k_pool"), (v_pool, "v_pool")):
+        _need(pool.dim() == 4 and tuple(pool.shape[1:]) == (nkv, page_size, hd) and pool.is_contiguous()
+              and pool.dtype == q.dtype, f"{nm} must be contiguous [pages, {nkv}, {page_size}, {hd}] of {q.dtype}")
+    _i32(positions, "positions", T)
+    _i32(token_entry, "token_entry", T)
+    _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.stride(1) == 1,
+          "block_table must be int32 [B, stride]")
+    if out is None:
+        out = torch.empty((T, nq * hd), dtype=q.dtype, device=q.device)
+    _need(out.shape == (T, nq * hd) and out.is_contiguous() and out.dtype == q.dtype, "bad attention output")
+    lib = build.load("attention_generic")
+    _check(lib.ullm_paged_attention_generic(
+        _p(q), _c_int(q.stride(0)), _p(out), _c_int(out.stride(0)), _p(k_pool), _p(v_pool), _p(positions),
+        _p(token_entry), _p(block_table), _c_int(block_table.stride(0)), _c_int(page_size), _c_int(T),
+        _c_int(nq), _c_int(nkv), _c_int(hd), _c_float(scale), _c_int(window), _c_int(_dt(q)), _stream()),
+        "paged_attention_generic")
+    return out
+
+
+# ---------------------------------------------------------------------------------- matrix products
+
+def gemm_simple(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
+                out_dtype: Optional[torch.dtype] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """a [M, K] times w [N, K] transposed (+ bias float32 [N]); 32-bit multiply-add in fixed K order."""
+    M, K = a.shape
+    N, K2 = w.shape
+    _need(K == K2, f"inner sizes differ: a is [{M}, {K}], w is [{N}, {K2}]")
+    _need(a.stride(1) == 1 and w.stride(1) == 1, "a and w must have unit stride along K")
+    if out is None:
+        out = torch.empty((M, N), dtype=out_dtype or a.dtype, device=a.device)
+    _need(out.shape == (M, N) and out.stride(1) == 1, "bad gemm output")
+    if bias is not None:
+        _need(bias.dtype == torch.float32 and bias.numel() == N and bias.is_contiguous(), "bias must be float32 [N]")
+    lib = build.load("gemm_simple")
+    _check(lib.ullm_gemm_simple(_p(a), _c_int(a.stride(0)), _p(w), _c_int(w.stride(0)), _p(bias), _p(out),
+                                _c_int(out.stride(0)), _c_int(M), _c_int(N), _c_int(K), _c_int(_dt(a)),
+                                _c_int(_dt(w)), _c_int(_dt(out)), _stream()), "gemm_simple")
+    return out
+
+
+def gemm_bf16(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
+              out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """bfloat16 operands, 32-bit accumulation.  Output in bfloat16 goes through the library product
+    (as the reference's linears do, ullm/layers/linear.py:165); 32-bit output (logits) through the
+    hand-written kernel, which keeps the accumulator's precision."""
+    out_dtype = out_dtype or a.dtype
+    if out_dtype == torch.bfloat16 and a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16:
+        y = torch.nn.functional.linear(a, w)
+        if bias is not None:
+            y = (y.float() + bias).to(torch.bfloat16)
+        return y
+    return gemm_simple(a, w, bias, out_dtype=out_dtype)
+
+
+def paged_attention(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, ctx, group, nq: int,
+                    nkv: int, hd: int, scale: float, window: int) -> torch.Tensor:
+    """Attention of the batch's queries over their requests' cached keys and values (the new
+    tokens' rows included).  Chooses the kernel by dtype and shape; every choice computes the same
+    function."""
+    return paged_attention_generic(q, k_pool, v_pool, ctx.positions, ctx.token_entry, group.block_table,
+                                   group.page_size, nq, nkv, hd, scale, window)

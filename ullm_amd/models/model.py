@@ -1,0 +1,132 @@
+"""A model as data: which parts make each layer, in which order layers run, whose cache a layer
+reads.  ``Model`` builds the parts named by a ``ModelPlan`` from the part registry, collects their
+declared weights and cache needs, and runs the layer list over a batch.
+
+Reference shape of the same thing: ullm/models/qwen3.py:199-286 (embedding, layer loop carrying
+(hidden, residual), final norm, lm_head on selected rows ullm/core/model_runner.py:339-341).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Dict, List, Optional, Sequence, Tuple
+
+import torch
+
+from ..cache.manager import CacheGroupSpec
+from ..kernels import ops
+from ..parts import (Block, KVNeed, LayerCache, Norm, Part, PartEnv, StateNeed, StepContext, WeightDecl,
+                     build_part, walk)
+from ..parts.linear import linear
+
+
+@dataclass(frozen=True)
+class Choice:
+    """A part chosen by name with its parameters; parameters may themselves be choices."""
+    kind: str
+    name: str
+    params: Dict[str, Any] = field(default_factory=dict)
+
+    def build(self) -> Part:
+        built = {k: (v.build() if isinstance(v, Choice) else v) for k, v in self.params.items()}
+        return build_part(self.kind, self.name, **built)
+
+
+@dataclass
+class ModelPlan:
+    vocab_size: int
+    hidden_size: int
+    embedding_weight: str                    # tensor name of the token table [vocab, hidden]
+    layers: List[Choice]                     # one "block" choice per layer
+    final_norm: Choice
+    head_weight: str                         # tensor name of the output matrix [vocab, hidden]
+    tie_head_to_embedding: bool = False      # bind the token table where the head tensor is absent
+    # The order layers run in: (layer, cache id).  A layer may appear more than once (with a cache id
+    # of its own each time, or the same one).  The first entry that names a cache id owns that cache
+    # and writes it; later entries with the same id only read it, so a layer can read the cache
+    # another layer wrote.  Default: every layer once, cache id = layer index.
+    run_order: Optional[List[Tuple[int, int]]] = None
+    init_std: float = 0.02                   # random-weights mode
+
+    def order(self) -> List[Tuple[int, int]]:
+        return self.run_order if self.run_order is not None else [(i, i) for i in range(len(self.layers))]
+
+
+class Model:
+    def __init__(self, plan: ModelPlan):
+        self.plan = plan
+        self.blocks: List[Block] = [c.build() for c in plan.layers]
+        self.final_norm: Norm = plan.final_norm.build()
+        self.run_order = plan.order()
+        self.cache_owner: Dict[int, int] = {}      # cache id -> index into run_order of its owner
+        for idx, (layer, cache_id) in enumerate(self.run_order):
+            if not (0 <= layer < len(self.blocks)):
+                raise ValueError(f"run order names layer {layer}: out of range")
+            self.cache_owner.setdefault(cache_id, idx)
+        self.embedding: Optional[torch.Tensor] = None
+        self.head: Optional[torch.Tensor] = None
+        self.env: Optional[PartEnv] = None
+
+    # ------------------------------------------------------------------ weights
+    def parts(self):
+        for b in self.blocks:
+            yield from walk(b)
+        yield from walk(self.final_norm)
+
+    def weight_decls(self) -> List[WeightDecl]:
+        p = self.plan
+        decls = [WeightDecl(p.embedding_weight, (p.vocab_size, p.hidden_size))]
+        for part in self.parts():
+            decls.extend(part.weights())
+        decls.append(WeightDecl(p.head_weight, (p.vocab_size, p.hidden_size),
+                                alias_of=p.embedding_weight if p.tie_head_to_embedding else None))
+        return decls
+
+    def bind(self, tensors: Dict[str, torch.Tensor], env: PartEnv) -> None:
+        self.env = env
+        self.embedding = tensors[self.plan.embedding_weight].contiguous()
+        self.head = tensors[self.plan.head_weight].contiguous()
+        for part in self.parts():
+            part.bind(tensors, env)
+
+    # ------------------------------------------------------------------ cache layout
+    def cache_layout(self):
+        """Groups of caches with equal needs, and the per-request state needs.
+        Returns (groups, {cache id: group index}, {cache id: StateNeed})."""
+        keyed: Dict[Tuple[int, int, int], List[int]] = {}
+        states: Dict[int, StateNeed] = {}
+        for cache_id, idx in self.cache_owner.items():
+            need = self.blocks[self.run_order[idx][0]].cache_need()
+            if isinstance(need, KVNeed):
+                keyed.setdefault((need.num_kv_heads, need.head_dim, need.window), []).append(cache_id)
+            elif isinstance(need, StateNeed):
+                states[cache_id] = need
+        groups, layer_group = [], {}
+        for (nkv, hd, window), ids in keyed.items():
+            for c in ids:
+                layer_group[c] = len(groups)
+            groups.append(CacheGroupSpec(nkv, hd, window, tuple(ids)))
+        for idx, (layer, cache_id) in enumerate(self.run_order):
+            owner_layer = self.run_order[self.cache_owner[cache_id]][0]
+            a, b = self.blocks[layer].cache_need(), self.blocks[owner_layer].cache_need()
+            if a != b:
+                raise ValueError(f"layer {layer} reads cache {cache_id} written by layer {owner_layer} "
+                                 f"but their needs differ: {a} vs {b}")
+        return groups, layer_group, states
+
+    # ------------------------------------------------------------------ forward
+    def forward(self, ctx: StepContext, caches: Dict[int, LayerCache], logit_rows: Optional[torch.Tensor]):
+        """Runs the batch through every layer of the run order and returns float32 logits
+        [len(logit_rows), vocab] (None if no row is wanted)."""
+        residual = ops.embedding(ctx.token_ids, self.embedding)
+        pending = None
+        for idx, (layer, cache_id) in enumerate(self.run_order):
+            cache = caches.get(cache_id)
+            if cache is None:
+                cache = LayerCache()
+            elif self.cache_owner[cache_id] != idx:
+                cache = LayerCache(cache.group, cache.k_pool, cache.v_pool, cache.state, owner=False)
+            residual, pending = self.blocks[layer].forward(residual, pending, ctx, cache)
+        if logit_rows is None or logit_rows.numel() == 0:
+            return None
+        x = self.final_norm.add_norm(pending, residual, rows=logit_rows, out_dtype=ctx.dtype)
+        return linear(x, self.head, out_dtype=torch.float32)

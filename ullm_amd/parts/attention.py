@@ -1,0 +1,82 @@
+"""Grouped-query attention over the paged cache, as a mixer.
+
+Reference: ullm/models/qwen3.py:49-130 (projection, per-head q/k norm, rotation, attention, output
+projection) and ullm/layers/attention.py:279-313 (write k, v to the cache, then attend over it).
+Head size is a parameter of its own (qwen3.py:78: not hidden/heads), the q/k norms and the position
+encoding are optional parts, and a window bounds how far back a query looks (0 = everything; the
+reference never windows).
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional
+
+import torch
+
+from ..kernels import ops
+from .base import KVNeed, LayerCache, Mixer, PartEnv, PositionEncoding, StepContext, WeightDecl, register_part
+from .linear import linear
+
+
+@register_part("mixer", "gqa_attention")
+class GQAttention(Mixer):
+    def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, prefix: str,
+                 position: Optional[PositionEncoding] = None, qk_norm_eps: Optional[float] = None,
+                 bias: bool = False, window: int = 0, scale: Optional[float] = None):
+        if num_heads % num_kv_heads:
+            raise ValueError(f"{num_heads} query heads are not a multiple of {num_kv_heads} kv heads")
+        if head_dim % 2 or head_dim > 512:
+            raise ValueError(f"head_dim={head_dim} must be even and at most 512")
+        self.hidden_size, self.nq, self.nkv, self.hd = hidden_size, num_heads, num_kv_heads, head_dim
+        self.prefix = prefix
+        self.position = position
+        self.qk_norm_eps = qk_norm_eps          # None: no per-head norm
+        self.bias = bias
+        self.window = int(window)
+        self.scale = float(scale) if scale is not None else head_dim ** -0.5   # qwen3.py:81
+        self.w_qkv = self.b_qkv = self.w_o = self.q_gain = self.k_gain = None
+
+    def children(self):
+        return [self.position] if self.position is not None else []
+
+    def cache_need(self):
+        return KVNeed(self.nkv, self.hd, self.window)
+
+    def weights(self) -> List[WeightDecl]:
+        p, H, hd = self.prefix, self.hidden_size, self.hd
+        out = [WeightDecl(f"{p}.q_proj.weight", (self.nq * hd, H)),
+               WeightDecl(f"{p}.k_proj.weight", (self.nkv * hd, H)),
+               WeightDecl(f"{p}.v_proj.weight", (self.nkv * hd, H)),
+               WeightDecl(f"{p}.o_proj.weight", (H, self.nq * hd))]
+        if self.bias:   # qwen3.py:146 (attention_bias): on q, k, v only; o_proj never has one (qwen3.py:94)
+            out += [WeightDecl(f"{p}.q_proj.bias", (self.nq * hd,), keep_fp32=True),
+                    WeightDecl(f"{p}.k_proj.bias", (self.nkv * hd,), keep_fp32=True),
+                    WeightDecl(f"{p}.v_proj.bias", (self.nkv * hd,), keep_fp32=True)]
+        if self.qk_norm_eps is not None:
+            out += [WeightDecl(f"{p}.q_norm.weight", (hd,), init="gain", keep_fp32=True),
+                    WeightDecl(f"{p}.k_norm.weight", (hd,), init="gain", keep_fp32=True)]
+        return out
+
+    def bind(self, tensors: Dict[str, torch.Tensor], env: PartEnv) -> None:
+        p = self.prefix
+        # one fused projection with rows q | k | v, as the reference merges them (linear.py:381-389)
+        self.w_qkv = torch.cat([tensors[f"{p}.{n}_proj.weight"] for n in "qkv"], dim=0).contiguous()
+        self.w_o = tensors[f"{p}.o_proj.weight"].contiguous()
+        if self.bias:
+            self.b_qkv = torch.cat([tensors[f"{p}.{n}_proj.bias"] for n in "qkv"], dim=0).contiguous()
+        if self.qk_norm_eps is not None:
+            self.q_gain = tensors[f"{p}.q_norm.weight"].contiguous()
+            self.k_gain = tensors[f"{p}.k_norm.weight"].contiguous()
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, cache: LayerCache) -> torch.Tensor:
+        T = x.shape[0]
+        group = ctx.groups[cache.group]
+        qkv = linear(x, self.w_qkv, self.b_qkv)
+        q = torch.empty((T, self.nq * self.hd), dtype=x.dtype, device=x.device)
+        table, rot, style = self.position.kernel_args() if self.position is not None else (None, 0, 0)
+        ops.qk_norm_rope_write(
+            qkv, q, self.q_gain, self.k_gain, self.qk_norm_eps if self.qk_norm_eps is not None else 0.0,
+            table, rot, style, ctx.positions, ctx.token_entry, group.block_table,
+            cache.k_pool, cache.v_pool, group.page_size, self.nq, self.nkv, self.hd, write_kv=cache.owner)
+        o = ops.paged_attention(q, cache.k_pool, cache.v_pool, ctx, group, self.nq, self.nkv, self.hd,
+                                self.scale, self.window)
+        return linear(o, self.w_o)

@@ -1,0 +1,199 @@
+"""What every part of a layer has in common: declared weights, declared cache needs,
+and a registry from (kind, name) to the class, so that a model is put together from a
+plan that names its parts layer by layer.
+
+Kinds: "mixer" (attention or anything else that mixes tokens), "ffn" (feed-forward),
+"norm", "position" (position encoding) and "block" (how norm, mixer and feed-forward are
+arranged around the residual stream).  No part knows which model it is in: sizes and
+constants arrive as constructor parameters, tensor names as a prefix.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Callable, Dict, List, Optional, Tuple, Union
+
+import torch
+
+
+# --------------------------------------------------------------------------- weights
+
+@dataclass(frozen=True)
+class WeightDecl:
+    """One tensor a part binds by its checkpoint name."""
+    name: str
+    shape: Tuple[int, ...]
+    init: str = "normal"          # random mode: "normal" N(0,s) | "gain" 1+N(0,s)
+    keep_fp32: bool = False       # held in 32-bit whatever the compute dtype (norm gains)
+    alias_of: Optional[str] = None  # if absent from the checkpoint, bind this tensor instead
+
+
+# --------------------------------------------------------------------------- cache needs
+
+@dataclass(frozen=True)
+class KVNeed:
+    """A mixer that keeps one key row and one value row per token and kv head."""
+    num_kv_heads: int
+    head_dim: int
+    window: int = 0               # keys a query looks back over, itself included; 0 = all
+
+
+@dataclass(frozen=True)
+class StateNeed:
+    """A mixer that keeps state of fixed size per request (zeroed at admission)."""
+    shape: Tuple[int, ...]
+    dtype: torch.dtype = torch.float32
+
+
+CacheNeed = Union[KVNeed, StateNeed, None]
+
+
+# --------------------------------------------------------------------------- step context
+
+@dataclass
+class GroupView:
+    """Block tables of the batch entries for one cache group (device tensors)."""
+    block_table: torch.Tensor     # int32 [B, stride]; entry = page id, -1 where none is held
+    stride: int
+    page_size: int
+    window: int
+
+
+@dataclass
+class LayerCache:
+    """What a mixer sees of the cache: its layer's pools or its layer's state rows."""
+    group: int = -1                        # index into StepContext.groups for KV mixers
+    k_pool: Optional[torch.Tensor] = None  # [num_pages, kv_heads, page_size, head_dim]
+    v_pool: Optional[torch.Tensor] = None
+    state: Optional[torch.Tensor] = None   # [num_slots, *StateNeed.shape]
+    owner: bool = True                     # False: reads another layer's cache, writes nothing
+
+
+@dataclass
+class StepContext:
+    """Device-side description of one batch: T tokens of B entries, flattened."""
+    num_tokens: int
+    num_entries: int
+    token_ids: torch.Tensor       # int32 [T]
+    positions: torch.Tensor       # int32 [T] absolute position of each token in its request
+    token_entry: torch.Tensor     # int32 [T] batch entry each token belongs to
+    q_start: torch.Tensor         # int32 [B+1] first token of each entry
+    entry_slot: torch.Tensor      # int32 [B] request slot of each entry (state rows)
+    entry_start: torch.Tensor     # int32 [B] position of the entry's first token
+    groups: List[GroupView]
+    max_q_len: int                # host copies, for grids
+    max_kv_len: int
+    decode_only: bool             # every entry brings exactly one token
+    dtype: torch.dtype = torch.bfloat16          # compute dtype of activations
+    host: dict = field(default_factory=dict)   # host-side copies for parts that want them
+
+
+# --------------------------------------------------------------------------- parts
+
+@dataclass(frozen=True)
+class PartEnv:
+    """Where and how a model is built: handed to every part with its tensors."""
+    device: torch.device
+    dtype: torch.dtype            # compute dtype: torch.bfloat16 or torch.float32
+    context_len: int              # most positions any request reaches
+
+
+class Part:
+    """Base of every part.  ``weights()`` declares tensors; ``bind`` receives them."""
+    kind = ""
+
+    def weights(self) -> List[WeightDecl]:
+        return []
+
+    def bind(self, tensors: Dict[str, torch.Tensor], env: PartEnv) -> None:
+        """Called once with {declared name: device tensor in its final dtype}."""
+
+    def children(self) -> List["Part"]:
+        return []
+
+
+class Mixer(Part):
+    """Token mixer: ``forward(x [T, hidden], ctx, cache) -> [T, hidden]`` in the compute dtype."""
+    kind = "mixer"
+
+    def cache_need(self) -> CacheNeed:
+        return None
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, cache: LayerCache) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    """``forward(x [T, hidden], ctx) -> [T, hidden]``; keeps nothing between steps."""
+    kind = "ffn"
+
+    def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Norm(Part):
+    """``add_norm(branch, residual, rows) -> normed``: adds the branch output (if any) into
+    the 32-bit residual stream, then normalises the sum; ``rows`` selects output rows."""
+    kind = "norm"
+
+    def add_norm(self, branch: Optional[torch.Tensor], residual: torch.Tensor,
+                 rows: Optional[torch.Tensor] = None, out_dtype: torch.dtype = None) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    """Describes how query and key vectors are marked with their position.
+    ``kernel_args()`` -> (table tensor or None, rotary_dim, style) for the fused
+    norm/rotate/cache-write kernel; style 0 = none, 1 = half-split pairs, 2 = adjacent pairs."""
+    kind = "position"
+
+    def kernel_args(self):
+        return None, 0, 0
+
+
+class Block(Part):
+    """Arrangement of norm, mixer and feed-forward around the residual stream.
+
+    ``forward(residual, pending, ctx, cache) -> (residual, pending)`` where ``residual`` is the
+    32-bit stream [T, hidden] and ``pending`` a branch output not yet added to it."""
+    kind = "block"
+
+    def cache_need(self) -> CacheNeed:
+        return None
+
+    def forward(self, residual, pending, ctx: StepContext, cache: LayerCache):
+        raise NotImplementedError
+
+
+# --------------------------------------------------------------------------- registry
+
+_PARTS: Dict[str, Dict[str, Callable]] = {k: {} for k in ("mixer", "ffn", "norm", "position", "block")}
+
+
+def register_part(kind: str, name: str):
+    """Class decorator: make ``build_part(kind, name, ...)`` construct this class."""
+    if kind not in _PARTS:
+        raise KeyError(f"unknown part kind {kind!r}; kinds are {sorted(_PARTS)}")
+
+    def deco(cls):
+        _PARTS[kind][name] = cls
+        return cls
+    return deco
+
+
+def build_part(kind: str, name: str, **params) -> Part:
+    try:
+        cls = _PARTS[kind][name]
+    except KeyError:
+        raise KeyError(f"no {kind} part named {name!r}; registered: {sorted(_PARTS.get(kind, {}))}") from None
+    return cls(**params)
+
+
+def registered_parts(kind: str) -> List[str]:
+    return sorted(_PARTS[kind])
+
+
+def walk(part: Part):
+    """The part and every part below it."""
+    yield part
+    for c in part.children():
+        yield from walk(c)

@@ -1,0 +1,28 @@
+"""Pre-norm residual block: h += mixer(norm1(h)); h += ffn(norm2(h)).
+
+The reference carries (branch output, residual) between layers and lets the next norm do the add
+(ullm/models/qwen3.py:159-178, ullm/layers/layernorm.py:24-26).  The same trick is kept: a branch
+output is left ``pending`` and added inside the next fused add+norm kernel, which saves one pass
+over the residual stream per branch.
+"""
+from __future__ import annotations
+
+from .base import Block, FeedForward, LayerCache, Mixer, Norm, StepContext, register_part
+
+
+@register_part("block", "prenorm")
+class PreNormBlock(Block):
+    def __init__(self, mixer_norm: Norm, mixer: Mixer, ffn_norm: Norm, ffn: FeedForward):
+        self.mixer_norm, self.mixer, self.ffn_norm, self.ffn = mixer_norm, mixer, ffn_norm, ffn
+
+    def children(self):
+        return [self.mixer_norm, self.mixer, self.ffn_norm, self.ffn]
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    def forward(self, residual, pending, ctx: StepContext, cache: LayerCache):
+        x = self.mixer_norm.add_norm(pending, residual, out_dtype=ctx.dtype)
+        a = self.mixer.forward(x, ctx, cache)
+        x = self.ffn_norm.add_norm(a, residual, out_dtype=ctx.dtype)
+        return residual, self.ffn.forward(x, ctx)

@@ -1,0 +1,34 @@
+"""Dense gated feed-forward: down(silu(gate(x)) * up(x)), no biases
+(ullm/models/qwen3.py:23-46, ullm/layers/activation.py:16-18).  gate and up are one fused
+projection with rows gate | up (qwen3.py:307-308).
+"""
+from __future__ import annotations
+
+from typing import Dict, List
+
+import torch
+
+from ..kernels import ops
+from .base import FeedForward, PartEnv, StepContext, WeightDecl, register_part
+from .linear import linear
+
+
+@register_part("ffn", "swiglu")
+class SwiGLU(FeedForward):
+    def __init__(self, hidden_size: int, intermediate_size: int, prefix: str):
+        self.hidden_size, self.intermediate_size, self.prefix = hidden_size, intermediate_size, prefix
+        self.w_gate_up = self.w_down = None
+
+    def weights(self) -> List[WeightDecl]:
+        p, H, I = self.prefix, self.hidden_size, self.intermediate_size
+        return [WeightDecl(f"{p}.gate_proj.weight", (I, H)), WeightDecl(f"{p}.up_proj.weight", (I, H)),
+                WeightDecl(f"{p}.down_proj.weight", (H, I))]
+
+    def bind(self, tensors: Dict[str, torch.Tensor], env: PartEnv) -> None:
+        p = self.prefix
+        self.w_gate_up = torch.cat([tensors[f"{p}.gate_proj.weight"], tensors[f"{p}.up_proj.weight"]],
+                                   dim=0).contiguous()
+        self.w_down = tensors[f"{p}.down_proj.weight"].contiguous()
+
+    def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
+        return linear(ops.silu_mul(linear(x, self.w_gate_up)), self.w_down)

@@ -1,0 +1,73 @@
+"""Random weights from a configuration and a seed (the reference has no such mode).
+
+``write_random_model`` writes a model folder (config.json, model.safetensors) that any loader of
+the format can read: tensors are drawn on the CPU in the order the parts declare them from one
+seeded generator, matrices and embeddings N(0, std), norm gains 1 + N(0, std), in float32, then
+stored in the requested dtype.  ``bind_random_weights`` draws straight on the device instead, for
+sizes where a file would only cost time (benchmarks).
+"""
+from __future__ import annotations
+
+import json
+import os
+from typing import Dict, Mapping, Optional
+
+import torch
+from safetensors.torch import save_file
+
+from ..models import build_model
+from ..parts import PartEnv
+
+_STORE = {"bfloat16": torch.bfloat16, "float32": torch.float32}
+
+
+def _draw(decl, std: float, gen: torch.Generator, device) -> torch.Tensor:
+    t = torch.empty(decl.shape, dtype=torch.float32, device=device).normal_(0.0, std, generator=gen)
+    if decl.init == "gain":
+        t += 1.0
+    return t
+
+
+def write_random_model(config: Mapping, out_dir: str, seed: int, std: Optional[float] = None,
+                       dtype: str = "bfloat16") -> str:
+    """Write ``out_dir/config.json`` and ``out_dir/model.safetensors``; returns ``out_dir``."""
+    if dtype not in _STORE:
+        raise ValueError(f"storage dtype {dtype!r}: choose bfloat16 or float32")
+    config = dict(config)
+    config.setdefault("torch_dtype", dtype)
+    _, model = build_model(config)
+    sigma = model.plan.init_std if std is None else float(std)
+    gen = torch.Generator(device="cpu").manual_seed(int(seed))
+    tensors: Dict[str, torch.Tensor] = {}
+    for d in model.weight_decls():
+        if d.name in tensors or d.alias_of is not None:
+            continue                                    # a tied head is not stored
+        tensors[d.name] = _draw(d, sigma, gen, "cpu").to(_STORE[dtype]).contiguous()
+    os.makedirs(out_dir, exist_ok=True)
+    with open(os.path.join(out_dir, "config.json"), "w", encoding="utf-8") as f:
+        json.dump(config, f, indent=1)
+    save_file(tensors, os.path.join(out_dir, "model.safetensors"), metadata={"format": "pt"})
+    return out_dir
+
+
+def bind_random_weights(model, env: PartEnv, seed: int, std: Optional[float] = None) -> None:
+    """Draw every declared tensor on ``env.device`` (own seeded generator) and bind the model."""
+    sigma = model.plan.init_std if std is None else float(std)
+    gen = torch.Generator(device=env.device).manual_seed(int(seed))
+    tensors: Dict[str, torch.Tensor] = {}
+    pending_alias = []
+    for d in model.weight_decls():
+        if d.name in tensors:
+            continue
+        if d.alias_of is not None:
+            pending_alias.append(d)
+            continue
+        final = torch.float32 if d.keep_fp32 else env.dtype
+        if final == torch.float32:
+            tensors[d.name] = _draw(d, sigma, gen, env.device)
+        else:   # large matrices: draw in the final dtype, no 32-bit copy
+            t = torch.empty(d.shape, dtype=final, device=env.device).normal_(0.0, sigma, generator=gen)
+            tensors[d.name] = t + 1.0 if d.init == "gain" else t
+    for d in pending_alias:
+        tensors[d.name] = tensors[d.alias_of]
+    model.bind(tensors, env)
