@@ -224,3 +224,27 @@ def paged_attention(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
     function."""
     return paged_attention_generic(q, k_pool, v_pool, ctx.positions, ctx.token_entry, group.block_table,
                                    group.page_size, nq, nkv, hd, scale, window)
+
+
+# ---------------------------------------------------------------------------------- sampling
+
+def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
+           min_p: torch.Tensor, seed_lo: torch.Tensor, seed_hi: torch.Tensor, position: torch.Tensor,
+           out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """One token id per row of float32 ``logits`` [n, V].  Per-row parameters: temperature (0 =
+    greedy), top_k (<= 0 = all), top_p, min_p (float32), seed halves and position (int32)."""
+    n, V = logits.shape
+    _need(logits.dtype == torch.float32 and logits.stride(1) == 1, "logits must be float32 with unit stride")
+    for t, nm, dt in ((temperature, "temperature", torch.float32), (top_k, "top_k", torch.int32),
+                      (top_p, "top_p", torch.float32), (min_p, "min_p", torch.float32),
+                      (seed_lo, "seed_lo", torch.int32), (seed_hi, "seed_hi", torch.int32),
+                      (position, "position", torch.int32)):
+        _need(t.dtype == dt and t.numel() >= n and t.is_contiguous(), f"{nm} must be contiguous {dt} [n]")
+    if out is None:
+        out = torch.empty((n,), dtype=torch.int32, device=logits.device)
+    _need(out.dtype == torch.int32 and out.numel() >= n and out.is_contiguous(), "bad sample output")
+    lib = build.load("sampling")
+    _check(lib.ullm_sample(_p(logits), _c_int(n), _c_int(V), _c_int(logits.stride(0)), _p(temperature), _p(top_k),
+                           _p(top_p), _p(min_p), _p(seed_lo), _p(seed_hi), _p(position), _p(out), _stream()),
+           "sample")
+    return out
