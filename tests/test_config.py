@@ -1,0 +1,106 @@
+"""Configuration, registry and command line (no GPU)."""
+import argparse
+import json
+
+import pytest
+
+from conftest import TINY_A, TINY_B, TINY_C
+from ullm_amd.config import ConfigError, EngineConfig, Qwen3Config, read_config_json
+from ullm_amd.models import MODEL_REGISTRY, build_model, resolve_architecture
+
+
+def test_reads_every_size_from_the_config():
+    for d in (TINY_A, TINY_B, TINY_C):
+        c = Qwen3Config.from_dict(d)
+        for key in ("vocab_size", "hidden_size", "num_hidden_layers", "num_attention_heads", "num_key_value_heads",
+                    "head_dim", "intermediate_size", "max_position_embeddings", "rms_norm_eps", "rope_theta",
+                    "tie_word_embeddings", "attention_bias"):
+            assert getattr(c, key) == d[key], key
+
+
+def test_defaults_follow_the_reference():
+    d = {k: v for k, v in TINY_A.items() if k not in ("head_dim", "rope_theta", "attention_bias",
+                                                      "tie_word_embeddings", "use_sliding_window")}
+    c = Qwen3Config.from_dict(d)
+    assert c.head_dim == d["hidden_size"] // d["num_attention_heads"]     # ullm/models/qwen3.py:78
+    assert c.rope_theta == 1000000.0                                       # ullm/models/qwen3.py:144
+    assert c.attention_bias is False and c.tie_word_embeddings is False
+    assert all(c.window_of_layer(i) == 0 for i in range(c.num_hidden_layers))
+
+
+@pytest.mark.parametrize("key", ["hidden_size", "num_hidden_layers", "num_attention_heads", "intermediate_size",
+                                 "vocab_size", "rms_norm_eps", "max_position_embeddings", "architectures"])
+def test_missing_required_key_is_named(key):
+    d = dict(TINY_B)
+    del d[key]
+    with pytest.raises(ConfigError, match=key):
+        Qwen3Config.from_dict(d)
+
+
+def test_bad_values_are_refused():
+    with pytest.raises(ConfigError, match="multiple"):
+        Qwen3Config.from_dict(dict(TINY_A, num_attention_heads=5))
+    with pytest.raises(ConfigError, match="hidden_act"):
+        Qwen3Config.from_dict(dict(TINY_A, hidden_act="gelu"))
+    with pytest.raises(ConfigError, match="sliding_window"):
+        Qwen3Config.from_dict(dict(TINY_A, use_sliding_window=True))
+    with pytest.raises(ConfigError, match="expected int"):
+        Qwen3Config.from_dict(dict(TINY_A, hidden_size="64"))
+
+
+def test_window_is_chosen_layer_by_layer():
+    c = Qwen3Config.from_dict(TINY_C)
+    assert [c.window_of_layer(i) for i in range(3)] == [0, 24, 24]
+    _, model = build_model(TINY_C)
+    groups, cache_group, states = model.cache_layout()
+    assert len(groups) == 2 and not states
+    by_window = {g.window: g for g in groups}
+    assert by_window[0].layers == (0,) and by_window[24].layers == (1, 2)
+
+
+def test_registry_maps_the_architecture_name():
+    assert "Qwen3ForCausalLM" in MODEL_REGISTRY
+    assert resolve_architecture(TINY_A).name == "Qwen3ForCausalLM"
+    with pytest.raises(ConfigError, match="not supported"):
+        resolve_architecture({"architectures": ["LlamaForCausalLM"]})
+    cfg, model = build_model(TINY_B)
+    assert len(model.blocks) == TINY_B["num_hidden_layers"]
+    names = {d.name: d.shape for d in model.weight_decls()}
+    assert names["model.layers.2.self_attn.q_proj.weight"] == (8 * 32, 96)     # heads*head_dim != hidden
+    assert names["model.layers.0.self_attn.q_norm.weight"] == (32,)
+    assert names["lm_head.weight"] == (503, 96)
+
+
+def test_read_config_json_errors(tmp_path):
+    with pytest.raises(ConfigError, match="no config.json"):
+        read_config_json(str(tmp_path))
+    (tmp_path / "config.json").write_text("{not json")
+    with pytest.raises(ConfigError, match="not valid JSON"):
+        read_config_json(str(tmp_path))
+
+
+def test_engine_config_names_and_checks(tmp_path):
+    ap = argparse.ArgumentParser()
+    EngineConfig.add_cli_args(ap)
+    args = ap.parse_args(["--model", str(tmp_path), "--max-bs", "7", "--context-len", "300", "--dtype", "fp32",
+                          "--page-size", "32", "--enforce-eager", "--gpu-memory-utilization", "0.5"])
+    ec = EngineConfig.from_args(args)
+    assert (ec.max_bs, ec.context_len, ec.dtype, ec.page_size, ec.enforce_eager) == (7, 300, "float32", 32, True)
+    # the reference's defaults (ullm/entrypoints/api_server.py:133-156)
+    base = EngineConfig.from_args(ap.parse_args(["--model", "x"]))
+    assert (base.gpu_memory_utilization, base.max_bs, base.context_len, base.tp_size, base.pp_size) == (0.9, 50, 2048, 1, 1)
+    with pytest.raises(ConfigError):
+        EngineConfig(model="x", tp_size=2)
+    with pytest.raises(ConfigError):
+        EngineConfig(model="x", page_size=12)
+    with pytest.raises(ConfigError):
+        EngineConfig(model="x", dtype="float16")
+    (tmp_path / "generation_config.json").write_text(json.dumps({"temperature": 0.6, "top_k": 20, "top_p": 0.95}))
+    assert EngineConfig(model=str(tmp_path)).generation_defaults() == {"temperature": 0.6, "top_k": 20, "top_p": 0.95}
+
+
+def test_cli_parser_has_sampling_options():
+    from ullm_amd.cli import build_parser
+    a = build_parser().parse_args(["--model", "m", "--prompt-ids", "1,2,3", "--temperature", "0", "--top-k", "5",
+                                   "--top-p", "0.9", "--min-p", "0.1", "--max-new-tokens", "4", "--ignore-eos"])
+    assert a.prompt_ids == ["1,2,3"] and a.temperature == 0 and a.top_k == 5 and a.ignore_eos

@@ -1,0 +1,254 @@
+"""Each HIP kernel alone against its plain reference, at sizes other than the engine's tests use."""
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+import plain_qwen3 as plain
+from gpu_util import DEV, paged_cache, table_tensor, tol
+
+pytestmark = pytest.mark.gpu
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from ullm_amd.kernels import ops as o
+    return o
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embedding(ops, dtype):
+    torch.manual_seed(0)
+    table = torch.randn(1003, 200).to(DEV, dtype)
+    ids = torch.tensor([0, 1002, 17, 17, 500], dtype=torch.int32, device=DEV)
+    out = ops.embedding(ids, table)
+    assert out.dtype == torch.float32 and torch.equal(out, table.float()[ids.long()])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H", [48, 1000, 5120])
+def test_add_rmsnorm(ops, dtype, H):
+    torch.manual_seed(1)
+    T, eps = 7, 1e-5
+    res = torch.randn(T, H, device=DEV) * 3
+    branch = torch.randn(T, H, device=DEV).to(dtype)
+    gain = (1 + 0.1 * torch.randn(H, device=DEV))
+    s = res + branch.float()
+    want = plain.rms_norm(s.cpu(), gain.cpu(), eps)
+    res_in = res.clone()
+    y = ops.add_rmsnorm(branch, res_in, gain, eps, dtype)
+    assert torch.equal(res_in, s)                                    # the stream is the unrounded 32-bit sum
+    assert (y.float().cpu() - want).abs().max() <= tol(dtype, want)
+    # rows: only the chosen rows, the stream untouched
+    rows = torch.tensor([6, 2, 2], dtype=torch.int32, device=DEV)
+    res_in = res.clone()
+    y = ops.add_rmsnorm(branch, res_in, gain, eps, dtype, rows=rows)
+    assert torch.equal(res_in, res)
+    assert (y.float().cpu() - want[[6, 2, 2]]).abs().max() <= tol(dtype, want)
+    # no branch: plain norm, equals the library routine
+    y = ops.add_rmsnorm(None, res.clone(), gain, eps, torch.float32)
+    assert torch.allclose(y, F.rms_norm(res, (H,), gain, eps), atol=1e-5, rtol=1e-5)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_silu_mul(ops, dtype):
+    torch.manual_seed(2)
+    gu = (torch.randn(5, 2 * 333, device=DEV) * 2).to(dtype)
+    want = plain.silu_and_mul(gu.float().cpu())
+    got = ops.silu_mul(gu)
+    assert (got.float().cpu() - want).abs().max() <= tol(dtype, want)
+    gu[:, :333] = 0
+    assert torch.all(ops.silu_mul(gu) == 0)
+
+
+@pytest.mark.parametrize("shape", [(1, 50, 70), (5, 129, 33), (70, 64, 16), (3, 503, 96)])
+def test_gemm_simple(ops, shape):
+    torch.manual_seed(3)
+    M, N, K = shape
+    a, w, b = torch.randn(M, K, device=DEV), torch.randn(N, K, device=DEV), torch.randn(N, device=DEV)
+    want = (a.double() @ w.double().T + b.double()).float()
+    got = ops.gemm_simple(a, w, b)
+    assert (got - want).abs().max() <= 2e-5 * want.abs().max()
+    # a row's result does not depend on the other rows (bitwise)
+    assert torch.equal(ops.gemm_simple(a[:1].contiguous(), w, b), got[:1])
+    ab, wb = a.bfloat16(), w.bfloat16()
+    want = ab.double() @ wb.double().T
+    got = ops.gemm_simple(ab, wb, out_dtype=torch.float32)
+    assert got.dtype == torch.float32 and (got - want.float()).abs().max() <= 2e-5 * want.abs().max()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("cfg", [dict(nq=6, nkv=2, hd=48, P=8, rot=48, style=1, norm=True),
+                                 dict(nq=5, nkv=5, hd=64, P=16, rot=32, style=1, norm=True),
+                                 dict(nq=4, nkv=1, hd=16, P=4, rot=16, style=2, norm=False),
+                                 dict(nq=2, nkv=2, hd=256, P=32, rot=0, style=0, norm=True)])
+def test_qk_norm_rope_write(ops, dtype, cfg):
+    torch.manual_seed(4)
+    nq, nkv, hd, P, rot, style = (cfg[k] for k in ("nq", "nkv", "hd", "P", "rot", "style"))
+    eps, theta = 1e-5, 5000.0
+    # two entries: positions 9..14 of request 0 and position 40 of request 1
+    positions = torch.tensor([9, 10, 11, 12, 13, 14, 40], dtype=torch.int32)
+    entry = torch.tensor([0, 0, 0, 0, 0, 0, 1], dtype=torch.int32)
+    T = positions.numel()
+    need = [14 // P + 1, 40 // P + 1]
+    ids = torch.randperm(sum(need) + 2).tolist()               # page ids in no order
+    tables = [ids[:need[0]], ids[need[0]:need[0] + need[1]]]
+    n_pages = len(ids)
+    bt = table_tensor(tables, DEV)
+    qkv = torch.randn(T, (nq + 2 * nkv) * hd).to(dtype)
+    qg, kg = 1 + 0.2 * torch.randn(hd), 1 + 0.2 * torch.randn(hd)
+    k_pool = torch.zeros(n_pages, nkv, P, hd, dtype=dtype, device=DEV)
+    v_pool = torch.zeros_like(k_pool)
+    q_out = torch.empty(T, nq * hd, dtype=dtype, device=DEV)
+    table = None
+    if style:
+        inv = 1.0 / (theta ** (torch.arange(0, rot, 2, dtype=torch.float32) / rot))
+        ang = torch.arange(64, dtype=torch.float32)[:, None] * inv[None]
+        table = torch.cat((ang.cos(), ang.sin()), -1).contiguous().to(DEV)
+    ops.qk_norm_rope_write(qkv.to(DEV), q_out, qg.to(DEV) if cfg["norm"] else None, kg.to(DEV) if cfg["norm"] else None,
+                           eps, table, rot, style, positions.to(DEV), entry.to(DEV), bt, k_pool, v_pool, P, nq, nkv,
+                           hd, write_kv=True)
+    x = qkv.float()
+    q, k, v = x[:, :nq * hd].view(T, nq, hd), x[:, nq * hd:(nq + nkv) * hd].view(T, nkv, hd), x[:, (nq + nkv) * hd:].view(T, nkv, hd)
+    if cfg["norm"]:
+        q, k = plain.rms_norm(q, qg, eps), plain.rms_norm(k, kg, eps)
+    if style:
+        cos, sin = plain.rope_cos_sin(positions, rot, theta)
+
+        def rotate(t):
+            r, rest = t[..., :rot], t[..., rot:]
+            if style == 1:
+                r = plain.apply_rope_concat_layout(r, cos, sin)
+            else:       # adjacent pairs (2i, 2i+1)
+                a, b = r[..., 0::2], r[..., 1::2]
+                c, s = cos.unsqueeze(1), sin.unsqueeze(1)
+                r = torch.stack((a * c - b * s, b * c + a * s), -1).flatten(-2)
+            return torch.cat((r, rest), -1)
+        q, k = rotate(q), rotate(k)
+    assert (q_out.float().cpu().view(T, nq, hd) - q).abs().max() <= tol(dtype, q)
+    for t in range(T):
+        pos, e = int(positions[t]), int(entry[t])
+        page, row = tables[e][pos // P], pos % P
+        assert (k_pool[page, :, row].float().cpu() - k[t]).abs().max() <= tol(dtype, k)
+        assert torch.equal(v_pool[page, :, row].float().cpu(), v[t])
+    written = sum(1 for _ in range(T))
+    assert int((k_pool.float().abs().sum(-1) > 0).sum()) == written * nkv       # nothing else was touched
+
+
+def reference_attention(qs, ks, vs, scale, window):
+    """qs[b]: [n_b, nq, hd] queries at the last n_b positions of sequence b (ks[b]: [S_b, nkv, hd])."""
+    outs = []
+    for q, k, v in zip(qs, ks, vs):
+        n, S = q.shape[0], k.shape[0]
+        full_q = torch.zeros(S, q.shape[1], q.shape[2])
+        full_q[S - n:] = q
+        outs.append(plain.causal_gqa_attention(full_q, k, v, scale, window)[S - n:])
+    return torch.cat(outs)
+
+
+ATT_CASES = [dict(nq=4, nkv=2, hd=16, P=4, lens=[(5, 5), (1, 37), (7, 20)], window=0),
+             dict(nq=6, nkv=2, hd=48, P=8, lens=[(1, 1), (2, 130), (33, 33), (1, 64)], window=0),
+             dict(nq=8, nkv=1, hd=128, P=16, lens=[(1, 300), (1, 17), (3, 48)], window=0),
+             dict(nq=3, nkv=3, hd=80, P=16, lens=[(9, 40), (1, 100)], window=11),
+             dict(nq=4, nkv=2, hd=256, P=32, lens=[(1, 70), (20, 64)], window=0)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("case", ATT_CASES)
+def test_paged_attention_generic(ops, dtype, case):
+    torch.manual_seed(5)
+    nq, nkv, hd, P, window = (case[k] for k in ("nq", "nkv", "hd", "P", "window"))
+    rnd = lambda *s: torch.randn(*s).to(dtype).float()   # noqa: E731
+    ks = [rnd(S, nkv, hd) for _, S in case["lens"]]
+    vs = [rnd(S, nkv, hd) for _, S in case["lens"]]
+    qs = [rnd(n, nq, hd) for n, _ in case["lens"]]
+    k_pool, v_pool, tables = paged_cache(ks, vs, P, dtype, DEV)          # unused rows are NaN
+    positions = torch.cat([torch.arange(S - n, S) for n, S in case["lens"]]).int().to(DEV)
+    entry = torch.cat([torch.full((n,), b) for b, (n, _) in enumerate(case["lens"])]).int().to(DEV)
+    q = torch.cat(qs).reshape(-1, nq * hd).to(DEV, dtype)
+    scale = hd ** -0.5
+    got = ops.paged_attention_generic(q, k_pool, v_pool, positions, entry, table_tensor(tables, DEV), P, nq, nkv,
+                                      hd, scale, window)
+    want = reference_attention(qs, ks, vs, scale, window).reshape(-1, nq * hd)
+    assert not torch.isnan(got).any()
+    assert (got.float().cpu() - want).abs().max() <= tol(dtype, want)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_finds_one_far_key_at_every_edge(ops, dtype):
+    """One key is made to dominate: the output must be its value row.  The key is placed at page edges,
+    at the first and last position and at both edges of a window, for a decoded token and for the last
+    token of a portion."""
+    torch.manual_seed(6)
+    nq, nkv, hd, P, S = 4, 2, 32, 8, 203
+    for window in (0, 50):
+        lo = 0 if window == 0 else S - window
+        for target in sorted(t for t in {lo, lo + 1, (lo // P + 1) * P - 1, (lo // P + 1) * P, 127, 128, 167, 168,
+                                        S - 2, S - 1} if t >= lo):
+            for n in (1, 5):
+                k = torch.randn(S, nkv, hd) * 0.1
+                v = torch.randn(S, nkv, hd).to(dtype).float()
+                q = torch.randn(n, nq, hd) * 0.1
+                direction = torch.randn(hd)
+                direction /= direction.norm()
+                k[target] = 30.0 * direction
+                q[-1] = 30.0 * direction                      # the last query looks at `target` only
+                k, q = k.to(dtype).float(), q.to(dtype).float()
+                k_pool, v_pool, tables = paged_cache([k], [v], P, dtype, DEV, seed=target)
+                positions = torch.arange(S - n, S).int().to(DEV)
+                entry = torch.zeros(n, dtype=torch.int32, device=DEV)
+                got = ops.paged_attention_generic(q.reshape(n, -1).to(DEV, dtype), k_pool, v_pool, positions, entry,
+                                                  table_tensor(tables, DEV), P, nq, nkv, hd, 1.0, window)
+                got = got.float().cpu().view(n, nq, hd)[-1]
+                for h in range(nq):
+                    assert (got[h] - v[target, h // 2]).abs().max() < 2e-2, (window, target, n, h)
+        if window:
+            # a dominant key just outside the window must NOT be seen
+            k = torch.randn(S, nkv, hd) * 0.1
+            direction = torch.ones(hd) / math.sqrt(hd)
+            k[lo - 1] = 30.0 * direction
+            q = (30.0 * direction).expand(1, nq, hd).clone()
+            v = torch.randn(S, nkv, hd)
+            k_pool, v_pool, tables = paged_cache([k], [v], P, dtype, DEV)
+            got = ops.paged_attention_generic(q.reshape(1, -1).to(DEV, dtype), k_pool, v_pool,
+                                              torch.tensor([S - 1], dtype=torch.int32, device=DEV),
+                                              torch.zeros(1, dtype=torch.int32, device=DEV), table_tensor(tables, DEV),
+                                              P, nq, nkv, hd, 1.0, window).float().cpu().view(nq, hd)
+            assert (got[0] - v[lo - 1, 0]).abs().max() > 0.1
+
+
+def test_sampler_kernel_against_the_plain_sampler(ops):
+    from ullm_amd.sampling import Sampler, SamplingParams
+    torch.manual_seed(7)
+    sampler = Sampler(torch.device(DEV))
+    configs = [(0.0, -1, 1.0, 0.0), (0.7, -1, 1.0, 0.0), (1.0, 5, 1.0, 0.0), (1.3, -1, 0.8, 0.0), (1.0, -1, 1.0, 0.1),
+               (0.9, 20, 0.9, 0.05), (1.0, 1, 1.0, 0.0), (1.0, -1, 0.01, 0.0), (1.0, 2000, 1.0, 0.0)]
+    for V in (503, 1537):
+        mismatches = 0
+        for trial in range(5):
+            logits = torch.randn(len(configs), V) * 3
+            ps = [SamplingParams(temperature=c[0], top_k=c[1], top_p=c[2], min_p=c[3]) for c in configs]
+            seeds = [trial * 100 + i for i in range(len(configs))]
+            pos = [trial * 7 + i for i in range(len(configs))]
+            got = sampler.sample(logits.to(DEV), ps, seeds, pos)
+            want = [plain.sample_token(logits[i], *configs[i], seeds[i], pos[i]) for i in range(len(configs))]
+            mismatches += sum(g != w for g, w in zip(got, want))
+            # the same row in another batch position draws the same token
+            again = sampler.sample(logits.flip(0).contiguous().to(DEV), ps[::-1], seeds[::-1], pos[::-1])
+            assert again[::-1] == got
+        assert mismatches == 0
+    # ties: greedy takes the first index of the maximum
+    logits = torch.zeros(2, 300)
+    logits[0, [40, 7, 200]] = 5.0
+    logits[1, 299] = 1.0
+    assert sampler.sample(logits.to(DEV), [SamplingParams(temperature=0.0)] * 2, [0, 0], [0, 0]) == [7, 299]
+    # frequencies follow the probabilities
+    logits = torch.tensor([[0.0, 1.0, 2.0, -1.0, 0.5]])
+    probs = torch.softmax(logits[0], -1)
+    n = 4000
+    rows = logits.expand(n, 5).contiguous().to(DEV)
+    got = sampler.sample(rows, [SamplingParams(temperature=1.0)] * n, [99] * n, list(range(n)))
+    counts = torch.bincount(torch.tensor(got), minlength=5).float()
+    assert float(((counts - n * probs) ** 2 / (n * probs)).sum()) < 25.0

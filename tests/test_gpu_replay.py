@@ -1,0 +1,206 @@
+"""Trace replay against the plain implementation: each request alone and whole; most of it in one
+step and the last 32 tokens one by one; portions of changing size down to two tokens; mixed with up
+to four live requests and so few pages that they are used again; long decoding; first tokens.
+In 32-bit and in bfloat16, for three tiny configurations."""
+import numpy as np
+import pytest
+import torch
+
+import plain_qwen3 as plain
+from gpu_util import DEV
+
+pytestmark = pytest.mark.gpu
+
+REL = {"float32": 2e-5, "bfloat16": 3e-2}
+
+
+def close(got, want, dtype):
+    want = want.numpy() if isinstance(want, torch.Tensor) else want
+    bound = REL[dtype] * float(np.abs(want).max()) + 1e-6
+    err = float(np.abs(got - want).max())
+    assert err <= bound, f"max |diff| {err:.3e} > {bound:.3e}"
+
+
+def make_tokens(vocab, n, seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, vocab, (n,), generator=g).tolist()
+
+
+@pytest.fixture(scope="module")
+def replayers(model_dirs):
+    from ullm_amd.replay import Replayer
+    cache = {}
+
+    def get(name, dtype, max_tokens=512, page_size=16):
+        key = (name, dtype, max_tokens, page_size)
+        if key not in cache:
+            cache[key] = Replayer(model_dirs[name], dtype, max_tokens, page_size, DEV)
+        rep = cache[key]
+        assert not rep.live and rep.runner.cache.num_free_pages() == rep.max_tokens // page_size
+        return rep
+    return get
+
+
+def oracle(plain_models, name, toks):
+    cfg, w = plain_models[name]
+    return plain.qwen3_forward(w, cfg, toks)
+
+
+CASES = [(n, d) for n in ("A", "B", "C") for d in ("float32", "bfloat16")]
+
+
+@pytest.mark.parametrize("name,dtype", CASES)
+def test_whole(replayers, plain_models, name, dtype):
+    rep = replayers(name, dtype)
+    vocab = plain_models[name][0]["vocab_size"]
+    for i, n in enumerate((1, 2, 17, 70, 113)):
+        toks = make_tokens(vocab, n, 10 + i)
+        got = rep.step({"step": i, "entries": [{"id": "r", "tokens": toks, "want": list(range(n))}], "end": ["r"]})
+        close(got, oracle(plain_models, name, toks), dtype)
+
+
+@pytest.mark.parametrize("name,dtype", CASES)
+def test_bulk_then_one_by_one(replayers, plain_models, name, dtype):
+    rep = replayers(name, dtype)
+    vocab = plain_models[name][0]["vocab_size"]
+    toks = make_tokens(vocab, 101, 20)
+    want = oracle(plain_models, name, toks)
+    head = len(toks) - 32
+    got = [rep.step({"step": 0, "entries": [{"id": "r", "tokens": toks[:head], "want": [head - 1]}], "end": []})]
+    for i in range(head, len(toks)):
+        got.append(rep.step({"step": i, "entries": [{"id": "r", "tokens": [toks[i]], "want": [0]}],
+                             "end": ["r"] if i == len(toks) - 1 else []}))
+    close(np.concatenate(got), want[head - 1:], dtype)
+
+
+@pytest.mark.parametrize("name,dtype", CASES)
+def test_changing_portions(replayers, plain_models, name, dtype):
+    rep = replayers(name, dtype)
+    vocab = plain_models[name][0]["vocab_size"]
+    toks = make_tokens(vocab, 150, 21)
+    want = oracle(plain_models, name, toks)
+    sizes = [2, 3, 16, 2, 15, 17, 1, 31, 2, 33, 5, 2, 2, 19]
+    assert sum(sizes) == 150
+    got, i = [], 0
+    for s, n in enumerate(sizes):
+        got.append(rep.step({"step": s, "entries": [{"id": "r", "tokens": toks[i:i + n], "want": list(range(n))}],
+                             "end": ["r"] if i + n == 150 else []}))
+        i += n
+    close(np.concatenate(got), want, dtype)
+
+
+@pytest.mark.parametrize("name,dtype", CASES)
+def test_mixed_with_page_reuse(replayers, plain_models, name, dtype):
+    """Seven requests, at most four live, portions of some beside decoded tokens of others.  The pool
+    holds 256 tokens while the requests need 2.4 times that in total, so pages are used again."""
+    rep = replayers(name, dtype, max_tokens=256, page_size=16)
+    vocab = plain_models[name][0]["vocab_size"]
+    lens = [70, 33, 90, 47, 61, 5, 64]
+    reqs = {f"q{i}": make_tokens(vocab, n, 30 + i) for i, n in enumerate(lens)}
+    wants = {r: oracle(plain_models, name, t) for r, t in reqs.items()}
+    done = {r: 0 for r in reqs}
+    got = {r: [] for r in reqs}
+    waiting = list(reqs)
+    live = []
+    rng = np.random.default_rng(0)
+    step = 0
+    freed_pages = set()
+    reused = False
+    while waiting or live:
+        while waiting and len(live) < 4:
+            cand = waiting[0]
+            held = sum(-(-max(done[r], 1) // 64) * 64 for r in live)
+            if held + -(-len(reqs[cand]) // 64) * 64 > 256:
+                break
+            live.append(waiting.pop(0))
+        entries, ends = [], []
+        for r in list(live):
+            rest = len(reqs[r]) - done[r]
+            if done[r] >= len(reqs[r]) - 8:
+                n = 1                                               # decode the tail token by token
+            else:
+                n = int(min(rest, rng.choice([2, 3, 7, 16, 29])))
+            if rng.random() < 0.15 and len(live) > 1:
+                continue                                            # left out of this step, goes on later
+            entries.append({"id": r, "tokens": reqs[r][done[r]:done[r] + n], "want": list(range(n))})
+            done[r] += n
+            if done[r] == len(reqs[r]):
+                ends.append(r)
+                live.remove(r)
+        for r in ends:                                              # pages about to be given back
+            freed_pages |= set(rep.live[r].tables[0]) if r in rep.live else set()
+        out = rep.step({"step": step, "entries": entries, "end": ends})
+        for rc in rep.live.values():
+            reused |= bool(freed_pages & {p for p in rc.tables[0] if p >= 0})
+        row = 0
+        for e in entries:
+            n = len(e["tokens"])
+            got[e["id"]].append(out[row:row + n])
+            row += n
+        step += 1
+        rep.runner.cache.check()
+    for r in reqs:
+        close(np.concatenate(got[r]), wants[r], dtype)
+    total_pages = sum(-(-n // 16) for n in lens)
+    assert total_pages > 256 // 16                                  # more pages were needed than exist
+    assert reused                                                   # a later request got a page an ended one had used
+
+
+@pytest.mark.parametrize("name,dtype", [("B", "float32"), ("C", "bfloat16"), ("C", "float32")])
+def test_long_decoding(replayers, plain_models, name, dtype):
+    rep = replayers(name, dtype)
+    vocab = plain_models[name][0]["vocab_size"]
+    toks = make_tokens(vocab, 230, 40)
+    want = oracle(plain_models, name, toks)
+    got = [rep.step({"step": 0, "entries": [{"id": "r", "tokens": toks[:3], "want": [0, 1, 2]}], "end": []})]
+    for i in range(3, len(toks)):
+        got.append(rep.step({"step": i, "entries": [{"id": "r", "tokens": [toks[i]], "want": [0]}],
+                             "end": ["r"] if i == len(toks) - 1 else []}))
+    close(np.concatenate(got), want, dtype)
+
+
+@pytest.mark.parametrize("name,dtype", CASES)
+def test_first_tokens_and_skipped_logits(replayers, plain_models, name, dtype):
+    rep = replayers(name, dtype)
+    vocab = plain_models[name][0]["vocab_size"]
+    toks = make_tokens(vocab, 20, 41)
+    want = oracle(plain_models, name, toks)
+    a = rep.step({"step": 0, "entries": [{"id": "r", "tokens": toks[:1], "want": [0]}], "end": []})
+    close(a, want[:1], dtype)
+    assert rep.step({"step": 1, "entries": [{"id": "r", "tokens": toks[1:9], "want": []}], "end": []}) is None
+    b = rep.step({"step": 2, "entries": [{"id": "r", "tokens": toks[9:20], "want": [10, 0]}], "end": ["r"]})
+    close(b, want[[19, 9]], dtype)                                   # order of `want` is kept
+
+
+def test_other_page_sizes(replayers, plain_models):
+    for page_size in (4, 64):
+        rep = replayers("B", "float32", max_tokens=128, page_size=page_size)
+        toks = make_tokens(503, 100, 42)
+        want = oracle(plain_models, "B", toks)
+        got = [rep.step({"step": 0, "entries": [{"id": "r", "tokens": toks[:61], "want": list(range(61))}], "end": []})]
+        for i in range(61, 100):
+            got.append(rep.step({"step": i, "entries": [{"id": "r", "tokens": [toks[i]], "want": [0]}],
+                                 "end": ["r"] if i == 99 else []}))
+        close(np.concatenate(got), want, "float32")
+
+
+def test_pool_too_small_is_an_error_not_a_wrong_result(replayers):
+    rep = replayers("A", "float32", max_tokens=64)
+    with pytest.raises(RuntimeError, match="pages"):
+        rep.step({"step": 0, "entries": [{"id": "r", "tokens": list(range(65)), "want": []}], "end": []})
+    rep.step({"step": 1, "entries": [], "end": ["r"]})
+
+
+def test_trace_run_program(trace_run, model_dirs, plain_models):
+    """The program itself: protocol on stdin/stdout, files in --out, exit code."""
+    for dtype in ("float32", "bfloat16"):
+        tr = trace_run(model_dirs["B"], dtype, 128)
+        toks = make_tokens(503, 40, 43)
+        want = oracle(plain_models, "B", toks)
+        a = tr.step([("x", toks[:30], [29]), ("y", toks[:5], [])])
+        b = tr.step([("x", toks[30:31], [0]), ("y", toks[5:40], [34, 0])], end=["y"])
+        c = tr.step([("x", toks[31:40], list(range(9)))], end=["x"])
+        tr.close()
+        close(a, want[29:30], dtype)
+        close(b, want[[30, 39, 5]], dtype)
+        close(c, want[31:], dtype)

@@ -1,0 +1,102 @@
+"""Weight binding by name, its one error, and the random-weights mode (no GPU)."""
+import json
+import os
+
+import pytest
+import torch
+from safetensors.torch import load_file, save_file
+
+from conftest import TINY_A, TINY_B
+from ullm_amd.models import build_model
+from ullm_amd.parts import PartEnv
+from ullm_amd.weights.loader import WeightError, checkpoint_index, load_weights
+from ullm_amd.weights.random_init import write_random_model
+
+CPU32 = PartEnv(torch.device("cpu"), torch.float32, 64)
+CPU16 = PartEnv(torch.device("cpu"), torch.bfloat16, 64)
+
+
+def test_random_folder_is_complete_and_deterministic(tmp_path):
+    a = write_random_model(TINY_B, str(tmp_path / "a"), seed=7)
+    b = write_random_model(TINY_B, str(tmp_path / "b"), seed=7)
+    c = write_random_model(TINY_B, str(tmp_path / "c"), seed=8)
+    assert json.load(open(os.path.join(a, "config.json")))["hidden_size"] == 96
+    wa, wb, wc = (load_file(os.path.join(d, "model.safetensors")) for d in (a, b, c))
+    assert set(wa) == {d.name for d in build_model(TINY_B)[1].weight_decls()}
+    assert all(torch.equal(wa[k], wb[k]) for k in wa)
+    assert any(not torch.equal(wa[k], wc[k]) for k in wa)
+    assert all(v.dtype == torch.bfloat16 for v in wa.values())
+    # gains are 1 + N(0, s), matrices N(0, s) with s = initializer_range
+    assert abs(wa["model.norm.weight"].float().mean() - 1.0) < 0.05
+    assert abs(wa["model.layers.0.mlp.down_proj.weight"].float().std() - 0.05) < 0.005
+
+
+def test_tied_model_stores_no_head_and_binds_the_embedding(tmp_path):
+    d = write_random_model(TINY_A, str(tmp_path / "a"), seed=0)
+    assert "lm_head.weight" not in checkpoint_index(d)
+    _, model = build_model(TINY_A)
+    load_weights(model, d, CPU16)
+    assert model.head.data_ptr() == model.embedding.data_ptr()
+    assert model.embedding.dtype == torch.bfloat16
+    assert model.final_norm.gain.dtype == torch.float32            # gains stay 32-bit
+
+
+def test_float32_mode_widens_exactly(tmp_path):
+    d = write_random_model(TINY_A, str(tmp_path / "a"), seed=0)
+    stored = load_file(os.path.join(d, "model.safetensors"))
+    _, model = build_model(TINY_A)
+    load_weights(model, d, CPU32)
+    assert model.embedding.dtype == torch.float32
+    assert torch.equal(model.embedding, stored["model.embed_tokens.weight"].float())
+    attn = model.blocks[0].mixer
+    want = torch.cat([stored[f"model.layers.0.self_attn.{n}_proj.weight"].float() for n in "qkv"])
+    assert torch.equal(attn.w_qkv, want)                           # rows q | k | v (ullm/layers/linear.py:381-389)
+    ffn = model.blocks[1].ffn
+    want = torch.cat([stored["model.layers.1.mlp.gate_proj.weight"].float(),
+                      stored["model.layers.1.mlp.up_proj.weight"].float()])
+    assert torch.equal(ffn.w_gate_up, want)                        # rows gate | up (ullm/models/qwen3.py:307-308)
+
+
+def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
+    d = write_random_model(TINY_B, str(tmp_path / "b"), seed=1)
+    path = os.path.join(d, "model.safetensors")
+    w = load_file(path)
+    del w["model.layers.1.self_attn.k_norm.weight"]
+    del w["lm_head.weight"]
+    w["model.layers.0.mlp.down_proj.weight"] = torch.zeros(96, 100, dtype=torch.bfloat16)
+    w["model.layers.9.mlp.down_proj.weight"] = torch.zeros(2, 2, dtype=torch.bfloat16)
+    w["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.zeros(16)      # known and ignorable
+    save_file(w, path)
+    _, model = build_model(TINY_B)
+    with pytest.raises(WeightError) as e:
+        load_weights(model, d, CPU32)
+    msg = str(e.value)
+    assert "missing tensors (2)" in msg and "model.layers.1.self_attn.k_norm.weight" in msg and "lm_head.weight" in msg
+    assert "unexpected tensors (1)" in msg and "model.layers.9.mlp.down_proj.weight" in msg
+    assert "wrong shapes (1)" in msg and "[96, 100]" in msg and "[96, 224]" in msg
+    assert "inv_freq" not in msg
+
+
+def test_no_safetensors_file(tmp_path):
+    (tmp_path / "config.json").write_text(json.dumps(TINY_A))
+    _, model = build_model(TINY_A)
+    with pytest.raises(WeightError, match="no \\*.safetensors"):
+        load_weights(model, str(tmp_path), CPU32)
+
+
+def test_tensors_may_be_spread_over_files_and_stored_in_32_bit(tmp_path):
+    d = write_random_model(TINY_A, str(tmp_path / "a"), seed=3, dtype="float32")
+    path = os.path.join(d, "model.safetensors")
+    w = load_file(path)
+    assert all(v.dtype == torch.float32 for v in w.values())
+    names = sorted(w)
+    save_file({k: w[k] for k in names[:10]}, os.path.join(d, "model-00001-of-00002.safetensors"))
+    save_file({k: w[k] for k in names[10:]}, os.path.join(d, "model-00002-of-00002.safetensors"))
+    os.unlink(path)
+    _, model = build_model(TINY_A)
+    load_weights(model, d, CPU32)
+    assert torch.equal(model.final_norm.gain, w["model.norm.weight"])
+    _, model16 = build_model(TINY_A)
+    load_weights(model16, d, CPU16)
+    assert model16.embedding.dtype == torch.bfloat16 and model16.final_norm.gain.dtype == torch.float32
+    assert torch.equal(model16.final_norm.gain, w["model.norm.weight"])     # a 32-bit gain stays as stored

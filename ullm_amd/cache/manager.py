@@ -134,11 +134,12 @@ class CacheManager:
         no later query can reach: page i is dead once (i+1)*page_size <= num_computed - window + 1."""
         if rc.released:
             raise PageError(f"request {rc.request_id!r} was released")
-        rc.num_computed += n_new
         P = self.page_size
-        for g, spec in enumerate(self.groups):
-            if rc.num_computed > len(rc.tables[g]) * P:
+        for g in range(len(self.groups)):
+            if rc.num_computed + n_new > len(rc.tables[g]) * P:
                 raise PageError(f"request {rc.request_id!r} computed past its reserved pages")
+        rc.num_computed += n_new
+        for g, spec in enumerate(self.groups):
             if spec.window > 0:
                 dead_upto = (rc.num_computed - spec.window + 1) // P   # pages [first_live, dead_upto) die
                 table = rc.tables[g]

@@ -58,10 +58,10 @@ class Scheduled:
     request: Request
     start: int
     num_tokens: int
+    samples: bool = False
 
-    @property
-    def samples(self) -> bool:
-        return self.start + self.num_tokens == self.request.num_tokens
+    def __post_init__(self):
+        self.samples = self.start + self.num_tokens == self.request.num_tokens
 
 
 @dataclass

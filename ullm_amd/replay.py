@@ -32,58 +32,73 @@ def parse_args(argv=None):
     return ap.parse_args(argv)
 
 
-def main(argv=None) -> int:
-    args = parse_args(argv)
-    if args.page_size < 1 or 64 % args.page_size:
-        print(f"trace_run: --page-size {args.page_size} must divide 64", file=sys.stderr)
-        return 2
-    if args.max_tokens < 1:
-        print("trace_run: --max-tokens must be positive", file=sys.stderr)
-        return 2
-    os.makedirs(args.out, exist_ok=True)
+class Replayer:
+    """The replay loop's state: the model, its runner and the live requests."""
 
-    import torch
-    from .engine.loading import load_model
-    from .engine.runner import ModelRunner, StepEntry
+    def __init__(self, model_dir: str, dtype: str, max_tokens: int, page_size: int = 16, device: str = "cuda:0",
+                 max_requests: int = 8):
+        from .engine.loading import load_model
+        from .engine.runner import ModelRunner
+        if page_size < 1 or 64 % page_size:
+            raise ValueError(f"page size {page_size} must divide 64")
+        if max_tokens < 1:
+            raise ValueError("max_tokens must be positive")
+        self.max_tokens = -(-max_tokens // 64) * 64
+        self.cfg, self.model, self.env = load_model(model_dir, dtype, device, context_len=self.max_tokens)
+        self.runner = ModelRunner(self.model, self.env, page_size=page_size,
+                                  num_pages=self.max_tokens // page_size, max_requests=max_requests)
+        self.live = {}
 
-    max_tokens = -(-args.max_tokens // 64) * 64
-    num_pages = max_tokens // args.page_size
-    cfg, model, env = load_model(args.model, args.dtype, args.device, context_len=max_tokens)
-    runner = ModelRunner(model, env, page_size=args.page_size, num_pages=num_pages, max_requests=8)
-    live = {}
-
-    for line in sys.stdin:
-        line = line.strip()
-        if not line:
-            continue
-        msg = json.loads(line)
-        step = msg["step"]
+    def step(self, msg: dict):
+        """Run one step object; returns float32 logits [wanted, vocab] on the host or None."""
+        from .engine.runner import StepEntry
+        step = msg.get("step")
         entries = []
         for ent in msg.get("entries", []):
             rid = str(ent["id"])
             tokens = [int(t) for t in ent["tokens"]]
             if not tokens:
                 continue
-            rc = live.get(rid)
+            rc = self.live.get(rid)
             if rc is None:
-                rc = runner.cache.admit(rid)
-                live[rid] = rc
-            if not runner.cache.reserve(rc, len(tokens)):
+                rc = self.runner.cache.admit(rid)
+                self.live[rid] = rc
+            if not self.runner.cache.reserve(rc, len(tokens)):
                 raise RuntimeError(
                     f"step {step}: request {rid!r} needs pages for {len(tokens)} more tokens but the pool made "
-                    f"for --max-tokens {args.max_tokens} has {runner.cache.num_free_pages()} pages left")
+                    f"for {self.max_tokens} tokens has {self.runner.cache.num_free_pages()} pages left")
             entries.append(StepEntry(rc, tokens, [int(w) for w in ent.get("want", [])]))
+        out = None
         if entries:
-            logits = runner.step(entries)
+            logits = self.runner.step(entries)
             if logits is not None:
-                arr = logits.to("cpu", torch.float32).contiguous().numpy().astype("<f4", copy=False)
-                tmp = os.path.join(args.out, f".{step}.f32.tmp")
-                arr.tofile(tmp)
-                os.replace(tmp, os.path.join(args.out, f"{step}.f32"))
+                out = logits.float().cpu().contiguous().numpy()
         for rid in msg.get("end", []):
-            rc = live.pop(str(rid), None)
+            rc = self.live.pop(str(rid), None)
             if rc is not None:
-                runner.cache.release(rc)
+                self.runner.cache.release(rc)
+        return out
+
+
+def main(argv=None) -> int:
+    args = parse_args(argv)
+    os.makedirs(args.out, exist_ok=True)
+    try:
+        rep = Replayer(args.model, args.dtype, args.max_tokens, args.page_size, args.device)
+    except ValueError as e:
+        print(f"trace_run: {e}", file=sys.stderr)
+        return 2
+    for line in sys.stdin:
+        line = line.strip()
+        if not line:
+            continue
+        msg = json.loads(line)
+        step = msg["step"]
+        arr = rep.step(msg)
+        if arr is not None:
+            tmp = os.path.join(args.out, f".{step}.f32.tmp")
+            arr.astype("<f4", copy=False).tofile(tmp)
+            os.replace(tmp, os.path.join(args.out, f"{step}.f32"))
         sys.stdout.write(f"done {step}\n")
         sys.stdout.flush()
     return 0
