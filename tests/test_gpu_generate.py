@@ -1,0 +1,148 @@
+"""Generation through the entry point: greedy tokens equal the plain implementation's; seeded
+temperature sampling equals the plain sampler run on the engine's own logits; finish rules;
+preemption and recomputation give the same tokens; the command line."""
+import json
+
+import pytest
+import torch
+
+import plain_qwen3 as plain
+from gpu_util import DEV
+
+pytestmark = pytest.mark.gpu
+
+
+def make_llm(model_dir, **kw):
+    from ullm_amd import LLM, EngineConfig
+    args = dict(model=model_dir, dtype="float32", max_bs=8, context_len=128, page_size=16, num_pages=64, device=DEV)
+    args.update(kw)
+    return LLM(EngineConfig(**args))
+
+
+def prompts_of(vocab, lens, seed):
+    g = torch.Generator().manual_seed(seed)
+    return [torch.randint(0, vocab, (n,), generator=g).tolist() for n in lens]
+
+
+@pytest.mark.parametrize("name,page_size,budget,chunk", [("A", 16, 64, 64), ("A", 16, 9, 4), ("B", 4, 16, 7),
+                                                          ("C", 8, 12, 5)])
+def test_greedy_generation_equals_the_plain_implementation(model_dirs, plain_models, name, page_size, budget, chunk):
+    from ullm_amd import SamplingParams
+    cfg, w = plain_models[name]
+    prompts = prompts_of(cfg["vocab_size"], (5, 11, 17, 1), 1)
+    llm = make_llm(model_dirs[name], page_size=page_size, max_num_batched_tokens=budget, max_prefill_chunk=chunk)
+    outs = llm.generate(prompts, SamplingParams(temperature=0.0, max_new_tokens=8, ignore_eos=True))
+    for p, o in zip(prompts, outs):
+        assert o.token_ids == plain.greedy_generate(w, cfg, p, 8)
+        assert o.finish_reason.name == "LENGTH" and o.num_prompt_tokens == len(p)
+    llm.engine.runner.cache.check()
+    assert llm.engine.runner.cache.num_free_pages() == 64
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_seeded_sampling_equals_the_plain_sampler_on_the_engines_logits(model_dirs, plain_models, dtype):
+    """Config B's workload: prompts of 1, 3, 9, 33 and 70 tokens, temperature 0.7, 12 new tokens each,
+    prompt portions of 7 with decodes beside them."""
+    from ullm_amd import SamplingParams
+    cfg, w = plain_models["B"]
+    prompts = prompts_of(503, (1, 3, 9, 33, 70), 3)
+    llm = make_llm(model_dirs["B"], dtype=dtype, page_size=4, num_pages=128, max_num_batched_tokens=24,
+                   max_prefill_chunk=7)
+    seen = {}
+
+    def hook(sampling, logits):
+        for s, row in zip(sampling, logits.float().cpu()):
+            seen.setdefault(s.request.request_id, []).append((s.request.num_tokens, row))
+    llm.engine.on_logits = hook
+    params = [SamplingParams(temperature=0.7, top_k=50 if i % 2 else -1, top_p=0.9 if i == 2 else 1.0,
+                             max_new_tokens=12, ignore_eos=True, seed=100 + i) for i in range(5)]
+    ids = [f"s{i}" for i in range(5)]
+    outs = llm.generate(prompts, params, ids)
+    for i, (p, o) in enumerate(zip(prompts, outs)):
+        assert len(o.token_ids) == 12
+        for (pos, row), tok in zip(seen[ids[i]], o.token_ids):
+            want = plain.sample_token(row, 0.7, params[i].top_k, params[i].top_p, 0.0, 100 + i, pos)
+            assert tok == want
+        # and the logits the engine sampled from are the plain implementation's
+        full = plain.qwen3_forward(w, cfg, p + o.token_ids)
+        for (pos, row) in seen[ids[i]]:
+            bound = (2e-5 if dtype == "float32" else 3e-2) * float(full.abs().max()) + 1e-6
+            assert float((row - full[pos - 1]).abs().max()) <= bound
+    # the same seeds give the same tokens in another batch composition
+    again = llm.generate(prompts[::-1], params[::-1])
+    assert [o.token_ids for o in again[::-1]] == [o.token_ids for o in outs]
+
+
+def test_preempted_requests_are_recomputed_to_the_same_tokens(model_dirs, plain_models):
+    from ullm_amd import SamplingParams
+    cfg, w = plain_models["B"]
+    prompts = prompts_of(503, (20, 22, 18), 5)
+    roomy = make_llm(model_dirs["B"], page_size=4, num_pages=128)
+    want = [o.token_ids for o in roomy.generate(prompts, SamplingParams(temperature=0.8, max_new_tokens=20,
+                                                                        ignore_eos=True, seed=7))]
+    tight = make_llm(model_dirs["B"], page_size=4, num_pages=22)       # 88 tokens for 3 x ~40
+    outs = tight.generate(prompts, SamplingParams(temperature=0.8, max_new_tokens=20, ignore_eos=True, seed=7))
+    assert [o.token_ids for o in outs] == want
+    assert tight.engine.scheduler.num_preemptions > 0 and roomy.engine.scheduler.num_preemptions == 0
+    assert tight.engine.runner.cache.num_free_pages() == 22
+    tight.engine.runner.cache.check()
+
+
+def test_finish_rules_and_abort(model_dirs, plain_models):
+    from ullm_amd import FinishReason, SamplingParams
+    cfg, w = plain_models["B"]
+    prompt = prompts_of(503, (6,), 8)[0]
+    greedy = plain.greedy_generate(w, cfg, prompt, 6)
+    llm = make_llm(model_dirs["B"], context_len=16)
+    # eos: stops at the first generated token equal to eos_token_id, which is emitted (ullm/core/engine.py:177-181)
+    out = llm.generate(prompt, SamplingParams(temperature=0.0, eos_token_id=greedy[2], max_new_tokens=6))
+    stop_at = greedy.index(greedy[2])
+    assert out.token_ids == greedy[:stop_at + 1] and out.finish_reason is FinishReason.STOP
+    # max_tokens caps prompt + generated (engine.py:184-189)
+    out = llm.generate(prompt, SamplingParams(temperature=0.0, max_tokens=9, ignore_eos=True))
+    assert len(out.token_ids) == 3 and out.finish_reason is FinishReason.LENGTH
+    # context_len caps the total (engine.py:196-198); a longer prompt keeps its last context_len tokens (:81-82)
+    out = llm.generate(prompt, SamplingParams(temperature=0.0, ignore_eos=True))
+    assert len(out.token_ids) == 10
+    long_prompt = prompts_of(503, (30,), 9)[0]
+    out = llm.generate(long_prompt, SamplingParams(temperature=0.0, max_new_tokens=1, ignore_eos=True))
+    assert out.prompt_token_ids == long_prompt[-16:]
+    # stream yields one record per token, the last one finished with its counts
+    recs = list(llm.stream(prompt, SamplingParams(temperature=0.0, max_new_tokens=4, ignore_eos=True)))
+    assert [r.token_id for r in recs] == greedy[:4] and [r.is_finished for r in recs] == [False] * 3 + [True]
+    assert recs[-1].num_prompt_tokens == 6 and recs[-1].num_generated_tokens == 4
+    # abort frees everything
+    eng = llm.engine
+    eng.add_request("gone", prompt, SamplingParams(max_new_tokens=50))
+    eng.step()
+    llm.abort("gone")
+    assert not eng.has_unfinished_requests() and eng.runner.cache.num_free_pages() == 64
+    with pytest.raises(ValueError):
+        eng.add_request("bad", [503], SamplingParams())
+
+
+def test_prefix_cache_gives_the_same_tokens(model_dirs, plain_models):
+    from ullm_amd import SamplingParams
+    cfg, w = plain_models["A"]
+    shared = prompts_of(256, (40,), 10)[0]
+    prompts = [shared + [1, 2, 3], shared + [9], shared[:33]]
+    llm = make_llm(model_dirs["A"], enable_prefix_cache=True, num_pages=32)
+    sp = SamplingParams(temperature=0.0, max_new_tokens=5, ignore_eos=True)
+    first = llm.generate(prompts[0], sp)
+    rest = llm.generate(prompts[1:], sp)
+    for p, o in zip(prompts, [first] + rest):
+        assert o.token_ids == plain.greedy_generate(w, cfg, p, 5)
+    assert llm.engine.runner.cache.prefix_tree.num_nodes >= 2
+    llm.engine.runner.cache.check()
+
+
+def test_command_line(model_dirs, plain_models, capsys):
+    from ullm_amd.cli import main
+    cfg, w = plain_models["A"]
+    rc = main(["--model", model_dirs["A"], "--dtype", "float32", "--prompt-ids", "5,17,3", "--prompt-ids", "9,8",
+               "--temperature", "0", "--max-new-tokens", "4", "--ignore-eos", "--context-len", "64", "--num-pages", "16",
+               "--max-bs", "4"])
+    assert rc == 0
+    lines = [json.loads(x) for x in capsys.readouterr().out.strip().splitlines() if x.startswith("{")]
+    assert [x["token_ids"] for x in lines] == [plain.greedy_generate(w, cfg, [5, 17, 3], 4),
+                                               plain.greedy_generate(w, cfg, [9, 8], 4)]

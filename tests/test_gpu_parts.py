@@ -1,0 +1,151 @@
+"""Each part alone, parts in other arrangements than Qwen3's, and a toy mixer with state of its own
+that is registered, built and stepped from outside the framework (tests/toy_arch.py)."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import plain_qwen3 as plain
+import toy_arch
+from gpu_util import DEV, tol
+
+pytestmark = pytest.mark.gpu
+DTYPES = ["float32", "bfloat16"]
+REL = {"float32": 2e-5, "bfloat16": 3e-2}
+
+
+def base_cfg(layers, **kw):
+    cfg = dict(architectures=["ToyStackForCausalLM"], vocab_size=211, hidden_size=72, eps=2e-6, theta=3000.0,
+               layers=layers, init_std=0.08)
+    cfg.update(kw)
+    return cfg
+
+
+ATT = dict(mixer="attention", heads=6, kv_heads=3, head_dim=16, ffn_size=100)
+TOY = dict(mixer="running_mean", ffn_size=60)
+
+
+def run_and_compare(tmp_path, cfg, dtype, cuts, n_tokens=75, page_size=8, seed=11):
+    """Write the toy model, replay one request in the given cuts beside a second request, compare
+    every position with the toy architecture's plain forward."""
+    from ullm_amd.replay import Replayer
+    from ullm_amd.weights.random_init import write_random_model
+    from safetensors.torch import load_file
+    d = write_random_model(cfg, str(tmp_path / f"m{seed}"), seed=seed)
+    w = load_file(os.path.join(d, "model.safetensors"))
+    g = torch.Generator().manual_seed(seed)
+    toks = torch.randint(0, cfg["vocab_size"], (n_tokens,), generator=g).tolist()
+    other = torch.randint(0, cfg["vocab_size"], (40,), generator=g).tolist()
+    want, want_other = toy_arch.toy_forward(w, cfg, toks), toy_arch.toy_forward(w, cfg, other)
+    rep = Replayer(d, dtype, 256, page_size, DEV)
+    got, got_other, i, j = [], [], 0, 0
+    assert sum(cuts) == n_tokens
+    for s, n in enumerate(cuts):
+        entries = [{"id": "a", "tokens": toks[i:i + n], "want": list(range(n))}]
+        m = min(7, len(other) - j)
+        if m > 0:
+            entries.insert(0, {"id": "b", "tokens": other[j:j + m], "want": list(range(m))})
+        out = rep.step({"step": s, "entries": entries, "end": []})
+        if m > 0:
+            got_other.append(out[:m])
+            out = out[m:]
+            j += m
+        got.append(out)
+        i += n
+    rep.step({"step": 999, "entries": [], "end": ["a", "b"]})
+    rep.runner.cache.check()
+    for g_, w_ in ((np.concatenate(got), want), (np.concatenate(got_other), want_other[:j])):
+        bound = REL[dtype] * float(w_.abs().max()) + 1e-6
+        assert float(np.abs(g_ - w_.numpy()).max()) <= bound
+    return rep, w
+
+
+CUTS = [75], [43] + [1] * 32, [2, 9, 1, 17, 2, 30, 3, 11]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("cuts", CUTS)
+def test_toy_mixer_with_state_registers_builds_and_steps(tmp_path, dtype, cuts):
+    """Layers 0 and 2 are attention, layer 1 is the toy mixer: different mixers in one model, state
+    carried across portion boundaries, zeroed when a slot is taken again."""
+    cfg = base_cfg([ATT, TOY, dict(ATT, heads=4, kv_heads=1, head_dim=32)])
+    rep, w = run_and_compare(tmp_path, cfg, dtype, cuts)
+    groups = rep.runner.cache.groups
+    assert len(groups) == 2 and any(c.state is not None for c in rep.runner.caches.values())
+    # the slots are used again by new requests: their state must start from zero
+    toks = list(range(3, 30))
+    out = rep.step({"step": 0, "entries": [{"id": "z", "tokens": toks, "want": [len(toks) - 1]}], "end": ["z"]})
+    want = toy_arch.toy_forward(w, cfg, toks)[-1:]
+    assert float(np.abs(out - want.numpy()).max()) <= REL[dtype] * float(want.abs().max()) + 1e-6
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_only_state_layers_need_no_pages(tmp_path, dtype):
+    cfg = base_cfg([TOY, TOY], tie=True)
+    rep, _ = run_and_compare(tmp_path, cfg, dtype, CUTS[2])
+    assert rep.runner.cache.groups == []
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("variant", [
+    dict(rope="adjacent"), dict(rope="none"), dict(rope="half", rotary_dim=8), dict(qk_norm=False),
+    dict(bias=True), dict(window=9), dict(scale=0.31), dict(heads=5, kv_heads=5, head_dim=48),
+    dict(heads=8, kv_heads=1, head_dim=64)])
+def test_attention_part_options(tmp_path, dtype, variant):
+    """The attention mixer with another position encoding (adjacent pairs, partial rotation, none),
+    without its norms, with biases, with a window, with a scale of its own, with other head shapes."""
+    cfg = base_cfg([dict(ATT, **variant), ATT])
+    run_and_compare(tmp_path, cfg, dtype, CUTS[2], seed=12)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_run_order_names_a_layer_twice_and_shares_a_cache(tmp_path, dtype):
+    # layer 1 runs twice with a cache of its own each time; layer 2 reads the cache layer 0 wrote
+    cfg = base_cfg([ATT, dict(ATT, window=13), ATT], run_order=[[0, 0], [1, 1], [1, 7], [2, 0]])
+    rep, _ = run_and_compare(tmp_path, cfg, dtype, CUTS[2], seed=13)
+    assert sorted(rep.runner.caches) == [0, 1, 7]
+    _, model = __import__("ullm_amd.models", fromlist=["build_model"]).build_model(cfg)
+    groups, cache_group, _ = model.cache_layout()
+    assert {g.window: g.layers for g in groups} == {0: (0,), 13: (1, 7)}
+
+
+def test_parts_are_found_by_name_and_unknown_names_fail():
+    from ullm_amd.parts import build_part, registered_parts
+    assert "toy_running_mean" in registered_parts("mixer") and "gqa_attention" in registered_parts("mixer")
+    assert registered_parts("ffn") == ["swiglu"] and registered_parts("block") == ["prenorm"]
+    with pytest.raises(KeyError, match="no mixer part named"):
+        build_part("mixer", "does_not_exist")
+    with pytest.raises(ValueError, match="needs differ"):
+        cfg = base_cfg([ATT, dict(ATT, window=5)], run_order=[[0, 0], [1, 0]])
+        from ullm_amd.models import build_model
+        build_model(cfg)[1].cache_layout()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_norm_part_and_block_wiring(dtype):
+    """The norm part alone: the pending branch is added into the 32-bit stream, then normalised."""
+    from ullm_amd.parts import PartEnv, build_part
+    env = PartEnv(torch.device(DEV), dtype, 16)
+    norm = build_part("norm", "rmsnorm", size=40, eps=1e-4, weight_name="g")
+    gain = 1 + 0.3 * torch.randn(40)
+    norm.bind({"g": gain.to(DEV)}, env)
+    res, br = torch.randn(6, 40), torch.randn(6, 40).to(dtype)
+    stream = res.clone().to(DEV)
+    y = norm.add_norm(br.to(DEV), stream, out_dtype=dtype)
+    s = res + br.float()
+    assert torch.equal(stream.cpu(), s)
+    want = plain.rms_norm(s, gain, 1e-4)
+    assert (y.float().cpu() - want).abs().max() <= tol(dtype, want)
+
+
+def test_rotary_part_table_matches_the_plain_angles():
+    from ullm_amd.parts import PartEnv, build_part
+    rot = build_part("position", "rotary", head_dim=24, theta=777.0, rotary_dim=12, pairing="half")
+    rot.bind({}, PartEnv(torch.device(DEV), torch.float32, 50))
+    table, dim, style = rot.kernel_args()
+    cos, sin = plain.rope_cos_sin(torch.arange(50), 12, 777.0)
+    assert (dim, style) == (12, 1) and table.shape == (50, 12)
+    assert torch.allclose(table.cpu(), torch.cat((cos, sin), -1), atol=1e-6)
+    with pytest.raises(ValueError):
+        build_part("position", "rotary", head_dim=24, theta=1.0, rotary_dim=13)

@@ -1,0 +1,137 @@
+"""A test-only architecture, registered from outside the framework: a stack whose layers are chosen
+one by one in the config (attention with any position encoding, window, norm and bias option, or a
+toy mixer with per-request state of fixed size), with an optional run order that names a layer
+twice or lets a layer read another layer's cache.  Beside it, its plain whole-sequence forward.
+Nothing here is a model of anyone's; it exists to show that the framework's parts, cache manager and
+step function take new parts without a change to the framework's files."""
+from typing import Dict, List
+
+import torch
+
+import plain_qwen3 as plain
+from ullm_amd.models import Choice, ModelPlan, register_architecture
+from ullm_amd.parts import Mixer, StateNeed, WeightDecl, register_part
+from ullm_amd.parts.linear import linear
+
+
+@register_part("mixer", "toy_running_mean")
+class RunningMean(Mixer):
+    """y_t = W * mean(x_0 .. x_t).  State per request: the running sum [hidden] and the count [1],
+    kept in float32; a portion continues from the state the previous portion left."""
+
+    def __init__(self, hidden_size: int, prefix: str):
+        self.hidden_size, self.prefix = hidden_size, prefix
+        self.w = None
+
+    def cache_need(self):
+        return StateNeed((self.hidden_size + 1,), torch.float32)
+
+    def weights(self):
+        return [WeightDecl(f"{self.prefix}.mean_proj.weight", (self.hidden_size, self.hidden_size))]
+
+    def bind(self, tensors, env):
+        self.w = tensors[f"{self.prefix}.mean_proj.weight"].contiguous()
+
+    def forward(self, x, ctx, cache):
+        H = self.hidden_size
+        means = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+        t = 0
+        for n, slot in zip(ctx.host["lens"], ctx.host["slots"]):
+            state = cache.state[slot]
+            sums = state[:H] + torch.cumsum(x[t:t + n].float(), dim=0)
+            counts = state[H] + torch.arange(1, n + 1, device=x.device, dtype=torch.float32)
+            means[t:t + n] = sums / counts[:, None]
+            if cache.owner:
+                state[:H] = sums[-1]
+                state[H] = counts[-1]
+            t += n
+        return linear(means.to(x.dtype), self.w)
+
+
+def toy_config_from_dict(d):
+    return dict(d)
+
+
+def toy_plan(cfg: dict) -> ModelPlan:
+    H, eps = cfg["hidden_size"], cfg["eps"]
+    layers = []
+    for i, L in enumerate(cfg["layers"]):
+        p = f"stack.{i}"
+        if L["mixer"] == "attention":
+            rope = L.get("rope", "half")
+            position = None if rope == "none" else Choice("position", "rotary", dict(
+                head_dim=L["head_dim"], theta=cfg["theta"], rotary_dim=L.get("rotary_dim", L["head_dim"]), pairing=rope))
+            mixer = Choice("mixer", "gqa_attention", dict(
+                hidden_size=H, num_heads=L["heads"], num_kv_heads=L["kv_heads"], head_dim=L["head_dim"],
+                prefix=f"{p}.attn", position=position, qk_norm_eps=eps if L.get("qk_norm", True) else None,
+                bias=L.get("bias", False), window=L.get("window", 0), scale=L.get("scale")))
+        else:
+            mixer = Choice("mixer", "toy_running_mean", dict(hidden_size=H, prefix=f"{p}.mix"))
+        norm = lambda n: Choice("norm", "rmsnorm", dict(size=H, eps=eps, weight_name=f"{p}.{n}.weight"))  # noqa: E731
+        layers.append(Choice("block", "prenorm", dict(
+            mixer_norm=norm("norm1"), mixer=mixer, ffn_norm=norm("norm2"),
+            ffn=Choice("ffn", "swiglu", dict(hidden_size=H, intermediate_size=L["ffn_size"], prefix=f"{p}.ffn")))))
+    order = [tuple(x) for x in cfg["run_order"]] if cfg.get("run_order") else None
+    return ModelPlan(vocab_size=cfg["vocab_size"], hidden_size=H, embedding_weight="tok.weight", layers=layers,
+                     final_norm=Choice("norm", "rmsnorm", dict(size=H, eps=eps, weight_name="out_norm.weight")),
+                     head_weight="head.weight", tie_head_to_embedding=cfg.get("tie", False), run_order=order,
+                     init_std=cfg.get("init_std", 0.05))
+
+
+register_architecture("ToyStackForCausalLM", toy_config_from_dict, toy_plan)
+
+
+# ---------------------------------------------------------------------------------------- plain forward
+
+def _rope(x, positions, L, theta):
+    rope = L.get("rope", "half")
+    if rope == "none":
+        return x
+    rot = L.get("rotary_dim", L["head_dim"])
+    cos, sin = plain.rope_cos_sin(positions, rot, theta)
+    r, rest = x[..., :rot], x[..., rot:]
+    if rope == "half":
+        r = plain.apply_rope_concat_layout(r, cos, sin)
+    else:
+        a, b = r[..., 0::2], r[..., 1::2]
+        c, s = cos.unsqueeze(1), sin.unsqueeze(1)
+        r = torch.stack((a * c - b * s, b * c + a * s), -1).flatten(-2)
+    return torch.cat((r, rest), -1)
+
+
+def toy_forward(w: Dict[str, torch.Tensor], cfg: dict, token_ids: List[int]) -> torch.Tensor:
+    w = {k: v.float() for k, v in w.items()}
+    T, eps = len(token_ids), cfg["eps"]
+    positions = torch.arange(T)
+    h = w["tok.weight"][torch.tensor(token_ids)]
+    order = cfg.get("run_order") or [[i, i] for i in range(len(cfg["layers"]))]
+    kv_of: Dict[int, tuple] = {}
+    for layer, cache_id in order:
+        L, p = cfg["layers"][layer], f"stack.{layer}"
+        x = plain.rms_norm(h, w[f"{p}.norm1.weight"], eps)
+        if L["mixer"] == "attention":
+            nq, nkv, d = L["heads"], L["kv_heads"], L["head_dim"]
+            b = (lambda n: w[f"{p}.attn.{n}_proj.bias"]) if L.get("bias", False) else (lambda n: None)
+            q = plain.linear(x, w[f"{p}.attn.q_proj.weight"], b("q")).view(T, nq, d)
+            if L.get("qk_norm", True):
+                q = plain.rms_norm(q, w[f"{p}.attn.q_norm.weight"], eps)
+            q = _rope(q, positions, L, cfg["theta"])
+            if cache_id not in kv_of:                     # the first layer that names a cache writes it
+                k = plain.linear(x, w[f"{p}.attn.k_proj.weight"], b("k")).view(T, nkv, d)
+                v = plain.linear(x, w[f"{p}.attn.v_proj.weight"], b("v")).view(T, nkv, d)
+                if L.get("qk_norm", True):
+                    k = plain.rms_norm(k, w[f"{p}.attn.k_norm.weight"], eps)
+                kv_of[cache_id] = (_rope(k, positions, L, cfg["theta"]), v)
+            k, v = kv_of[cache_id]
+            scale = L.get("scale") or d ** -0.5
+            o = plain.causal_gqa_attention(q, k, v, scale, L.get("window", 0))
+            a = plain.linear(o.reshape(T, nq * d), w[f"{p}.attn.o_proj.weight"])
+        else:
+            means = torch.cumsum(x, 0) / torch.arange(1, T + 1, dtype=torch.float32)[:, None]
+            a = plain.linear(means, w[f"{p}.mix.mean_proj.weight"])
+        h = h + a
+        x = plain.rms_norm(h, w[f"{p}.norm2.weight"], eps)
+        gu = torch.cat((plain.linear(x, w[f"{p}.ffn.gate_proj.weight"]), plain.linear(x, w[f"{p}.ffn.up_proj.weight"])), -1)
+        h = h + plain.linear(plain.silu_and_mul(gu), w[f"{p}.ffn.down_proj.weight"])
+    x = plain.rms_norm(h, w["out_norm.weight"], eps)
+    return plain.linear(x, w["head.weight"] if "head.weight" in w else w["tok.weight"])

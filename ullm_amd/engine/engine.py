@@ -60,6 +60,7 @@ class Engine:
                                    config.max_bs)
         self.sampler = Sampler(env.device)
         self._arrivals = 0
+        self.on_logits = None      # optional callable(scheduled that sample, float32 logits): for inspection
         logger.info("cache: %s pages of %d tokens per group, %.2f GiB", num_pages, config.page_size,
                     self.runner.cache_bytes() / 2 ** 30)
 
@@ -107,6 +108,8 @@ class Engine:
         logits = self.runner.step(entries)
         sampling = [s for s in scheduled if s.samples]
         if sampling:
+            if self.on_logits is not None:
+                self.on_logits(sampling, logits)
             ids = self.sampler.sample(logits, [s.request.params for s in sampling],
                                       [s.request.seed for s in sampling],
                                       [s.request.num_tokens for s in sampling])

@@ -33,6 +33,7 @@ class Scheduler:
         self.running: List[Request] = []              # in admission order: oldest first
         self.requests: Dict[str, Request] = {}
         self.finished_by_scheduler: List[Request] = []   # ended because the pool cannot hold more
+        self.num_preemptions = 0
 
     # ------------------------------------------------------------------ queue
     def add(self, req: Request) -> None:
@@ -107,6 +108,7 @@ class Scheduler:
         req.cache = None
         req.status = RequestStatus.WAITING
         req.num_preemptions += 1
+        self.num_preemptions += 1
         self.waiting.appendleft(req)
 
     def _finish_for_capacity(self, req: Request) -> None:
