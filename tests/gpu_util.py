@@ -14,7 +14,8 @@ def tol(dtype, ref):
 
 
 def paged_cache(seqs_k, seqs_v, page_size, dtype, device, spare_pages=3, seed=0, fill=None):
-    """seqs_k/v: list of [S_b, nkv, hd] float tensors.  Returns k_pool, v_pool [pages, nkv, P, hd] and
+    """seqs_k/v: list of [S_b, nkv, hd] float tensors.  Returns k_pool [pages, nkv, P, hd], v_pool
+    [pages, nkv, hd, P] (values are transposed inside a page) and
     block tables (list of page-id lists) with page ids shuffled; unused rows hold ``fill`` (NaN by
     default so that any read of them shows)."""
     nkv, hd = seqs_k[0].shape[1:]
@@ -23,7 +24,7 @@ def paged_cache(seqs_k, seqs_v, page_size, dtype, device, spare_pages=3, seed=0,
     random.Random(seed).shuffle(ids)
     fillv = float("nan") if fill is None else fill
     k_pool = torch.full((n_pages, nkv, page_size, hd), fillv, dtype=torch.float32)
-    v_pool = torch.full((n_pages, nkv, page_size, hd), fillv, dtype=torch.float32)
+    v_pool = torch.full((n_pages, nkv, hd, page_size), fillv, dtype=torch.float32)
     tables = []
     for k, v in zip(seqs_k, seqs_v):
         table = []
@@ -32,7 +33,7 @@ def paged_cache(seqs_k, seqs_v, page_size, dtype, device, spare_pages=3, seed=0,
             table.append(page)
             rows = k[i * page_size:(i + 1) * page_size]
             k_pool[page, :, :rows.shape[0]] = rows.transpose(0, 1)
-            v_pool[page, :, :rows.shape[0]] = v[i * page_size:(i + 1) * page_size].transpose(0, 1)
+            v_pool[page, :, :, :rows.shape[0]] = v[i * page_size:(i + 1) * page_size].permute(1, 2, 0)
         tables.append(table)
     return k_pool.to(device, dtype), v_pool.to(device, dtype), tables
 

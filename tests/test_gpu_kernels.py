@@ -100,7 +100,7 @@ def test_qk_norm_rope_write(ops, dtype, cfg):
     qkv = torch.randn(T, (nq + 2 * nkv) * hd).to(dtype)
     qg, kg = 1 + 0.2 * torch.randn(hd), 1 + 0.2 * torch.randn(hd)
     k_pool = torch.zeros(n_pages, nkv, P, hd, dtype=dtype, device=DEV)
-    v_pool = torch.zeros_like(k_pool)
+    v_pool = torch.zeros(n_pages, nkv, hd, P, dtype=dtype, device=DEV)
     q_out = torch.empty(T, nq * hd, dtype=dtype, device=DEV)
     table = None
     if style:
@@ -132,7 +132,7 @@ def test_qk_norm_rope_write(ops, dtype, cfg):
         pos, e = int(positions[t]), int(entry[t])
         page, row = tables[e][pos // P], pos % P
         assert (k_pool[page, :, row].float().cpu() - k[t]).abs().max() <= tol(dtype, k)
-        assert torch.equal(v_pool[page, :, row].float().cpu(), v[t])
+        assert torch.equal(v_pool[page, :, :, row].float().cpu(), v[t])
     written = sum(1 for _ in range(T))
     assert int((k_pool.float().abs().sum(-1) > 0).sum()) == written * nkv       # nothing else was touched
 
@@ -252,3 +252,93 @@ def test_sampler_kernel_against_the_plain_sampler(ops):
     got = sampler.sample(rows, [SamplingParams(temperature=1.0)] * n, [99] * n, list(range(n)))
     counts = torch.bincount(torch.tensor(got), minlength=5).float()
     assert float(((counts - n * probs) ** 2 / (n * probs)).sum()) < 25.0
+
+
+MFMA_CASES = [dict(nq=8, nkv=2, hd=32, P=16, lens=[(1, 1), (1, 37), (1, 300), (1, 64)], window=0),
+              dict(nq=32, nkv=8, hd=128, P=16, lens=[(1, 1153), (1, 31), (1, 32), (1, 33)], window=0),
+              dict(nq=8, nkv=1, hd=64, P=32, lens=[(1, 500), (1, 97)], window=0),
+              dict(nq=40, nkv=2, hd=64, P=16, lens=[(1, 130), (1, 17)], window=0),          # 20 heads per kv head
+              dict(nq=4, nkv=4, hd=96, P=64, lens=[(1, 200), (1, 64)], window=0),
+              dict(nq=6, nkv=2, hd=256, P=16, lens=[(1, 77)], window=0),
+              dict(nq=8, nkv=2, hd=64, P=16, lens=[(1, 300), (1, 40), (1, 9)], window=50),
+              dict(nq=8, nkv=2, hd=32, P=16, lens=[(5, 5), (33, 70), (16, 16), (2, 130), (17, 49)], window=0),
+              dict(nq=32, nkv=8, hd=128, P=16, lens=[(100, 100), (7, 260)], window=0),
+              dict(nq=6, nkv=2, hd=64, P=32, lens=[(40, 90), (3, 3)], window=21),
+              dict(nq=8, nkv=2, hd=32, P=16, lens=[(1, 45), (9, 40), (1, 200), (20, 20), (1, 1)], window=0),  # mixed
+              dict(nq=8, nkv=2, hd=32, P=16, lens=[(1, 45), (9, 40), (1, 200), (20, 50)], window=13)]
+
+
+@pytest.mark.parametrize("case", MFMA_CASES)
+def test_attention_on_the_matrix_cores(ops, case):
+    """Decoded tokens (split over the keys and reduced), prompt portions, and both in one batch."""
+    torch.manual_seed(8)
+    dtype = torch.bfloat16
+    nq, nkv, hd, P, window = (case[k] for k in ("nq", "nkv", "hd", "P", "window"))
+    assert ops.attention_mfma_supports(dtype, hd, P, nq, nkv)
+    rnd = lambda *s: torch.randn(*s).to(dtype).float()   # noqa: E731
+    ks = [rnd(S, nkv, hd) for _, S in case["lens"]]
+    vs = [rnd(S, nkv, hd) for _, S in case["lens"]]
+    qs = [rnd(n, nq, hd) for n, _ in case["lens"]]
+    k_pool, v_pool, tables = paged_cache(ks, vs, P, dtype, DEV)          # unused rows are NaN
+    positions = torch.cat([torch.arange(S - n, S) for n, S in case["lens"]]).int().to(DEV)
+    entry = torch.cat([torch.full((n,), b) for b, (n, _) in enumerate(case["lens"])]).int().to(DEV)
+    q = torch.cat(qs).reshape(-1, nq * hd).to(DEV, dtype)
+    scale = hd ** -0.5
+    want = reference_attention(qs, ks, vs, scale, window).reshape(-1, nq * hd)
+    bt = table_tensor(tables, DEV)
+    dec, tiles, t0, max_kv = [], [], 0, 0
+    for n, S in case["lens"]:
+        if n == 1:
+            dec.append(t0)
+            max_kv = max(max_kv, S)
+        else:
+            for f in range(0, n, 16):
+                tiles += [t0 + f, min(16, n - f)]
+        t0 += n
+    for chunk in (None, 32, 64, 4096):
+        out = torch.full((q.shape[0], nq * hd), float("nan"), dtype=dtype, device=DEV)
+        if dec:
+            ops.attention_decode_mfma(q, out, k_pool, v_pool, torch.tensor(dec, dtype=torch.int32, device=DEV),
+                                      len(dec), positions, entry, bt, P, nq, nkv, hd, scale, window, max_kv, chunk=chunk)
+        if tiles:
+            ops.attention_prefill_mfma(q, out, k_pool, v_pool, torch.tensor(tiles, dtype=torch.int32, device=DEV),
+                                       len(tiles) // 2, positions, entry, bt, P, nq, nkv, hd, scale, window)
+        assert not torch.isnan(out).any()
+        assert (out.float().cpu() - want).abs().max() <= tol(dtype, want), chunk
+        if not dec:
+            break
+
+
+def test_matrix_core_attention_finds_one_far_key_at_every_edge(ops):
+    torch.manual_seed(9)
+    dtype = torch.bfloat16
+    nq, nkv, hd, P, S = 8, 2, 64, 16, 403
+    for window in (0, 70):
+        lo = 0 if window == 0 else S - window
+        targets = sorted(t for t in {lo, lo + 1, (lo // P + 1) * P - 1, (lo // P + 1) * P, 31, 32, 255, 256, 383, 384,
+                                     S - 2, S - 1} if t >= lo)
+        for target in targets:
+            for n in (1, 5):
+                k = torch.randn(S, nkv, hd) * 0.1
+                v = torch.randn(S, nkv, hd).to(dtype).float()
+                q = torch.randn(n, nq, hd) * 0.1
+                direction = torch.randn(hd)
+                direction /= direction.norm()
+                k[target] = 30.0 * direction
+                q[-1] = 30.0 * direction
+                k, q = k.to(dtype).float(), q.to(dtype).float()
+                k_pool, v_pool, tables = paged_cache([k], [v], P, dtype, DEV, seed=target)
+                positions = torch.arange(S - n, S).int().to(DEV)
+                entry = torch.zeros(n, dtype=torch.int32, device=DEV)
+                qd = q.reshape(n, -1).to(DEV, dtype)
+                out = torch.zeros(n, nq * hd, dtype=dtype, device=DEV)
+                bt = table_tensor(tables, DEV)
+                if n == 1:
+                    ops.attention_decode_mfma(qd, out, k_pool, v_pool, None, 1, positions, entry, bt, P, nq, nkv, hd,
+                                              1.0, window, S, chunk=64)
+                else:
+                    ops.attention_prefill_mfma(qd, out, k_pool, v_pool, torch.tensor([0, n], dtype=torch.int32, device=DEV),
+                                               1, positions, entry, bt, P, nq, nkv, hd, 1.0, window)
+                got = out.float().cpu().view(n, nq, hd)[-1]
+                for h in range(nq):
+                    assert (got[h] - v[target, h // 4]).abs().max() < 3e-2, (window, target, n, h)

@@ -3,6 +3,7 @@
 // One block per (token, query head); keys are visited in tiles of the block size in a fixed order
 // that depends only on the token's own position, so the result for a token is the same however
 // the batch was cut.  Scores, running maximum, sum and output are 32-bit.
+// Pools: keys [page, kv_head, row, head_dim]; values [page, kv_head, head_dim, row].
 //
 // Semantics as the reference asks of its attention library (ullm/layers/attention.py:76-104,
 // 298-309): scale = given (head_dim^-0.5, ullm/models/qwen3.py:81), causal with the queries at the
@@ -73,7 +74,7 @@ paged_attention_generic_kernel(const T* __restrict__ q, int q_stride, T* __restr
         float a = acc[r] * alpha;
         for (int jj = 0; jj < n_tile; ++jj) {
           const long long vr = row_s[jj];
-          if (vr >= 0) a += p_s[jj] * ld_f32(v_pool + vr * hd + d);
+          if (vr >= 0) a += p_s[jj] * ld_f32(v_pool + (vr / page_size) * page_size * hd + (size_t)d * page_size + vr % page_size);
         }
         acc[r] = a;
       }

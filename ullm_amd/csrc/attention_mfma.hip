@@ -1,0 +1,334 @@
+// Paged grouped-query attention on the matrix cores (bfloat16 operands, 32-bit accumulation),
+// for decoded tokens (split over the keys, then reduced) and for prompt portions.
+//
+// One wave owns 16 "columns": in decode mode the query heads of one token that share a kv head,
+// in prompt mode 16 consecutive tokens of one request for one query head.  Per 32 keys it computes
+//   S^T[key, col]   = K[key, :] . Q[col, :]        (v_mfma_f32_16x16x32_bf16: A = K rows, B = Q columns)
+//   O^T[dim, col]  += V^T[dim, key] * P^T[key, col] (A = values, transposed inside the page, B = P)
+// In the 16x16 result layout a lane holds 4 keys of one column, so the probabilities a lane has are
+// exactly the ones it must feed as the B operand of the second product: nothing moves between lanes.
+// Both operands of both products are plain 8- or 16-byte loads from the paged cache:
+//   keys   [page, kv_head, row, head_dim],  values [page, kv_head, head_dim, row].
+// Softmax state (maximum, sum) is 32-bit and per column; the scale and log2(e) are folded into one
+// multiply so that the exponential is a single v_exp_f32.
+//
+// Semantics as in the general kernel: causal with the queries at the end of the keys, optional
+// window, query head h reads kv head h / (nq / nkv) (ullm/layers/attention.py:76-104,271,298-309).
+#include "common.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+
+#define NEG_BIG (-1.0e30f)
+
+union Pack8 {
+  bf16x8_t v;
+  uint4 u4;
+  uint2 u2[2];
+  bf16_t h[8];
+};
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// The work of one wave.  NQK = head_dim / 32.
+//   col_q      : pointer to this lane's column's query row (null if the column is padding)
+//   col_lo/hi  : first and last key the column may see (hi < lo for padding)
+//   key_begin/key_end : the wave's key range [begin, end), begin a multiple of 32
+//   max_hi     : largest key position that holds written data for this request
+// Results: acc[n][r] = O^T[16n + 4g + r][col] (unnormalised), m (log2 domain), l (this lane's share
+// of the sum; the four lanes of a column add up to the column's sum).
+template <int NQK>
+__device__ __forceinline__ void attend_range(
+    const bf16_t* __restrict__ col_q, int col_lo, int col_hi, int key_begin, int key_end, int max_hi,
+    const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool, const int* __restrict__ bt,
+    int page_size, int nkv, int kvh, float scale_log2e, f32x4_t (&acc)[2 * NQK], float& m, float& l) {
+  constexpr int HD = 32 * NQK;
+  const int lane = threadIdx.x & 63, g = lane >> 4, c = lane & 15;
+  Pack8 qreg[NQK];
+#pragma unroll
+  for (int ch = 0; ch < NQK; ++ch) {
+    if (col_q) qreg[ch].u4 = *reinterpret_cast<const uint4*>(col_q + 32 * ch + 8 * g);
+    else qreg[ch].u4 = make_uint4(0, 0, 0, 0);
+  }
+#pragma unroll
+  for (int n = 0; n < 2 * NQK; ++n) acc[n] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  m = NEG_BIG;
+  l = 0.f;
+
+  for (int key0 = key_begin; key0 < key_end; key0 += 32) {
+    // the two 16-key halves of the tile; each lies inside one page (page_size is a multiple of 16)
+    int page[2], off[2];
+#pragma unroll
+    for (int sb = 0; sb < 2; ++sb) {
+      const int kb = key0 + 16 * sb;
+      page[sb] = kb < key_end ? bt[kb / page_size] : -1;
+      off[sb] = kb % page_size;
+    }
+    f32x4_t s[2];
+#pragma unroll
+    for (int sb = 0; sb < 2; ++sb) {
+      s[sb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      if (page[sb] >= 0) {
+        const bf16_t* kp = k_pool + (((size_t)page[sb] * nkv + kvh) * page_size + off[sb] + c) * HD + 8 * g;
+#pragma unroll
+        for (int ch = 0; ch < NQK; ++ch) {
+          Pack8 a;
+          a.u4 = *reinterpret_cast<const uint4*>(kp + 32 * ch);
+          s[sb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, qreg[ch].v, s[sb], 0, 0, 0);
+        }
+      }
+    }
+    // scores of keys key0 + 16 sb + 4 g + r for column c; mask, running maximum
+    float tile_max = NEG_BIG;
+#pragma unroll
+    for (int sb = 0; sb < 2; ++sb)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int kk = key0 + 16 * sb + 4 * g + r;
+        const bool ok = page[sb] >= 0 && kk >= col_lo && kk <= col_hi;
+        const float v = ok ? s[sb][r] * scale_log2e : NEG_BIG;
+        s[sb][r] = v;
+        tile_max = fmaxf(tile_max, v);
+      }
+    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, 64));
+    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, 64));
+    const float m_new = fmaxf(m, tile_max);
+    const float alpha = fast_exp2(m - m_new);
+    Pack8 p;
+    float psum = 0.f;
+#pragma unroll
+    for (int sb = 0; sb < 2; ++sb)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        // a masked score stays at NEG_BIG: its weight is zero even while m_new is still NEG_BIG
+        const float e = s[sb][r] > 0.5f * NEG_BIG ? fast_exp2(s[sb][r] - m_new) : 0.f;
+        psum += e;
+        p.h[4 * sb + r] = f32_to_bf16_bits(e);
+      }
+    l = l * alpha + psum;
+    m = m_new;
+    // values: lane (c, g) feeds V^T[dim 16n + c][keys key0 + 16 sb + 4g .. +4]
+    const bool edge = key0 + 32 > max_hi + 1;     // some keys of the tile hold no written data
+#pragma unroll
+    for (int n = 0; n < 2 * NQK; ++n) {
+      Pack8 a;
+#pragma unroll
+      for (int sb = 0; sb < 2; ++sb) {
+        if (page[sb] >= 0) {
+          const bf16_t* vp = v_pool + (((size_t)page[sb] * nkv + kvh) * HD + 16 * n + c) * page_size + off[sb] + 4 * g;
+          a.u2[sb] = *reinterpret_cast<const uint2*>(vp);
+        } else {
+          a.u2[sb] = make_uint2(0, 0);
+        }
+      }
+      if (edge) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          if (key0 + 16 * (j >> 2) + 4 * g + (j & 3) > max_hi) a.h[j] = 0;
+      }
+      f32x4_t o = acc[n];
+      o[0] *= alpha; o[1] *= alpha; o[2] *= alpha; o[3] *= alpha;
+      acc[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, p.v, o, 0, 0, 0);
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------- decode
+// grid (ceil(splits / 4), nkv * col_groups, n_tokens), block 256: wave w of block x works on split
+// 4 x + w of the token's keys: [split * chunk, (split + 1) * chunk) cut to [lo, pos].
+// With one split the result is final; otherwise (O, m, l) go to the workspace for the reduce kernel.
+template <int NQK>
+__global__ void __launch_bounds__(256)
+attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
+                        const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
+                        const int* __restrict__ token_list, const int* __restrict__ positions,
+                        const int* __restrict__ token_entry, const int* __restrict__ block_table,
+                        int bt_stride, int page_size, int nq, int nkv, float scale_log2e, int window,
+                        int chunk, int num_splits, float* __restrict__ part_o, float* __restrict__ part_ml) {
+  constexpr int HD = 32 * NQK;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, g = lane >> 4, c = lane & 15;
+  const int split = blockIdx.x * 4 + wave;
+  if (split >= num_splits) return;
+  const int G = nq / nkv;
+  const int groups = (G + 15) / 16;
+  const int kvh = blockIdx.y / groups, cg = blockIdx.y % groups;
+  const int item = blockIdx.z;
+  const int t = token_list ? token_list[item] : item;
+  const int pos = positions[t];
+  const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  int begin = split * chunk, end = begin + chunk;
+  if (end > pos + 1) end = pos + 1;
+  if (begin < (lo & ~31)) begin = lo & ~31;
+  const int head_in_group = cg * 16 + c;
+  const bool col_ok = head_in_group < G;
+  const int head = kvh * G + head_in_group;
+  const bool empty = begin >= end;
+  f32x4_t acc[2 * NQK];
+  float m = NEG_BIG, l = 0.f;
+  if (!empty) {
+    attend_range<NQK>(col_ok ? q + (size_t)t * q_stride + (size_t)head * HD : nullptr, lo, col_ok ? pos : -1,
+                      begin, end, pos, k_pool, v_pool, block_table + (size_t)token_entry[t] * bt_stride,
+                      page_size, nkv, kvh, scale_log2e, acc, m, l);
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+  } else {
+#pragma unroll
+    for (int n = 0; n < 2 * NQK; ++n) acc[n] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  }
+  if (!col_ok) return;
+  if (num_splits == 1) {
+    const float inv = l > 0.f ? 1.f / l : 0.f;
+    bf16_t* op = out + (size_t)t * out_stride + (size_t)head * HD;
+#pragma unroll
+    for (int n = 0; n < 2 * NQK; ++n) {
+      uint2 w;
+      w.x = (uint32_t)f32_to_bf16_bits(acc[n][0] * inv) | ((uint32_t)f32_to_bf16_bits(acc[n][1] * inv) << 16);
+      w.y = (uint32_t)f32_to_bf16_bits(acc[n][2] * inv) | ((uint32_t)f32_to_bf16_bits(acc[n][3] * inv) << 16);
+      *reinterpret_cast<uint2*>(op + 16 * n + 4 * g) = w;
+    }
+  } else {
+    const size_t slot = ((size_t)item * nq + head) * num_splits + split;
+    float* po = part_o + slot * HD;
+#pragma unroll
+    for (int n = 0; n < 2 * NQK; ++n)
+      *reinterpret_cast<float4*>(po + 16 * n + 4 * g) = make_float4(acc[n][0], acc[n][1], acc[n][2], acc[n][3]);
+    if (g == 0) {
+      part_ml[slot * 2] = m;
+      part_ml[slot * 2 + 1] = l;
+    }
+  }
+}
+
+// Combine the splits of one (token, head): out = sum_s O_s 2^(m_s - M) / sum_s l_s 2^(m_s - M).
+__global__ void __launch_bounds__(64)
+attention_reduce_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                        bf16_t* __restrict__ out, int out_stride, const int* __restrict__ token_list,
+                        int nq, int hd, int num_splits) {
+  const int item = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+  const int t = token_list ? token_list[item] : item;
+  const size_t base = ((size_t)item * nq + head) * num_splits;
+  float M = NEG_BIG;
+  for (int s = 0; s < num_splits; ++s) M = fmaxf(M, part_ml[(base + s) * 2]);
+  float L = 0.f;
+  for (int s = 0; s < num_splits; ++s) L += part_ml[(base + s) * 2 + 1] * fast_exp2(part_ml[(base + s) * 2] - M);
+  const float inv = L > 0.f ? 1.f / L : 0.f;
+  for (int d = lane; d < hd; d += 64) {
+    float o = 0.f;
+    for (int s = 0; s < num_splits; ++s)
+      o += part_o[(base + s) * hd + d] * fast_exp2(part_ml[(base + s) * 2] - M);
+    out[(size_t)t * out_stride + (size_t)head * hd + d] = f32_to_bf16_bits(o * inv);
+  }
+}
+
+// ------------------------------------------------------------------------------- prompt portions
+// grid (n_tiles, nkv * ceil(G / waves)), block 64 * waves with waves = min(G, 4): one wave per query
+// head, the waves of a block share a kv head (and so the cache lines they read); tile = (first
+// token, number of tokens <= 16) of one request; every wave walks all keys its tokens see.
+template <int NQK>
+__global__ void __launch_bounds__(256)
+attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
+                         const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
+                         const int* __restrict__ tiles, const int* __restrict__ positions,
+                         const int* __restrict__ token_entry, const int* __restrict__ block_table,
+                         int bt_stride, int page_size, int nq, int nkv, float scale_log2e, int window) {
+  constexpr int HD = 32 * NQK;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, g = lane >> 4, c = lane & 15;
+  const int G = nq / nkv;
+  const int waves = blockDim.x >> 6, hgroups = (G + waves - 1) / waves;
+  const int kvh = blockIdx.y / hgroups;
+  const int head_in_group = (blockIdx.y % hgroups) * waves + wave;
+  if (head_in_group >= G) return;
+  const int head = kvh * G + head_in_group;
+  const int first = tiles[2 * blockIdx.x], count = tiles[2 * blockIdx.x + 1];
+  const bool col_ok = c < count;
+  const int t = first + (col_ok ? c : 0);
+  const int pos = positions[t];
+  const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int last_pos = positions[first + count - 1];
+  const int first_pos = positions[first];
+  const int tile_lo = (window > 0 && first_pos - window + 1 > 0) ? first_pos - window + 1 : 0;
+  f32x4_t acc[2 * NQK];
+  float m, l;
+  attend_range<NQK>(col_ok ? q + (size_t)t * q_stride + (size_t)head * HD : nullptr, lo, col_ok ? pos : -1,
+                    tile_lo & ~31, last_pos + 1, last_pos, k_pool, v_pool,
+                    block_table + (size_t)token_entry[first] * bt_stride, page_size, nkv, kvh, scale_log2e,
+                    acc, m, l);
+  l += __shfl_xor(l, 16, 64);
+  l += __shfl_xor(l, 32, 64);
+  if (!col_ok) return;
+  const float inv = l > 0.f ? 1.f / l : 0.f;
+  bf16_t* op = out + (size_t)t * out_stride + (size_t)head * HD;
+#pragma unroll
+  for (int n = 0; n < 2 * NQK; ++n) {
+    uint2 w;
+    w.x = (uint32_t)f32_to_bf16_bits(acc[n][0] * inv) | ((uint32_t)f32_to_bf16_bits(acc[n][1] * inv) << 16);
+    w.y = (uint32_t)f32_to_bf16_bits(acc[n][2] * inv) | ((uint32_t)f32_to_bf16_bits(acc[n][3] * inv) << 16);
+    *reinterpret_cast<uint2*>(op + 16 * n + 4 * g) = w;
+  }
+}
+
+static bool supported_hd(int hd) { return hd == 32 || hd == 64 || hd == 96 || hd == 128 || hd == 256; }
+
+#define DISPATCH_NQK(hd, CALL)            \
+  switch ((hd) / 32) {                    \
+    case 1: { CALL(1); break; }           \
+    case 2: { CALL(2); break; }           \
+    case 3: { CALL(3); break; }           \
+    case 4: { CALL(4); break; }           \
+    case 8: { CALL(8); break; }           \
+    default: return ULLM_ERR_UNSUPPORTED; \
+  }
+
+// 1 if this family takes the shape (bfloat16 only), else 0.
+extern "C" int ullm_attention_mfma_supports(int hd, int page_size, int nq, int nkv) {
+  return supported_hd(hd) && page_size > 0 && page_size % 16 == 0 && nkv > 0 && nq % nkv == 0;
+}
+
+// Workspace floats needed for `n_items` tokens split `num_splits` ways.
+extern "C" long long ullm_attention_decode_workspace(int n_items, int nq, int hd, int num_splits) {
+  return num_splits <= 1 ? 0 : (long long)n_items * nq * num_splits * (hd + 2);
+}
+
+extern "C" int ullm_attention_decode(
+    const void* q, int q_stride, void* out, int out_stride, const void* k_pool, const void* v_pool,
+    const int* token_list, int n_items, const int* positions, const int* token_entry,
+    const int* block_table, int bt_stride, int page_size, int nq, int nkv, int hd, float scale, int window,
+    int chunk, int num_splits, float* workspace, hipStream_t stream) {
+  if (n_items <= 0) return 0;
+  if (!ullm_attention_mfma_supports(hd, page_size, nq, nkv)) return ULLM_ERR_UNSUPPORTED;
+  if (chunk <= 0 || chunk % 32 != 0 || num_splits < 1 || window < 0) return ULLM_ERR_SHAPE;
+  if (num_splits > 1 && !workspace) return ULLM_ERR_SHAPE;
+  const int G = nq / nkv, groups = (G + 15) / 16;
+  float* part_o = workspace;
+  float* part_ml = workspace ? workspace + (size_t)n_items * nq * num_splits * hd : nullptr;
+  const float sl = scale * 1.4426950408889634f;
+  dim3 grid((num_splits + 3) / 4, nkv * groups, n_items), block(256);
+#define CALL(N) hipLaunchKernelGGL(attention_decode_kernel<N>, grid, block, 0, stream, (const bf16_t*)q, q_stride, \
+    (bf16_t*)out, out_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool, token_list, positions, token_entry, \
+    block_table, bt_stride, page_size, nq, nkv, sl, window, chunk, num_splits, part_o, part_ml)
+  DISPATCH_NQK(hd, CALL)
+#undef CALL
+  int rc = (int)hipGetLastError();
+  if (rc != 0 || num_splits == 1) return rc;
+  hipLaunchKernelGGL(attention_reduce_kernel, dim3(n_items, nq), dim3(64), 0, stream, part_o, part_ml,
+                     (bf16_t*)out, out_stride, token_list, nq, hd, num_splits);
+  ULLM_LAUNCH_CHECK();
+}
+
+extern "C" int ullm_attention_prefill(
+    const void* q, int q_stride, void* out, int out_stride, const void* k_pool, const void* v_pool,
+    const int* tiles, int n_tiles, const int* positions, const int* token_entry, const int* block_table,
+    int bt_stride, int page_size, int nq, int nkv, int hd, float scale, int window, hipStream_t stream) {
+  if (n_tiles <= 0) return 0;
+  if (!ullm_attention_mfma_supports(hd, page_size, nq, nkv)) return ULLM_ERR_UNSUPPORTED;
+  if (window < 0) return ULLM_ERR_SHAPE;
+  const int G = nq / nkv, waves = G < 4 ? G : 4, hgroups = (G + waves - 1) / waves;
+  const float sl = scale * 1.4426950408889634f;
+  dim3 grid(n_tiles, nkv * hgroups), block(64 * waves);
+#define CALL(N) hipLaunchKernelGGL(attention_prefill_kernel<N>, grid, block, 0, stream, (const bf16_t*)q, q_stride, \
+    (bf16_t*)out, out_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool, tiles, positions, token_entry, \
+    block_table, bt_stride, page_size, nq, nkv, sl, window)
+  DISPATCH_NQK(hd, CALL)
+#undef CALL
+  ULLM_LAUNCH_CHECK();
+}

@@ -122,8 +122,10 @@ extern "C" int ullm_silu_mul(const void* gu, void* out, int T_, int I, int dtype
 // Rotation: pair (i, i + rot/2) for style 1 (half split), (2i, 2i+1) for style 2, i < rot/2;
 //   o_a = a cos - b sin, o_b = b cos + a sin with cos/sin = table[pos, i], table[pos, rot/2 + i];
 //   dims >= rot pass through.  style 0: no rotation.
-// Cache page of token t: block_table[entry[t], pos / page_size], row pos % page_size;
-// pool layout [page, kv_head, row, head_dim].  Tokens whose page id is negative are not written.
+// Cache page of token t: block_table[entry[t], pos / page_size], row pos % page_size.
+// Key pool layout [page, kv_head, row, head_dim]; value pool layout [page, kv_head, head_dim, row]
+// (values are kept transposed inside a page so that the attention kernels can load eight keys of
+// one dimension as one vector).  Tokens whose page id is negative are not written.
 #define MAX_HEAD_DIM 512
 template <typename T>
 __global__ void qk_norm_rope_write_kernel(
@@ -146,12 +148,12 @@ __global__ void qk_norm_rope_write_kernel(
     const int kvh = is_k ? head - nq : head - nq - nkv;
     const int page = block_table[(size_t)token_entry[t] * bt_stride + pos / page_size];
     if (page < 0) return;
-    T* pool = is_k ? k_pool : v_pool;
-    dst = pool + (((size_t)page * nkv + kvh) * page_size + (pos % page_size)) * hd;
-  }
-  if (!is_q && !is_k) {  // v: plain copy
-    for (int i = lane; i < hd; i += WAVE) dst[i] = src[i];
-    return;
+    if (!is_k) {  // v: transposed copy
+      T* vdst = v_pool + ((size_t)page * nkv + kvh) * hd * page_size + (pos % page_size);
+      for (int i = lane; i < hd; i += WAVE) vdst[(size_t)i * page_size] = src[i];
+      return;
+    }
+    dst = k_pool + (((size_t)page * nkv + kvh) * page_size + (pos % page_size)) * hd;
   }
   const float* gain = is_q ? q_gain : k_gain;
   float ss = 0.f;

@@ -32,6 +32,9 @@ class StepError(RuntimeError):
     pass
 
 
+Q_TILE = 16     # tokens of one request that the prompt-portion attention kernel handles per wave
+
+
 class ModelRunner:
     def __init__(self, model: Model, env: PartEnv, page_size: int, num_pages, max_requests: int,
                  enable_prefix_cache: bool = False):
@@ -48,12 +51,13 @@ class ModelRunner:
         self.max_table = -(-env.context_len // page_size)
         self.caches: Dict[int, LayerCache] = {}
         for g, spec in enumerate(groups):
-            shape = (num_pages[g], spec.num_kv_heads, page_size, spec.head_dim)
+            k_shape = (num_pages[g], spec.num_kv_heads, page_size, spec.head_dim)
+            v_shape = (num_pages[g], spec.num_kv_heads, spec.head_dim, page_size)   # transposed inside a page
             for cache_id in spec.layers:
                 # zeroed once so that no row ever holds a non-finite bit pattern before it is written
                 self.caches[cache_id] = LayerCache(
-                    group=g, k_pool=torch.zeros(shape, dtype=env.dtype, device=env.device),
-                    v_pool=torch.zeros(shape, dtype=env.dtype, device=env.device))
+                    group=g, k_pool=torch.zeros(k_shape, dtype=env.dtype, device=env.device),
+                    v_pool=torch.zeros(v_shape, dtype=env.dtype, device=env.device))
         for cache_id, need in states.items():
             self.caches[cache_id] = LayerCache(
                 state=torch.zeros((max_requests,) + tuple(need.shape), dtype=need.dtype, device=env.device))
@@ -105,8 +109,18 @@ class ModelRunner:
         for g in range(len(groups)):
             strides.append(max(1, max(len(e.cache.tables[g]) for e in entries)))
         n_want = sum(len(e.want) for e in entries)
+        # attention work lists: tokens of one-token entries; tiles of <= 16 tokens of longer entries
+        dec_list, tile_list, max_dec_kv, t0 = [], [], 0, 0
+        for e, n in zip(entries, lens):
+            if n == 1:
+                dec_list.append(t0)
+                max_dec_kv = max(max_dec_kv, e.cache.num_computed + 1)
+            else:
+                for first in range(0, n, Q_TILE):
+                    tile_list.extend((t0 + first, min(Q_TILE, n - first)))
+            t0 += n
         # layout of the packed int32 buffer
-        sizes = [T, T, T, B + 1, B, B, n_want] + [B * s for s in strides]
+        sizes = [T, T, T, B + 1, B, B, n_want] + [B * s for s in strides] + [len(dec_list), len(tile_list)]
         offs = np.concatenate(([0], np.cumsum(sizes)))
         host = np.empty(int(offs[-1]), dtype=np.int32)
         ids, pos, ent = host[offs[0]:offs[1]], host[offs[1]:offs[2]], host[offs[2]:offs[3]]
@@ -154,6 +168,9 @@ class ModelRunner:
             for b, e in enumerate(entries):
                 tab = e.cache.tables[g]
                 bt[b, :len(tab)] = tab
+        ng = len(groups)
+        host[offs[7 + ng]:offs[8 + ng]] = dec_list
+        host[offs[8 + ng]:offs[9 + ng]] = tile_list
         dev = self._upload(host)
         view = lambda i: dev[int(offs[i]):int(offs[i + 1])]  # noqa: E731
         gviews = [GroupView(view(7 + g).view(B, strides[g]), strides[g], P, groups[g].window)
@@ -163,6 +180,9 @@ class ModelRunner:
             q_start=view(3), entry_slot=view(4), entry_start=view(5), groups=gviews,
             max_q_len=max(lens), max_kv_len=max_kv, decode_only=all(n == 1 for n in lens),
             dtype=self.env.dtype,
+            decode_tokens=view(7 + ng) if (dec_list and len(dec_list) < T) else None, num_decode=len(dec_list),
+            max_decode_kv=max_dec_kv, tiles=view(8 + ng).view(-1, 2) if tile_list else None,
+            num_tiles=len(tile_list) // 2,
             host={"lens": lens, "starts": [e.cache.num_computed for e in entries],
                   "slots": [e.cache.slot for e in entries]})
         return ctx, (view(6) if n_want else None)

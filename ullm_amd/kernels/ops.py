@@ -58,6 +58,16 @@ def _i32(t: torch.Tensor, name: str, n: Optional[int] = None) -> None:
 _c_int, _c_float = ctypes.c_int, ctypes.c_float
 
 
+def _check_pools(k_pool, v_pool, nkv: int, page_size: int, hd: int, dtype) -> None:
+    """Keys are [pages, nkv, page_size, hd]; values are kept transposed inside a page: [pages, nkv, hd, page_size]."""
+    _need(k_pool is not None and k_pool.dim() == 4 and tuple(k_pool.shape[1:]) == (nkv, page_size, hd)
+          and k_pool.is_contiguous() and k_pool.dtype == dtype,
+          f"k_pool must be contiguous [pages, {nkv}, {page_size}, {hd}] of {dtype}")
+    _need(v_pool is not None and v_pool.dim() == 4 and tuple(v_pool.shape[1:]) == (nkv, hd, page_size)
+          and v_pool.is_contiguous() and v_pool.dtype == dtype and v_pool.shape[0] == k_pool.shape[0],
+          f"v_pool must be contiguous [pages, {nkv}, {hd}, {page_size}] of {dtype}")
+
+
 # ---------------------------------------------------------------------------------- elementwise
 
 def embedding(ids: torch.Tensor, table: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -121,7 +131,8 @@ def qk_norm_rope_write(qkv: torch.Tensor, q_out: torch.Tensor, q_gain: Optional[
                        block_table: torch.Tensor, k_pool: Optional[torch.Tensor], v_pool: Optional[torch.Tensor],
                        page_size: int, nq: int, nkv: int, hd: int, write_kv: bool) -> None:
     """Per-head norm and rotation of q (to ``q_out`` [T, nq*hd]) and k, and the cache write of k and v.
-    ``qkv`` is [T, (nq + 2 nkv) * hd]; pools are [pages, nkv, page_size, hd]; ``block_table`` is
+    ``qkv`` is [T, (nq + 2 nkv) * hd]; key pool [pages, nkv, page_size, hd], value pool
+    [pages, nkv, hd, page_size]; ``block_table`` is
     int32 [B, stride] with one row per batch entry."""
     T = qkv.shape[0]
     _need(qkv.dim() == 2 and qkv.shape[1] == (nq + 2 * nkv) * hd and qkv.stride(1) == 1, "bad qkv shape")
@@ -141,10 +152,7 @@ def qk_norm_rope_write(qkv: torch.Tensor, q_out: torch.Tensor, q_gain: Optional[
               "cos_sin must be float32 [positions, rotary_dim]")
         table_rows = cos_sin.shape[0]
     if write_kv:
-        for pool, nm in ((k_pool, "k_pool"), (v_pool, "v_pool")):
-            _need(pool is not None and pool.dim() == 4 and tuple(pool.shape[1:]) == (nkv, page_size, hd)
-                  and pool.is_contiguous() and pool.dtype == qkv.dtype,
-                  f"{nm} must be contiguous [pages, {nkv}, {page_size}, {hd}] of {qkv.dtype}")
+        _check_pools(k_pool, v_pool, nkv, page_size, hd, qkv.dtype)
     lib = build.load("elementwise")
     _check(lib.ullm_qk_norm_rope_write(
         _p(qkv), _c_int(qkv.stride(0)), _p(q_out), _c_int(q_out.stride(0)), _p(q_gain), _p(k_gain),
@@ -163,9 +171,7 @@ def paged_attention_generic(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch
     T = q.shape[0]
     _need(q.shape == (T, nq * hd) and q.stride(1) == 1, "q must be [T, nq*hd]")
     _need(hd <= 512 and nq % nkv == 0, "head_dim > 512 or heads not a multiple of kv heads")
-    for pool, nm in ((k_pool, "k_pool"), (v_pool, "v_pool")):
-        _need(pool.dim() == 4 and tuple(pool.shape[1:]) == (nkv, page_size, hd) and pool.is_contiguous()
-              and pool.dtype == q.dtype, f"{nm} must be contiguous [pages, {nkv}, {page_size}, {hd}] of {q.dtype}")
+    _check_pools(k_pool, v_pool, nkv, page_size, hd, q.dtype)
     _i32(positions, "positions", T)
     _i32(token_entry, "token_entry", T)
     _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.stride(1) == 1,
@@ -217,13 +223,97 @@ def gemm_bf16(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = N
     return gemm_simple(a, w, bias, out_dtype=out_dtype)
 
 
+def attention_mfma_supports(dtype: torch.dtype, hd: int, page_size: int, nq: int, nkv: int) -> bool:
+    """True if the matrix-core attention kernels take this shape (bfloat16, head_dim in
+    {32, 64, 96, 128, 256}, page size a multiple of 16)."""
+    if dtype != torch.bfloat16:
+        return False
+    return bool(build.load("attention_mfma").ullm_attention_mfma_supports(
+        _c_int(hd), _c_int(page_size), _c_int(nq), _c_int(nkv)))
+
+
+def decode_split(n_items: int, nkv: int, groups: int, max_kv: int, target_waves: int = 2048):
+    """(chunk, num_splits): keys per split (32 * a power of two) so that the launch has about
+    ``target_waves`` waves."""
+    want = max(1, target_waves // max(1, n_items * nkv * groups))
+    chunk = 32
+    while -(-max_kv // chunk) > want:
+        chunk *= 2
+    return chunk, max(1, -(-max_kv // chunk))
+
+
+def attention_decode_mfma(q, out, k_pool, v_pool, token_list: Optional[torch.Tensor], n_items: int,
+                          positions, token_entry, block_table, page_size: int, nq: int, nkv: int, hd: int,
+                          scale: float, window: int, max_kv: int, chunk: Optional[int] = None) -> None:
+    """One query token per item (``token_list`` int32 [n_items] names the tokens, None = tokens
+    0..n_items-1) against its request's cache, keys split into chunks and reduced."""
+    _check_pools(k_pool, v_pool, nkv, page_size, hd, torch.bfloat16)
+    _need(q.dtype == torch.bfloat16 and q.stride(1) == 1 and q.shape[1] == nq * hd, "q must be bfloat16 [T, nq*hd]")
+    _need(out.dtype == torch.bfloat16 and out.stride(1) == 1 and out.shape == q.shape, "bad attention output")
+    _i32(positions, "positions")
+    _i32(token_entry, "token_entry")
+    if token_list is not None:
+        _i32(token_list, "token_list", n_items)
+    else:
+        _need(n_items <= q.shape[0], "more items than tokens")
+    _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.stride(1) == 1,
+          "block_table must be int32 [B, stride]")
+    _need(-(-max_kv // page_size) <= block_table.shape[1], "block table narrower than the longest context")
+    groups = -(-(nq // nkv) // 16)
+    if chunk is None:
+        chunk, splits = decode_split(n_items, nkv, groups, max_kv)
+    else:
+        splits = max(1, -(-max_kv // chunk))
+    lib = build.load("attention_mfma")
+    ws = None
+    if splits > 1:
+        ws = torch.empty(n_items * nq * splits * (hd + 2), dtype=torch.float32, device=q.device)
+    _check(lib.ullm_attention_decode(
+        _p(q), _c_int(q.stride(0)), _p(out), _c_int(out.stride(0)), _p(k_pool), _p(v_pool), _p(token_list),
+        _c_int(n_items), _p(positions), _p(token_entry), _p(block_table), _c_int(block_table.stride(0)),
+        _c_int(page_size), _c_int(nq), _c_int(nkv), _c_int(hd), _c_float(scale), _c_int(window), _c_int(chunk),
+        _c_int(splits), _p(ws), _stream()), "attention_decode")
+
+
+def attention_prefill_mfma(q, out, k_pool, v_pool, tiles: torch.Tensor, n_tiles: int, positions, token_entry,
+                           block_table, page_size: int, nq: int, nkv: int, hd: int, scale: float,
+                           window: int) -> None:
+    """Tiles (first token, count <= 16) of consecutive tokens of one request each, every token
+    against the keys up to its own position."""
+    _check_pools(k_pool, v_pool, nkv, page_size, hd, torch.bfloat16)
+    _need(q.dtype == torch.bfloat16 and q.stride(1) == 1 and q.shape[1] == nq * hd, "q must be bfloat16 [T, nq*hd]")
+    _need(out.dtype == torch.bfloat16 and out.stride(1) == 1 and out.shape == q.shape, "bad attention output")
+    _need(tiles.dtype == torch.int32 and tiles.is_contiguous() and tiles.numel() >= 2 * n_tiles, "tiles must be int32 [n, 2]")
+    _i32(positions, "positions")
+    _i32(token_entry, "token_entry")
+    _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.stride(1) == 1,
+          "block_table must be int32 [B, stride]")
+    lib = build.load("attention_mfma")
+    _check(lib.ullm_attention_prefill(
+        _p(q), _c_int(q.stride(0)), _p(out), _c_int(out.stride(0)), _p(k_pool), _p(v_pool), _p(tiles),
+        _c_int(n_tiles), _p(positions), _p(token_entry), _p(block_table), _c_int(block_table.stride(0)),
+        _c_int(page_size), _c_int(nq), _c_int(nkv), _c_int(hd), _c_float(scale), _c_int(window), _stream()),
+        "attention_prefill")
+
+
 def paged_attention(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, ctx, group, nq: int,
                     nkv: int, hd: int, scale: float, window: int) -> torch.Tensor:
     """Attention of the batch's queries over their requests' cached keys and values (the new
-    tokens' rows included).  Chooses the kernel by dtype and shape; every choice computes the same
-    function."""
-    return paged_attention_generic(q, k_pool, v_pool, ctx.positions, ctx.token_entry, group.block_table,
-                                   group.page_size, nq, nkv, hd, scale, window)
+    tokens' rows included).  bfloat16 shapes the matrix-core kernels take go there (one launch for
+    the one-token entries, one for the tiles of longer entries); everything else, and float32
+    always, takes the general kernel.  Every choice computes the same function."""
+    if not attention_mfma_supports(q.dtype, hd, group.page_size, nq, nkv):
+        return paged_attention_generic(q, k_pool, v_pool, ctx.positions, ctx.token_entry, group.block_table,
+                                       group.page_size, nq, nkv, hd, scale, window)
+    out = torch.empty((q.shape[0], nq * hd), dtype=q.dtype, device=q.device)
+    if ctx.num_decode:
+        attention_decode_mfma(q, out, k_pool, v_pool, ctx.decode_tokens, ctx.num_decode, ctx.positions,
+                              ctx.token_entry, group.block_table, group.page_size, nq, nkv, hd, scale, window,
+                              ctx.max_decode_kv)
+    if ctx.num_tiles:
+        attention_prefill_mfma(q, out, k_pool, v_pool, ctx.tiles, ctx.num_tiles, ctx.positions, ctx.token_entry,
+                               group.block_table, group.page_size, nq, nkv, hd, scale, window)
+    return out
 
 
 # ---------------------------------------------------------------------------------- sampling

@@ -63,7 +63,7 @@ class LayerCache:
     """What a mixer sees of the cache: its layer's pools or its layer's state rows."""
     group: int = -1                        # index into StepContext.groups for KV mixers
     k_pool: Optional[torch.Tensor] = None  # [num_pages, kv_heads, page_size, head_dim]
-    v_pool: Optional[torch.Tensor] = None
+    v_pool: Optional[torch.Tensor] = None  # [num_pages, kv_heads, head_dim, page_size]
     state: Optional[torch.Tensor] = None   # [num_slots, *StateNeed.shape]
     owner: bool = True                     # False: reads another layer's cache, writes nothing
 
@@ -85,6 +85,13 @@ class StepContext:
     decode_only: bool             # every entry brings exactly one token
     dtype: torch.dtype = torch.bfloat16          # compute dtype of activations
     host: dict = field(default_factory=dict)   # host-side copies for parts that want them
+    # how attention kernels split the batch: tokens of one-token entries, and tiles of up to 16
+    # consecutive tokens (first token, count) of the longer entries
+    decode_tokens: Optional[torch.Tensor] = None   # int32 [n_decode]; None when every token is one
+    num_decode: int = 0
+    max_decode_kv: int = 0
+    tiles: Optional[torch.Tensor] = None           # int32 [n_tiles, 2]
+    num_tiles: int = 0
 
 
 # --------------------------------------------------------------------------- parts
