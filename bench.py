@@ -91,10 +91,12 @@ def main():
 
     def run_decode(batch, steps, warmup):
         """tokens/s, ms per step, bytes read per step (mean over the timed steps)."""
-        new_tokens = warmup + steps + 2
+        budget = max(8192, batch)
+        # requests that finish their prompt early decode while the others are still in theirs
+        new_tokens = warmup + steps + 4 + -(-batch * args.prompt_len // budget)
         ec = EngineConfig(model="(random)", dtype=args.dtype, max_bs=batch, context_len=args.context_len,
                           page_size=16, num_pages=batch * (-(-(args.prompt_len + new_tokens + 16) // 16)),
-                          max_num_batched_tokens=max(8192, batch), max_prefill_chunk=2048, enforce_eager=args.eager)
+                          max_num_batched_tokens=budget, max_prefill_chunk=2048, enforce_eager=args.eager)
         eng = Engine(ec, model=model, env=env, model_config=cfg)
         for i in range(batch):
             prompt = torch.randint(0, cfg.vocab_size, (args.prompt_len,), generator=gen).tolist()

@@ -295,7 +295,7 @@ def test_attention_on_the_matrix_cores(ops, case):
             for f in range(0, n, 16):
                 tiles += [t0 + f, min(16, n - f)]
         t0 += n
-    for chunk in (None, 32, 64, 4096):
+    for chunk in (None, 128, 256, 4096):
         out = torch.full((q.shape[0], nq * hd), float("nan"), dtype=dtype, device=DEV)
         if dec:
             ops.attention_decode_mfma(q, out, k_pool, v_pool, torch.tensor(dec, dtype=torch.int32, device=DEV),
@@ -335,10 +335,42 @@ def test_matrix_core_attention_finds_one_far_key_at_every_edge(ops):
                 bt = table_tensor(tables, DEV)
                 if n == 1:
                     ops.attention_decode_mfma(qd, out, k_pool, v_pool, None, 1, positions, entry, bt, P, nq, nkv, hd,
-                                              1.0, window, S, chunk=64)
+                                              1.0, window, S, chunk=128)
                 else:
                     ops.attention_prefill_mfma(qd, out, k_pool, v_pool, torch.tensor([0, n], dtype=torch.int32, device=DEV),
                                                1, positions, entry, bt, P, nq, nkv, hd, 1.0, window)
                 got = out.float().cpu().view(n, nq, hd)[-1]
                 for h in range(nq):
                     assert (got[h] - v[target, h // 4]).abs().max() < 3e-2, (window, target, n, h)
+
+
+@pytest.mark.parametrize("shape", [(1, 48, 64), (8, 503, 96), (16, 256, 4096), (17, 100, 224), (33, 64, 1032),
+                                   (64, 130, 520), (5, 4096, 128), (3, 16, 8), (2, 9496, 72)])
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+def test_gemm_skinny(ops, shape, out_dtype):
+    torch.manual_seed(10)
+    M, N, K = shape
+    a = torch.randn(M, K, device=DEV).bfloat16()
+    w = torch.randn(N, K, device=DEV).bfloat16()
+    b = torch.randn(N, device=DEV)
+    want = (a.double() @ w.double().T + b.double()).float()
+    got = ops.gemm_skinny(a, w, b, out_dtype=out_dtype)
+    assert got.dtype == out_dtype
+    bound = (1e-2 if out_dtype == torch.bfloat16 else 2e-5) * float(want.abs().max())
+    assert (got.float() - want).abs().max() <= bound
+    assert torch.equal(ops.gemm_skinny(a, w, b, out_dtype=out_dtype), got)          # repeatable bit for bit
+    # strided activations (a column slice of a wider buffer)
+    wide = torch.randn(M, K + 64, device=DEV).bfloat16()
+    wide[:, 32:32 + K] = a
+    got2 = ops.gemm_skinny(wide[:, 32:32 + K], w, b, out_dtype=out_dtype)
+    assert torch.equal(got2, got)
+
+
+def test_gemm_dispatch_refuses_nothing_silently(ops):
+    a = torch.randn(4, 20, device=DEV).bfloat16()          # K not a multiple of 8: the general kernel takes it
+    w = torch.randn(6, 20, device=DEV).bfloat16()
+    assert not ops.gemm_skinny_supports(a, w)
+    got = ops.gemm_bf16(a, w, out_dtype=torch.float32)
+    assert (got - a.float() @ w.float().T).abs().max() < 1e-4
+    with pytest.raises(ops.KernelError):
+        ops.gemm_skinny(a, w)

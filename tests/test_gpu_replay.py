@@ -204,3 +204,43 @@ def test_trace_run_program(trace_run, model_dirs, plain_models):
         close(a, want[29:30], dtype)
         close(b, want[[30, 39, 5]], dtype)
         close(c, want[31:], dtype)
+
+
+@pytest.mark.parametrize("name,dtype", [("B", "float32"), ("B", "bfloat16"), ("C", "bfloat16")])
+def test_graph_replays_equal_eager_steps(model_dirs, plain_models, name, dtype):
+    """Decode steps replayed from HIP graphs: every replay is checked against the same step run
+    eagerly by a second runner, with eager work (prompt portions, other batch sizes) between the
+    replays, and against the plain implementation."""
+    from ullm_amd.replay import Replayer
+    graphs = Replayer(model_dirs[name], dtype, 512, 16, DEV, use_graphs=True)
+    eager = Replayer(model_dirs[name], dtype, 512, 16, DEV, use_graphs=False)
+    if not graphs.runner.use_graphs:
+        pytest.skip("graphs need the GPU")
+    vocab = plain_models[name][0]["vocab_size"]
+    reqs = {r: make_tokens(vocab, n, 50 + i) for i, (r, n) in enumerate([("a", 60), ("b", 45), ("c", 80)])}
+    wants = {r: oracle(plain_models, name, t) for r, t in reqs.items()}
+    done = {r: 0 for r in reqs}
+    got = {r: [] for r in reqs}
+    plan = [[("a", 20), ("b", 30)], [("a", 1), ("b", 1)], [("a", 1), ("b", 1), ("c", 50)], [("a", 1), ("b", 1), ("c", 1)],
+            [("a", 1), ("c", 1)], [("a", 7), ("c", 1)], [("a", 1), ("b", 1), ("c", 1)], [("a", 1)], [("a", 1), ("b", 1), ("c", 1)]]
+    for i in range(12):
+        plan.append([(r, 1) for r in reqs])
+    for s, step in enumerate(plan):
+        entries = []
+        for r, n in step:
+            n = min(n, len(reqs[r]) - done[r])
+            if n > 0:
+                entries.append({"id": r, "tokens": reqs[r][done[r]:done[r] + n], "want": list(range(n))})
+                done[r] += n
+        if not entries:
+            continue
+        a = graphs.step({"step": s, "entries": entries, "end": []})
+        b = eager.step({"step": s, "entries": entries, "end": []})
+        close(a, b, dtype)
+        row = 0
+        for e in entries:
+            got[e["id"]].append(a[row:row + len(e["tokens"])])
+            row += len(e["tokens"])
+    assert len(graphs.runner._graphs) >= 2 and not eager.runner._graphs
+    for r in reqs:
+        close(np.concatenate(got[r]), wants[r][:done[r]], dtype)

@@ -30,6 +30,42 @@ union Pack8 {
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// One 32-key tile of a request's cache in registers: the operands of both products.
+template <int NQK>
+struct KVTile {
+  Pack8 k[2][NQK];        // k[sb][ch]: keys key0 + 16 sb + (lane & 15), dims 32 ch + 8 g .. +8
+  uint2 v[2 * NQK][2];    // v[n][sb]: dim 16 n + (lane & 15), keys key0 + 16 sb + 4 g .. +4
+  int ok[2];              // the 16-key half holds a page
+};
+
+template <int NQK>
+__device__ __forceinline__ void load_tile(KVTile<NQK>& t, int key0, int key_end, const bf16_t* __restrict__ k_pool,
+                                          const bf16_t* __restrict__ v_pool, const int* __restrict__ bt,
+                                          int page_size, int nkv, int kvh) {
+  constexpr int HD = 32 * NQK;
+  const int lane = threadIdx.x & 63, g = lane >> 4, c = lane & 15;
+#pragma unroll
+  for (int sb = 0; sb < 2; ++sb) {
+    const int kb = key0 + 16 * sb;
+    const int page = kb < key_end ? bt[kb / page_size] : -1;
+    const int off = kb % page_size;
+    t.ok[sb] = page >= 0;
+    if (page >= 0) {
+      const bf16_t* kp = k_pool + (((size_t)page * nkv + kvh) * page_size + off + c) * HD + 8 * g;
+#pragma unroll
+      for (int ch = 0; ch < NQK; ++ch) t.k[sb][ch].u4 = *reinterpret_cast<const uint4*>(kp + 32 * ch);
+      const bf16_t* vp = v_pool + (((size_t)page * nkv + kvh) * HD + c) * page_size + off + 4 * g;
+#pragma unroll
+      for (int n = 0; n < 2 * NQK; ++n) t.v[n][sb] = *reinterpret_cast<const uint2*>(vp + (size_t)16 * n * page_size);
+    } else {
+#pragma unroll
+      for (int ch = 0; ch < NQK; ++ch) t.k[sb][ch].u4 = make_uint4(0, 0, 0, 0);
+#pragma unroll
+      for (int n = 0; n < 2 * NQK; ++n) t.v[n][sb] = make_uint2(0, 0);
+    }
+  }
+}
+
 // The work of one wave.  NQK = head_dim / 32.
 //   col_q      : pointer to this lane's column's query row (null if the column is padding)
 //   col_lo/hi  : first and last key the column may see (hi < lo for padding)
@@ -37,13 +73,13 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 //   max_hi     : largest key position that holds written data for this request
 // Results: acc[n][r] = O^T[16n + 4g + r][col] (unnormalised), m (log2 domain), l (this lane's share
 // of the sum; the four lanes of a column add up to the column's sum).
+// The loads of the next tile are issued before the arithmetic on the current one.
 template <int NQK>
 __device__ __forceinline__ void attend_range(
     const bf16_t* __restrict__ col_q, int col_lo, int col_hi, int key_begin, int key_end, int max_hi,
     const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool, const int* __restrict__ bt,
     int page_size, int nkv, int kvh, float scale_log2e, f32x4_t (&acc)[2 * NQK], float& m, float& l) {
-  constexpr int HD = 32 * NQK;
-  const int lane = threadIdx.x & 63, g = lane >> 4, c = lane & 15;
+  const int lane = threadIdx.x & 63, g = lane >> 4;
   Pack8 qreg[NQK];
 #pragma unroll
   for (int ch = 0; ch < NQK; ++ch) {
@@ -54,38 +90,29 @@ __device__ __forceinline__ void attend_range(
   for (int n = 0; n < 2 * NQK; ++n) acc[n] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   m = NEG_BIG;
   l = 0.f;
+  if (key_begin >= key_end) return;
 
+  KVTile<NQK> cur, nxt;
+  load_tile<NQK>(cur, key_begin, key_end, k_pool, v_pool, bt, page_size, nkv, kvh);
   for (int key0 = key_begin; key0 < key_end; key0 += 32) {
-    // the two 16-key halves of the tile; each lies inside one page (page_size is a multiple of 16)
-    int page[2], off[2];
-#pragma unroll
-    for (int sb = 0; sb < 2; ++sb) {
-      const int kb = key0 + 16 * sb;
-      page[sb] = kb < key_end ? bt[kb / page_size] : -1;
-      off[sb] = kb % page_size;
-    }
+    const bool more = key0 + 32 < key_end;
+    if (more) load_tile<NQK>(nxt, key0 + 32, key_end, k_pool, v_pool, bt, page_size, nkv, kvh);
     f32x4_t s[2];
 #pragma unroll
     for (int sb = 0; sb < 2; ++sb) {
       s[sb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-      if (page[sb] >= 0) {
-        const bf16_t* kp = k_pool + (((size_t)page[sb] * nkv + kvh) * page_size + off[sb] + c) * HD + 8 * g;
 #pragma unroll
-        for (int ch = 0; ch < NQK; ++ch) {
-          Pack8 a;
-          a.u4 = *reinterpret_cast<const uint4*>(kp + 32 * ch);
-          s[sb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, qreg[ch].v, s[sb], 0, 0, 0);
-        }
-      }
+      for (int ch = 0; ch < NQK; ++ch)
+        s[sb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.k[sb][ch].v, qreg[ch].v, s[sb], 0, 0, 0);
     }
-    // scores of keys key0 + 16 sb + 4 g + r for column c; mask, running maximum
+    // scores of keys key0 + 16 sb + 4 g + r for this lane's column; mask, running maximum
     float tile_max = NEG_BIG;
 #pragma unroll
     for (int sb = 0; sb < 2; ++sb)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int kk = key0 + 16 * sb + 4 * g + r;
-        const bool ok = page[sb] >= 0 && kk >= col_lo && kk <= col_hi;
+        const bool ok = cur.ok[sb] && kk >= col_lo && kk <= col_hi;
         const float v = ok ? s[sb][r] * scale_log2e : NEG_BIG;
         s[sb][r] = v;
         tile_max = fmaxf(tile_max, v);
@@ -107,20 +134,12 @@ __device__ __forceinline__ void attend_range(
       }
     l = l * alpha + psum;
     m = m_new;
-    // values: lane (c, g) feeds V^T[dim 16n + c][keys key0 + 16 sb + 4g .. +4]
     const bool edge = key0 + 32 > max_hi + 1;     // some keys of the tile hold no written data
 #pragma unroll
     for (int n = 0; n < 2 * NQK; ++n) {
       Pack8 a;
-#pragma unroll
-      for (int sb = 0; sb < 2; ++sb) {
-        if (page[sb] >= 0) {
-          const bf16_t* vp = v_pool + (((size_t)page[sb] * nkv + kvh) * HD + 16 * n + c) * page_size + off[sb] + 4 * g;
-          a.u2[sb] = *reinterpret_cast<const uint2*>(vp);
-        } else {
-          a.u2[sb] = make_uint2(0, 0);
-        }
-      }
+      a.u2[0] = cur.v[n][0];
+      a.u2[1] = cur.v[n][1];
       if (edge) {
 #pragma unroll
         for (int j = 0; j < 8; ++j)
@@ -130,13 +149,17 @@ __device__ __forceinline__ void attend_range(
       o[0] *= alpha; o[1] *= alpha; o[2] *= alpha; o[3] *= alpha;
       acc[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, p.v, o, 0, 0, 0);
     }
+    if (more) cur = nxt;
   }
 }
 
 // ------------------------------------------------------------------------------- decode
-// grid (ceil(splits / 4), nkv * col_groups, n_tokens), block 256: wave w of block x works on split
-// 4 x + w of the token's keys: [split * chunk, (split + 1) * chunk) cut to [lo, pos].
-// With one split the result is final; otherwise (O, m, l) go to the workspace for the reduce kernel.
+// grid (num_splits, nkv * col_groups, n_tokens), block 256.  Block x works on keys
+// [x * chunk, (x + 1) * chunk) cut to [lo, pos]; its four waves take a quarter each and combine
+// their (maximum, sum, output) through shared memory.  With one split that is the result.  Otherwise
+// the block writes its partial to the workspace and a second, small kernel adds the partials in
+// split order.  (A single kernel in which the last block to finish does that sum needs a device-wide
+// memory fence per block, which on a part with one L2 per XCD costs far more than the second launch.)
 template <int NQK>
 __global__ void __launch_bounds__(256)
 attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
@@ -144,11 +167,13 @@ attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __re
                         const int* __restrict__ token_list, const int* __restrict__ positions,
                         const int* __restrict__ token_entry, const int* __restrict__ block_table,
                         int bt_stride, int page_size, int nq, int nkv, float scale_log2e, int window,
-                        int chunk, int num_splits, float* __restrict__ part_o, float* __restrict__ part_ml) {
+                        int chunk, int num_splits, float* __restrict__ part) {
   constexpr int HD = 32 * NQK;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, g = lane >> 4, c = lane & 15;
-  const int split = blockIdx.x * 4 + wave;
-  if (split >= num_splits) return;
+  constexpr int ROW = HD + 2;                       // output dims, then maximum and sum
+  __shared__ float comb[4][16][ROW];
+  __shared__ float res[16][ROW];                    // the four waves' rows combined
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g = lane >> 4, c = lane & 15;
+  const int split = blockIdx.x;
   const int G = nq / nkv;
   const int groups = (G + 15) / 16;
   const int kvh = blockIdx.y / groups, cg = blockIdx.y % groups;
@@ -156,67 +181,87 @@ attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __re
   const int t = token_list ? token_list[item] : item;
   const int pos = positions[t];
   const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
-  int begin = split * chunk, end = begin + chunk;
+  const int quarter = chunk / 4;
+  int begin = split * chunk + wave * quarter, end = begin + quarter;
   if (end > pos + 1) end = pos + 1;
   if (begin < (lo & ~31)) begin = lo & ~31;
   const int head_in_group = cg * 16 + c;
   const bool col_ok = head_in_group < G;
   const int head = kvh * G + head_in_group;
-  const bool empty = begin >= end;
   f32x4_t acc[2 * NQK];
-  float m = NEG_BIG, l = 0.f;
-  if (!empty) {
-    attend_range<NQK>(col_ok ? q + (size_t)t * q_stride + (size_t)head * HD : nullptr, lo, col_ok ? pos : -1,
-                      begin, end, pos, k_pool, v_pool, block_table + (size_t)token_entry[t] * bt_stride,
-                      page_size, nkv, kvh, scale_log2e, acc, m, l);
-    l += __shfl_xor(l, 16, 64);
-    l += __shfl_xor(l, 32, 64);
-  } else {
+  float m, l;
+  attend_range<NQK>(col_ok ? q + (size_t)t * q_stride + (size_t)head * HD : nullptr, lo, col_ok ? pos : -1,
+                    begin, end, pos, k_pool, v_pool, block_table + (size_t)token_entry[t] * bt_stride,
+                    page_size, nkv, kvh, scale_log2e, acc, m, l);
+  l += __shfl_xor(l, 16, 64);
+  l += __shfl_xor(l, 32, 64);
 #pragma unroll
-    for (int n = 0; n < 2 * NQK; ++n) acc[n] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  for (int n = 0; n < 2 * NQK; ++n)
+    *reinterpret_cast<float4*>(&comb[wave][c][16 * n + 4 * g]) = make_float4(acc[n][0], acc[n][1], acc[n][2], acc[n][3]);
+  if (g == 0) {
+    comb[wave][c][HD] = m;
+    comb[wave][c][HD + 1] = l;
   }
-  if (!col_ok) return;
+  __syncthreads();
+  // combine the four waves: wave -> column, lane -> dims
+  const int ncols = G - cg * 16 < 16 ? G - cg * 16 : 16;
+  for (int col = wave; col < ncols; col += 4) {
+    float M = comb[0][col][HD];
+#pragma unroll
+    for (int w = 1; w < 4; ++w) M = fmaxf(M, comb[w][col][HD]);
+    float f[4];
+#pragma unroll
+    for (int w = 0; w < 4; ++w) f[w] = fast_exp2(comb[w][col][HD] - M);
+    for (int d = lane; d < HD; d += 64) {
+      float o = 0.f;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) o += comb[w][col][d] * f[w];
+      res[col][d] = o;
+    }
+    float L = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) L += comb[w][col][HD + 1] * f[w];
+    if (lane == 0) {
+      res[col][HD] = M;
+      res[col][HD + 1] = L;
+    }
+  }
+  __syncthreads();
+  const int head0 = kvh * G + cg * 16;
   if (num_splits == 1) {
-    const float inv = l > 0.f ? 1.f / l : 0.f;
-    bf16_t* op = out + (size_t)t * out_stride + (size_t)head * HD;
-#pragma unroll
-    for (int n = 0; n < 2 * NQK; ++n) {
-      uint2 w;
-      w.x = (uint32_t)f32_to_bf16_bits(acc[n][0] * inv) | ((uint32_t)f32_to_bf16_bits(acc[n][1] * inv) << 16);
-      w.y = (uint32_t)f32_to_bf16_bits(acc[n][2] * inv) | ((uint32_t)f32_to_bf16_bits(acc[n][3] * inv) << 16);
-      *reinterpret_cast<uint2*>(op + 16 * n + 4 * g) = w;
+    for (int col = wave; col < ncols; col += 4) {
+      const float L = res[col][HD + 1];
+      const float inv = L > 0.f ? 1.f / L : 0.f;
+      bf16_t* op = out + (size_t)t * out_stride + (size_t)(head0 + col) * HD;
+      for (int d = lane; d < HD; d += 64) op[d] = f32_to_bf16_bits(res[col][d] * inv);
     }
-  } else {
-    const size_t slot = ((size_t)item * nq + head) * num_splits + split;
-    float* po = part_o + slot * HD;
-#pragma unroll
-    for (int n = 0; n < 2 * NQK; ++n)
-      *reinterpret_cast<float4*>(po + 16 * n + 4 * g) = make_float4(acc[n][0], acc[n][1], acc[n][2], acc[n][3]);
-    if (g == 0) {
-      part_ml[slot * 2] = m;
-      part_ml[slot * 2 + 1] = l;
-    }
+    return;
+  }
+  // partial of this block: [item][head][split][ROW]
+  for (int col = wave; col < ncols; col += 4) {
+    float* pp = part + (((size_t)item * nq + head0 + col) * num_splits + split) * ROW;
+    for (int d = lane; d < ROW; d += 64) pp[d] = res[col][d];
   }
 }
 
-// Combine the splits of one (token, head): out = sum_s O_s 2^(m_s - M) / sum_s l_s 2^(m_s - M).
+// Adds the splits' partials [item][head][split][head_dim + 2] in split order.  grid (n_items, nq).
 __global__ void __launch_bounds__(64)
-attention_reduce_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                        bf16_t* __restrict__ out, int out_stride, const int* __restrict__ token_list,
-                        int nq, int hd, int num_splits) {
+attention_reduce_kernel(const float* __restrict__ part, bf16_t* __restrict__ out, int out_stride,
+                        const int* __restrict__ token_list, int nq, int hd, int num_splits) {
   const int item = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
   const int t = token_list ? token_list[item] : item;
-  const size_t base = ((size_t)item * nq + head) * num_splits;
+  const int row = hd + 2;
+  const float* pp = part + ((size_t)item * nq + head) * num_splits * row;
   float M = NEG_BIG;
-  for (int s = 0; s < num_splits; ++s) M = fmaxf(M, part_ml[(base + s) * 2]);
+  for (int sp = 0; sp < num_splits; ++sp) M = fmaxf(M, pp[sp * row + hd]);
   float L = 0.f;
-  for (int s = 0; s < num_splits; ++s) L += part_ml[(base + s) * 2 + 1] * fast_exp2(part_ml[(base + s) * 2] - M);
+  for (int sp = 0; sp < num_splits; ++sp) L += pp[sp * row + hd + 1] * fast_exp2(pp[sp * row + hd] - M);
   const float inv = L > 0.f ? 1.f / L : 0.f;
+  bf16_t* op = out + (size_t)t * out_stride + (size_t)head * hd;
   for (int d = lane; d < hd; d += 64) {
     float o = 0.f;
-    for (int s = 0; s < num_splits; ++s)
-      o += part_o[(base + s) * hd + d] * fast_exp2(part_ml[(base + s) * 2] - M);
-    out[(size_t)t * out_stride + (size_t)head * hd + d] = f32_to_bf16_bits(o * inv);
+    for (int sp = 0; sp < num_splits; ++sp) o += pp[sp * row + d] * fast_exp2(pp[sp * row + hd] - M);
+    op[d] = f32_to_bf16_bits(o * inv);
   }
 }
 
@@ -288,7 +333,6 @@ extern "C" int ullm_attention_mfma_supports(int hd, int page_size, int nq, int n
 extern "C" long long ullm_attention_decode_workspace(int n_items, int nq, int hd, int num_splits) {
   return num_splits <= 1 ? 0 : (long long)n_items * nq * num_splits * (hd + 2);
 }
-
 extern "C" int ullm_attention_decode(
     const void* q, int q_stride, void* out, int out_stride, const void* k_pool, const void* v_pool,
     const int* token_list, int n_items, const int* positions, const int* token_entry,
@@ -296,22 +340,21 @@ extern "C" int ullm_attention_decode(
     int chunk, int num_splits, float* workspace, hipStream_t stream) {
   if (n_items <= 0) return 0;
   if (!ullm_attention_mfma_supports(hd, page_size, nq, nkv)) return ULLM_ERR_UNSUPPORTED;
-  if (chunk <= 0 || chunk % 32 != 0 || num_splits < 1 || window < 0) return ULLM_ERR_SHAPE;
+  if (chunk <= 0 || chunk % 128 != 0 || num_splits < 1 || window < 0) return ULLM_ERR_SHAPE;
   if (num_splits > 1 && !workspace) return ULLM_ERR_SHAPE;
   const int G = nq / nkv, groups = (G + 15) / 16;
-  float* part_o = workspace;
-  float* part_ml = workspace ? workspace + (size_t)n_items * nq * num_splits * hd : nullptr;
+  if (n_items > 65535 || nkv * groups > 65535) return ULLM_ERR_SHAPE;
   const float sl = scale * 1.4426950408889634f;
-  dim3 grid((num_splits + 3) / 4, nkv * groups, n_items), block(256);
+  dim3 grid(num_splits, nkv * groups, n_items), block(256);
 #define CALL(N) hipLaunchKernelGGL(attention_decode_kernel<N>, grid, block, 0, stream, (const bf16_t*)q, q_stride, \
     (bf16_t*)out, out_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool, token_list, positions, token_entry, \
-    block_table, bt_stride, page_size, nq, nkv, sl, window, chunk, num_splits, part_o, part_ml)
+    block_table, bt_stride, page_size, nq, nkv, sl, window, chunk, num_splits, workspace)
   DISPATCH_NQK(hd, CALL)
 #undef CALL
   int rc = (int)hipGetLastError();
   if (rc != 0 || num_splits == 1) return rc;
-  hipLaunchKernelGGL(attention_reduce_kernel, dim3(n_items, nq), dim3(64), 0, stream, part_o, part_ml,
-                     (bf16_t*)out, out_stride, token_list, nq, hd, num_splits);
+  hipLaunchKernelGGL(attention_reduce_kernel, dim3(n_items, nq), dim3(64), 0, stream, workspace, (bf16_t*)out,
+                     out_stride, token_list, nq, hd, num_splits);
   ULLM_LAUNCH_CHECK();
 }
 

@@ -55,7 +55,8 @@ class Engine:
             num_pages = pages_from_memory(model, env, config.page_size, config.gpu_memory_utilization,
                                           config.context_len, config.max_bs)
         self.runner = ModelRunner(model, env, config.page_size, num_pages, config.max_bs,
-                                  enable_prefix_cache=config.enable_prefix_cache)
+                                  enable_prefix_cache=config.enable_prefix_cache,
+                                  use_graphs=not config.enforce_eager)
         self.scheduler = Scheduler(self.runner.cache, config.max_num_batched_tokens, config.max_prefill_chunk,
                                    config.max_bs)
         self.sampler = Sampler(env.device)

@@ -37,7 +37,7 @@ Q_TILE = 16     # tokens of one request that the prompt-portion attention kernel
 
 class ModelRunner:
     def __init__(self, model: Model, env: PartEnv, page_size: int, num_pages, max_requests: int,
-                 enable_prefix_cache: bool = False):
+                 enable_prefix_cache: bool = False, use_graphs: bool = True, max_graph_batch: int = 256):
         if model.env is None:
             raise StepError("the model has no weights bound")
         self.model, self.env = model, env
@@ -66,6 +66,13 @@ class ModelRunner:
         self._staging_done: List[Optional[torch.cuda.Event]] = [None, None]
         self._turn = 0
         self.vocab_size = model.plan.vocab_size
+        # Steps in which every entry brings one token are replayed from HIP graphs, one graph per
+        # (batch size bucket, context length bucket).  Padding entries would disturb per-request state,
+        # so a model with state mixers always runs eagerly.
+        self.use_graphs = bool(use_graphs) and env.device.type == "cuda" and not states
+        self.max_graph_batch = max_graph_batch
+        self._graphs: Dict[tuple, "_DecodeGraph"] = {}
+        self._graph_pool = None
 
     # ------------------------------------------------------------------ helpers
     def cache_bytes(self) -> int:
@@ -76,9 +83,9 @@ class ModelRunner:
                     total += t.numel() * t.element_size()
         return total
 
-    def _upload(self, host: np.ndarray) -> torch.Tensor:
-        """Copy the packed batch description to the device through one of two pinned buffers; a
-        buffer is written again only after the copy that last read it has finished."""
+    def _upload(self, host: np.ndarray, into: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Copy the packed batch description to the device (into ``into`` if given) through one of two
+        pinned buffers; a buffer is written again only after the copy that last read it has finished."""
         i = self._turn
         self._turn ^= 1
         if self._staging_done[i] is not None:
@@ -87,7 +94,11 @@ class ModelRunner:
             self._staging[i] = torch.empty(max(host.size, 4096), dtype=torch.int32, pin_memory=self._pin)
         stage = self._staging[i][:host.size]
         stage.numpy()[:] = host
-        dev = stage.to(self.env.device, non_blocking=True)
+        if into is not None:
+            into.copy_(stage, non_blocking=True)
+            dev = into
+        else:
+            dev = stage.to(self.env.device, non_blocking=True)
         if self._pin:
             ev = torch.cuda.Event()
             ev.record()
@@ -96,20 +107,29 @@ class ModelRunner:
             dev = dev.clone()
         return dev
 
-    def build_context(self, entries: Sequence[StepEntry]):
-        """Flatten the entries into device tensors (one host-to-device copy)."""
+    def _pack(self, entries: Sequence[StepEntry], pad_entries: int = 0, table_stride: Optional[int] = None):
+        """Flatten the entries into one int32 host array.  Returns (host array, offsets, facts).
+        ``pad_entries`` > len(entries) appends one-token entries that hold no pages (their cache
+        writes are skipped and their outputs ignored), so that a batch fits a captured graph."""
         P = self.page_size
-        B = len(entries)
+        n_real = len(entries)
         lens = [len(e.tokens) for e in entries]
-        T = sum(lens)
-        if B == 0 or T == 0:
+        if n_real == 0 or sum(lens) == 0:
             raise StepError("a step needs at least one token")
+        n_pad = max(0, pad_entries - n_real)
+        B = n_real + n_pad
+        T = sum(lens) + n_pad
         groups = self.cache.groups
         strides = []
         for g in range(len(groups)):
-            strides.append(max(1, max(len(e.cache.tables[g]) for e in entries)))
-        n_want = sum(len(e.want) for e in entries)
-        # attention work lists: tokens of one-token entries; tiles of <= 16 tokens of longer entries
+            widest = max(1, max(len(e.cache.tables[g]) for e in entries))
+            if table_stride is not None:
+                if widest > table_stride:
+                    raise StepError("a block table is wider than the captured graph's")
+                widest = table_stride
+            strides.append(widest)
+        n_want = sum(len(e.want) for e in entries) + n_pad
+        # attention work lists: tokens of one-token entries; tiles of <= Q_TILE tokens of longer entries
         dec_list, tile_list, max_dec_kv, t0 = [], [], 0, 0
         for e, n in zip(entries, lens):
             if n == 1:
@@ -119,10 +139,11 @@ class ModelRunner:
                 for first in range(0, n, Q_TILE):
                     tile_list.extend((t0 + first, min(Q_TILE, n - first)))
             t0 += n
-        # layout of the packed int32 buffer
+        dec_list.extend(range(t0, t0 + n_pad))
+        ng = len(groups)
         sizes = [T, T, T, B + 1, B, B, n_want] + [B * s for s in strides] + [len(dec_list), len(tile_list)]
         offs = np.concatenate(([0], np.cumsum(sizes)))
-        host = np.empty(int(offs[-1]), dtype=np.int32)
+        host = np.zeros(int(offs[-1]), dtype=np.int32)
         ids, pos, ent = host[offs[0]:offs[1]], host[offs[1]:offs[2]], host[offs[2]:offs[3]]
         q_start, slot, start = host[offs[3]:offs[4]], host[offs[4]:offs[5]], host[offs[5]:offs[6]]
         rows = host[offs[6]:offs[7]]
@@ -142,7 +163,7 @@ class ModelRunner:
             s0 = rc.num_computed
             if s0 + n > self.env.context_len:
                 raise StepError(f"request {rc.request_id!r}: {s0 + n} tokens exceed context_len={self.env.context_len}")
-            for g in range(len(groups)):
+            for g in range(ng):
                 if len(rc.tables[g]) * P < s0 + n:
                     raise StepError(f"request {rc.request_id!r}: no pages reserved for positions up to {s0 + n - 1}")
             tok = np.asarray(e.tokens, dtype=np.int64)
@@ -161,6 +182,12 @@ class ModelRunner:
                 r += 1
             max_kv = max(max_kv, s0 + n)
             t += n
+        for b in range(n_real, B):                       # padding entries: token 0 at position 0, no pages
+            ent[t] = b
+            q_start[b] = t
+            rows[r] = t
+            t += 1
+            r += 1
         q_start[B] = T
         for g, s in enumerate(strides):
             bt = host[offs[7 + g]:offs[8 + g]].reshape(B, s)
@@ -168,24 +195,38 @@ class ModelRunner:
             for b, e in enumerate(entries):
                 tab = e.cache.tables[g]
                 bt[b, :len(tab)] = tab
-        ng = len(groups)
         host[offs[7 + ng]:offs[8 + ng]] = dec_list
         host[offs[8 + ng]:offs[9 + ng]] = tile_list
-        dev = self._upload(host)
+        facts = dict(T=T, B=B, strides=strides, n_want=n_want, num_decode=len(dec_list), max_dec_kv=max_dec_kv,
+                     num_tiles=len(tile_list) // 2, max_q=max(lens), max_kv=max_kv,
+                     decode_only=all(n == 1 for n in lens), lens=lens + [1] * n_pad,
+                     starts=[e.cache.num_computed for e in entries] + [0] * n_pad,
+                     slots=[e.cache.slot for e in entries] + [0] * n_pad)
+        return host, offs, facts
+
+    def _context(self, dev: torch.Tensor, offs, facts) -> tuple:
+        """Views into the uploaded buffer as a StepContext, and the wanted rows."""
+        groups = self.cache.groups
+        ng = len(groups)
+        B, T = facts["B"], facts["T"]
         view = lambda i: dev[int(offs[i]):int(offs[i + 1])]  # noqa: E731
-        gviews = [GroupView(view(7 + g).view(B, strides[g]), strides[g], P, groups[g].window)
-                  for g in range(len(groups))]
+        gviews = [GroupView(view(7 + g).view(B, facts["strides"][g]), facts["strides"][g], self.page_size,
+                            groups[g].window) for g in range(ng)]
         ctx = StepContext(
             num_tokens=T, num_entries=B, token_ids=view(0), positions=view(1), token_entry=view(2),
             q_start=view(3), entry_slot=view(4), entry_start=view(5), groups=gviews,
-            max_q_len=max(lens), max_kv_len=max_kv, decode_only=all(n == 1 for n in lens),
+            max_q_len=facts["max_q"], max_kv_len=facts["max_kv"], decode_only=facts["decode_only"],
             dtype=self.env.dtype,
-            decode_tokens=view(7 + ng) if (dec_list and len(dec_list) < T) else None, num_decode=len(dec_list),
-            max_decode_kv=max_dec_kv, tiles=view(8 + ng).view(-1, 2) if tile_list else None,
-            num_tiles=len(tile_list) // 2,
-            host={"lens": lens, "starts": [e.cache.num_computed for e in entries],
-                  "slots": [e.cache.slot for e in entries]})
-        return ctx, (view(6) if n_want else None)
+            decode_tokens=view(7 + ng) if 0 < facts["num_decode"] < T else None, num_decode=facts["num_decode"],
+            max_decode_kv=facts["max_dec_kv"], tiles=view(8 + ng).view(-1, 2) if facts["num_tiles"] else None,
+            num_tiles=facts["num_tiles"],
+            host={"lens": facts["lens"], "starts": facts["starts"], "slots": facts["slots"]})
+        return ctx, (view(6) if facts["n_want"] else None)
+
+    def build_context(self, entries: Sequence[StepEntry]):
+        """Flatten the entries into device tensors (one host-to-device copy)."""
+        host, offs, facts = self._pack(entries)
+        return self._context(self._upload(host), offs, facts)
 
     # ------------------------------------------------------------------ the step
     def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
@@ -198,9 +239,68 @@ class ModelRunner:
             for c in self.caches.values():
                 if c.state is not None:
                     c.state[torch.tensor(fresh, device=c.state.device)] = 0
-        ctx, rows = self.build_context(entries)
-        with torch.no_grad():
-            logits = self.model.forward(ctx, self.caches, rows)
+        if (self.use_graphs and len(entries) <= self.max_graph_batch and all(len(e.tokens) == 1 for e in entries)):
+            logits = self._step_from_graph(entries)
+        else:
+            ctx, rows = self.build_context(entries)
+            with torch.no_grad():
+                logits = self.model.forward(ctx, self.caches, rows)
         for e in entries:
             self.cache.commit(e.cache, len(e.tokens))
         return logits
+
+    # ------------------------------------------------------------------ HIP graphs for decode steps
+    def _step_from_graph(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+        B = len(entries)
+        b_pad = 1
+        while b_pad < B:
+            b_pad *= 2
+        longest = max(e.cache.num_computed + 1 for e in entries)
+        kv_bucket = 256
+        while kv_bucket < longest:
+            kv_bucket *= 2
+        kv_bucket = min(kv_bucket, self.max_table * self.page_size)
+        packed = [StepEntry(e.cache, e.tokens, [0]) for e in entries]
+        host, offs, facts = self._pack(packed, pad_entries=b_pad, table_stride=self.max_table)
+        key = (b_pad, kv_bucket)
+        graph = self._graphs.get(key)
+        if graph is None:
+            graph = self._capture(key, host, offs, facts)
+        else:
+            self._upload(host, into=graph.static_dev)
+        graph.graph.replay()
+        wanted = [b for b, e in enumerate(entries) if len(e.want)]
+        if not wanted:
+            return None
+        if len(wanted) == B:
+            return graph.logits[:B]
+        return graph.logits[torch.tensor(wanted, device=graph.logits.device)]
+
+    def _capture(self, key, host: np.ndarray, offs, facts) -> "_DecodeGraph":
+        b_pad, kv_bucket = key
+        facts = dict(facts, max_dec_kv=kv_bucket, max_kv=kv_bucket)    # the kernels' split of the keys is fixed
+        static_dev = torch.empty(host.size, dtype=torch.int32, device=self.env.device)
+        self._upload(host, into=static_dev)
+        ctx, rows = self._context(static_dev, offs, facts)
+        with torch.no_grad():
+            # once eagerly on a side stream: loads the kernels and sizes the library's workspaces
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                self.model.forward(ctx, self.caches, rows)
+            torch.cuda.current_stream().wait_stream(side)
+            if self._graph_pool is None:
+                self._graph_pool = torch.cuda.graph_pool_handle()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g, pool=self._graph_pool):
+                logits = self.model.forward(ctx, self.caches, rows)
+        graph = _DecodeGraph(g, static_dev, logits)
+        self._graphs[key] = graph
+        return graph
+
+
+@dataclass
+class _DecodeGraph:
+    graph: "torch.cuda.CUDAGraph"
+    static_dev: torch.Tensor          # the packed batch description the captured kernels read
+    logits: torch.Tensor              # float32 [batch bucket, vocab], rewritten by every replay

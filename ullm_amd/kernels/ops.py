@@ -209,12 +209,46 @@ def gemm_simple(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] =
     return out
 
 
+def gemm_skinny_supports(a: torch.Tensor, w: torch.Tensor) -> bool:
+    M, K = a.shape
+    return (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and 1 <= M <= 64 and K % 8 == 0 and K >= 8
+            and a.stride(1) == 1 and w.stride(1) == 1 and a.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
+            and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
+
+
+def gemm_skinny(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
+                out_dtype: Optional[torch.dtype] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """a [M <= 64, K] times w [N, K] transposed, bfloat16 operands streamed once through the matrix
+    cores, 32-bit accumulation; output bfloat16 or float32."""
+    M, K = a.shape
+    N, K2 = w.shape
+    _need(K == K2, f"inner sizes differ: a is [{M}, {K}], w is [{N}, {K2}]")
+    _need(gemm_skinny_supports(a, w), "gemm_skinny takes bfloat16, M <= 64, K a multiple of 8, 16-byte aligned rows")
+    if out is None:
+        out = torch.empty((M, N), dtype=out_dtype or a.dtype, device=a.device)
+    _need(out.shape == (M, N) and out.stride(1) == 1, "bad gemm output")
+    if bias is not None:
+        _need(bias.dtype == torch.float32 and bias.numel() == N and bias.is_contiguous(), "bias must be float32 [N]")
+    lib = build.load("gemm_skinny")
+    _check(lib.ullm_gemm_skinny(_p(a), _c_int(a.stride(0)), _p(w), _c_int(w.stride(0)), _p(bias), _p(out),
+                                _c_int(out.stride(0)), _c_int(M), _c_int(N), _c_int(K), _c_int(_dt(out)), _stream()),
+           "gemm_skinny")
+    return out
+
+
+SKINNY_MAX_ROWS = 16     # up to here the weight-streaming kernel beats the library product
+
+
 def gemm_bf16(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
               out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
-    """bfloat16 operands, 32-bit accumulation.  Output in bfloat16 goes through the library product
-    (as the reference's linears do, ullm/layers/linear.py:165); 32-bit output (logits) through the
-    hand-written kernel, which keeps the accumulator's precision."""
+    """bfloat16 operands, 32-bit accumulation.  Few rows go to the weight-streaming kernel; many
+    rows with bfloat16 output go through the library product (as the reference's linears do,
+    ullm/layers/linear.py:165); 32-bit output (logits) always comes from a hand-written kernel,
+    which keeps the accumulator's precision."""
     out_dtype = out_dtype or a.dtype
+    M = a.shape[0]
+    if (M <= SKINNY_MAX_ROWS or (out_dtype == torch.float32 and M <= 64)) and gemm_skinny_supports(a, w):
+        return gemm_skinny(a, w, bias, out_dtype=out_dtype)
     if out_dtype == torch.bfloat16 and a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16:
         y = torch.nn.functional.linear(a, w)
         if bias is not None:
@@ -232,11 +266,11 @@ def attention_mfma_supports(dtype: torch.dtype, hd: int, page_size: int, nq: int
         _c_int(hd), _c_int(page_size), _c_int(nq), _c_int(nkv)))
 
 
-def decode_split(n_items: int, nkv: int, groups: int, max_kv: int, target_waves: int = 2048):
-    """(chunk, num_splits): keys per split (32 * a power of two) so that the launch has about
-    ``target_waves`` waves."""
-    want = max(1, target_waves // max(1, n_items * nkv * groups))
-    chunk = 32
+def decode_split(n_items: int, nkv: int, groups: int, max_kv: int, target_blocks: int = 768):
+    """(chunk, num_splits): keys per block (128 * a power of two; a block's four waves take a
+    quarter each) so that the launch has about ``target_blocks`` blocks."""
+    want = max(1, target_blocks // max(1, n_items * nkv * groups))
+    chunk = 128
     while -(-max_kv // chunk) > want:
         chunk *= 2
     return chunk, max(1, -(-max_kv // chunk))
@@ -246,7 +280,8 @@ def attention_decode_mfma(q, out, k_pool, v_pool, token_list: Optional[torch.Ten
                           positions, token_entry, block_table, page_size: int, nq: int, nkv: int, hd: int,
                           scale: float, window: int, max_kv: int, chunk: Optional[int] = None) -> None:
     """One query token per item (``token_list`` int32 [n_items] names the tokens, None = tokens
-    0..n_items-1) against its request's cache, keys split into chunks and reduced."""
+    0..n_items-1) against its request's cache; the keys are split into chunks whose partial results
+    a second small kernel adds up."""
     _check_pools(k_pool, v_pool, nkv, page_size, hd, torch.bfloat16)
     _need(q.dtype == torch.bfloat16 and q.stride(1) == 1 and q.shape[1] == nq * hd, "q must be bfloat16 [T, nq*hd]")
     _need(out.dtype == torch.bfloat16 and out.stride(1) == 1 and out.shape == q.shape, "bad attention output")
@@ -263,6 +298,7 @@ def attention_decode_mfma(q, out, k_pool, v_pool, token_list: Optional[torch.Ten
     if chunk is None:
         chunk, splits = decode_split(n_items, nkv, groups, max_kv)
     else:
+        _need(chunk % 128 == 0, "chunk must be a multiple of 128")
         splits = max(1, -(-max_kv // chunk))
     lib = build.load("attention_mfma")
     ws = None

@@ -29,6 +29,7 @@ def parse_args(argv=None):
                     help="most tokens live requests hold at any time (each rounded up to 64)")
     ap.add_argument("--page-size", type=int, default=16, help="tokens per cache page (divides 64)")
     ap.add_argument("--device", default="cuda:0")
+    ap.add_argument("--enforce-eager", action="store_true", help="never replay decode steps from HIP graphs")
     return ap.parse_args(argv)
 
 
@@ -36,7 +37,7 @@ class Replayer:
     """The replay loop's state: the model, its runner and the live requests."""
 
     def __init__(self, model_dir: str, dtype: str, max_tokens: int, page_size: int = 16, device: str = "cuda:0",
-                 max_requests: int = 8):
+                 max_requests: int = 8, use_graphs: bool = True):
         from .engine.loading import load_model
         from .engine.runner import ModelRunner
         if page_size < 1 or 64 % page_size:
@@ -46,7 +47,8 @@ class Replayer:
         self.max_tokens = -(-max_tokens // 64) * 64
         self.cfg, self.model, self.env = load_model(model_dir, dtype, device, context_len=self.max_tokens)
         self.runner = ModelRunner(self.model, self.env, page_size=page_size,
-                                  num_pages=self.max_tokens // page_size, max_requests=max_requests)
+                                  num_pages=self.max_tokens // page_size, max_requests=max_requests,
+                                  use_graphs=use_graphs)
         self.live = {}
 
     def step(self, msg: dict):
@@ -84,7 +86,8 @@ def main(argv=None) -> int:
     args = parse_args(argv)
     os.makedirs(args.out, exist_ok=True)
     try:
-        rep = Replayer(args.model, args.dtype, args.max_tokens, args.page_size, args.device)
+        rep = Replayer(args.model, args.dtype, args.max_tokens, args.page_size, args.device,
+                       use_graphs=not args.enforce_eager)
     except ValueError as e:
         print(f"trace_run: {e}", file=sys.stderr)
         return 2
