@@ -225,7 +225,7 @@ def test_sampler_kernel_against_the_plain_sampler(ops):
     sampler = Sampler(torch.device(DEV))
     configs = [(0.0, -1, 1.0, 0.0), (0.7, -1, 1.0, 0.0), (1.0, 5, 1.0, 0.0), (1.3, -1, 0.8, 0.0), (1.0, -1, 1.0, 0.1),
                (0.9, 20, 0.9, 0.05), (1.0, 1, 1.0, 0.0), (1.0, -1, 0.01, 0.0), (1.0, 2000, 1.0, 0.0)]
-    for V in (503, 1537):
+    for V in (503, 1537, 4100):            # 4100: rows aligned for the 16-byte path
         mismatches = 0
         for trial in range(5):
             logits = torch.randn(len(configs), V) * 3
@@ -356,6 +356,9 @@ def test_gemm_skinny(ops, shape, out_dtype):
     want = (a.double() @ w.double().T + b.double()).float()
     got = ops.gemm_skinny(a, w, b, out_dtype=out_dtype)
     assert got.dtype == out_dtype
+    for nt, waves in ((1, 1), (2, 2), (2, 16), (4 if M > 16 else 2, 4)):
+        assert (ops.gemm_skinny(a, w, b, out_dtype=out_dtype, nt=nt, waves=waves).float() - got.float()).abs().max() \
+            <= 1e-2 * float(want.abs().max())
     bound = (1e-2 if out_dtype == torch.bfloat16 else 2e-5) * float(want.abs().max())
     assert (got.float() - want).abs().max() <= bound
     assert torch.equal(ops.gemm_skinny(a, w, b, out_dtype=out_dtype), got)          # repeatable bit for bit
@@ -374,3 +377,30 @@ def test_gemm_dispatch_refuses_nothing_silently(ops):
     assert (got - a.float() @ w.float().T).abs().max() < 1e-4
     with pytest.raises(ops.KernelError):
         ops.gemm_skinny(a, w)
+
+
+@pytest.mark.parametrize("shape", [(1, 48, 64), (8, 503, 96), (16, 256, 4096), (17, 100, 224), (40, 96, 1032),
+                                   (64, 2100, 520), (5, 4096, 128)])
+@pytest.mark.parametrize("nt", [0, 1, 2, 4])
+def test_gemm_skinny_fused_forms(ops, shape, nt):
+    """The folded forms against the separate kernels' references: silu*up in front, add into the
+    32-bit residual behind."""
+    torch.manual_seed(11)
+    M, N, K = shape
+    if nt == 4 and M <= 16:
+        nt = 2
+    w = (torch.randn(N, K, device=DEV) * 0.3).bfloat16()
+    # add into the residual (whose rows must be 16-byte aligned), plain and with silu(gate) * up in front
+    N -= N % 4
+    w = w[:N]
+    a = torch.randn(M, K, device=DEV).bfloat16()
+    stream = torch.randn(M, N, device=DEV)
+    want = stream.cpu() + a.float().cpu() @ w.float().cpu().T
+    ops.gemm_skinny_add(a, w, stream, nt=nt)
+    assert (stream.cpu() - want).abs().max() <= 1e-4 * want.abs().max() + 1e-4
+    gu = torch.randn(M, 2 * K, device=DEV).bfloat16()
+    stream = torch.randn(M, N, device=DEV)
+    act = plain.silu_and_mul(gu.float().cpu()).bfloat16().float()
+    want = stream.cpu() + act @ w.float().cpu().T
+    ops.gemm_skinny_add(gu, w, stream, silu=True, nt=nt)
+    assert (stream.cpu() - want).abs().max() <= 2e-2 * want.abs().max()

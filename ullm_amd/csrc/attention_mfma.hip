@@ -25,6 +25,7 @@ union Pack8 {
   bf16x8_t v;
   uint4 u4;
   uint2 u2[2];
+  uint32_t w[4];
   bf16_t h[8];
 };
 
@@ -124,14 +125,17 @@ __device__ __forceinline__ void attend_range(
     Pack8 p;
     float psum = 0.f;
 #pragma unroll
-    for (int sb = 0; sb < 2; ++sb)
+    for (int sb = 0; sb < 2; ++sb) {
+      float e[4];
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         // a masked score stays at NEG_BIG: its weight is zero even while m_new is still NEG_BIG
-        const float e = s[sb][r] > 0.5f * NEG_BIG ? fast_exp2(s[sb][r] - m_new) : 0.f;
-        psum += e;
-        p.h[4 * sb + r] = f32_to_bf16_bits(e);
+        e[r] = s[sb][r] > 0.5f * NEG_BIG ? fast_exp2(s[sb][r] - m_new) : 0.f;
+        psum += e[r];
       }
+      p.w[2 * sb] = pack2_bf16(e[0], e[1]);
+      p.w[2 * sb + 1] = pack2_bf16(e[2], e[3]);
+    }
     l = l * alpha + psum;
     m = m_new;
     const bool edge = key0 + 32 > max_hi + 1;     // some keys of the tile hold no written data
@@ -244,7 +248,9 @@ attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __re
   }
 }
 
-// Adds the splits' partials [item][head][split][head_dim + 2] in split order.  grid (n_items, nq).
+// Adds the splits' partials [item][head][split][head_dim + 2] in split order.  grid (n_items, nq),
+// one wave: lane s first reads split s's maximum and sum (64 splits at a time), then every lane sums
+// its output dims over the splits with the splits' weights passed round by shuffles.
 __global__ void __launch_bounds__(64)
 attention_reduce_kernel(const float* __restrict__ part, bf16_t* __restrict__ out, int out_stride,
                         const int* __restrict__ token_list, int nq, int hd, int num_splits) {
@@ -253,16 +259,31 @@ attention_reduce_kernel(const float* __restrict__ part, bf16_t* __restrict__ out
   const int row = hd + 2;
   const float* pp = part + ((size_t)item * nq + head) * num_splits * row;
   float M = NEG_BIG;
-  for (int sp = 0; sp < num_splits; ++sp) M = fmaxf(M, pp[sp * row + hd]);
+  for (int s0 = 0; s0 < num_splits; s0 += 64) {
+    const int sp = s0 + lane;
+    M = fmaxf(M, wave_max(sp < num_splits ? pp[sp * row + hd] : NEG_BIG));
+  }
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};       // head_dim <= 256: dims lane, lane + 64, ...
   float L = 0.f;
-  for (int sp = 0; sp < num_splits; ++sp) L += pp[sp * row + hd + 1] * fast_exp2(pp[sp * row + hd] - M);
+  for (int s0 = 0; s0 < num_splits; s0 += 64) {
+    const int sp = s0 + lane;
+    const bool ok = sp < num_splits;
+    const float f = ok ? fast_exp2(pp[sp * row + hd] - M) : 0.f;
+    L += wave_sum(ok ? pp[sp * row + hd + 1] * f : 0.f);
+    const int n = num_splits - s0 < 64 ? num_splits - s0 : 64;
+    for (int j = 0; j < n; ++j) {
+      const float fj = __shfl(f, j, 64);
+      const float* pj = pp + (size_t)(s0 + j) * row;
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (lane + 64 * r < hd) acc[r] += pj[lane + 64 * r] * fj;
+    }
+  }
   const float inv = L > 0.f ? 1.f / L : 0.f;
   bf16_t* op = out + (size_t)t * out_stride + (size_t)head * hd;
-  for (int d = lane; d < hd; d += 64) {
-    float o = 0.f;
-    for (int sp = 0; sp < num_splits; ++sp) o += pp[sp * row + d] * fast_exp2(pp[sp * row + hd] - M);
-    op[d] = f32_to_bf16_bits(o * inv);
-  }
+#pragma unroll
+  for (int r = 0; r < 4; ++r)
+    if (lane + 64 * r < hd) op[lane + 64 * r] = f32_to_bf16_bits(acc[r] * inv);
 }
 
 // ------------------------------------------------------------------------------- prompt portions

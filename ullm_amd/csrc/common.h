@@ -17,12 +17,21 @@ __device__ __forceinline__ float bf16_bits_to_f32(bf16_t v) {
   return __uint_as_float(((uint32_t)v) << 16);
 }
 
-// round to nearest even; NaN stays NaN
+// round to nearest even; NaN stays NaN.  gfx950 converts in hardware (v_cvt_pk_bf16_f32).
 __device__ __forceinline__ bf16_t f32_to_bf16_bits(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x0040u);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (bf16_t)(u >> 16);
+  return __builtin_bit_cast(bf16_t, (__bf16)f);
+}
+typedef __attribute__((ext_vector_type(2))) float ullm_f32x2;
+typedef __attribute__((ext_vector_type(2))) __bf16 ullm_bf16x2;
+// two values in one instruction: low half = a, high half = b
+__device__ __forceinline__ uint32_t pack2_bf16(float a, float b) {
+  const ullm_f32x2 v = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, ullm_bf16x2));
+}
+// silu with the hardware exponential and reciprocal (about 1 ulp each); for results that are rounded
+// to bfloat16 afterwards
+__device__ __forceinline__ float fast_silu(float g) {
+  return g * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-1.4426950408889634f * g));
 }
 
 __device__ __forceinline__ float ld_f32(const float* p) { return *p; }

@@ -8,6 +8,18 @@
 // (ullm/layers/attention.py:288-296).
 #include "common.h"
 
+__device__ __forceinline__ float4 ld4_f32(const float* p) { return *reinterpret_cast<const float4*>(p); }
+__device__ __forceinline__ float4 ld4_f32(const bf16_t* p) {
+  const uint2 u = *reinterpret_cast<const uint2*>(p);
+  return make_float4(__uint_as_float(u.x << 16), __uint_as_float(u.x & 0xffff0000u),
+                     __uint_as_float(u.y << 16), __uint_as_float(u.y & 0xffff0000u));
+}
+__device__ __forceinline__ void st4_f32(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
+__device__ __forceinline__ void st4_f32(bf16_t* p, float4 v) {
+  *reinterpret_cast<uint2*>(p) = make_uint2(pack2_bf16(v.x, v.y), pack2_bf16(v.z, v.w));
+}
+
+
 // ------------------------------------------------------------------ embedding
 // residual[t, :] = float(table[ids[t], :]); ids outside [0, V) give a zero row.
 template <typename T>
@@ -21,6 +33,11 @@ __global__ void embedding_kernel(const int* __restrict__ ids, const T* __restric
     return;
   }
   const T* row = table + (size_t)id * H;
+  if (H % 4 == 0 && !(((uintptr_t)table | (uintptr_t)residual) & 15)) {
+    for (int i = 4 * threadIdx.x; i < H; i += 4 * blockDim.x)
+      *reinterpret_cast<float4*>(out + i) = ld4_f32(row + i);
+    return;
+  }
   for (int i = threadIdx.x; i < H; i += blockDim.x) out[i] = ld_f32(row + i);
 }
 
@@ -43,6 +60,9 @@ extern "C" int ullm_embedding(const int* ids, const void* table, float* residual
 //   s = residual[i] + float(branch[i])      (branch may be null: s = residual[i])
 //   if write_res: residual[i] = s           (the stream stays 32-bit, never rounded)
 //   y[r] = s * rsqrt(mean(s^2) + eps) * gain
+// One block per row.  The general kernel walks the row twice with scalar loads; the fast one
+// (H a multiple of 4 and at most 4 * 4 * blockDim) keeps the row's sums in registers between the
+// reduction and the scaling and moves 16 bytes per lane and access.
 template <typename TB, typename TY>
 __global__ void add_rmsnorm_kernel(const TB* __restrict__ branch, float* __restrict__ residual,
                                    const float* __restrict__ gain, float eps, TY* __restrict__ y,
@@ -69,21 +89,83 @@ __global__ void add_rmsnorm_kernel(const TB* __restrict__ branch, float* __restr
   }
 }
 
+#define NORM_VEC_MAX 4     // float4 groups per thread
+template <typename TB, typename TY>
+__global__ void add_rmsnorm_vec_kernel(const TB* __restrict__ branch, float* __restrict__ residual,
+                                       const float* __restrict__ gain, float eps, TY* __restrict__ y,
+                                       const int* __restrict__ rows, int H, int write_res) {
+  __shared__ float scratch[16];
+  const int r = blockIdx.x;
+  const int i = rows ? rows[r] : r;
+  float* res = residual + (size_t)i * H;
+  const TB* br = branch ? branch + (size_t)i * H : nullptr;
+  float4 v[NORM_VEC_MAX];
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < NORM_VEC_MAX; ++j) {
+    const int c = 4 * (threadIdx.x + j * blockDim.x);
+    if (c < H) {
+      float4 s = ld4_f32(res + c);
+      if (br) {
+        const float4 b = ld4_f32(br + c);
+        s.x += b.x; s.y += b.y; s.z += b.z; s.w += b.w;
+        if (write_res) st4_f32(res + c, s);
+      }
+      v[j] = s;
+      ss += s.x * s.x + s.y * s.y + s.z * s.z + s.w * s.w;
+    }
+  }
+  const float rs = rsqrtf(block_sum(ss, scratch) / (float)H + eps);
+  TY* out = y + (size_t)r * H;
+#pragma unroll
+  for (int j = 0; j < NORM_VEC_MAX; ++j) {
+    const int c = 4 * (threadIdx.x + j * blockDim.x);
+    if (c < H) {
+      const float4 g = ld4_f32(gain + c);
+      st4_f32(out + c, make_float4((v[j].x * rs) * g.x, (v[j].y * rs) * g.y, (v[j].z * rs) * g.z, (v[j].w * rs) * g.w));
+    }
+  }
+}
+
 extern "C" int ullm_add_rmsnorm(const void* branch, float* residual, const float* gain, float eps,
                                 void* y, const int* rows, int n_rows, int H, int branch_dtype,
                                 int y_dtype, int write_res, hipStream_t stream) {
   if (n_rows <= 0) return 0;
   if (H <= 0) return ULLM_ERR_SHAPE;
   if (rows && write_res) return ULLM_ERR_UNSUPPORTED;  // a gathered row could be updated twice
-  dim3 grid(n_rows), block(H >= 2048 ? 512 : 256);
-#define GO(TB, TY) hipLaunchKernelGGL((add_rmsnorm_kernel<TB, TY>), grid, block, 0, stream, \
-    (const TB*)branch, residual, gain, eps, (TY*)y, rows, H, write_res)
+  const int threads = H >= 4096 ? 512 : 256;
+  const bool vec = H % 4 == 0 && H <= 4 * NORM_VEC_MAX * threads && !(((uintptr_t)residual | (uintptr_t)gain |
+                   (uintptr_t)y | (uintptr_t)branch) & 15);
+  dim3 grid(n_rows), block(threads);
+#define GO(TB, TY) do { if (vec) hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TB, TY>), grid, block, 0, stream, \
+    (const TB*)branch, residual, gain, eps, (TY*)y, rows, H, write_res); \
+  else hipLaunchKernelGGL((add_rmsnorm_kernel<TB, TY>), grid, block, 0, stream, \
+    (const TB*)branch, residual, gain, eps, (TY*)y, rows, H, write_res); } while (0)
   if (branch_dtype == ULLM_F32 && y_dtype == ULLM_F32) GO(float, float);
   else if (branch_dtype == ULLM_BF16 && y_dtype == ULLM_BF16) GO(bf16_t, bf16_t);
   else if (branch_dtype == ULLM_BF16 && y_dtype == ULLM_F32) GO(bf16_t, float);
   else if (branch_dtype == ULLM_F32 && y_dtype == ULLM_BF16) GO(float, bf16_t);
   else return ULLM_ERR_DTYPE;
 #undef GO
+  ULLM_LAUNCH_CHECK();
+}
+
+// ------------------------------------------------------------------ residual += branch
+template <typename T>
+__global__ void residual_add_kernel(const T* __restrict__ branch, float* __restrict__ residual, size_t total) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx < total) residual[idx] += ld_f32(branch + idx);
+}
+
+extern "C" int ullm_residual_add(const void* branch, float* residual, long long total, int dtype, hipStream_t stream) {
+  if (total <= 0) return 0;
+  dim3 block(256), grid((unsigned)((total + 255) / 256));
+  if (dtype == ULLM_F32)
+    hipLaunchKernelGGL(residual_add_kernel<float>, grid, block, 0, stream, (const float*)branch, residual, (size_t)total);
+  else if (dtype == ULLM_BF16)
+    hipLaunchKernelGGL(residual_add_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)branch, residual, (size_t)total);
+  else
+    return ULLM_ERR_DTYPE;
   ULLM_LAUNCH_CHECK();
 }
 
@@ -96,14 +178,45 @@ __global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, i
   const int i = (int)(idx - t * I);
   const T* row = gu + t * (size_t)(2 * I);
   const float g = ld_f32(row + i), u = ld_f32(row + I + i);
-  const float s = g / (1.f + expf(-g));
+  // 32-bit mode: exact exponential and division; bfloat16: the hardware's, then rounded
+  const float s = sizeof(T) == 4 ? g / (1.f + expf(-g)) : fast_silu(g);
   st_f32(out + idx, s * u);
+}
+
+template <typename T>
+__global__ void silu_mul_vec_kernel(const T* __restrict__ gu, T* __restrict__ out, int I, size_t total4) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;    // group of 4 consecutive outputs
+  if (idx >= total4) return;
+  const size_t per_row = (size_t)(I / 4);
+  const size_t t = idx / per_row;
+  const int i = 4 * (int)(idx - t * per_row);
+  const T* row = gu + t * (size_t)(2 * I);
+  const float4 g = ld4_f32(row + i), u = ld4_f32(row + I + i);
+  float4 o;
+  if (sizeof(T) == 4) {
+    o = make_float4(g.x / (1.f + expf(-g.x)) * u.x, g.y / (1.f + expf(-g.y)) * u.y,
+                    g.z / (1.f + expf(-g.z)) * u.z, g.w / (1.f + expf(-g.w)) * u.w);
+  } else {
+    o = make_float4(fast_silu(g.x) * u.x, fast_silu(g.y) * u.y, fast_silu(g.z) * u.z, fast_silu(g.w) * u.w);
+  }
+  st4_f32(out + t * (size_t)I + i, o);
 }
 
 extern "C" int ullm_silu_mul(const void* gu, void* out, int T_, int I, int dtype, hipStream_t stream) {
   if (T_ <= 0) return 0;
   if (I <= 0) return ULLM_ERR_SHAPE;
   const size_t total = (size_t)T_ * I;
+  if (I % 4 == 0 && !(((uintptr_t)gu | (uintptr_t)out) & 15)) {
+    const size_t total4 = total / 4;
+    dim3 vblock(256), vgrid((unsigned)((total4 + 255) / 256));
+    if (dtype == ULLM_F32)
+      hipLaunchKernelGGL(silu_mul_vec_kernel<float>, vgrid, vblock, 0, stream, (const float*)gu, (float*)out, I, total4);
+    else if (dtype == ULLM_BF16)
+      hipLaunchKernelGGL(silu_mul_vec_kernel<bf16_t>, vgrid, vblock, 0, stream, (const bf16_t*)gu, (bf16_t*)out, I, total4);
+    else
+      return ULLM_ERR_DTYPE;
+    ULLM_LAUNCH_CHECK();
+  }
   dim3 block(256), grid((unsigned)((total + 255) / 256));
   if (dtype == ULLM_F32)
     hipLaunchKernelGGL(silu_mul_kernel<float>, grid, block, 0, stream, (const float*)gu, (float*)out, I, total);

@@ -1,14 +1,24 @@
-// C[M, N] = A[M, K] * W[N, K]^T (+ bias) for few rows (M <= 64), bfloat16 operands, 32-bit
-// accumulation, output bfloat16 or float32.  This is the decode-time matrix product: its time is the
-// time to stream W once from HBM, so the kernel is built around the weight loads.
+// C[M, N] = X[M, K] * W[N, K]^T for few rows (M <= 64), bfloat16 weights streamed once from HBM through
+// the matrix cores, 32-bit accumulation.  This is the decode-time matrix product: its time is the time
+// to read W, so the kernel is built around the weight loads, and the small row-wise operations that
+// surround a projection in a decoder layer are folded into it so that they cost no launch and no
+// pass over memory of their own:
 //
-// A block owns 16 consecutive rows of W (16 output columns); its waves split K between them.  Per 32
-// values of K a wave issues one 16-byte load per lane straight from global memory for the W tile
-// (A operand of v_mfma_f32_16x16x32_bf16: lane (r, g) holds W[n0 + r][k + 8g .. +8]) and one per
-// 16 rows of the activations (B operand: lane (m, g) holds A[m][k + 8g .. +8]; the activations are
-// small and stay in cache).  The loop is unrolled so that many loads are in flight.  The waves'
-// partial 16x16 results are added in wave order through shared memory, so the result does not depend
-// on timing.  Weights are [out, in] (ullm/layers/linear.py:165).
+//   how X is produced (PRO)
+//     PLAIN : X is a bfloat16 matrix
+//     SILU  : X = silu(G[:, :K]) * G[:, K:] with G the bfloat16 [M, 2K] gate|up matrix
+//             (ullm/layers/activation.py:16-18 followed by down_proj, ullm/models/qwen3.py:44-45)
+//   what happens to the result (EPI)
+//     STORE : C = result (+ bias), bfloat16 or float32
+//     RESADD: R[M, N] += result, the 32-bit residual stream (the add the reference leaves to the next
+//             norm, ullm/layers/layernorm.py:24-26)
+//
+// A block owns NT x 16 consecutive rows of W; its waves split K between them.  Per 32 values of K a
+// wave issues one 16-byte load per lane and W tile straight from global memory (A operand of
+// v_mfma_f32_16x16x32_bf16: lane (r, g) holds W[n0 + r][k + 8g .. +8]) and builds the B operand
+// (lane (m, g) holds X[m][k + 8g .. +8]) per 16 rows of X.  The waves' partial results are added in
+// wave order through shared memory, so the result does not depend on timing.
+// Weights are [out, in] (ullm/layers/linear.py:165).
 #include "common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
@@ -17,122 +27,214 @@ typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 union Pack8 {
   bf16x8_t v;
   uint4 u4;
+  uint32_t w[4];
+  bf16_t h[8];
 };
 
-#define SK_MAX_WAVES 16
-#define SK_UNROLL 4
+enum { PRO_PLAIN = 0, PRO_SILU = 2 };
+enum { EPI_STORE = 0, EPI_RESADD = 1 };
 
-// MT = number of 16-row tiles of A (M <= 16 * MT).
-template <int MT, typename TC>
-__global__ void __launch_bounds__(64 * SK_MAX_WAVES)
-gemm_skinny_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, int ldw,
-                   const float* __restrict__ bias, TC* __restrict__ C, int ldc, int M, int N, int K,
-                   int k_per_wave) {
-  __shared__ float red[SK_MAX_WAVES - 1][MT][64 * 4];   // wave 0 adds the others' partials to its own
+// most waves per block for a tile shape: bounded by the shared memory that holds the waves' partials
+__host__ __device__ constexpr int sk_max_waves(int mt, int nt) { return mt * nt >= 8 ? 4 : (mt * nt >= 4 ? 8 : 16); }
+
+template <int PRO>
+__device__ __forceinline__ Pack8 load_x(const bf16_t* __restrict__ X, size_t row_off, int k, int silu_off) {
+  Pack8 x;
+  if (PRO == PRO_PLAIN) {
+    x.u4 = *reinterpret_cast<const uint4*>(X + row_off + k);
+  } else {
+    Pack8 gt, up;
+    gt.u4 = *reinterpret_cast<const uint4*>(X + row_off + k);
+    up.u4 = *reinterpret_cast<const uint4*>(X + row_off + silu_off + k);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      // low and high halves of a 32-bit word are two bfloat16 values
+      const float g0 = __uint_as_float(gt.w[j] << 16), g1 = __uint_as_float(gt.w[j] & 0xffff0000u);
+      const float u0 = __uint_as_float(up.w[j] << 16), u1 = __uint_as_float(up.w[j] & 0xffff0000u);
+      x.w[j] = pack2_bf16(fast_silu(g0) * u0, fast_silu(g1) * u1);
+    }
+  }
+  return x;
+}
+
+// MT = 16-row tiles of X (M <= 16 MT); NT = 16-row tiles of W per block.
+template <int MT, int NT, int PRO, int EPI, typename TC>
+__global__ void __launch_bounds__(64 * sk_max_waves(MT, NT))
+gemm_skinny_kernel(const bf16_t* __restrict__ X, int ldx, const bf16_t* __restrict__ W, int ldw,
+                   const float* __restrict__ bias, TC* __restrict__ C, float* __restrict__ R, int ldc, int M,
+                   int N, int K, int k_per_wave) {
+  constexpr int MAXW = sk_max_waves(MT, NT);
+  __shared__ float red[MAXW - 1][NT * MT][64 * 4];   // wave 0 adds the others' partials to its own
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
   const int g = lane >> 4, r = lane & 15;
-  const int n0 = blockIdx.x * 16;
-  const int n = n0 + r < N ? n0 + r : N - 1;          // rows past N repeat the last row; never stored
-  const bf16_t* wp = W + (size_t)n * ldw + 8 * g;
-  const bf16_t* ap[MT];
+  const int n0 = blockIdx.x * (16 * NT);
+  const bf16_t* wp[NT];
+#pragma unroll
+  for (int i = 0; i < NT; ++i) {
+    const int n = n0 + 16 * i + r < N ? n0 + 16 * i + r : N - 1;   // rows past N repeat the last row; never stored
+    wp[i] = W + (size_t)n * ldw + 8 * g;
+  }
+  size_t xo[MT];
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
     const int m = 16 * t + r < M ? 16 * t + r : M - 1;
-    ap[t] = A + (size_t)m * lda + 8 * g;
+    xo[t] = (size_t)m * ldx + 8 * g;
   }
-  f32x4_t acc[MT];
+  f32x4_t acc[NT][MT];
 #pragma unroll
-  for (int t = 0; t < MT; ++t) acc[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-
+  for (int t = 0; t < MT; ++t)
+#pragma unroll
+    for (int i = 0; i < NT; ++i) acc[i][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   const int k_begin = wave * k_per_wave;
   int k_end = k_begin + k_per_wave;
   if (k_end > K) k_end = K;
   int k = k_begin;
-  // full steps of SK_UNROLL * 32 values
-  for (; k + 32 * SK_UNROLL <= k_end; k += 32 * SK_UNROLL) {
-    Pack8 w[SK_UNROLL], a[SK_UNROLL][MT];
+  constexpr int U = (NT * MT >= 8) ? 1 : ((NT + MT >= 5) ? 2 : 4);       // steps of 32 in flight per wave
+  for (; k + 32 * U <= k_end; k += 32 * U) {
+    Pack8 w[U][NT], x[U][MT];
 #pragma unroll
-    for (int u = 0; u < SK_UNROLL; ++u) w[u].u4 = *reinterpret_cast<const uint4*>(wp + k + 32 * u);
+    for (int u = 0; u < U; ++u)
 #pragma unroll
-    for (int u = 0; u < SK_UNROLL; ++u)
+      for (int i = 0; i < NT; ++i) w[u][i].u4 = *reinterpret_cast<const uint4*>(wp[i] + k + 32 * u);
 #pragma unroll
-      for (int t = 0; t < MT; ++t) a[u][t].u4 = *reinterpret_cast<const uint4*>(ap[t] + k + 32 * u);
+    for (int u = 0; u < U; ++u)
 #pragma unroll
-    for (int u = 0; u < SK_UNROLL; ++u)
+      for (int t = 0; t < MT; ++t) x[u][t] = load_x<PRO>(X, xo[t], k + 32 * u, K);
 #pragma unroll
-      for (int t = 0; t < MT; ++t)
-        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[u].v, a[u][t].v, acc[t], 0, 0, 0);
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int i = 0; i < NT; ++i)
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+          acc[i][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[u][i].v, x[u][t].v, acc[i][t], 0, 0, 0);
   }
   // remaining steps of 32, the last one possibly short (K is a multiple of 8)
   for (; k < k_end; k += 32) {
-    Pack8 w;
     const bool in = k + 8 * g < k_end;
-    w.u4 = in ? *reinterpret_cast<const uint4*>(wp + k) : make_uint4(0, 0, 0, 0);
+    Pack8 w[NT], x[MT];
+#pragma unroll
+    for (int i = 0; i < NT; ++i) w[i].u4 = in ? *reinterpret_cast<const uint4*>(wp[i] + k) : make_uint4(0, 0, 0, 0);
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
-      Pack8 a;
-      a.u4 = in ? *reinterpret_cast<const uint4*>(ap[t] + k) : make_uint4(0, 0, 0, 0);
-      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w.v, a.v, acc[t], 0, 0, 0);
+      if (in) x[t] = load_x<PRO>(X, xo[t], k, K);
+      else x[t].u4 = make_uint4(0, 0, 0, 0);
     }
+#pragma unroll
+    for (int i = 0; i < NT; ++i)
+#pragma unroll
+      for (int t = 0; t < MT; ++t)
+        acc[i][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[i].v, x[t].v, acc[i][t], 0, 0, 0);
   }
-  // acc[t][j] = partial C[m = 16 t + r][n0 + 4 g + j]; add the waves' partials in wave order
+  // acc[i][t][j] = partial C[m = 16 t + r][n0 + 16 i + 4 g + j]; add the waves' partials in wave order
   if (nwaves > 1) {
     if (wave != 0) {
 #pragma unroll
-      for (int t = 0; t < MT; ++t)
-        *reinterpret_cast<float4*>(&red[wave - 1][t][lane * 4]) = make_float4(acc[t][0], acc[t][1], acc[t][2], acc[t][3]);
+      for (int i = 0; i < NT; ++i)
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+          *reinterpret_cast<float4*>(&red[wave - 1][i * MT + t][lane * 4]) =
+              make_float4(acc[i][t][0], acc[i][t][1], acc[i][t][2], acc[i][t][3]);
     }
     __syncthreads();
     if (wave != 0) return;
 #pragma unroll
-    for (int t = 0; t < MT; ++t)
-      for (int w = 1; w < nwaves; ++w) {
-        const float4 o = *reinterpret_cast<const float4*>(&red[w - 1][t][lane * 4]);
-        acc[t][0] += o.x; acc[t][1] += o.y; acc[t][2] += o.z; acc[t][3] += o.w;
-      }
+    for (int i = 0; i < NT; ++i)
+#pragma unroll
+      for (int t = 0; t < MT; ++t)
+        for (int w = 1; w < nwaves; ++w) {
+          const float4 o = *reinterpret_cast<const float4*>(&red[w - 1][i * MT + t][lane * 4]);
+          acc[i][t][0] += o.x; acc[i][t][1] += o.y; acc[i][t][2] += o.z; acc[i][t][3] += o.w;
+        }
   }
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
     const int m = 16 * t + r;
     if (m >= M) continue;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int nn = n0 + 4 * g + j;
-      if (nn < N) st_f32(C + (size_t)m * ldc + nn, acc[t][j] + (bias ? bias[nn] : 0.f));
+    for (int i = 0; i < NT; ++i) {
+      const int nn = n0 + 16 * i + 4 * g;
+      if (EPI == EPI_RESADD) {
+        float* rp = R + (size_t)m * ldc + nn;
+        if (nn + 3 < N) {
+          float4 o = *reinterpret_cast<float4*>(rp);
+          o.x += acc[i][t][0]; o.y += acc[i][t][1]; o.z += acc[i][t][2]; o.w += acc[i][t][3];
+          *reinterpret_cast<float4*>(rp) = o;
+        } else {
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            if (nn + j < N) rp[j] += acc[i][t][j];
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          if (nn + j < N) st_f32(C + (size_t)m * ldc + nn + j, acc[i][t][j] + (bias ? bias[nn + j] : 0.f));
+      }
     }
   }
 }
 
-extern "C" int ullm_gemm_skinny_supports(int M, int N, int K, int lda, int ldw) {
-  return M >= 1 && M <= 64 && N >= 1 && K >= 8 && K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0;
+extern "C" int ullm_gemm_skinny_supports(int M, int N, int K, int ldx, int ldw) {
+  return M >= 1 && M <= 64 && N >= 1 && K >= 8 && K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0;
 }
 
-extern "C" int ullm_gemm_skinny(const void* A, int lda, const void* W, int ldw, const float* bias, void* C,
-                                int ldc, int M, int N, int K, int c_dtype, hipStream_t stream) {
+// pro: 0 plain (X bfloat16 [M, K]), 2 silu (X bfloat16 [M, 2K]).  epi: 0 store to C (c_dtype, bias
+// optional), 1 add into R (float32 [M, N], row stride ldc).  force_nt / force_waves: 0 = chosen here.
+extern "C" int ullm_gemm_skinny(const void* X, int ldx, const void* W, int ldw, const float* bias, void* C,
+                                int ldc, int M, int N, int K, int pro, int epi, int c_dtype, int force_nt,
+                                int force_waves, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
-  if (!ullm_gemm_skinny_supports(M, N, K, lda, ldw) || ldc < N) return ULLM_ERR_SHAPE;
-  if (((uintptr_t)A & 15) || ((uintptr_t)W & 15)) return ULLM_ERR_SHAPE;
-  const int tiles = (N + 15) / 16;
+  if (!ullm_gemm_skinny_supports(M, N, K, ldx, ldw) || ldc < N) return ULLM_ERR_SHAPE;
+  if (((uintptr_t)X & 15) || ((uintptr_t)W & 15)) return ULLM_ERR_SHAPE;
+  if ((pro != PRO_PLAIN && pro != PRO_SILU) || epi < 0 || epi > 1) return ULLM_ERR_UNSUPPORTED;
+  if (pro == PRO_SILU && ldx < 2 * K) return ULLM_ERR_SHAPE;
+  if (epi == EPI_RESADD && (((uintptr_t)C & 15) || ldc % 4 != 0 || bias)) return ULLM_ERR_SHAPE;
+  int mt = (M + 15) / 16;
+  if (mt == 3) mt = 4;                                  // instantiated for 1, 2 and 4 tiles of rows
+  const int tiles16 = (N + 15) / 16;
+  int nt = 1;
+  if (force_nt > 0) nt = force_nt;
+  else if (tiles16 >= 4096) nt = mt >= 2 ? 4 : 2;
+  else if (tiles16 >= 1024 && mt >= 2) nt = 2;
+  if (nt != 1 && nt != 2 && nt != 4) return ULLM_ERR_UNSUPPORTED;
+  if (nt == 4 && mt == 1) nt = 2;                       // not instantiated
+  const int tiles = (tiles16 + nt - 1) / nt;
   // waves per block: enough blocks x waves to fill the chip, each wave with at least 128 values of K
+  const int max_waves = sk_max_waves(mt, nt);
   int waves = 1;
-  while (waves < SK_MAX_WAVES && tiles * waves < 4096 && K / (waves * 2) >= 128) waves *= 2;
+  while (waves < max_waves && tiles * waves < 4096 && K / (waves * 2) >= 128) waves *= 2;
+  if (force_waves > 0) waves = force_waves < max_waves ? force_waves : max_waves;
   int k_per_wave = (K + waves - 1) / waves;
   k_per_wave = (k_per_wave + 31) / 32 * 32;
-  const int mt = (M + 15) / 16;
   dim3 grid(tiles), block(64 * waves);
-#define GO(MT, TC) hipLaunchKernelGGL((gemm_skinny_kernel<MT, TC>), grid, block, 0, stream, (const bf16_t*)A, lda, \
-    (const bf16_t*)W, ldw, bias, (TC*)C, ldc, M, N, K, k_per_wave)
-#define GO_MT(TC)                 \
-  switch (mt) {                   \
-    case 1: GO(1, TC); break;     \
-    case 2: GO(2, TC); break;     \
-    case 3: GO(3, TC); break;     \
-    default: GO(4, TC); break;    \
+  float* R = (float*)C;
+#define GO(MT, NT, PRO, EPI, TC) hipLaunchKernelGGL((gemm_skinny_kernel<MT, NT, PRO, EPI, TC>), grid, block, 0, stream, \
+    (const bf16_t*)X, ldx, (const bf16_t*)W, ldw, bias, (TC*)C, R, ldc, M, N, K, k_per_wave)
+#define GO_SHAPE(PRO, EPI, TC)                                              \
+  switch (mt * 8 + nt) {                                                    \
+    case 1 * 8 + 1: GO(1, 1, PRO, EPI, TC); break;                          \
+    case 1 * 8 + 2: GO(1, 2, PRO, EPI, TC); break;                          \
+    case 2 * 8 + 1: GO(2, 1, PRO, EPI, TC); break;                          \
+    case 2 * 8 + 2: GO(2, 2, PRO, EPI, TC); break;                          \
+    case 2 * 8 + 4: GO(2, 4, PRO, EPI, TC); break;                          \
+    case 4 * 8 + 1: GO(4, 1, PRO, EPI, TC); break;                          \
+    case 4 * 8 + 2: GO(4, 2, PRO, EPI, TC); break;                          \
+    case 4 * 8 + 4: GO(4, 4, PRO, EPI, TC); break;                          \
+    default: return ULLM_ERR_UNSUPPORTED;                                   \
   }
-  if (c_dtype == ULLM_BF16) { GO_MT(bf16_t) }
-  else if (c_dtype == ULLM_F32) { GO_MT(float) }
-  else return ULLM_ERR_DTYPE;
-#undef GO_MT
+  if (epi == EPI_STORE) {
+    if (pro == PRO_PLAIN) {
+      if (c_dtype == ULLM_BF16) { GO_SHAPE(PRO_PLAIN, EPI_STORE, bf16_t) }
+      else if (c_dtype == ULLM_F32) { GO_SHAPE(PRO_PLAIN, EPI_STORE, float) }
+      else return ULLM_ERR_DTYPE;
+    } else {
+      return ULLM_ERR_UNSUPPORTED;
+    }
+  } else {
+    if (pro == PRO_PLAIN) { GO_SHAPE(PRO_PLAIN, EPI_RESADD, float) }
+    else if (pro == PRO_SILU) { GO_SHAPE(PRO_SILU, EPI_RESADD, float) }
+    else return ULLM_ERR_UNSUPPORTED;
+  }
+#undef GO_SHAPE
 #undef GO
   ULLM_LAUNCH_CHECK();
 }

@@ -41,6 +41,40 @@ __device__ __forceinline__ float uniform_from_seed(uint64_t seed, uint32_t posit
   return (float)(uint32_t)(z >> 40) * (1.0f / 16777216.0f);
 }
 
+// Visits the elements [wbeg, wend) of a wave's range, lane-strided, with several independent loads
+// in flight per lane.  VEC: 16-byte loads (the row must be 16-byte aligned and wbeg, wend multiples
+// of 4): a lane gets 4 consecutive values, the wave 256 consecutive values per access.
+template <bool VEC, typename F>
+__device__ __forceinline__ void for_range(const float* __restrict__ x, int wbeg, int wend, int lane, F f) {
+  if (VEC) {
+    for (int i0 = wbeg + 4 * lane; i0 < wend; i0 += 4 * 4 * WAVE) {
+      float4 v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int ii = i0 + u * 4 * WAVE;
+        v[u] = ii < wend ? *reinterpret_cast<const float4*>(x + ii) : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int ii = i0 + u * 4 * WAVE;
+        if (ii < wend) { f(ii, v[u].x); f(ii + 1, v[u].y); f(ii + 2, v[u].z); f(ii + 3, v[u].w); }
+      }
+    }
+  } else {
+    for (int i0 = wbeg + lane; i0 < wend; i0 += 4 * WAVE) {
+      float v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) v[u] = i0 + u * WAVE < wend ? x[i0 + u * WAVE] : 0.f;
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        if (i0 + u * WAVE < wend) f(i0 + u * WAVE, v[u]);
+    }
+  }
+}
+
+// Each wave owns a contiguous range of the vocabulary, so sums over a wave's range are sums over
+// consecutive indices and the draw can walk the index order wave by wave.
+template <bool VEC>
 __global__ void __launch_bounds__(SAMPLE_THREADS)
 sample_kernel(const float* __restrict__ logits, int V, int ld, const float* __restrict__ temperature,
               const int* __restrict__ top_k, const float* __restrict__ top_p,
@@ -49,45 +83,47 @@ sample_kernel(const float* __restrict__ logits, int V, int ld, const float* __re
               int* __restrict__ out) {
   __shared__ float fscratch[16];
   __shared__ int iscratch[16];
-  __shared__ float wave_incl[16];
+  __shared__ float wave_tot[16];
   __shared__ int chosen;
-  __shared__ float part[SAMPLE_THREADS];
-  const int row = blockIdx.x, tid = threadIdx.x, nthreads = blockDim.x;
+  constexpr int STEP = VEC ? 4 * WAVE : WAVE;        // values a wave reads per access
+  const int row = blockIdx.x, tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
+  const int nwaves = blockDim.x / WAVE;
   const float* x = logits + (size_t)row * ld;
   const float t = temperature[row];
-  const int chunk = (V + nthreads - 1) / nthreads;
-  const int begin = tid * chunk < V ? tid * chunk : V;
-  const int end = begin + chunk < V ? begin + chunk : V;
+  const int per = ((V + nwaves - 1) / nwaves + STEP - 1) / STEP * STEP;
+  const int wbeg = wave * per < V ? wave * per : V;
+  const int wend = wbeg + per < V ? wbeg + per : V;
 
   if (t == 0.f) {  // greedy: first index of the maximum
     float best = -INFINITY;
     int best_i = 0x7fffffff;
-    for (int i = begin; i < end; ++i) {
-      const float v = x[i];
+    for_range<VEC>(x, wbeg, wend, lane, [&](int i, float v) {
       if (v > best || best_i == 0x7fffffff) { best = v; best_i = i; }
-    }
+    });
     const float m = block_max(best, fscratch);
     int cand = (best == m && best_i != 0x7fffffff) ? best_i : 0x7fffffff;
-    // smallest index among the holders of the maximum
 #pragma unroll
     for (int s = WAVE / 2; s > 0; s >>= 1) { const int o = __shfl_xor(cand, s, WAVE); cand = o < cand ? o : cand; }
     __syncthreads();
-    if ((tid & (WAVE - 1)) == 0) iscratch[tid / WAVE] = cand;
+    if (lane == 0) iscratch[wave] = cand;
     __syncthreads();
     if (tid == 0) {
       int r = 0x7fffffff;
-      for (int w = 0; w < (nthreads + WAVE - 1) / WAVE; ++w) r = iscratch[w] < r ? iscratch[w] : r;
+      for (int w = 0; w < nwaves; ++w) r = iscratch[w] < r ? iscratch[w] : r;
       out[row] = r == 0x7fffffff ? 0 : r;
     }
     return;
   }
 
-  const float temp = t < 0.f ? 1.f : t;  // the reference maps T <= 0 to 1 (sampler.py:41)
+  // z = x / T is taken as x * (1 / T); the exponential is the hardware's 2^x
+  const float inv_t = 1.f / (t < 0.f ? 1.f : t);  // the reference maps T <= 0 to 1 (sampler.py:41)
+  const float L2E = 1.4426950408889634f;
   float mloc = -INFINITY;
-  for (int i = begin; i < end; ++i) mloc = fmaxf(mloc, x[i] / temp);
+  for_range<VEC>(x, wbeg, wend, lane, [&](int, float v) { mloc = fmaxf(mloc, v * inv_t); });
   const float m = block_max(mloc, fscratch);
   const uint32_t key_max = order_key(m);
   uint32_t kmin = 0;
+#define E_OF(z) __builtin_amdgcn_exp2f(((z) - m) * L2E)
 
   const int k = top_k[row];
   if (k > 0 && k < V) {  // largest key v with #{key >= v} >= k
@@ -95,7 +131,7 @@ sample_kernel(const float* __restrict__ logits, int V, int ld, const float* __re
     while (lo < hi) {
       const uint32_t mid = lo + (hi - lo + 1) / 2;
       int c = 0;
-      for (int i = begin; i < end; ++i) c += order_key(x[i] / temp) >= mid;
+      for_range<VEC>(x, wbeg, wend, lane, [&](int, float v) { c += order_key(v * inv_t) >= mid; });
       if (block_sum_int(c, iscratch) >= k) lo = mid; else hi = mid - 1;
     }
     kmin = lo;
@@ -104,77 +140,101 @@ sample_kernel(const float* __restrict__ logits, int V, int ld, const float* __re
   const float p = top_p[row];
   if (p > 0.f && p < 1.f) {  // smallest key v with (mass of keys > v) < p * (mass kept so far)
     float s = 0.f;
-    for (int i = begin; i < end; ++i) {
-      const float z = x[i] / temp;
-      if (order_key(z) >= kmin) s += expf(z - m);
-    }
+    for_range<VEC>(x, wbeg, wend, lane, [&](int, float v) {
+      const float z = v * inv_t;
+      if (order_key(z) >= kmin) s += E_OF(z);
+    });
     const float bound = p * block_sum(s, fscratch);
     uint32_t lo = kmin, hi = key_max;
     while (lo < hi) {
       const uint32_t mid = lo + (hi - lo) / 2;
       float a = 0.f;
-      for (int i = begin; i < end; ++i) {
-        const float z = x[i] / temp;
-        if (order_key(z) > mid) a += expf(z - m);
-      }
+      for_range<VEC>(x, wbeg, wend, lane, [&](int, float v) {
+        const float z = v * inv_t;
+        if (order_key(z) > mid) a += E_OF(z);
+      });
       if (block_sum(a, fscratch) < bound) hi = mid; else lo = mid + 1;
     }
     kmin = lo;
   }
 
   const float mp = min_p[row];
-  // partial sums over contiguous index ranges, then a scan in thread (= index) order
   float s = 0.f;
-  for (int i = begin; i < end; ++i) {
-    const float z = x[i] / temp;
-    const float e = expf(z - m);
+  for_range<VEC>(x, wbeg, wend, lane, [&](int, float v) {
+    const float z = v * inv_t;
+    const float e = E_OF(z);
     if (order_key(z) >= kmin && e >= mp) s += e;
-  }
-  // inclusive scan in thread order, built from sequential sums only, so that it never decreases
-  const int lane = tid & (WAVE - 1), wave = tid / WAVE;
-  const int nwaves = (nthreads + WAVE - 1) / WAVE;
+  });
+  s = wave_sum(s);
   if (tid == 0) chosen = -1;
-  part[tid] = s;
+  if (lane == 0) wave_tot[wave] = s;
   __syncthreads();
-  if (lane == 0) {
-    float run = 0.f;
-    const int stop = (wave + 1) * WAVE < nthreads ? (wave + 1) * WAVE : nthreads;
-    for (int j = wave * WAVE; j < stop; ++j) { run += part[j]; part[j] = run; }
-    wave_incl[wave] = run;
+  float base = 0.f, total = 0.f;
+  for (int w = 0; w < nwaves; ++w) {       // sequential sums: the running total never decreases
+    if (w == wave) base = total;
+    total += wave_tot[w];
   }
-  __syncthreads();
-  float wave_base = 0.f, total = 0.f;
-  for (int w = 0; w < nwaves; ++w) {
-    if (w == wave) wave_base = total;
-    total += wave_incl[w];
-  }
-  const float incl = wave_base + part[tid];
-  const float prev_incl = lane == 0 ? wave_base : wave_base + part[tid - 1];
   const uint64_t seed = ((uint64_t)seed_hi[row] << 32) | (uint64_t)seed_lo[row];
   const float target = uniform_from_seed(seed, (uint32_t)position[row]) * total;
-  const bool mine = s > 0.f && incl > target && !(prev_incl > target);
+  const bool mine = s > 0.f && base + s > target && !(base > target);   // exactly one wave
   if (mine) {
-    // walk this thread's range from the exact running value of the scan
-    float run = prev_incl;
+    // walk this wave's range in index order, STEP values at a time (the next ones already loading)
+    constexpr int PER = VEC ? 4 : 1;
+    float run = base;
     int pick = -1, last_kept = -1;
-    for (int i = begin; i < end; ++i) {
-      const float z = x[i] / temp;
-      const float e = expf(z - m);
-      if (order_key(z) >= kmin && e >= mp) {
-        run += e;
-        last_kept = i;
-        if (run > target) { pick = i; break; }
+    float nxt[PER];
+    auto fetch = [&](int i0, float (&dst)[PER]) {
+      if (VEC) {
+        const int ii = i0 + 4 * lane;
+        const float4 v = ii < wend ? *reinterpret_cast<const float4*>(x + ii) : make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+        dst[0] = v.x; if (PER > 1) { dst[1] = v.y; dst[2] = v.z; dst[3] = v.w; }
+      } else {
+        dst[0] = i0 + lane < wend ? x[i0 + lane] : -INFINITY;
+      }
+    };
+    fetch(wbeg, nxt);
+    for (int i0 = wbeg; i0 < wend && pick < 0; i0 += STEP) {
+      float cur[PER];
+#pragma unroll
+      for (int c = 0; c < PER; ++c) cur[c] = nxt[c];
+      if (i0 + STEP < wend) fetch(i0 + STEP, nxt);
+      float e[PER], esum = 0.f;
+      int kept_hi = -1;
+#pragma unroll
+      for (int c = 0; c < PER; ++c) {
+        const int i = i0 + PER * lane + c;
+        const float z = cur[c] * inv_t;
+        const float ev = E_OF(z);
+        e[c] = (i < wend && order_key(z) >= kmin && ev >= mp) ? ev : 0.f;
+        if (e[c] > 0.f) kept_hi = i;
+        esum += e[c];
+      }
+#pragma unroll
+      for (int sft = WAVE / 2; sft > 0; sft >>= 1) { const int o = __shfl_xor(kept_hi, sft, WAVE); kept_hi = o > kept_hi ? o : kept_hi; }
+      if (kept_hi >= 0) last_kept = kept_hi;
+      const float step = wave_sum(esum);
+      if (run + step > target) {            // the crossing is among these: add them one by one
+        for (int j = 0; j < WAVE && pick < 0; ++j) {
+#pragma unroll
+          for (int c = 0; c < PER; ++c) {
+            const float ej = __shfl(e[c], j, WAVE);
+            run += ej;
+            if (pick < 0 && ej > 0.f && run > target) pick = i0 + PER * j + c;
+          }
+        }
+      } else {
+        run += step;
       }
     }
-    chosen = pick >= 0 ? pick : last_kept;
+    if (lane == 0) chosen = pick >= 0 ? pick : last_kept;
   }
   __syncthreads();
   if (chosen < 0) {  // rounding pushed the target past the total: take the last kept index
     int last = -1;
-    for (int i = begin; i < end; ++i) {
-      const float z = x[i] / temp;
-      if (order_key(z) >= kmin && expf(z - m) >= mp) last = i;
-    }
+    for_range<VEC>(x, wbeg, wend, lane, [&](int i, float v) {
+      const float z = v * inv_t;
+      if (order_key(z) >= kmin && E_OF(z) >= mp) last = i > last ? i : last;
+    });
 #pragma unroll
     for (int sft = WAVE / 2; sft > 0; sft >>= 1) { const int o = __shfl_xor(last, sft, WAVE); last = o > last ? o : last; }
     __syncthreads();
@@ -188,6 +248,7 @@ sample_kernel(const float* __restrict__ logits, int V, int ld, const float* __re
   } else if (tid == 0) {
     out[row] = chosen;
   }
+#undef E_OF
 }
 
 extern "C" int ullm_sample(const float* logits, int n_rows, int V, int ld, const float* temperature,
@@ -196,7 +257,12 @@ extern "C" int ullm_sample(const float* logits, int n_rows, int V, int ld, const
                            int* out, hipStream_t stream) {
   if (n_rows <= 0) return 0;
   if (V <= 0 || ld < V) return ULLM_ERR_SHAPE;
-  hipLaunchKernelGGL(sample_kernel, dim3(n_rows), dim3(SAMPLE_THREADS), 0, stream, logits, V, ld,
-                     temperature, top_k, top_p, min_p, seed_lo, seed_hi, position, out);
+  const bool vec = V % 4 == 0 && ld % 4 == 0 && !((uintptr_t)logits & 15);
+  if (vec)
+    hipLaunchKernelGGL(sample_kernel<true>, dim3(n_rows), dim3(SAMPLE_THREADS), 0, stream, logits, V, ld,
+                       temperature, top_k, top_p, min_p, seed_lo, seed_hi, position, out);
+  else
+    hipLaunchKernelGGL(sample_kernel<false>, dim3(n_rows), dim3(SAMPLE_THREADS), 0, stream, logits, V, ld,
+                       temperature, top_k, top_p, min_p, seed_lo, seed_hi, position, out);
   ULLM_LAUNCH_CHECK();
 }

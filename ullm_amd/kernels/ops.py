@@ -111,6 +111,15 @@ def add_rmsnorm(branch: Optional[torch.Tensor], residual: torch.Tensor, gain: to
     return out
 
 
+def residual_add(branch: torch.Tensor, residual: torch.Tensor) -> None:
+    """residual (float32, contiguous) += branch (same shape, contiguous)."""
+    _need(residual.dtype == torch.float32 and residual.is_contiguous() and branch.is_contiguous()
+          and branch.shape == residual.shape, "residual_add takes contiguous tensors of one shape")
+    lib = build.load("elementwise")
+    _check(lib.ullm_residual_add(_p(branch), _p(residual), ctypes.c_longlong(residual.numel()), _c_int(_dt(branch)),
+                                 _stream()), "residual_add")
+
+
 def silu_mul(gate_up: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """silu(gate_up[:, :I]) * gate_up[:, I:] for a contiguous [T, 2I] input."""
     T, two_i = gate_up.shape
@@ -209,15 +218,27 @@ def gemm_simple(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] =
     return out
 
 
+def _skinny_ok(M: int, K: int, x: torch.Tensor, w: torch.Tensor) -> bool:
+    return (w.dtype == torch.bfloat16 and 1 <= M <= 64 and K % 8 == 0 and K >= 8 and x.stride(1) == 1
+            and w.stride(1) == 1 and x.stride(0) % 8 == 0 and w.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0
+            and w.data_ptr() % 16 == 0)
+
+
 def gemm_skinny_supports(a: torch.Tensor, w: torch.Tensor) -> bool:
-    M, K = a.shape
-    return (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and 1 <= M <= 64 and K % 8 == 0 and K >= 8
-            and a.stride(1) == 1 and w.stride(1) == 1 and a.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
-            and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
+    return a.dtype == torch.bfloat16 and _skinny_ok(a.shape[0], a.shape[1], a, w)
+
+
+def _gemm_skinny(x, w, bias, c, M, N, K, pro, epi, c_dtype, nt=0, waves=0) -> None:
+    lib = build.load("gemm_skinny")
+    _check(lib.ullm_gemm_skinny(_p(x), _c_int(x.stride(0)), _p(w), _c_int(w.stride(0)), _p(bias),
+                                _p(c), _c_int(c.stride(0)), _c_int(M), _c_int(N), _c_int(K),
+                                _c_int(pro), _c_int(epi), _c_int(c_dtype), _c_int(nt), _c_int(waves), _stream()),
+           "gemm_skinny")
 
 
 def gemm_skinny(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
-                out_dtype: Optional[torch.dtype] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                out_dtype: Optional[torch.dtype] = None, out: Optional[torch.Tensor] = None,
+                nt: int = 0, waves: int = 0) -> torch.Tensor:
     """a [M <= 64, K] times w [N, K] transposed, bfloat16 operands streamed once through the matrix
     cores, 32-bit accumulation; output bfloat16 or float32."""
     M, K = a.shape
@@ -229,11 +250,21 @@ def gemm_skinny(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] =
     _need(out.shape == (M, N) and out.stride(1) == 1, "bad gemm output")
     if bias is not None:
         _need(bias.dtype == torch.float32 and bias.numel() == N and bias.is_contiguous(), "bias must be float32 [N]")
-    lib = build.load("gemm_skinny")
-    _check(lib.ullm_gemm_skinny(_p(a), _c_int(a.stride(0)), _p(w), _c_int(w.stride(0)), _p(bias), _p(out),
-                                _c_int(out.stride(0)), _c_int(M), _c_int(N), _c_int(K), _c_int(_dt(out)), _stream()),
-           "gemm_skinny")
+    _gemm_skinny(a, w, bias, out, M, N, K, 0, 0, _dt(out), nt, waves)
     return out
+
+
+def gemm_skinny_add(a: torch.Tensor, w: torch.Tensor, residual: torch.Tensor, silu: bool = False,
+                    nt: int = 0, waves: int = 0) -> None:
+    """residual (float32 [M, N]) += x times w transposed, where x = a (bfloat16 [M, K]) or, with
+    ``silu``, x = silu(a[:, :K]) * a[:, K:] for a = gate|up (bfloat16 [M, 2K])."""
+    M = a.shape[0]
+    N, K = w.shape
+    _need(a.dtype == torch.bfloat16 and a.shape[1] == (2 * K if silu else K) and _skinny_ok(M, K, a, w),
+          "gemm_skinny_add takes bfloat16 activations [M <= 64, K] (or [M, 2K] with silu)")
+    _need(residual.dtype == torch.float32 and residual.shape == (M, N) and residual.stride(1) == 1
+          and residual.stride(0) % 4 == 0 and residual.data_ptr() % 16 == 0, "residual must be float32 [M, N]")
+    _gemm_skinny(a, w, None, residual, M, N, K, 2 if silu else 0, 1, F32, nt, waves)
 
 
 SKINNY_MAX_ROWS = 16     # up to here the weight-streaming kernel beats the library product

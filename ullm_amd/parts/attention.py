@@ -14,7 +14,7 @@ import torch
 
 from ..kernels import ops
 from .base import KVNeed, LayerCache, Mixer, PartEnv, PositionEncoding, StepContext, WeightDecl, register_part
-from .linear import linear
+from .linear import can_fuse, linear
 
 
 @register_part("mixer", "gqa_attention")
@@ -68,15 +68,26 @@ class GQAttention(Mixer):
             self.k_gain = tensors[f"{p}.k_norm.weight"].contiguous()
 
     def forward(self, x: torch.Tensor, ctx: StepContext, cache: LayerCache) -> torch.Tensor:
-        T = x.shape[0]
-        group = ctx.groups[cache.group]
+        return linear(self._attend(linear(x, self.w_qkv, self.b_qkv), ctx, cache), self.w_o)
+
+    def fusable(self, residual, ctx: StepContext) -> bool:
+        return can_fuse(residual, ctx.dtype, self.w_qkv, self.w_o)
+
+    def forward_fused(self, x, residual, ctx: StepContext, cache: LayerCache) -> None:
         qkv = linear(x, self.w_qkv, self.b_qkv)
+        ops.gemm_skinny_add(self._attend(qkv, ctx, cache), self.w_o, residual)        # residual add folded behind
+
+    def _attend(self, qkv: torch.Tensor, ctx: StepContext, cache: LayerCache) -> torch.Tensor:
+        """Per-head norm, rotation, cache write and attention for a fused projection [T, (nq+2nkv)*hd];
+        returns the heads' outputs [T, nq*hd]."""
+        T = qkv.shape[0]
+        x = qkv
+        group = ctx.groups[cache.group]
         q = torch.empty((T, self.nq * self.hd), dtype=x.dtype, device=x.device)
         table, rot, style = self.position.kernel_args() if self.position is not None else (None, 0, 0)
         ops.qk_norm_rope_write(
             qkv, q, self.q_gain, self.k_gain, self.qk_norm_eps if self.qk_norm_eps is not None else 0.0,
             table, rot, style, ctx.positions, ctx.token_entry, group.block_table,
             cache.k_pool, cache.v_pool, group.page_size, self.nq, self.nkv, self.hd, write_kv=cache.owner)
-        o = ops.paged_attention(q, cache.k_pool, cache.v_pool, ctx, group, self.nq, self.nkv, self.hd,
-                                self.scale, self.window)
-        return linear(o, self.w_o)
+        return ops.paged_attention(q, cache.k_pool, cache.v_pool, ctx, group, self.nq, self.nkv, self.hd,
+                                   self.scale, self.window)

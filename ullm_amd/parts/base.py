@@ -119,7 +119,11 @@ class Part:
 
 
 class Mixer(Part):
-    """Token mixer: ``forward(x [T, hidden], ctx, cache) -> [T, hidden]`` in the compute dtype."""
+    """Token mixer: ``forward(x [T, hidden], ctx, cache) -> [T, hidden]`` in the compute dtype.
+
+    A mixer may also offer ``forward_fused(x, residual, ctx, cache)``: add mixer(x) into the 32-bit
+    residual in place, with the add folded into its last kernel.  It is called only when
+    ``fusable(residual, ctx)`` says so."""
     kind = "mixer"
 
     def cache_need(self) -> CacheNeed:
@@ -128,12 +132,25 @@ class Mixer(Part):
     def forward(self, x: torch.Tensor, ctx: StepContext, cache: LayerCache) -> torch.Tensor:
         raise NotImplementedError
 
+    def fusable(self, residual: torch.Tensor, ctx: StepContext) -> bool:
+        return False
+
+    def forward_fused(self, x, residual, ctx: StepContext, cache: LayerCache) -> None:
+        raise NotImplementedError
+
 
 class FeedForward(Part):
-    """``forward(x [T, hidden], ctx) -> [T, hidden]``; keeps nothing between steps."""
+    """``forward(x [T, hidden], ctx) -> [T, hidden]``; keeps nothing between steps.
+    ``fusable`` and ``forward_fused(x, residual, ctx)`` as for mixers."""
     kind = "ffn"
 
     def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
+        raise NotImplementedError
+
+    def fusable(self, residual: torch.Tensor, ctx: StepContext) -> bool:
+        return False
+
+    def forward_fused(self, x, residual, ctx: StepContext) -> None:
         raise NotImplementedError
 
 

@@ -22,7 +22,17 @@ class PreNormBlock(Block):
         return self.mixer.cache_need()
 
     def forward(self, residual, pending, ctx: StepContext, cache: LayerCache):
+        # Each half: the norm kernel adds the pending branch into the stream and normalises; the
+        # part then either adds its result into the stream itself (folded into its last kernel,
+        # where it offers that for this batch) or returns it as the next pending branch.
         x = self.mixer_norm.add_norm(pending, residual, out_dtype=ctx.dtype)
-        a = self.mixer.forward(x, ctx, cache)
-        x = self.ffn_norm.add_norm(a, residual, out_dtype=ctx.dtype)
+        if self.mixer.fusable(residual, ctx):
+            self.mixer.forward_fused(x, residual, ctx, cache)
+            pending = None
+        else:
+            pending = self.mixer.forward(x, ctx, cache)
+        x = self.ffn_norm.add_norm(pending, residual, out_dtype=ctx.dtype)
+        if self.ffn.fusable(residual, ctx):
+            self.ffn.forward_fused(x, residual, ctx)
+            return residual, None
         return residual, self.ffn.forward(x, ctx)

@@ -10,7 +10,7 @@ import torch
 
 from ..kernels import ops
 from .base import FeedForward, PartEnv, StepContext, WeightDecl, register_part
-from .linear import linear
+from .linear import can_fuse, linear
 
 
 @register_part("ffn", "swiglu")
@@ -32,3 +32,10 @@ class SwiGLU(FeedForward):
 
     def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
         return linear(ops.silu_mul(linear(x, self.w_gate_up)), self.w_down)
+
+    def fusable(self, residual, ctx: StepContext) -> bool:
+        return can_fuse(residual, ctx.dtype, self.w_gate_up, self.w_down)
+
+    def forward_fused(self, x, residual, ctx: StepContext) -> None:
+        gate_up = linear(x, self.w_gate_up)
+        ops.gemm_skinny_add(gate_up, self.w_down, residual, silu=True)                  # silu*up in front, add behind

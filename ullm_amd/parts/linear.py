@@ -18,3 +18,16 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
     if x.dtype == torch.float32 or weight.dtype == torch.float32:
         return ops.gemm_simple(x, weight, bias, out_dtype=out_dtype)
     return ops.gemm_bf16(x, weight, bias, out_dtype=out_dtype)
+
+
+FUSED_MAX_ROWS = 16      # batches up to this many tokens take the projections with folded norm / add
+
+
+def can_fuse(residual: torch.Tensor, dtype: torch.dtype, *weights: torch.Tensor) -> bool:
+    """True if the folded projection kernels take this batch: bfloat16 compute, few rows, row lengths
+    that keep 16-byte alignment."""
+    T, H = residual.shape
+    if dtype != torch.bfloat16 or T > FUSED_MAX_ROWS or H % 8:
+        return False
+    return all(w.dtype == torch.bfloat16 and w.shape[1] % 8 == 0 and w.shape[0] % 4 == 0 and w.data_ptr() % 16 == 0
+               for w in weights)
