@@ -295,16 +295,17 @@ def test_attention_on_the_matrix_cores(ops, case):
             for f in range(0, n, 16):
                 tiles += [t0 + f, min(16, n - f)]
         t0 += n
-    for chunk in (None, 128, 256, 4096):
+    for splits, waves in ((0, 0), (1, 4), (1, 8), (2, 8), (3, 4), (7, 8)):
         out = torch.full((q.shape[0], nq * hd), float("nan"), dtype=dtype, device=DEV)
         if dec:
             ops.attention_decode_mfma(q, out, k_pool, v_pool, torch.tensor(dec, dtype=torch.int32, device=DEV),
-                                      len(dec), positions, entry, bt, P, nq, nkv, hd, scale, window, max_kv, chunk=chunk)
+                                      len(dec), positions, entry, bt, P, nq, nkv, hd, scale, window, max_kv,
+                                      splits=splits, waves=waves)
         if tiles:
             ops.attention_prefill_mfma(q, out, k_pool, v_pool, torch.tensor(tiles, dtype=torch.int32, device=DEV),
                                        len(tiles) // 2, positions, entry, bt, P, nq, nkv, hd, scale, window)
         assert not torch.isnan(out).any()
-        assert (out.float().cpu() - want).abs().max() <= tol(dtype, want), chunk
+        assert (out.float().cpu() - want).abs().max() <= tol(dtype, want), (splits, waves)
         if not dec:
             break
 
@@ -335,7 +336,7 @@ def test_matrix_core_attention_finds_one_far_key_at_every_edge(ops):
                 bt = table_tensor(tables, DEV)
                 if n == 1:
                     ops.attention_decode_mfma(qd, out, k_pool, v_pool, None, 1, positions, entry, bt, P, nq, nkv, hd,
-                                              1.0, window, S, chunk=128)
+                                              1.0, window, S, splits=1 + target % 3, waves=8 if target % 2 else 4)
                 else:
                     ops.attention_prefill_mfma(qd, out, k_pool, v_pool, torch.tensor([0, n], dtype=torch.int32, device=DEV),
                                                1, positions, entry, bt, P, nq, nkv, hd, 1.0, window)

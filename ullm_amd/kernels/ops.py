@@ -297,22 +297,23 @@ def attention_mfma_supports(dtype: torch.dtype, hd: int, page_size: int, nq: int
         _c_int(hd), _c_int(page_size), _c_int(nq), _c_int(nkv)))
 
 
-def decode_split(n_items: int, nkv: int, groups: int, max_kv: int, target_blocks: int = 768):
-    """(chunk, num_splits): keys per block (128 * a power of two; a block's four waves take a
-    quarter each) so that the launch has about ``target_blocks`` blocks."""
-    want = max(1, target_blocks // max(1, n_items * nkv * groups))
-    chunk = 128
-    while -(-max_kv // chunk) > want:
-        chunk *= 2
-    return chunk, max(1, -(-max_kv // chunk))
+def decode_split(n_items: int, nkv: int, groups: int, max_kv: int, hd: int = 128):
+    """(waves, num_splits) of the decode attention launch.  Few (token, kv head) pairs get 8 waves a
+    block; a token's keys are cut evenly over splits * waves waves.  Keys go to several blocks (whose
+    partial results a second kernel adds up) only when a wave would otherwise get more than 512."""
+    pairs = max(1, n_items * nkv * groups)
+    waves = 8 if (pairs <= 512 and hd != 256) else 4
+    if pairs >= 256:
+        return waves, 1
+    return waves, max(1, -(-max_kv // (512 * waves)))
 
 
 def attention_decode_mfma(q, out, k_pool, v_pool, token_list: Optional[torch.Tensor], n_items: int,
                           positions, token_entry, block_table, page_size: int, nq: int, nkv: int, hd: int,
-                          scale: float, window: int, max_kv: int, chunk: Optional[int] = None) -> None:
+                          scale: float, window: int, max_kv: int, splits: int = 0, waves: int = 0) -> None:
     """One query token per item (``token_list`` int32 [n_items] names the tokens, None = tokens
-    0..n_items-1) against its request's cache; the keys are split into chunks whose partial results
-    a second small kernel adds up."""
+    0..n_items-1) against its request's cache; with ``splits`` > 1 the keys go to several blocks whose
+    partial results a second small kernel adds up."""
     _check_pools(k_pool, v_pool, nkv, page_size, hd, torch.bfloat16)
     _need(q.dtype == torch.bfloat16 and q.stride(1) == 1 and q.shape[1] == nq * hd, "q must be bfloat16 [T, nq*hd]")
     _need(out.dtype == torch.bfloat16 and out.stride(1) == 1 and out.shape == q.shape, "bad attention output")
@@ -326,20 +327,20 @@ def attention_decode_mfma(q, out, k_pool, v_pool, token_list: Optional[torch.Ten
           "block_table must be int32 [B, stride]")
     _need(-(-max_kv // page_size) <= block_table.shape[1], "block table narrower than the longest context")
     groups = -(-(nq // nkv) // 16)
-    if chunk is None:
-        chunk, splits = decode_split(n_items, nkv, groups, max_kv)
-    else:
-        _need(chunk % 128 == 0, "chunk must be a multiple of 128")
-        splits = max(1, -(-max_kv // chunk))
+    auto_waves, auto_splits = decode_split(n_items, nkv, groups, max_kv, hd)
+    waves = waves or auto_waves
+    if hd == 256:
+        waves = 4
+    splits = splits or auto_splits
     lib = build.load("attention_mfma")
     ws = None
     if splits > 1:
-        ws = torch.empty(n_items * nq * splits * (hd + 2), dtype=torch.float32, device=q.device)
+        ws = torch.empty(n_items * nq * splits * (hd + 4), dtype=torch.float32, device=q.device)
     _check(lib.ullm_attention_decode(
         _p(q), _c_int(q.stride(0)), _p(out), _c_int(out.stride(0)), _p(k_pool), _p(v_pool), _p(token_list),
         _c_int(n_items), _p(positions), _p(token_entry), _p(block_table), _c_int(block_table.stride(0)),
-        _c_int(page_size), _c_int(nq), _c_int(nkv), _c_int(hd), _c_float(scale), _c_int(window), _c_int(chunk),
-        _c_int(splits), _p(ws), _stream()), "attention_decode")
+        _c_int(page_size), _c_int(nq), _c_int(nkv), _c_int(hd), _c_float(scale), _c_int(window),
+        _c_int(splits), _c_int(waves), _p(ws), _stream()), "attention_decode")
 
 
 def attention_prefill_mfma(q, out, k_pool, v_pool, tiles: torch.Tensor, n_tiles: int, positions, token_entry,
