@@ -263,6 +263,7 @@ MFMA_CASES = [dict(nq=8, nkv=2, hd=32, P=16, lens=[(1, 1), (1, 37), (1, 300), (1
               dict(nq=8, nkv=2, hd=64, P=16, lens=[(1, 300), (1, 40), (1, 9)], window=50),
               dict(nq=8, nkv=2, hd=32, P=16, lens=[(5, 5), (33, 70), (16, 16), (2, 130), (17, 49)], window=0),
               dict(nq=32, nkv=8, hd=128, P=16, lens=[(100, 100), (7, 260)], window=0),
+              dict(nq=32, nkv=16, hd=32, P=16, lens=[(70, 70), (33, 90), (1, 5)], window=0),      # kv heads 2 x 8
               dict(nq=6, nkv=2, hd=64, P=32, lens=[(40, 90), (3, 3)], window=21),
               dict(nq=8, nkv=2, hd=32, P=16, lens=[(1, 45), (9, 40), (1, 200), (20, 20), (1, 1)], window=0),  # mixed
               dict(nq=8, nkv=2, hd=32, P=16, lens=[(1, 45), (9, 40), (1, 200), (20, 50)], window=13)]
@@ -292,8 +293,8 @@ def test_attention_on_the_matrix_cores(ops, case):
             dec.append(t0)
             max_kv = max(max_kv, S)
         else:
-            for f in range(0, n, 16):
-                tiles += [t0 + f, min(16, n - f)]
+            for f in range(0, n, ops.PREFILL_TILE):
+                tiles += [t0 + f, min(ops.PREFILL_TILE, n - f)]
         t0 += n
     for splits, waves in ((0, 0), (1, 4), (1, 8), (2, 8), (3, 4), (7, 8)):
         out = torch.full((q.shape[0], nq * hd), float("nan"), dtype=dtype, device=DEV)

@@ -82,125 +82,184 @@ __device__ __forceinline__ void load_tile(KVTile<NQK>& t, int key0, const PageWi
   }
 }
 
-// Scores, softmax update and value product for one tile held in registers.
-template <int NQK>
-__device__ __forceinline__ void process_tile(const KVTile<NQK>& cur, int key0, const Pack8 (&qreg)[NQK], int col_lo,
-                                             int col_hi, int max_hi, float scale_log2e, f32x4_t (&acc)[2 * NQK],
-                                             float& m, float& l) {
+// Scores, softmax update and value product for one tile held in registers, for NG groups of 16
+// columns that share the tile (each group has its own queries, limits, maximum, sum and output).
+template <int NQK, int NG>
+__device__ __forceinline__ void process_tile(const KVTile<NQK>& cur, int key0, const Pack8 (&qreg)[NG][NQK],
+                                             const int (&col_lo)[NG], const int (&col_hi)[NG], int max_hi,
+                                             float scale_log2e, f32x4_t (&acc)[NG][2 * NQK], float (&m)[NG],
+                                             float (&l)[NG]) {
   const int lane = threadIdx.x & 63, g = lane >> 4;
-  f32x4_t s[2];
-#pragma unroll
-  for (int sb = 0; sb < 2; ++sb) {
-    s[sb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int ch = 0; ch < NQK; ++ch)
-      s[sb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.k[sb][ch].v, qreg[ch].v, s[sb], 0, 0, 0);
-  }
-  // scores of keys key0 + 16 sb + 4 g + r for this lane's column; mask, running maximum
-  float tile_max = NEG_BIG;
-#pragma unroll
-  for (int sb = 0; sb < 2; ++sb)
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const int kk = key0 + 16 * sb + 4 * g + r;
-      const bool ok = cur.ok[sb] && kk >= col_lo && kk <= col_hi;
-      const float v = ok ? s[sb][r] * scale_log2e : NEG_BIG;
-      s[sb][r] = v;
-      tile_max = fmaxf(tile_max, v);
-    }
-  tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, 64));
-  tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, 64));
-  const float m_new = fmaxf(m, tile_max);
-  const float alpha = fast_exp2(m - m_new);
-  Pack8 p;
-  float psum = 0.f;
-#pragma unroll
-  for (int sb = 0; sb < 2; ++sb) {
-    float e[4];
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      // a masked score stays at NEG_BIG: its weight is zero even while m_new is still NEG_BIG
-      e[r] = s[sb][r] > 0.5f * NEG_BIG ? fast_exp2(s[sb][r] - m_new) : 0.f;
-      psum += e[r];
-    }
-    p.w[2 * sb] = pack2_bf16(e[0], e[1]);
-    p.w[2 * sb + 1] = pack2_bf16(e[2], e[3]);
-  }
-  l = l * alpha + psum;
-  m = m_new;
   const bool edge = key0 + 32 > max_hi + 1;     // some keys of the tile hold no written data
+  Pack8 vals[2 * NQK];
 #pragma unroll
   for (int n = 0; n < 2 * NQK; ++n) {
-    Pack8 a;
-    a.u2[0] = cur.v[n][0];
-    a.u2[1] = cur.v[n][1];
+    vals[n].u2[0] = cur.v[n][0];
+    vals[n].u2[1] = cur.v[n][1];
     if (edge) {
 #pragma unroll
       for (int j = 0; j < 8; ++j)
-        if (key0 + 16 * (j >> 2) + 4 * g + (j & 3) > max_hi) a.h[j] = 0;
+        if (key0 + 16 * (j >> 2) + 4 * g + (j & 3) > max_hi) vals[n].h[j] = 0;
     }
-    f32x4_t o = acc[n];
-    o[0] *= alpha; o[1] *= alpha; o[2] *= alpha; o[3] *= alpha;
-    acc[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, p.v, o, 0, 0, 0);
+  }
+#pragma unroll
+  for (int q = 0; q < NG; ++q) {
+    f32x4_t s[2];
+#pragma unroll
+    for (int sb = 0; sb < 2; ++sb) {
+      s[sb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ch = 0; ch < NQK; ++ch)
+        s[sb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.k[sb][ch].v, qreg[q][ch].v, s[sb], 0, 0, 0);
+    }
+    // scores of keys key0 + 16 sb + 4 g + r for this lane's column; mask, running maximum
+    float tile_max = NEG_BIG;
+#pragma unroll
+    for (int sb = 0; sb < 2; ++sb)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int kk = key0 + 16 * sb + 4 * g + r;
+        const bool ok = cur.ok[sb] && kk >= col_lo[q] && kk <= col_hi[q];
+        const float v = ok ? s[sb][r] * scale_log2e : NEG_BIG;
+        s[sb][r] = v;
+        tile_max = fmaxf(tile_max, v);
+      }
+    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, 64));
+    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, 64));
+    const float m_new = fmaxf(m[q], tile_max);
+    const float alpha = fast_exp2(m[q] - m_new);
+    Pack8 p;
+    float psum = 0.f;
+#pragma unroll
+    for (int sb = 0; sb < 2; ++sb) {
+      float e[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        // a masked score stays at NEG_BIG: its weight is zero even while m_new is still NEG_BIG
+        e[r] = s[sb][r] > 0.5f * NEG_BIG ? fast_exp2(s[sb][r] - m_new) : 0.f;
+        psum += e[r];
+      }
+      p.w[2 * sb] = pack2_bf16(e[0], e[1]);
+      p.w[2 * sb + 1] = pack2_bf16(e[2], e[3]);
+    }
+    l[q] = l[q] * alpha + psum;
+    m[q] = m_new;
+#pragma unroll
+    for (int n = 0; n < 2 * NQK; ++n) {
+      f32x4_t o = acc[q][n];
+      o[0] *= alpha; o[1] *= alpha; o[2] *= alpha; o[3] *= alpha;
+      acc[q][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vals[n].v, p.v, o, 0, 0, 0);
+    }
   }
 }
 
-// The work of one wave.  NQK = head_dim / 32.
-//   col_q      : pointer to this lane's column's query row (null if the column is padding)
-//   col_lo/hi  : first and last key the column may see (hi < lo for padding)
+// The work of one wave.  NQK = head_dim / 32; NG groups of 16 columns share every tile.
+//   col_q[q]      : pointer to this lane's column's query row in group q (null if padding)
+//   col_lo/hi[q]  : first and last key the column may see (hi < lo for padding)
 //   key_begin/key_end : the wave's key range [begin, end), begin a multiple of 32
 //   max_hi     : largest key position that holds written data for this request
-// Results: acc[n][r] = O^T[16n + 4g + r][col] (unnormalised), m (log2 domain), l (this lane's share
-// of the sum; the four lanes of a column add up to the column's sum).
+// Results per group: acc[q][n][r] = O^T[16n + 4g + r][col] (unnormalised), m (log2 domain), l (this
+// lane's share of the sum; the four lanes of a column add up to the column's sum).
 // Page ids are fetched 1024 keys at a time; the loads of the next DEPTH (1 or 2) tiles are in flight
-// while the current one is worked on (2 needs about 230 registers, 1 about 130).
-template <int NQK, int DEPTH = 2>
+// while the current one is worked on.
+template <int NQK, int NG, int DEPTH>
 __device__ __forceinline__ void attend_range(
-    const bf16_t* __restrict__ col_q, int col_lo, int col_hi, int key_begin, int key_end, int max_hi,
-    const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool, const int* __restrict__ bt,
-    int page_size, int nkv, int kvh, float scale_log2e, f32x4_t (&acc)[2 * NQK], float& m, float& l) {
+    const bf16_t* const (&col_q)[NG], const int (&col_lo)[NG], const int (&col_hi)[NG], int key_begin, int key_end,
+    int max_hi, const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool, const int* __restrict__ bt,
+    int page_size, int nkv, int kvh, float scale_log2e, f32x4_t (&acc)[NG][2 * NQK], float (&m)[NG], float (&l)[NG]) {
   const int lane = threadIdx.x & 63, g = lane >> 4;
 #pragma unroll
-  for (int n = 0; n < 2 * NQK; ++n) acc[n] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-  m = NEG_BIG;
-  l = 0.f;
+  for (int q = 0; q < NG; ++q) {
+#pragma unroll
+    for (int n = 0; n < 2 * NQK; ++n) acc[q][n] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    m[q] = NEG_BIG;
+    l[q] = 0.f;
+  }
   if (key_begin >= key_end) return;
   PageWindow pw = load_pages(key_begin, key_end, bt, page_size);
-  Pack8 qreg[NQK];
+  Pack8 qreg[NG][NQK];
 #pragma unroll
-  for (int ch = 0; ch < NQK; ++ch) {
-    if (col_q) qreg[ch].u4 = *reinterpret_cast<const uint4*>(col_q + 32 * ch + 8 * g);
-    else qreg[ch].u4 = make_uint4(0, 0, 0, 0);
-  }
+  for (int q = 0; q < NG; ++q)
+#pragma unroll
+    for (int ch = 0; ch < NQK; ++ch) {
+      if (col_q[q]) qreg[q][ch].u4 = *reinterpret_cast<const uint4*>(col_q[q] + 32 * ch + 8 * g);
+      else qreg[q][ch].u4 = make_uint4(0, 0, 0, 0);
+    }
+#define TILE_LOAD(T, K0) load_tile<NQK>(T, K0, pw, k_pool, v_pool, page_size, nkv, kvh)
+#define TILE_WORK(T, K0) process_tile<NQK, NG>(T, K0, qreg, col_lo, col_hi, max_hi, scale_log2e, acc, m, l)
   for (int base = key_begin; base < key_end; base += 1024) {
     if (base != key_begin) pw = load_pages(base, key_end, bt, page_size);
     const int stop = base + 1024 < key_end ? base + 1024 : key_end;
     if (DEPTH == 1) {
       KVTile<NQK> a, b;
-      load_tile<NQK>(a, base, pw, k_pool, v_pool, page_size, nkv, kvh);
+      TILE_LOAD(a, base);
       for (int key0 = base; key0 < stop; key0 += 64) {
-        if (key0 + 32 < stop) load_tile<NQK>(b, key0 + 32, pw, k_pool, v_pool, page_size, nkv, kvh);
-        process_tile<NQK>(a, key0, qreg, col_lo, col_hi, max_hi, scale_log2e, acc, m, l);
+        if (key0 + 32 < stop) TILE_LOAD(b, key0 + 32);
+        TILE_WORK(a, key0);
         if (key0 + 32 >= stop) break;
-        if (key0 + 64 < stop) load_tile<NQK>(a, key0 + 64, pw, k_pool, v_pool, page_size, nkv, kvh);
-        process_tile<NQK>(b, key0 + 32, qreg, col_lo, col_hi, max_hi, scale_log2e, acc, m, l);
+        if (key0 + 64 < stop) TILE_LOAD(a, key0 + 64);
+        TILE_WORK(b, key0 + 32);
       }
       continue;
     }
     KVTile<NQK> t0, t1, t2;
-    load_tile<NQK>(t0, base, pw, k_pool, v_pool, page_size, nkv, kvh);
-    if (base + 32 < stop) load_tile<NQK>(t1, base + 32, pw, k_pool, v_pool, page_size, nkv, kvh);
+    TILE_LOAD(t0, base);
+    if (base + 32 < stop) TILE_LOAD(t1, base + 32);
     // three buffers in rotation: while tile i is worked on, tiles i+1 and i+2 are loading
     for (int key0 = base; key0 < stop; key0 += 96) {
-      if (key0 + 64 < stop) load_tile<NQK>(t2, key0 + 64, pw, k_pool, v_pool, page_size, nkv, kvh);
-      process_tile<NQK>(t0, key0, qreg, col_lo, col_hi, max_hi, scale_log2e, acc, m, l);
+      if (key0 + 64 < stop) TILE_LOAD(t2, key0 + 64);
+      TILE_WORK(t0, key0);
       if (key0 + 32 >= stop) break;
-      if (key0 + 96 < stop) load_tile<NQK>(t0, key0 + 96, pw, k_pool, v_pool, page_size, nkv, kvh);
-      process_tile<NQK>(t1, key0 + 32, qreg, col_lo, col_hi, max_hi, scale_log2e, acc, m, l);
+      if (key0 + 96 < stop) TILE_LOAD(t0, key0 + 96);
+      TILE_WORK(t1, key0 + 32);
       if (key0 + 64 >= stop) break;
-      if (key0 + 128 < stop) load_tile<NQK>(t1, key0 + 128, pw, k_pool, v_pool, page_size, nkv, kvh);
-      process_tile<NQK>(t2, key0 + 64, qreg, col_lo, col_hi, max_hi, scale_log2e, acc, m, l);
+      if (key0 + 128 < stop) TILE_LOAD(t1, key0 + 128);
+      TILE_WORK(t2, key0 + 64);
     }
+  }
+#undef TILE_LOAD
+#undef TILE_WORK
+}
+
+// Merge the waves of a block pairwise, lane by lane (a lane's values mean the same in every wave),
+// halving the number of live waves each round in a fixed order; wave 0 ends with the block's result.
+// `buf` holds (WAVES / 2) x (NG * (8 NQK + 2)) x 64 floats.  Every wave of the block must call this.
+template <int NQK, int NG, int WAVES>
+__device__ __forceinline__ void merge_waves(f32x4_t (&acc)[NG][2 * NQK], float (&m)[NG], float (&l)[NG], float* buf) {
+  constexpr int PER_LANE = NG * (8 * NQK + 2);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int half = WAVES / 2; half >= 1; half >>= 1) {
+    if (wave >= half && wave < 2 * half) {          // the upper half of the live waves hands over
+      float* w = buf + (size_t)(wave - half) * PER_LANE * 64 + lane;
+#pragma unroll
+      for (int q = 0; q < NG; ++q) {
+#pragma unroll
+        for (int n = 0; n < 2 * NQK; ++n)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) w[(q * (8 * NQK + 2) + 4 * n + r) * 64] = acc[q][n][r];
+        w[(q * (8 * NQK + 2) + 8 * NQK) * 64] = m[q];
+        w[(q * (8 * NQK + 2) + 8 * NQK + 1) * 64] = l[q];
+      }
+    }
+    __syncthreads();
+    if (wave < half) {
+      const float* w = buf + (size_t)wave * PER_LANE * 64 + lane;
+#pragma unroll
+      for (int q = 0; q < NG; ++q) {
+        const float m_b = w[(q * (8 * NQK + 2) + 8 * NQK) * 64], l_b = w[(q * (8 * NQK + 2) + 8 * NQK + 1) * 64];
+        const float M = fmaxf(m[q], m_b);
+        const float fa = fast_exp2(m[q] - M), fb = fast_exp2(m_b - M);
+#pragma unroll
+        for (int n = 0; n < 2 * NQK; ++n)
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            acc[q][n][r] = acc[q][n][r] * fa + w[(q * (8 * NQK + 2) + 4 * n + r) * 64] * fb;
+        l[q] = l[q] * fa + l_b * fb;
+        m[q] = M;
+      }
+    }
+    __syncthreads();
   }
 }
 
@@ -224,8 +283,7 @@ attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __re
                         int num_splits, float* __restrict__ part) {
   constexpr int HD = 32 * NQK;
   constexpr int ROW = HD + 4;                       // output dims, then maximum and sum (rows stay 16-byte aligned)
-  constexpr int PER_LANE = 8 * NQK + 2;             // a lane's accumulators, maximum and sum share
-  __shared__ float merge[WAVES / 2][PER_LANE][64];  // [writer][value][lane]: conflict-free
+  __shared__ float merge[(WAVES / 2) * (8 * NQK + 2) * 64];   // [writer][value][lane]: conflict-free
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g = lane >> 4, c = lane & 15;
   const int split = blockIdx.x;
   const int G = nq / nkv;
@@ -243,37 +301,19 @@ attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __re
   const int head_in_group = cg * 16 + c;
   const bool col_ok = head_in_group < G;
   const int head = kvh * G + head_in_group;
-  f32x4_t acc[2 * NQK];
-  float m, l;
-  attend_range<NQK, (WAVES > 4 ? 1 : 2)>(
-      col_ok ? q + (size_t)t * q_stride + (size_t)head * HD : nullptr, lo, col_ok ? pos : -1, begin, end, pos,
-      k_pool, v_pool, block_table + (size_t)token_entry[t] * bt_stride, page_size, nkv, kvh, scale_log2e, acc, m, l);
-#pragma unroll
-  for (int half = WAVES / 2; half >= 1; half >>= 1) {
-    if (wave >= half && wave < 2 * half) {          // the upper half of the live waves hands over
-      float (*w)[64] = merge[wave - half];
-#pragma unroll
-      for (int n = 0; n < 2 * NQK; ++n)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) w[4 * n + r][lane] = acc[n][r];
-      w[8 * NQK][lane] = m;
-      w[8 * NQK + 1][lane] = l;
-    }
-    __syncthreads();
-    if (wave < half) {
-      const float (*w)[64] = merge[wave];
-      const float m_b = w[8 * NQK][lane], l_b = w[8 * NQK + 1][lane];
-      const float M = fmaxf(m, m_b);
-      const float fa = fast_exp2(m - M), fb = fast_exp2(m_b - M);
-#pragma unroll
-      for (int n = 0; n < 2 * NQK; ++n)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) acc[n][r] = acc[n][r] * fa + w[4 * n + r][lane] * fb;
-      l = l * fa + l_b * fb;
-      m = M;
-    }
-    __syncthreads();
+  f32x4_t accs[1][2 * NQK];
+  float ms[1], ls[1];
+  {
+    const bf16_t* const cq[1] = {col_ok ? q + (size_t)t * q_stride + (size_t)head * HD : nullptr};
+    const int clo[1] = {lo}, chi[1] = {col_ok ? pos : -1};
+    attend_range<NQK, 1, (WAVES > 4 ? 1 : 2)>(cq, clo, chi, begin, end, pos, k_pool, v_pool,
+                                              block_table + (size_t)token_entry[t] * bt_stride, page_size, nkv, kvh,
+                                              scale_log2e, accs, ms, ls);
   }
+  merge_waves<NQK, 1, WAVES>(accs, ms, ls, merge);
+  f32x4_t (&acc)[2 * NQK] = accs[0];
+  float& m = ms[0];
+  float& l = ls[0];
   if (wave != 0) return;
   l += __shfl_xor(l, 16, 64);
   l += __shfl_xor(l, 32, 64);
@@ -337,51 +377,90 @@ attention_reduce_kernel(const float* __restrict__ part, bf16_t* __restrict__ out
 }
 
 // ------------------------------------------------------------------------------- prompt portions
-// grid (n_tiles, nkv * ceil(G / waves)), block 64 * waves with waves = min(G, 4): one wave per query
-// head, the waves of a block share a kv head (and so the cache lines they read); tile = (first
-// token, number of tokens <= 16) of one request; every wave walks all keys its tokens see.
+// grid (n_tiles * nq), block 256 (128 for head_dim 256).  Workgroups go to the 8 XCDs round-robin by
+// their linear id and each XCD has an L2 of its own, so the id is decoded such that all work on one kv
+// head lands on one XCD (kv head = id mod 8 when the kv heads are a multiple of 8): that head's keys
+// and values then stay in that L2 instead of every XCD streaming every head from memory.  Tiles are
+// taken last first (under the causal mask they see the most keys).
+// Tile = (first token, number of tokens <= 32) of one request: two
+// groups of 16 tokens share every key/value tile a wave loads.  The keys the tile's tokens see are
+// cut into equal shares of whole 32-key tiles, one per wave (under a causal mask the last tiles of
+// a long prompt see far more keys than the first; cutting by keys keeps every wave's walk short),
+// and the waves merge as in the decode kernel.
+#define PREFILL_GROUPS 2
+// waves per block: four, or two for head_dim 256 (shared memory of the merge)
+__host__ __device__ constexpr int prefill_waves(int nqk) { return nqk >= 8 ? 2 : 4; }
 template <int NQK>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(64 * prefill_waves(NQK))
 attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
                          const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
                          const int* __restrict__ tiles, const int* __restrict__ positions,
                          const int* __restrict__ token_entry, const int* __restrict__ block_table,
-                         int bt_stride, int page_size, int nq, int nkv, float scale_log2e, int window) {
+                         int bt_stride, int page_size, int nq, int nkv, float scale_log2e, int window,
+                         int n_tiles) {
   constexpr int HD = 32 * NQK;
+  constexpr int NG = PREFILL_GROUPS;
+  constexpr int PREFILL_WAVES = prefill_waves(NQK);
+  __shared__ float merge[(PREFILL_WAVES / 2) * NG * (8 * NQK + 2) * 64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, g = lane >> 4, c = lane & 15;
   const int G = nq / nkv;
-  const int waves = blockDim.x >> 6, hgroups = (G + waves - 1) / waves;
-  const int kvh = blockIdx.y / hgroups;
-  const int head_in_group = (blockIdx.y % hgroups) * waves + wave;
-  if (head_in_group >= G) return;
-  const int head = kvh * G + head_in_group;
-  const int first = tiles[2 * blockIdx.x], count = tiles[2 * blockIdx.x + 1];
-  const bool col_ok = c < count;
-  const int t = first + (col_ok ? c : 0);
-  const int pos = positions[t];
-  const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  int kvh, tile_idx, head;
+  if (nkv % 8 == 0) {
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, per_kv = n_tiles * G;
+    kvh = (slot / per_kv) * 8 + xcd;
+    tile_idx = (slot % per_kv) / G;
+    head = kvh * G + (slot % per_kv) % G;
+  } else {
+    tile_idx = blockIdx.x / nq;
+    head = blockIdx.x % nq;
+    kvh = head / G;
+  }
+  tile_idx = n_tiles - 1 - tile_idx;
+  const int first = tiles[2 * tile_idx], count = tiles[2 * tile_idx + 1];
+  const bf16_t* cq[NG];
+  int clo[NG], chi[NG], tok[NG];
+#pragma unroll
+  for (int qg = 0; qg < NG; ++qg) {
+    const bool ok = 16 * qg + c < count;
+    tok[qg] = first + (ok ? 16 * qg + c : 0);
+    const int pos = positions[tok[qg]];
+    clo[qg] = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+    chi[qg] = ok ? pos : -1;
+    cq[qg] = ok ? q + (size_t)tok[qg] * q_stride + (size_t)head * HD : nullptr;
+  }
   const int last_pos = positions[first + count - 1];
   const int first_pos = positions[first];
-  const int tile_lo = (window > 0 && first_pos - window + 1 > 0) ? first_pos - window + 1 : 0;
-  f32x4_t acc[2 * NQK];
-  float m, l;
-  attend_range<NQK>(col_ok ? q + (size_t)t * q_stride + (size_t)head * HD : nullptr, lo, col_ok ? pos : -1,
-                    tile_lo & ~31, last_pos + 1, last_pos, k_pool, v_pool,
-                    block_table + (size_t)token_entry[first] * bt_stride, page_size, nkv, kvh, scale_log2e,
-                    acc, m, l);
-  l += __shfl_xor(l, 16, 64);
-  l += __shfl_xor(l, 32, 64);
-  if (!col_ok) return;
-  const float inv = l > 0.f ? 1.f / l : 0.f;
-  bf16_t* op = out + (size_t)t * out_stride + (size_t)head * HD;
+  const int tile_lo = ((window > 0 && first_pos - window + 1 > 0) ? first_pos - window + 1 : 0) & ~31;
+  const int n32 = (last_pos + 1 - tile_lo + 31) / 32;
+  const int share = 32 * ((n32 + PREFILL_WAVES - 1) / PREFILL_WAVES);
+  int begin = tile_lo + wave * share, end = begin + share;
+  if (end > last_pos + 1) end = last_pos + 1;
+  f32x4_t acc[NG][2 * NQK];
+  float m[NG], l[NG];
+  const bf16_t* const (&cqr)[NG] = cq;
+  attend_range<NQK, NG, 1>(cqr, clo, chi, begin, end, last_pos, k_pool, v_pool,
+                           block_table + (size_t)token_entry[first] * bt_stride, page_size, nkv, kvh, scale_log2e,
+                           acc, m, l);
+  merge_waves<NQK, NG, PREFILL_WAVES>(acc, m, l, merge);
+  if (wave != 0) return;
 #pragma unroll
-  for (int n = 0; n < 2 * NQK; ++n) {
-    uint2 w;
-    w.x = (uint32_t)f32_to_bf16_bits(acc[n][0] * inv) | ((uint32_t)f32_to_bf16_bits(acc[n][1] * inv) << 16);
-    w.y = (uint32_t)f32_to_bf16_bits(acc[n][2] * inv) | ((uint32_t)f32_to_bf16_bits(acc[n][3] * inv) << 16);
-    *reinterpret_cast<uint2*>(op + 16 * n + 4 * g) = w;
+  for (int qg = 0; qg < NG; ++qg) {
+    float lt = l[qg];
+    lt += __shfl_xor(lt, 16, 64);
+    lt += __shfl_xor(lt, 32, 64);
+    if (chi[qg] < 0) continue;
+    const float inv = lt > 0.f ? 1.f / lt : 0.f;
+    bf16_t* op = out + (size_t)tok[qg] * out_stride + (size_t)head * HD;
+#pragma unroll
+    for (int n = 0; n < 2 * NQK; ++n)
+      *reinterpret_cast<uint2*>(op + 16 * n + 4 * g) =
+          make_uint2(pack2_bf16(acc[qg][n][0] * inv, acc[qg][n][1] * inv),
+                     pack2_bf16(acc[qg][n][2] * inv, acc[qg][n][3] * inv));
   }
 }
+
+// tokens of one request a prompt tile may hold
+extern "C" int ullm_attention_prefill_tile(void) { return 16 * PREFILL_GROUPS; }
 
 static bool supported_hd(int hd) { return hd == 32 || hd == 64 || hd == 96 || hd == 128 || hd == 256; }
 
@@ -442,12 +521,12 @@ extern "C" int ullm_attention_prefill(
   if (n_tiles <= 0) return 0;
   if (!ullm_attention_mfma_supports(hd, page_size, nq, nkv)) return ULLM_ERR_UNSUPPORTED;
   if (window < 0) return ULLM_ERR_SHAPE;
-  const int G = nq / nkv, waves = G < 4 ? G : 4, hgroups = (G + waves - 1) / waves;
+  if ((long long)n_tiles * nq > 0x7fffffffLL) return ULLM_ERR_SHAPE;
   const float sl = scale * 1.4426950408889634f;
-  dim3 grid(n_tiles, nkv * hgroups), block(64 * waves);
+  dim3 grid(n_tiles * nq), block(64 * prefill_waves(hd / 32));
 #define CALL(N) hipLaunchKernelGGL(attention_prefill_kernel<N>, grid, block, 0, stream, (const bf16_t*)q, q_stride, \
     (bf16_t*)out, out_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool, tiles, positions, token_entry, \
-    block_table, bt_stride, page_size, nq, nkv, sl, window)
+    block_table, bt_stride, page_size, nq, nkv, sl, window, n_tiles)
   DISPATCH_NQK(hd, CALL)
 #undef CALL
   ULLM_LAUNCH_CHECK();

@@ -32,7 +32,7 @@ class StepError(RuntimeError):
     pass
 
 
-Q_TILE = 16     # tokens of one request that the prompt-portion attention kernel handles per wave
+from ..kernels.ops import PREFILL_TILE as Q_TILE   # tokens of one request per prompt-portion attention tile
 
 
 class ModelRunner:

@@ -343,11 +343,14 @@ def attention_decode_mfma(q, out, k_pool, v_pool, token_list: Optional[torch.Ten
         _c_int(splits), _c_int(waves), _p(ws), _stream()), "attention_decode")
 
 
+PREFILL_TILE = 32      # tokens of one request per prompt tile (two groups of 16 columns per wave)
+
+
 def attention_prefill_mfma(q, out, k_pool, v_pool, tiles: torch.Tensor, n_tiles: int, positions, token_entry,
                            block_table, page_size: int, nq: int, nkv: int, hd: int, scale: float,
                            window: int) -> None:
-    """Tiles (first token, count <= 16) of consecutive tokens of one request each, every token
-    against the keys up to its own position."""
+    """Tiles (first token, count <= PREFILL_TILE) of consecutive tokens of one request each, every
+    token against the keys up to its own position."""
     _check_pools(k_pool, v_pool, nkv, page_size, hd, torch.bfloat16)
     _need(q.dtype == torch.bfloat16 and q.stride(1) == 1 and q.shape[1] == nq * hd, "q must be bfloat16 [T, nq*hd]")
     _need(out.dtype == torch.bfloat16 and out.stride(1) == 1 and out.shape == q.shape, "bad attention output")

@@ -85,7 +85,7 @@ class StepContext:
     decode_only: bool             # every entry brings exactly one token
     dtype: torch.dtype = torch.bfloat16          # compute dtype of activations
     host: dict = field(default_factory=dict)   # host-side copies for parts that want them
-    # how attention kernels split the batch: tokens of one-token entries, and tiles of up to 16
+    # how attention kernels split the batch: tokens of one-token entries, and tiles of up to 32
     # consecutive tokens (first token, count) of the longer entries
     decode_tokens: Optional[torch.Tensor] = None   # int32 [n_decode]; None when every token is one
     num_decode: int = 0
