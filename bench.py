@@ -40,6 +40,8 @@ def parse_args():
     ap.add_argument("--dtype", default="bfloat16")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
     ap.add_argument("--eager", action="store_true", help="no HIP graphs")
+    ap.add_argument("--prefill-only", type=int, default=0, metavar="T",
+                    help="only time a T-token prompt and print its figures (for profiling)")
     return ap.parse_args()
 
 
@@ -144,6 +146,11 @@ def main():
         flops = step_flops(cfg, n_tokens, n_tokens * (n_tokens + 1) // 2, 1)
         return n_tokens / best, best * 1e3, flops / best / PEAK_FLOPS[args.dtype]
 
+    if args.prefill_only:
+        p_tok_s, p_ms, p_frac = run_prefill(args.prefill_only)
+        print(json.dumps({"prefill": {"value": round(p_tok_s, 1), "tokens": args.prefill_only, "ms": round(p_ms, 3),
+                                      "frac": round(p_frac, 4)}}))
+        return 0
     tok_s, ms, bytes_step = run_decode(args.batch, args.steps, args.warmup)
     achieved = bytes_step / (ms * 1e-3) / 1e9
     line = {
