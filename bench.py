@@ -27,6 +27,15 @@ QWEN3_8B = dict(architectures=["Qwen3ForCausalLM"], hidden_size=4096, num_hidden
                 tie_word_embeddings=False, attention_bias=False, use_sliding_window=False,
                 initializer_range=0.02, torch_dtype="bfloat16")
 
+# the reference's own benchmark (bench.py:10-45, README.md:129-147): Qwen3-0.6B, 256 requests, prompt and
+# generation lengths uniform in 100..1024, temperature 0.6, no end-of-sequence; 9032.37 tokens/s on an A100 40GB
+QWEN3_0P6B = dict(architectures=["Qwen3ForCausalLM"], hidden_size=1024, num_hidden_layers=28,
+                  num_attention_heads=16, num_key_value_heads=8, head_dim=128, intermediate_size=3072,
+                  vocab_size=151936, rope_theta=1000000.0, rms_norm_eps=1e-6, max_position_embeddings=40960,
+                  tie_word_embeddings=True, attention_bias=False, use_sliding_window=False,
+                  initializer_range=0.02, torch_dtype="bfloat16")
+REFERENCE_MIXED_TOK_S = 9032.37
+
 
 def parse_args():
     ap = argparse.ArgumentParser()
@@ -40,6 +49,8 @@ def parse_args():
     ap.add_argument("--dtype", default="bfloat16")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
     ap.add_argument("--eager", action="store_true", help="no HIP graphs")
+    ap.add_argument("--mixed-only", action="store_true",
+                    help="only the reference's own workload: 256 requests of mixed lengths, Qwen3-0.6B sizes")
     ap.add_argument("--prefill-only", type=int, default=0, metavar="T",
                     help="only time a T-token prompt and print its figures (for profiling)")
     return ap.parse_args()
@@ -67,6 +78,46 @@ def step_flops(cfg, n_tokens, kv_lens_sum_causal, n_logit_rows):
     return L * (per_token * n_tokens + attn) + 2 * H * V * n_logit_rows
 
 
+def run_mixed(dtype, eager):
+    """Output tokens per second over 256 requests arriving at once, continuous batching; returns
+    (tokens/s, output tokens, seconds, engine steps)."""
+    import random
+    import torch
+    from ullm_amd import EngineConfig, SamplingParams
+    from ullm_amd.engine.engine import Engine
+    from ullm_amd.engine.loading import make_env
+    from ullm_amd.models import build_model
+    from ullm_amd.weights.random_init import bind_random_weights
+
+    cfg, model = build_model(dict(QWEN3_0P6B))
+    env = make_env(dtype, "cuda:0", 4096)
+    bind_random_weights(model, env, seed=0)
+    rng = random.Random(0)
+    n = 256
+    prompts = [[rng.randint(0, 10000) for _ in range(rng.randint(100, 1024))] for _ in range(n)]
+    new_tokens = [rng.randint(100, 1024) for _ in range(n)]
+    ec = EngineConfig(model="(random)", dtype=dtype, max_bs=256, context_len=4096, page_size=16,
+                      num_pages=n * 130, max_num_batched_tokens=8192, max_prefill_chunk=2048, enforce_eager=eager)
+    eng = Engine(ec, model=model, env=env, model_config=cfg)
+    eng.add_request("warm", prompts[0][:64], SamplingParams(temperature=0.6, ignore_eos=True, max_new_tokens=10))
+    while eng.has_unfinished_requests():
+        eng.step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(n):
+        eng.add_request(f"m{i}", prompts[i], SamplingParams(temperature=0.6, ignore_eos=True, seed=i,
+                                                            max_new_tokens=new_tokens[i]))
+    steps = 0
+    while eng.has_unfinished_requests():
+        eng.step()
+        steps += 1
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    del eng
+    torch.cuda.empty_cache()
+    return sum(new_tokens) / dt, sum(new_tokens), dt, steps
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -79,6 +130,14 @@ def main():
     from ullm_amd.models import build_model
     from ullm_amd.weights.random_init import bind_random_weights
 
+    if args.mixed_only:
+        tok_s, n_out, secs, steps = run_mixed(args.dtype, args.eager)
+        print(json.dumps({"metric": "output tok/s, 256 requests, lengths 100..1024 in and out, Qwen3-0.6B sizes",
+                          "value": round(tok_s, 1), "unit": "tokens/s", "output_tokens": n_out,
+                          "seconds": round(secs, 3), "engine_steps": steps,
+                          "vs_baseline": round(tok_s / REFERENCE_MIXED_TOK_S, 3),
+                          "baseline": "9032.37 tokens/s, the reference on an A100 40GB"}))
+        return 0
     config = dict(QWEN3_8B)
     full_layers = config["num_hidden_layers"]
     if args.layers is not None:

@@ -18,6 +18,8 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 from typing import Dict, List, Optional, Sequence
 
+import numpy as np
+
 from .pages import PageAllocator, PageError
 from .prefix_tree import PrefixTree
 
@@ -64,6 +66,9 @@ class CacheManager:
         self.allocators = [PageAllocator(n) for n in num_pages]
         self._free_slots: List[int] = list(range(max_requests - 1, -1, -1))
         self._fresh_slots: List[int] = []
+        # the block tables once more as one int32 matrix per group, row = slot, -1 where a table holds
+        # no page: a step gathers its rows from here instead of converting Python lists
+        self._rows = [np.full((max_requests, 16), -1, dtype=np.int32) for _ in groups]
         self.requests: Dict[str, RequestCache] = {}
         shareable = all(g.window == 0 for g in groups) and len(groups) > 0
         self.prefix_tree: Optional[PrefixTree] = (
@@ -89,10 +94,31 @@ class CacheManager:
             for per_group in matched:
                 for g, page in enumerate(per_group):
                     rc.tables[g].append(page)
+            for g in range(len(self.groups)):
+                self._put_row(g, slot, 0, rc.tables[g])
             rc.num_computed = len(matched) * self.page_size
         self.requests[request_id] = rc
         self._fresh_slots.append(slot)
         return rc
+
+    def _put_row(self, g: int, slot: int, start: int, pages: Sequence[int]) -> None:
+        rows = self._rows[g]
+        end = start + len(pages)
+        if end > rows.shape[1]:
+            wider = np.full((rows.shape[0], max(end, 2 * rows.shape[1])), -1, dtype=np.int32)
+            wider[:, :rows.shape[1]] = rows
+            self._rows[g] = rows = wider
+        rows[slot, start:end] = pages
+
+    def table_rows(self, group: int, slots: Sequence[int], width: int) -> np.ndarray:
+        """int32 [len(slots), width]: the block tables of the requests in these slots, -1 where a
+        table holds no page."""
+        rows = self._rows[group]
+        if width <= rows.shape[1]:
+            return rows[slots, :width]
+        out = np.full((len(slots), width), -1, dtype=np.int32)
+        out[:, :rows.shape[1]] = rows[slots]
+        return out
 
     def take_fresh_slots(self) -> List[int]:
         """Slots admitted since the last call: their state rows must be zeroed before they step."""
@@ -117,6 +143,8 @@ class CacheManager:
         if n_new < 1:
             raise ValueError("reserve needs at least one token")
         needs = self.pages_needed(rc, n_new)
+        if not any(needs):
+            return True
         for g, need in enumerate(needs):
             short = need - self.allocators[g].num_free
             if short > 0 and self.prefix_tree is not None:
@@ -124,9 +152,11 @@ class CacheManager:
             if need > self.allocators[g].num_free:
                 return False
         for g, need in enumerate(needs):
-            pages = self.allocators[g].alloc(need)
-            assert pages is not None
-            rc.tables[g].extend(pages)
+            if need:
+                pages = self.allocators[g].alloc(need)
+                assert pages is not None
+                self._put_row(g, rc.slot, len(rc.tables[g]), pages)
+                rc.tables[g].extend(pages)
         return True
 
     def commit(self, rc: RequestCache, n_new: int) -> None:
@@ -147,6 +177,7 @@ class CacheManager:
                     if table[i] >= 0:
                         self.allocators[g].decref(table[i])
                         table[i] = -1
+                        self._rows[g][rc.slot, i] = -1
                 rc.first_live[g] = max(rc.first_live[g], min(dead_upto, len(table)))
 
     def release(self, rc: RequestCache, tokens: Optional[Sequence[int]] = None) -> None:
@@ -162,6 +193,7 @@ class CacheManager:
                 if p >= 0:
                     self.allocators[g].decref(p)
             table.clear()
+            self._rows[g][rc.slot] = -1
         rc.released = True
         self._free_slots.append(rc.slot)
         if rc.slot in self._fresh_slots:
@@ -175,6 +207,7 @@ class CacheManager:
                 if p >= 0:
                     self.allocators[g].decref(p)
             table.clear()
+            self._rows[g][rc.slot] = -1
             rc.first_live[g] = 0
         rc.num_computed = 0
         if rc.slot not in self._fresh_slots:
@@ -213,6 +246,12 @@ class CacheManager:
                     raise PageError(f"group {g} page {p}: {holders[p]} holders found, count says {alloc.refcount(p)}")
                 if holders[p] > 1 and p not in tree_pages:
                     raise PageError(f"group {g} page {p} is in {holders[p]} block tables without a shared prefix")
+        for g in range(len(self.groups)):
+            held = np.full_like(self._rows[g], -1)
+            for rc in self.requests.values():
+                held[rc.slot, :len(rc.tables[g])] = rc.tables[g]
+            if not np.array_equal(held, self._rows[g]):
+                raise PageError(f"group {g}: the table matrix differs from the requests' block tables")
         slots = [rc.slot for rc in self.requests.values()]
         if len(set(slots)) != len(slots) or set(slots) & set(self._free_slots):
             raise PageError("a request slot is held twice")

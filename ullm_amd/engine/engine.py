@@ -106,14 +106,16 @@ class Engine:
             return results
         entries = [StepEntry(s.request.cache, s.request.token_ids[s.start:s.start + s.num_tokens],
                              [s.num_tokens - 1] if s.samples else []) for s in scheduled]
-        logits = self.runner.step(entries)
         sampling = [s for s in scheduled if s.samples]
+        prepared = None
+        if sampling:                                      # uploaded ahead of the model step
+            prepared = self.sampler.prepare([s.request.params for s in sampling], [s.request.seed for s in sampling],
+                                            [s.request.num_tokens for s in sampling])
+        logits = self.runner.step(entries)
         if sampling:
             if self.on_logits is not None:
                 self.on_logits(sampling, logits)
-            ids = self.sampler.sample(logits, [s.request.params for s in sampling],
-                                      [s.request.seed for s in sampling],
-                                      [s.request.num_tokens for s in sampling])
+            ids = self.sampler.sample(logits, prepared=prepared)
             for s, tok in zip(sampling, ids):
                 req = s.request
                 self.scheduler.append_token(req, tok)

@@ -17,6 +17,7 @@ import torch
 from ..cache.manager import CacheManager, RequestCache
 from ..models.model import Model
 from ..parts import GroupView, LayerCache, PartEnv, StepContext
+from ..staging import StagedUpload
 
 
 @dataclass
@@ -61,10 +62,7 @@ class ModelRunner:
         for cache_id, need in states.items():
             self.caches[cache_id] = LayerCache(
                 state=torch.zeros((max_requests,) + tuple(need.shape), dtype=need.dtype, device=env.device))
-        self._pin = env.device.type == "cuda"
-        self._staging: List[Optional[torch.Tensor]] = [None, None]   # two host buffers, used in turn
-        self._staging_done: List[Optional[torch.cuda.Event]] = [None, None]
-        self._turn = 0
+        self._upload = StagedUpload(env.device)
         self.vocab_size = model.plan.vocab_size
         # Steps in which every entry brings one token are replayed from HIP graphs, one graph per
         # (batch size bucket, context length bucket).  Padding entries would disturb per-request state,
@@ -82,30 +80,6 @@ class ModelRunner:
                 if t is not None:
                     total += t.numel() * t.element_size()
         return total
-
-    def _upload(self, host: np.ndarray, into: Optional[torch.Tensor] = None) -> torch.Tensor:
-        """Copy the packed batch description to the device (into ``into`` if given) through one of two
-        pinned buffers; a buffer is written again only after the copy that last read it has finished."""
-        i = self._turn
-        self._turn ^= 1
-        if self._staging_done[i] is not None:
-            self._staging_done[i].synchronize()
-        if self._staging[i] is None or self._staging[i].numel() < host.size:
-            self._staging[i] = torch.empty(max(host.size, 4096), dtype=torch.int32, pin_memory=self._pin)
-        stage = self._staging[i][:host.size]
-        stage.numpy()[:] = host
-        if into is not None:
-            into.copy_(stage, non_blocking=True)
-            dev = into
-        else:
-            dev = stage.to(self.env.device, non_blocking=True)
-        if self._pin:
-            ev = torch.cuda.Event()
-            ev.record()
-            self._staging_done[i] = ev
-        elif dev.data_ptr() == stage.data_ptr():
-            dev = dev.clone()
-        return dev
 
     def _pack(self, entries: Sequence[StepEntry], pad_entries: int = 0, table_stride: Optional[int] = None):
         """Flatten the entries into one int32 host array.  Returns (host array, offsets, facts).
@@ -147,41 +121,57 @@ class ModelRunner:
         ids, pos, ent = host[offs[0]:offs[1]], host[offs[1]:offs[2]], host[offs[2]:offs[3]]
         q_start, slot, start = host[offs[3]:offs[4]], host[offs[4]:offs[5]], host[offs[5]:offs[6]]
         rows = host[offs[6]:offs[7]]
-        t = 0
-        r = 0
-        max_kv = 0
-        seen = set()
-        for b, e in enumerate(entries):
-            rc, n = e.cache, lens[b]
+        caches = [e.cache for e in entries]
+        starts = [rc.num_computed for rc in caches]
+        slots = [rc.slot for rc in caches]
+        for rc, n, s0 in zip(caches, lens, starts):
             if n < 1:
                 raise StepError(f"request {rc.request_id!r}: an entry needs at least one token")
             if rc.released:
                 raise StepError(f"request {rc.request_id!r} was released")
-            if id(rc) in seen:
-                raise StepError(f"request {rc.request_id!r} appears twice in one step")
-            seen.add(id(rc))
-            s0 = rc.num_computed
             if s0 + n > self.env.context_len:
                 raise StepError(f"request {rc.request_id!r}: {s0 + n} tokens exceed context_len={self.env.context_len}")
-            for g in range(ng):
-                if len(rc.tables[g]) * P < s0 + n:
+            for tab in rc.tables:
+                if len(tab) * P < s0 + n:
                     raise StepError(f"request {rc.request_id!r}: no pages reserved for positions up to {s0 + n - 1}")
-            tok = np.asarray(e.tokens, dtype=np.int64)
-            if tok.min() < 0 or tok.max() >= self.vocab_size:
-                raise StepError(f"request {rc.request_id!r}: token id outside [0, {self.vocab_size})")
-            ids[t:t + n] = tok
-            pos[t:t + n] = np.arange(s0, s0 + n)
-            ent[t:t + n] = b
-            q_start[b] = t
-            slot[b] = rc.slot
-            start[b] = s0
+        if len(set(slots)) != n_real:
+            seen = set()
+            for rc in caches:
+                if rc.slot in seen:
+                    raise StepError(f"request {rc.request_id!r} appears twice in one step")
+                seen.add(rc.slot)
+        n_tok = T - n_pad
+        tok = np.empty(n_tok, dtype=np.int64)
+        if n_tok == n_real:                              # one token each: no per-entry array work
+            tok[:] = [e.tokens[0] for e in entries]
+            pos[:n_real] = starts
+            ent[:n_real] = np.arange(n_real)
+            q_start[:n_real] = ent[:n_real]
+        else:
+            first = np.zeros(n_real + 1, dtype=np.int64)
+            np.cumsum(lens, out=first[1:])
+            q_start[:n_real] = first[:n_real]
+            ent[:n_tok] = np.repeat(np.arange(n_real), lens)
+            pos[:n_tok] = np.arange(n_tok) - np.repeat(first[:n_real] - np.asarray(starts, dtype=np.int64), lens)
+            t = 0
+            for e, n in zip(entries, lens):
+                tok[t:t + n] = e.tokens
+                t += n
+        if int(tok.min()) < 0 or int(tok.max()) >= self.vocab_size:
+            bad = next(rc for rc, e in zip(caches, entries) if min(e.tokens) < 0 or max(e.tokens) >= self.vocab_size)
+            raise StepError(f"request {bad.request_id!r}: token id outside [0, {self.vocab_size})")
+        ids[:n_tok] = tok
+        slot[:n_real] = slots
+        start[:n_real] = starts
+        r = 0
+        for b, e in enumerate(entries):
             for w in e.want:
-                if not (0 <= w < n):
-                    raise StepError(f"request {rc.request_id!r}: wanted place {w} outside its {n} tokens")
-                rows[r] = t + w
+                if not (0 <= w < lens[b]):
+                    raise StepError(f"request {caches[b].request_id!r}: wanted place {w} outside its {lens[b]} tokens")
+                rows[r] = q_start[b] + w
                 r += 1
-            max_kv = max(max_kv, s0 + n)
-            t += n
+        max_kv = max(s0 + n for s0, n in zip(starts, lens))
+        t = n_tok
         for b in range(n_real, B):                       # padding entries: token 0 at position 0, no pages
             ent[t] = b
             q_start[b] = t
@@ -191,17 +181,14 @@ class ModelRunner:
         q_start[B] = T
         for g, s in enumerate(strides):
             bt = host[offs[7 + g]:offs[8 + g]].reshape(B, s)
-            bt.fill(-1)
-            for b, e in enumerate(entries):
-                tab = e.cache.tables[g]
-                bt[b, :len(tab)] = tab
+            bt[:n_real] = self.cache.table_rows(g, slots, s)
+            bt[n_real:] = -1
         host[offs[7 + ng]:offs[8 + ng]] = dec_list
         host[offs[8 + ng]:offs[9 + ng]] = tile_list
         facts = dict(T=T, B=B, strides=strides, n_want=n_want, num_decode=len(dec_list), max_dec_kv=max_dec_kv,
                      num_tiles=len(tile_list) // 2, max_q=max(lens), max_kv=max_kv,
                      decode_only=all(n == 1 for n in lens), lens=lens + [1] * n_pad,
-                     starts=[e.cache.num_computed for e in entries] + [0] * n_pad,
-                     slots=[e.cache.slot for e in entries] + [0] * n_pad)
+                     starts=starts + [0] * n_pad, slots=slots + [0] * n_pad)
         return host, offs, facts
 
     def _context(self, dev: torch.Tensor, offs, facts) -> tuple:

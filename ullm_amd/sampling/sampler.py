@@ -4,36 +4,57 @@ One kernel launch per step for all rows; each row carries its own parameters and
 (seed, position), so what a request draws does not depend on the rest of the batch."""
 from __future__ import annotations
 
-from typing import List, Sequence
+from dataclasses import dataclass
+from typing import List, Optional, Sequence
 
 import numpy as np
 import torch
 
 from ..kernels import ops
+from ..staging import StagedUpload
 from .params import SamplingParams
+
+
+@dataclass
+class SamplerInputs:
+    """Per-row parameters on the device: rows of one int32 buffer (the float ones bit-cast)."""
+    n: int
+    packed: torch.Tensor      # int32 [7, n]: temperature, top_p, min_p (float bits), top_k, seed low, seed high, position
 
 
 class Sampler:
     def __init__(self, device: torch.device):
         self.device = device
+        self._upload = StagedUpload(device)
 
-    def sample(self, logits: torch.Tensor, params: Sequence[SamplingParams], seeds: Sequence[int],
-               positions: Sequence[int]) -> List[int]:
-        """``logits`` float32 [n, V]; ``positions[i]`` = index the new token of row i will take in its
-        request (the counter of the row's random stream).  Returns n token ids."""
-        n = logits.shape[0]
-        if not (len(params) == len(seeds) == len(positions) == n):
+    def prepare(self, params: Sequence[SamplingParams], seeds: Sequence[int], positions: Sequence[int]) -> SamplerInputs:
+        """Queue the upload of the rows' parameters.  Called before the model step is launched, the
+        copy does not wait for the step, and sampling can follow it without the host in between.
+        ``positions[i]`` = index the new token of row i will take in its request (the counter of
+        the row's random stream)."""
+        n = len(params)
+        if not (len(seeds) == len(positions) == n):
             raise ValueError("one parameter set, seed and position per logits row is needed")
-        f = np.empty((3, n), dtype=np.float32)
-        i = np.empty((4, n), dtype=np.int32)
-        for r, (p, s, pos) in enumerate(zip(params, seeds, positions)):
-            f[0, r], f[1, r], f[2, r] = p.temperature, p.top_p, p.min_p
-            s &= (1 << 64) - 1
-            i[0, r] = p.top_k
-            i[1, r] = np.uint32(s & 0xFFFFFFFF).astype(np.int32)
-            i[2, r] = np.uint32(s >> 32).astype(np.int32)
-            i[3, r] = pos
-        fd = torch.from_numpy(f).to(self.device)
-        idev = torch.from_numpy(i).to(self.device)
-        out = ops.sample(logits, fd[0], idev[0], fd[1], fd[2], idev[1], idev[2], idev[3])
+        host = np.empty((7, n), dtype=np.int32)
+        host[0:3].view(np.float32)[:] = [[p.temperature for p in params], [p.top_p for p in params],
+                                         [p.min_p for p in params]]
+        host[3] = [p.top_k for p in params]
+        s64 = np.array([s & 0xFFFFFFFFFFFFFFFF for s in seeds], dtype=np.uint64)
+        host[4] = (s64 & np.uint64(0xFFFFFFFF)).astype(np.uint32).view(np.int32)
+        host[5] = (s64 >> np.uint64(32)).astype(np.uint32).view(np.int32)
+        host[6] = positions
+        return SamplerInputs(n, self._upload(host.reshape(-1)).view(7, n))
+
+    def sample(self, logits: torch.Tensor, params: Optional[Sequence[SamplingParams]] = None,
+               seeds: Optional[Sequence[int]] = None, positions: Optional[Sequence[int]] = None,
+               prepared: Optional[SamplerInputs] = None) -> List[int]:
+        """``logits`` float32 [n, V]; the rows' parameters either as lists or as the result of
+        :meth:`prepare`.  Returns n token ids."""
+        if prepared is None:
+            prepared = self.prepare(params, seeds, positions)
+        if prepared.n != logits.shape[0]:
+            raise ValueError("one parameter set, seed and position per logits row is needed")
+        f = prepared.packed[0:3].view(torch.float32)
+        i = prepared.packed
+        out = ops.sample(logits, f[0], i[3], f[1], f[2], i[4], i[5], i[6])
         return out.tolist()
