@@ -233,6 +233,13 @@ def main():
         b1, _, _ = run_decode(1, min(args.steps, 32), min(args.warmup, 4))
         b64, _, _ = run_decode(64, min(args.steps, 32), min(args.warmup, 4))
         line["points"] = {"decode_b1": round(b1, 2), "decode_b64": round(b64, 2)}
+        del model
+        torch.cuda.empty_cache()
+        m_tok_s, m_out, m_secs, _ = run_mixed(args.dtype, args.eager)
+        # the reference's own benchmark (Qwen3-0.6B, 256 requests); its 9032.37 tokens/s are from an A100 40GB
+        line["mixed_qwen3_0p6b"] = {"value": round(m_tok_s, 1), "unit": "output tokens/s", "output_tokens": m_out,
+                                    "seconds": round(m_secs, 3),
+                                    "vs_reference_a100": round(m_tok_s / REFERENCE_MIXED_TOK_S, 3)}
     print(json.dumps(line))
     return 0
 

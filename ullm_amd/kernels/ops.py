@@ -273,18 +273,22 @@ SKINNY_MAX_ROWS = 16     # up to here the weight-streaming kernel beats the libr
 def gemm_bf16(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
               out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
     """bfloat16 operands, 32-bit accumulation.  Few rows go to the weight-streaming kernel; many
-    rows with bfloat16 output go through the library product (as the reference's linears do,
-    ullm/layers/linear.py:165); 32-bit output (logits) always comes from a hand-written kernel,
-    which keeps the accumulator's precision."""
+    rows go through the library product (as the reference's linears do, ullm/layers/linear.py:165),
+    which for 32-bit output (logits) stores the accumulator unrounded."""
     out_dtype = out_dtype or a.dtype
     M = a.shape[0]
-    if (M <= SKINNY_MAX_ROWS or (out_dtype == torch.float32 and M <= 64)) and gemm_skinny_supports(a, w):
+    library = a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and a.is_cuda
+    if library and out_dtype == torch.float32 and a.is_contiguous() and w.is_contiguous():
+        # the widest product of a step (the vocabulary): the library streams it a little faster at any M
+        y = torch.mm(a, w.t(), out_dtype=torch.float32)
+        return y if bias is None else y + bias
+    if M <= SKINNY_MAX_ROWS and gemm_skinny_supports(a, w):
         return gemm_skinny(a, w, bias, out_dtype=out_dtype)
-    if out_dtype == torch.bfloat16 and a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16:
+    if library and out_dtype == torch.bfloat16:
         y = torch.nn.functional.linear(a, w)
-        if bias is not None:
-            y = (y.float() + bias).to(torch.bfloat16)
-        return y
+        return y if bias is None else (y.float() + bias).to(torch.bfloat16)
+    if out_dtype == torch.float32 and M <= 64 and gemm_skinny_supports(a, w):
+        return gemm_skinny(a, w, bias, out_dtype=out_dtype)
     return gemm_simple(a, w, bias, out_dtype=out_dtype)
 
 
