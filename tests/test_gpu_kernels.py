@@ -265,6 +265,10 @@ MFMA_CASES = [dict(nq=8, nkv=2, hd=32, P=16, lens=[(1, 1), (1, 37), (1, 300), (1
               dict(nq=32, nkv=8, hd=128, P=16, lens=[(100, 100), (7, 260)], window=0),
               dict(nq=32, nkv=16, hd=32, P=16, lens=[(70, 70), (33, 90), (1, 5)], window=0),      # kv heads 2 x 8
               dict(nq=6, nkv=2, hd=64, P=32, lens=[(40, 90), (3, 3)], window=21),
+              dict(nq=10, nkv=2, hd=96, P=16, lens=[(45, 45), (2, 66)], window=0),       # 5 heads per kv head: 4 + 1 waves
+              dict(nq=3, nkv=3, hd=256, P=16, lens=[(37, 80)], window=0),               # one head per kv head
+              dict(nq=4, nkv=1, hd=128, P=16, lens=[(40, 1200), (64, 64)], window=0),   # page ids refetched past 1024 keys
+              dict(nq=4, nkv=2, hd=64, P=48, lens=[(50, 1100)], window=300),
               dict(nq=8, nkv=2, hd=32, P=16, lens=[(1, 45), (9, 40), (1, 200), (20, 20), (1, 1)], window=0),  # mixed
               dict(nq=8, nkv=2, hd=32, P=16, lens=[(1, 45), (9, 40), (1, 200), (20, 50)], window=13)]
 

@@ -377,72 +377,253 @@ attention_reduce_kernel(const float* __restrict__ part, bf16_t* __restrict__ out
 }
 
 // ------------------------------------------------------------------------------- prompt portions
-// grid (n_tiles * nq), block 256 (128 for head_dim 256).  Workgroups go to the 8 XCDs round-robin by
-// their linear id and each XCD has an L2 of its own, so the id is decoded such that all work on one kv
-// head lands on one XCD (kv head = id mod 8 when the kv heads are a multiple of 8): that head's keys
-// and values then stay in that L2 instead of every XCD streaming every head from memory.  Tiles are
-// taken last first (under the causal mask they see the most keys).
-// Tile = (first token, number of tokens <= 32) of one request: two
-// groups of 16 tokens share every key/value tile a wave loads.  The keys the tile's tokens see are
-// cut into equal shares of whole 32-key tiles, one per wave (under a causal mask the last tiles of
-// a long prompt see far more keys than the first; cutting by keys keeps every wave's walk short),
-// and the waves merge as in the decode kernel.
+// Tile = (first token, number of tokens <= 32) of one request.  A block of PREFILL_WAVES waves works
+// on one tile for up to PREFILL_WAVES query heads that share a kv head, one head per wave (two groups
+// of 16 tokens each), so every 32-key tile of keys and values is fetched from memory once per block
+// and shared through LDS:
+//   keys   LDS row = one key, head_dim values + 16 bytes of padding
+//   values LDS row = one dim, its 32 keys in the order [g][half][4] (the 8 keys lane group g feeds to
+//          one product are 16 adjacent bytes) + 16 bytes of padding
+// With these paddings the 16 lanes that the hardware serves together read 16 different bank groups.
+// Loads run two tiles ahead of the products (two register sets in rotation), the single LDS tile is
+// rewritten between two barriers.
+// grid (n_tiles * nkv * head_chunks).  Workgroups go to the 8 XCDs round-robin by their linear id and
+// each XCD has an L2 of its own, so the id is decoded such that all work on one kv head lands on one
+// XCD (kv head = id mod 8 when the kv heads are a multiple of 8): that head's keys and values then
+// stay in that L2 instead of every XCD streaming every head from memory.  Tiles are taken last first
+// (under the causal mask they see the most keys).
 #define PREFILL_GROUPS 2
-// waves per block: four, or two for head_dim 256 (shared memory of the merge)
-__host__ __device__ constexpr int prefill_waves(int nqk) { return nqk >= 8 ? 2 : 4; }
+#define PREFILL_WAVES 4
+
 template <int NQK>
-__global__ void __launch_bounds__(64 * prefill_waves(NQK))
+struct PrefillStage {                     // one 32-key tile on its way from the cache to LDS
+  static constexpr int HD = 32 * NQK;
+  static constexpr int THREADS = 64 * PREFILL_WAVES;
+  static constexpr int CHUNKS = 4 * HD;   // 16-byte pieces of the key tile, and as many of the value tile
+  static constexpr int PER_THREAD = (CHUNKS + THREADS - 1) / THREADS;
+  static constexpr int KROW = 2 * HD + 16, VROW = 64 + 16;     // bytes
+  static constexpr int KBYTES = 32 * KROW, VBYTES = HD * VROW;
+  uint4 k[PER_THREAD], v[PER_THREAD];
+};
+
+// Queue the loads of the tile at key0.  A wave's 64 pieces of one round lie in one 16-key sub-block,
+// so its page id is a single lane of the page window.
+template <int NQK>
+__device__ __forceinline__ void stage_load(PrefillStage<NQK>& st, int key0, const PageWindow& pw,
+                                           const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
+                                           int page_size, int nkv, int kvh) {
+  using S = PrefillStage<NQK>;
+  constexpr int HD = S::HD;
+  const int tid = threadIdx.x;
+#pragma unroll
+  for (int j = 0; j < S::PER_THREAD; ++j) {
+    const int piece = tid + j * S::THREADS;
+    st.k[j] = make_uint4(0, 0, 0, 0);
+    st.v[j] = make_uint4(0, 0, 0, 0);
+    if (piece >= S::CHUNKS) continue;
+    const int sb = __builtin_amdgcn_readfirstlane(piece / (2 * HD));      // 2 HD pieces per sub-block
+    const int kb = key0 + 16 * sb;
+    const int page = __builtin_amdgcn_readlane(pw.page, (kb >> 4) - pw.base);
+    if (page < 0) continue;
+    const int off = kb % page_size, rem = piece % (2 * HD);
+    const size_t base = ((size_t)page * nkv + kvh) * page_size * HD;
+    // keys: row rem / (HD / 8) of the sub-block, 8 values at column 8 (rem % (HD / 8))
+    st.k[j] = *reinterpret_cast<const uint4*>(k_pool + base + (size_t)(off + rem / (HD / 8)) * HD + 8 * (rem % (HD / 8)));
+    // values: dim rem / 2, keys off + 8 (rem % 2) .. +8 of the sub-block
+    st.v[j] = *reinterpret_cast<const uint4*>(v_pool + base + (size_t)(rem / 2) * page_size + off + 8 * (rem % 2));
+  }
+}
+
+// Write a loaded tile to LDS; values of keys past max_hi (never written, may hold anything) become 0.
+template <int NQK>
+__device__ __forceinline__ void stage_store(const PrefillStage<NQK>& st, int key0, int max_hi,
+                                            unsigned char* __restrict__ kl, unsigned char* __restrict__ vl) {
+  using S = PrefillStage<NQK>;
+  constexpr int HD = S::HD;
+  const int tid = threadIdx.x;
+  const bool edge = key0 + 32 > max_hi + 1;
+#pragma unroll
+  for (int j = 0; j < S::PER_THREAD; ++j) {
+    const int piece = tid + j * S::THREADS;
+    if (piece >= S::CHUNKS) continue;
+    const int sb = piece / (2 * HD), rem = piece % (2 * HD);
+    *reinterpret_cast<uint4*>(kl + (16 * sb + rem / (HD / 8)) * S::KROW + 16 * (rem % (HD / 8))) = st.k[j];
+    Pack8 v;
+    v.u4 = st.v[j];
+    const int half = rem % 2;
+    if (edge) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        if (key0 + 16 * sb + 8 * half + e > max_hi) v.h[e] = 0;
+    }
+    unsigned char* row = vl + (rem / 2) * S::VROW + 8 * sb;
+    *reinterpret_cast<uint2*>(row + 16 * (2 * half)) = v.u2[0];         // keys 8 half .. +4 -> lane group 2 half
+    *reinterpret_cast<uint2*>(row + 16 * (2 * half + 1)) = v.u2[1];     // keys 8 half + 4 .. +4 -> group 2 half + 1
+  }
+}
+
+// Scores, softmax update and value product of one wave for the tile in LDS.  `masked` = some key of
+// the tile is hidden from some column (diagonal, window or end of data); otherwise no per-score test.
+template <int NQK, int NG>
+__device__ __forceinline__ void process_tile_lds(const unsigned char* __restrict__ kl, const unsigned char* __restrict__ vl,
+                                                 int key0, bool masked, const Pack8 (&qreg)[NG][NQK],
+                                                 const int (&col_lo)[NG], const int (&col_hi)[NG], float scale_log2e,
+                                                 f32x4_t (&acc)[NG][2 * NQK], float (&m)[NG], float (&l)[NG]) {
+  using S = PrefillStage<NQK>;
+  const int lane = threadIdx.x & 63, g = lane >> 4, c = lane & 15;
+  f32x4_t s[NG][2];
+#pragma unroll
+  for (int q = 0; q < NG; ++q) s[q][0] = s[q][1] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int sb = 0; sb < 2; ++sb)
+#pragma unroll
+    for (int ch = 0; ch < NQK; ++ch) {
+      Pack8 kf;
+      kf.u4 = *reinterpret_cast<const uint4*>(kl + (16 * sb + c) * S::KROW + 64 * ch + 16 * g);
+#pragma unroll
+      for (int q = 0; q < NG; ++q)
+        s[q][sb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qreg[q][ch].v, s[q][sb], 0, 0, 0);
+    }
+  Pack8 p[NG];
+  float alpha[NG];
+#pragma unroll
+  for (int q = 0; q < NG; ++q) {
+    float tile_max = NEG_BIG;
+#pragma unroll
+    for (int sb = 0; sb < 2; ++sb)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        float v = s[q][sb][r] * scale_log2e;
+        if (masked) {
+          const int kk = key0 + 16 * sb + 4 * g + r;
+          v = (kk >= col_lo[q] && kk <= col_hi[q]) ? v : NEG_BIG;
+        }
+        s[q][sb][r] = v;
+        tile_max = fmaxf(tile_max, v);
+      }
+    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, 64));
+    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, 64));
+    const float m_new = fmaxf(m[q], tile_max);
+    alpha[q] = fast_exp2(m[q] - m_new);
+    float psum = 0.f;
+#pragma unroll
+    for (int sb = 0; sb < 2; ++sb) {
+      float e[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        // a masked score stays at NEG_BIG: its weight is zero even while m_new is still NEG_BIG
+        e[r] = (!masked || s[q][sb][r] > 0.5f * NEG_BIG) ? fast_exp2(s[q][sb][r] - m_new) : 0.f;
+        psum += e[r];
+      }
+      p[q].w[2 * sb] = pack2_bf16(e[0], e[1]);
+      p[q].w[2 * sb + 1] = pack2_bf16(e[2], e[3]);
+    }
+    l[q] = l[q] * alpha[q] + psum;
+    m[q] = m_new;
+  }
+#pragma unroll
+  for (int n = 0; n < 2 * NQK; ++n) {
+    Pack8 vf;
+    vf.u4 = *reinterpret_cast<const uint4*>(vl + (16 * n + c) * S::VROW + 16 * g);
+#pragma unroll
+    for (int q = 0; q < NG; ++q) {
+      f32x4_t o = acc[q][n];
+      o[0] *= alpha[q]; o[1] *= alpha[q]; o[2] *= alpha[q]; o[3] *= alpha[q];
+      acc[q][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, p[q].v, o, 0, 0, 0);
+    }
+  }
+}
+
+template <int NQK>
+__global__ void __launch_bounds__(64 * PREFILL_WAVES)
 attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
                          const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
                          const int* __restrict__ tiles, const int* __restrict__ positions,
                          const int* __restrict__ token_entry, const int* __restrict__ block_table,
                          int bt_stride, int page_size, int nq, int nkv, float scale_log2e, int window,
                          int n_tiles) {
+  using S = PrefillStage<NQK>;
   constexpr int HD = 32 * NQK;
   constexpr int NG = PREFILL_GROUPS;
-  constexpr int PREFILL_WAVES = prefill_waves(NQK);
-  __shared__ float merge[(PREFILL_WAVES / 2) * NG * (8 * NQK + 2) * 64];
+  __shared__ __attribute__((aligned(16))) unsigned char k_lds[S::KBYTES];
+  __shared__ __attribute__((aligned(16))) unsigned char v_lds[S::VBYTES];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, g = lane >> 4, c = lane & 15;
-  const int G = nq / nkv;
-  int kvh, tile_idx, head;
+  const int G = nq / nkv, chunks = (G + PREFILL_WAVES - 1) / PREFILL_WAVES, per_kv = n_tiles * chunks;
+  int kvh, rest;
   if (nkv % 8 == 0) {
-    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, per_kv = n_tiles * G;
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
     kvh = (slot / per_kv) * 8 + xcd;
-    tile_idx = (slot % per_kv) / G;
-    head = kvh * G + (slot % per_kv) % G;
+    rest = slot % per_kv;
   } else {
-    tile_idx = blockIdx.x / nq;
-    head = blockIdx.x % nq;
-    kvh = head / G;
+    kvh = blockIdx.x / per_kv;
+    rest = blockIdx.x % per_kv;
   }
-  tile_idx = n_tiles - 1 - tile_idx;
+  const int tile_idx = n_tiles - 1 - rest / chunks;
+  const int head_in_group = (rest % chunks) * PREFILL_WAVES + wave;
+  const bool head_ok = head_in_group < G;                 // a wave without a head still helps to load
+  const int head = kvh * G + (head_ok ? head_in_group : G - 1);
   const int first = tiles[2 * tile_idx], count = tiles[2 * tile_idx + 1];
-  const bf16_t* cq[NG];
   int clo[NG], chi[NG], tok[NG];
+  Pack8 qreg[NG][NQK];
 #pragma unroll
   for (int qg = 0; qg < NG; ++qg) {
-    const bool ok = 16 * qg + c < count;
-    tok[qg] = first + (ok ? 16 * qg + c : 0);
+    const bool ok = head_ok && 16 * qg + c < count;
+    tok[qg] = first + (16 * qg + c < count ? 16 * qg + c : 0);
     const int pos = positions[tok[qg]];
     clo[qg] = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
     chi[qg] = ok ? pos : -1;
-    cq[qg] = ok ? q + (size_t)tok[qg] * q_stride + (size_t)head * HD : nullptr;
+    const bf16_t* qp = q + (size_t)tok[qg] * q_stride + (size_t)head * HD + 8 * g;
+#pragma unroll
+    for (int ch = 0; ch < NQK; ++ch) {
+      if (ok) qreg[qg][ch].u4 = *reinterpret_cast<const uint4*>(qp + 32 * ch);
+      else qreg[qg][ch].u4 = make_uint4(0, 0, 0, 0);
+    }
   }
   const int last_pos = positions[first + count - 1];
   const int first_pos = positions[first];
-  const int tile_lo = ((window > 0 && first_pos - window + 1 > 0) ? first_pos - window + 1 : 0) & ~31;
-  const int n32 = (last_pos + 1 - tile_lo + 31) / 32;
-  const int share = 32 * ((n32 + PREFILL_WAVES - 1) / PREFILL_WAVES);
-  int begin = tile_lo + wave * share, end = begin + share;
-  if (end > last_pos + 1) end = last_pos + 1;
+  // keys every column of the tile sees without a test: from the last column's window start up to the first column
+  const int open_lo = (window > 0 && last_pos - window + 1 > 0) ? last_pos - window + 1 : 0;
+  const int key_begin = ((window > 0 && first_pos - window + 1 > 0) ? first_pos - window + 1 : 0) & ~31;
+  const int key_end = last_pos + 1;
+  const int* bt = block_table + (size_t)token_entry[first] * bt_stride;
   f32x4_t acc[NG][2 * NQK];
   float m[NG], l[NG];
-  const bf16_t* const (&cqr)[NG] = cq;
-  attend_range<NQK, NG, 1>(cqr, clo, chi, begin, end, last_pos, k_pool, v_pool,
-                           block_table + (size_t)token_entry[first] * bt_stride, page_size, nkv, kvh, scale_log2e,
-                           acc, m, l);
-  merge_waves<NQK, NG, PREFILL_WAVES>(acc, m, l, merge);
-  if (wave != 0) return;
+#pragma unroll
+  for (int qg = 0; qg < NG; ++qg) {
+#pragma unroll
+    for (int n = 0; n < 2 * NQK; ++n) acc[qg][n] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    m[qg] = NEG_BIG;
+    l[qg] = 0.f;
+  }
+  // the page window serves the loads, which run ahead of the products
+  PageWindow pw = load_pages(key_begin, key_end, bt, page_size);
+  PrefillStage<NQK> st0, st1;
+#define STAGE_LOAD(ST, K0)                                                         \
+  do {                                                                             \
+    if ((K0) < key_end) {                                                          \
+      if ((K0) >= 16 * (pw.base + 64)) pw = load_pages((K0), key_end, bt, page_size); \
+      stage_load<NQK>(ST, (K0), pw, k_pool, v_pool, page_size, nkv, kvh);          \
+    }                                                                              \
+  } while (0)
+#define STAGE_WORK(ST, K0)                                                         \
+  do {                                                                             \
+    __syncthreads();                         /* the previous tile has been read by every wave */ \
+    stage_store<NQK>(ST, (K0), last_pos, k_lds, v_lds);                            \
+    STAGE_LOAD(ST, (K0) + 64);                                                     \
+    __syncthreads();                                                               \
+    if (head_ok)                                                                   \
+      process_tile_lds<NQK, NG>(k_lds, v_lds, (K0), (K0) + 31 > first_pos || (K0) < open_lo, qreg, clo, chi, \
+                                scale_log2e, acc, m, l);                           \
+  } while (0)
+  STAGE_LOAD(st0, key_begin);
+  STAGE_LOAD(st1, key_begin + 32);
+  for (int key0 = key_begin; key0 < key_end; key0 += 64) {
+    STAGE_WORK(st0, key0);
+    if (key0 + 32 >= key_end) break;
+    STAGE_WORK(st1, key0 + 32);
+  }
+#undef STAGE_LOAD
+#undef STAGE_WORK
 #pragma unroll
   for (int qg = 0; qg < NG; ++qg) {
     float lt = l[qg];
@@ -521,9 +702,10 @@ extern "C" int ullm_attention_prefill(
   if (n_tiles <= 0) return 0;
   if (!ullm_attention_mfma_supports(hd, page_size, nq, nkv)) return ULLM_ERR_UNSUPPORTED;
   if (window < 0) return ULLM_ERR_SHAPE;
-  if ((long long)n_tiles * nq > 0x7fffffffLL) return ULLM_ERR_SHAPE;
+  const int chunks = (nq / nkv + PREFILL_WAVES - 1) / PREFILL_WAVES;
+  if ((long long)n_tiles * nkv * chunks > 0x7fffffffLL) return ULLM_ERR_SHAPE;
   const float sl = scale * 1.4426950408889634f;
-  dim3 grid(n_tiles * nq), block(64 * prefill_waves(hd / 32));
+  dim3 grid(n_tiles * nkv * chunks), block(64 * PREFILL_WAVES);
 #define CALL(N) hipLaunchKernelGGL(attention_prefill_kernel<N>, grid, block, 0, stream, (const bf16_t*)q, q_stride, \
     (bf16_t*)out, out_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool, tiles, positions, token_entry, \
     block_table, bt_stride, page_size, nq, nkv, sl, window, n_tiles)
