@@ -269,6 +269,7 @@ MFMA_CASES = [dict(nq=8, nkv=2, hd=32, P=16, lens=[(1, 1), (1, 37), (1, 300), (1
               dict(nq=3, nkv=3, hd=256, P=16, lens=[(37, 80)], window=0),               # one head per kv head
               dict(nq=4, nkv=1, hd=128, P=16, lens=[(40, 1200), (64, 64)], window=0),   # page ids refetched past 1024 keys
               dict(nq=4, nkv=2, hd=64, P=48, lens=[(50, 1100)], window=300),
+              dict(nq=2, nkv=2, hd=32, P=16, lens=[(2200, 2200), (70, 70)], window=0),  # 72 tiles: three rounds of blocks
               dict(nq=8, nkv=2, hd=32, P=16, lens=[(1, 45), (9, 40), (1, 200), (20, 20), (1, 1)], window=0),  # mixed
               dict(nq=8, nkv=2, hd=32, P=16, lens=[(1, 45), (9, 40), (1, 200), (20, 50)], window=13)]
 
@@ -348,6 +349,38 @@ def test_matrix_core_attention_finds_one_far_key_at_every_edge(ops):
                 got = out.float().cpu().view(n, nq, hd)[-1]
                 for h in range(nq):
                     assert (got[h] - v[target, h // 4]).abs().max() < 3e-2, (window, target, n, h)
+
+
+def test_matrix_core_attention_with_scores_that_climb(ops):
+    """The reference value of the exponentials follows the running maximum only in steps: scores that
+    rise a little with every tile (so it lags, then jumps) and scores that fall must both come out right."""
+    torch.manual_seed(12)
+    dtype = torch.bfloat16
+    nq, nkv, hd, P, S = 4, 2, 32, 16, 640
+    for slope in (0.09, -0.09, 0.4):                      # natural-log units per key: 2.9, -2.9, 12.8 per 32-key tile
+        k = torch.randn(S, nkv, hd) * 0.05
+        k[:, :, 0] = slope * torch.arange(S).float()[:, None]
+        v = torch.randn(S, nkv, hd)
+        k, v = k.to(dtype).float(), v.to(dtype).float()
+        for n in (1, 40):
+            q = torch.randn(n, nq, hd) * 0.05
+            q[:, :, 0] = 1.0
+            q = q.to(dtype).float()
+            want = reference_attention([q], [k], [v], 1.0, 0).reshape(n, nq * hd)
+            k_pool, v_pool, tables = paged_cache([k], [v], P, dtype, DEV)
+            positions = torch.arange(S - n, S).int().to(DEV)
+            entry = torch.zeros(n, dtype=torch.int32, device=DEV)
+            qd = q.reshape(n, -1).to(DEV, dtype)
+            out = torch.zeros(n, nq * hd, dtype=dtype, device=DEV)
+            bt = table_tensor(tables, DEV)
+            if n == 1:
+                ops.attention_decode_mfma(qd, out, k_pool, v_pool, None, 1, positions, entry, bt, P, nq, nkv, hd,
+                                          1.0, 0, S, splits=1, waves=4)
+            else:
+                tiles = [x for f in range(0, n, ops.PREFILL_TILE) for x in (f, min(ops.PREFILL_TILE, n - f))]
+                ops.attention_prefill_mfma(qd, out, k_pool, v_pool, torch.tensor(tiles, dtype=torch.int32, device=DEV),
+                                           len(tiles) // 2, positions, entry, bt, P, nq, nkv, hd, 1.0, 0)
+            assert (out.float().cpu() - want).abs().max() <= tol(dtype, want), (slope, n)
 
 
 @pytest.mark.parametrize("shape", [(1, 48, 64), (8, 503, 96), (16, 256, 4096), (17, 100, 224), (33, 64, 1032),

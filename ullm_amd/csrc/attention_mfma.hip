@@ -9,8 +9,11 @@
 // exactly the ones it must feed as the B operand of the second product: nothing moves between lanes.
 // Both operands of both products are plain 8- or 16-byte loads from the paged cache:
 //   keys   [page, kv_head, row, head_dim],  values [page, kv_head, head_dim, row].
-// Softmax state (maximum, sum) is 32-bit and per column; the scale and log2(e) are folded into one
-// multiply so that the exponential is a single v_exp_f32.
+// Softmax state (reference value, sum) is 32-bit and per column; the scale and log2(e) are folded into
+// one multiply so that the exponential is a single v_exp_f32.  The reference value a column's
+// exponentials are taken against follows the column's running maximum lazily: it moves only when a
+// tile's maximum exceeds it by more than RESCALE_STEP (so weights stay below 2^RESCALE_STEP), and the
+// output is rescaled only then: the result is the same sum, and most tiles skip the rescaling.
 //
 // Semantics as in the general kernel: causal with the queries at the end of the keys, optional
 // window, query head h reads kv head h / (nq / nkv) (ullm/layers/attention.py:76-104,271,298-309).
@@ -20,6 +23,7 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 
 #define NEG_BIG (-1.0e30f)
+#define RESCALE_STEP 8.0f
 
 union Pack8 {
   bf16x8_t v;
@@ -390,8 +394,9 @@ attention_reduce_kernel(const float* __restrict__ part, bf16_t* __restrict__ out
 // grid (n_tiles * nkv * head_chunks).  Workgroups go to the 8 XCDs round-robin by their linear id and
 // each XCD has an L2 of its own, so the id is decoded such that all work on one kv head lands on one
 // XCD (kv head = id mod 8 when the kv heads are a multiple of 8): that head's keys and values then
-// stay in that L2 instead of every XCD streaming every head from memory.  Tiles are taken last first
-// (under the causal mask they see the most keys).
+// stay in that L2 instead of every XCD streaming every head from memory.
+// The caller lists the tiles by rising number of keys; blocks take them from the end, the longest
+// first (measured against orders that alternate long and short tiles, this one was the fastest).
 #define PREFILL_GROUPS 2
 #define PREFILL_WAVES 4
 
@@ -464,9 +469,9 @@ __device__ __forceinline__ void stage_store(const PrefillStage<NQK>& st, int key
 
 // Scores, softmax update and value product of one wave for the tile in LDS.  `masked` = some key of
 // the tile is hidden from some column (diagonal, window or end of data); otherwise no per-score test.
-template <int NQK, int NG>
+template <int NQK, int NG, bool masked>
 __device__ __forceinline__ void process_tile_lds(const unsigned char* __restrict__ kl, const unsigned char* __restrict__ vl,
-                                                 int key0, bool masked, const Pack8 (&qreg)[NG][NQK],
+                                                 int key0, const Pack8 (&qreg)[NG][NQK],
                                                  const int (&col_lo)[NG], const int (&col_hi)[NG], float scale_log2e,
                                                  f32x4_t (&acc)[NG][2 * NQK], float (&m)[NG], float (&l)[NG]) {
   using S = PrefillStage<NQK>;
@@ -486,6 +491,7 @@ __device__ __forceinline__ void process_tile_lds(const unsigned char* __restrict
     }
   Pack8 p[NG];
   float alpha[NG];
+  bool rescale = false;
 #pragma unroll
   for (int q = 0; q < NG; ++q) {
     float tile_max = NEG_BIG;
@@ -503,8 +509,10 @@ __device__ __forceinline__ void process_tile_lds(const unsigned char* __restrict
       }
     tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, 64));
     tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, 64));
-    const float m_new = fmaxf(m[q], tile_max);
-    alpha[q] = fast_exp2(m[q] - m_new);
+    const bool moves = tile_max > m[q] + RESCALE_STEP;
+    const float m_new = moves ? tile_max : m[q];
+    alpha[q] = moves ? fast_exp2(m[q] - m_new) : 1.f;
+    rescale = rescale || moves;
     float psum = 0.f;
 #pragma unroll
     for (int sb = 0; sb < 2; ++sb) {
@@ -521,16 +529,21 @@ __device__ __forceinline__ void process_tile_lds(const unsigned char* __restrict
     l[q] = l[q] * alpha[q] + psum;
     m[q] = m_new;
   }
+  if (__any(rescale)) {
+#pragma unroll
+    for (int q = 0; q < NG; ++q)
+#pragma unroll
+      for (int n = 0; n < 2 * NQK; ++n) {
+        acc[q][n][0] *= alpha[q]; acc[q][n][1] *= alpha[q]; acc[q][n][2] *= alpha[q]; acc[q][n][3] *= alpha[q];
+      }
+  }
 #pragma unroll
   for (int n = 0; n < 2 * NQK; ++n) {
     Pack8 vf;
     vf.u4 = *reinterpret_cast<const uint4*>(vl + (16 * n + c) * S::VROW + 16 * g);
 #pragma unroll
-    for (int q = 0; q < NG; ++q) {
-      f32x4_t o = acc[q][n];
-      o[0] *= alpha[q]; o[1] *= alpha[q]; o[2] *= alpha[q]; o[3] *= alpha[q];
-      acc[q][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, p[q].v, o, 0, 0, 0);
-    }
+    for (int q = 0; q < NG; ++q)
+      acc[q][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, p[q].v, acc[q][n], 0, 0, 0);
   }
 }
 
@@ -611,9 +624,12 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __r
     stage_store<NQK>(ST, (K0), last_pos, k_lds, v_lds);                            \
     STAGE_LOAD(ST, (K0) + 64);                                                     \
     __syncthreads();                                                               \
-    if (head_ok)                                                                   \
-      process_tile_lds<NQK, NG>(k_lds, v_lds, (K0), (K0) + 31 > first_pos || (K0) < open_lo, qreg, clo, chi, \
-                                scale_log2e, acc, m, l);                           \
+    if (head_ok) {                                                                 \
+      if ((K0) + 31 > first_pos || (K0) < open_lo)                                 \
+        process_tile_lds<NQK, NG, true>(k_lds, v_lds, (K0), qreg, clo, chi, scale_log2e, acc, m, l);  \
+      else                                                                         \
+        process_tile_lds<NQK, NG, false>(k_lds, v_lds, (K0), qreg, clo, chi, scale_log2e, acc, m, l); \
+    }                                                                              \
   } while (0)
   STAGE_LOAD(st0, key_begin);
   STAGE_LOAD(st1, key_begin + 32);

@@ -104,15 +104,18 @@ class ModelRunner:
             strides.append(widest)
         n_want = sum(len(e.want) for e in entries) + n_pad
         # attention work lists: tokens of one-token entries; tiles of <= Q_TILE tokens of longer entries
-        dec_list, tile_list, max_dec_kv, t0 = [], [], 0, 0
+        dec_list, tile_keys, max_dec_kv, t0 = [], [], 0, 0
         for e, n in zip(entries, lens):
             if n == 1:
                 dec_list.append(t0)
                 max_dec_kv = max(max_dec_kv, e.cache.num_computed + 1)
             else:
                 for first in range(0, n, Q_TILE):
-                    tile_list.extend((t0 + first, min(Q_TILE, n - first)))
+                    count = min(Q_TILE, n - first)
+                    tile_keys.append((e.cache.num_computed + first + count, t0 + first, count))
             t0 += n
+        tile_keys.sort()                                  # the attention kernel wants rising numbers of keys
+        tile_list = [x for _, first, count in tile_keys for x in (first, count)]
         dec_list.extend(range(t0, t0 + n_pad))
         ng = len(groups)
         sizes = [T, T, T, B + 1, B, B, n_want] + [B * s for s in strides] + [len(dec_list), len(tile_list)]

@@ -25,6 +25,9 @@ HIPCC_FLAGS = [
     f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", "-shared",
     # hipcc -O3 may form packed 32-bit float ops from ordinary code; they are switched off
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # matrix-core results stay in ordinary vector registers: accumulators that are also scaled by
+    # vector instructions otherwise travel between the two register classes around every product
+    "-mllvm", "-amdgpu-mfma-vgpr-form",
     "-Wno-unused-command-line-argument",
 ]
 HEADERS = ["common.h"]
