@@ -419,7 +419,7 @@ __device__ __forceinline__ void stage_load(PrefillStage<NQK>& st, int key0, cons
                                            int page_size, int nkv, int kvh) {
   using S = PrefillStage<NQK>;
   constexpr int HD = S::HD;
-  const int tid = threadIdx.x;
+  const int tid = threadIdx.x & (S::THREADS - 1);
 #pragma unroll
   for (int j = 0; j < S::PER_THREAD; ++j) {
     const int piece = tid + j * S::THREADS;
@@ -445,7 +445,7 @@ __device__ __forceinline__ void stage_store(const PrefillStage<NQK>& st, int key
                                             unsigned char* __restrict__ kl, unsigned char* __restrict__ vl) {
   using S = PrefillStage<NQK>;
   constexpr int HD = S::HD;
-  const int tid = threadIdx.x;
+  const int tid = threadIdx.x & (S::THREADS - 1);
   const bool edge = key0 + 32 > max_hi + 1;
 #pragma unroll
   for (int j = 0; j < S::PER_THREAD; ++j) {
@@ -547,8 +547,12 @@ __device__ __forceinline__ void process_tile_lds(const unsigned char* __restrict
   }
 }
 
-template <int NQK>
-__global__ void __launch_bounds__(64 * PREFILL_WAVES)
+// KS = 2: eight waves; the upper four take the second half of the tile's keys through an LDS tile of
+// their own and hand their (reference value, sum, output) to the lower four at the end.  A block then
+// lasts half as long and a compute unit holds one block at a time, so that blocks that finish early
+// (tiles with few keys) make room for the next ones instead of idling beside a long one.
+template <int NQK, int KS>
+__global__ void __launch_bounds__(64 * PREFILL_WAVES * KS)
 attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
                          const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
                          const int* __restrict__ tiles, const int* __restrict__ positions,
@@ -558,9 +562,14 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __r
   using S = PrefillStage<NQK>;
   constexpr int HD = 32 * NQK;
   constexpr int NG = PREFILL_GROUPS;
-  __shared__ __attribute__((aligned(16))) unsigned char k_lds[S::KBYTES];
-  __shared__ __attribute__((aligned(16))) unsigned char v_lds[S::VBYTES];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, g = lane >> 4, c = lane & 15;
+  constexpr int TILE_BYTES = S::KBYTES + S::VBYTES;
+  constexpr int PER_LANE = NG * (8 * NQK + 2);            // floats a lane hands over in the merge
+  static_assert(KS == 1 || 2 * PER_LANE * 64 * 4 <= 2 * TILE_BYTES, "the merge reuses the tiles' memory");
+  __shared__ __attribute__((aligned(16))) unsigned char lds[KS * TILE_BYTES];
+  const int lane = threadIdx.x & 63, wave = (threadIdx.x >> 6) % PREFILL_WAVES, half = threadIdx.x / S::THREADS;
+  const int g = lane >> 4, c = lane & 15;
+  unsigned char* const k_lds = lds + half * TILE_BYTES;
+  unsigned char* const v_lds = k_lds + S::KBYTES;
   const int G = nq / nkv, chunks = (G + PREFILL_WAVES - 1) / PREFILL_WAVES, per_kv = n_tiles * chunks;
   int kvh, rest;
   if (nkv % 8 == 0) {
@@ -598,6 +607,10 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __r
   const int open_lo = (window > 0 && last_pos - window + 1 > 0) ? last_pos - window + 1 : 0;
   const int key_begin = ((window > 0 && first_pos - window + 1 > 0) ? first_pos - window + 1 : 0) & ~31;
   const int key_end = last_pos + 1;
+  // this half's share of the 32-key tiles
+  const int steps = ((key_end - key_begin + 31) / 32 + KS - 1) / KS;
+  const int my_begin = key_begin + half * steps * 32;
+  const int my_end = my_begin + steps * 32 < key_end ? my_begin + steps * 32 : key_end;
   const int* bt = block_table + (size_t)token_entry[first] * bt_stride;
   f32x4_t acc[NG][2 * NQK];
   float m[NG], l[NG];
@@ -609,11 +622,11 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __r
     l[qg] = 0.f;
   }
   // the page window serves the loads, which run ahead of the products
-  PageWindow pw = load_pages(key_begin, key_end, bt, page_size);
+  PageWindow pw = load_pages(my_begin < key_end ? my_begin : key_begin, key_end, bt, page_size);
   PrefillStage<NQK> st0, st1;
 #define STAGE_LOAD(ST, K0)                                                         \
   do {                                                                             \
-    if ((K0) < key_end) {                                                          \
+    if ((K0) < my_end) {                                                           \
       if ((K0) >= 16 * (pw.base + 64)) pw = load_pages((K0), key_end, bt, page_size); \
       stage_load<NQK>(ST, (K0), pw, k_pool, v_pool, page_size, nkv, kvh);          \
     }                                                                              \
@@ -621,25 +634,62 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __r
 #define STAGE_WORK(ST, K0)                                                         \
   do {                                                                             \
     __syncthreads();                         /* the previous tile has been read by every wave */ \
-    stage_store<NQK>(ST, (K0), last_pos, k_lds, v_lds);                            \
+    if ((K0) < my_end) stage_store<NQK>(ST, (K0), last_pos, k_lds, v_lds);         \
     STAGE_LOAD(ST, (K0) + 64);                                                     \
     __syncthreads();                                                               \
-    if (head_ok) {                                                                 \
+    if (head_ok && (K0) < my_end) {                                                \
       if ((K0) + 31 > first_pos || (K0) < open_lo)                                 \
         process_tile_lds<NQK, NG, true>(k_lds, v_lds, (K0), qreg, clo, chi, scale_log2e, acc, m, l);  \
       else                                                                         \
         process_tile_lds<NQK, NG, false>(k_lds, v_lds, (K0), qreg, clo, chi, scale_log2e, acc, m, l); \
     }                                                                              \
   } while (0)
-  STAGE_LOAD(st0, key_begin);
-  STAGE_LOAD(st1, key_begin + 32);
-  for (int key0 = key_begin; key0 < key_end; key0 += 64) {
-    STAGE_WORK(st0, key0);
-    if (key0 + 32 >= key_end) break;
-    STAGE_WORK(st1, key0 + 32);
+  STAGE_LOAD(st0, my_begin);
+  STAGE_LOAD(st1, my_begin + 32);
+  for (int i = 0; i < steps; i += 2) {                    // the same number of barriers in both halves
+    STAGE_WORK(st0, my_begin + 32 * i);
+    if (i + 1 >= steps) break;
+    STAGE_WORK(st1, my_begin + 32 * i + 32);
   }
 #undef STAGE_LOAD
 #undef STAGE_WORK
+  if (KS == 2) {
+    // waves 4..7 hand over to waves 0..3, two at a time through the tiles' memory, lane by lane
+    float* buf = reinterpret_cast<float*>(lds);
+#pragma unroll
+    for (int r = 0; r < PREFILL_WAVES / 2; ++r) {
+      __syncthreads();
+      float* w = buf + (size_t)(wave & 1) * PER_LANE * 64 + lane;
+      if (half == 1 && (wave >> 1) == r) {
+#pragma unroll
+        for (int qg = 0; qg < NG; ++qg) {
+#pragma unroll
+          for (int n = 0; n < 2 * NQK; ++n)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) w[(qg * (8 * NQK + 2) + 4 * n + e) * 64] = acc[qg][n][e];
+          w[(qg * (8 * NQK + 2) + 8 * NQK) * 64] = m[qg];
+          w[(qg * (8 * NQK + 2) + 8 * NQK + 1) * 64] = l[qg];
+        }
+      }
+      __syncthreads();
+      if (half == 0 && (wave >> 1) == r) {
+#pragma unroll
+        for (int qg = 0; qg < NG; ++qg) {
+          const float m_b = w[(qg * (8 * NQK + 2) + 8 * NQK) * 64], l_b = w[(qg * (8 * NQK + 2) + 8 * NQK + 1) * 64];
+          const float M = fmaxf(m[qg], m_b);
+          const float fa = fast_exp2(m[qg] - M), fb = fast_exp2(m_b - M);
+#pragma unroll
+          for (int n = 0; n < 2 * NQK; ++n)
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              acc[qg][n][e] = acc[qg][n][e] * fa + w[(qg * (8 * NQK + 2) + 4 * n + e) * 64] * fb;
+          l[qg] = l[qg] * fa + l_b * fb;
+          m[qg] = M;
+        }
+      }
+    }
+    if (half == 1) return;
+  }
 #pragma unroll
   for (int qg = 0; qg < NG; ++qg) {
     float lt = l[qg];
@@ -721,11 +771,14 @@ extern "C" int ullm_attention_prefill(
   const int chunks = (nq / nkv + PREFILL_WAVES - 1) / PREFILL_WAVES;
   if ((long long)n_tiles * nkv * chunks > 0x7fffffffLL) return ULLM_ERR_SHAPE;
   const float sl = scale * 1.4426950408889634f;
-  dim3 grid(n_tiles * nkv * chunks), block(64 * PREFILL_WAVES);
-#define CALL(N) hipLaunchKernelGGL(attention_prefill_kernel<N>, grid, block, 0, stream, (const bf16_t*)q, q_stride, \
-    (bf16_t*)out, out_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool, tiles, positions, token_entry, \
-    block_table, bt_stride, page_size, nq, nkv, sl, window, n_tiles)
+  const int ks = hd <= 128 ? 2 : 1;                      // keys split over two halves of a block (LDS allows it)
+  dim3 grid(n_tiles * nkv * chunks), block(64 * PREFILL_WAVES * ks);
+#define ARGS (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool, tiles, \
+    positions, token_entry, block_table, bt_stride, page_size, nq, nkv, sl, window, n_tiles
+#define CALL(N) do { if (N <= 4) hipLaunchKernelGGL((attention_prefill_kernel<N, (N <= 4 ? 2 : 1)>), grid, block, 0, stream, ARGS); \
+    else hipLaunchKernelGGL((attention_prefill_kernel<N, 1>), grid, block, 0, stream, ARGS); } while (0)
   DISPATCH_NQK(hd, CALL)
+#undef ARGS
 #undef CALL
   ULLM_LAUNCH_CHECK();
 }
