@@ -231,6 +231,22 @@ def sample_token(logits: torch.Tensor, temperature: float, top_k: int, top_p: fl
     return tok
 
 
+def sample_token_set(logits: torch.Tensor, temperature: float, top_k: int, top_p: float, min_p: float,
+                     seed: int, position: int, slack: float = 2e-5) -> set:
+    """The tokens an inverse-CDF draw may give when the sums are taken in 32-bit in another order:
+    every kept token whose CDF interval comes within ``slack`` of the seeded uniform.  Almost always
+    one token (the one :func:`sample_token` returns); two when the draw falls on a boundary."""
+    if temperature == 0:
+        return {sample_token(logits, temperature, top_k, top_p, min_p, seed, position)}
+    probs = torch.softmax(filter_logits(logits, temperature, top_k, top_p, min_p).double(), dim=-1)
+    cdf = probs.cumsum(dim=-1)
+    u = uniform_from_seed(seed, position) * float(cdf[-1])
+    lower = cdf - probs
+    near = (probs > 0) & (lower - slack <= u) & (u < cdf + slack)
+    return set(torch.nonzero(near).flatten().tolist()) | {sample_token(logits, temperature, top_k, top_p, min_p,
+                                                                        seed, position)}
+
+
 def greedy_generate(w, cfg, prompt: List[int], n_new: int) -> List[int]:
     ids = list(prompt)
     for _ in range(n_new):

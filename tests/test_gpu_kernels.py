@@ -422,24 +422,26 @@ def test_gemm_dispatch_refuses_nothing_silently(ops):
                                    (64, 2100, 520), (5, 4096, 128)])
 @pytest.mark.parametrize("nt", [0, 1, 2, 4])
 def test_gemm_skinny_fused_forms(ops, shape, nt):
-    """The folded forms against the separate kernels' references: silu*up in front, add into the
-    32-bit residual behind."""
+    """The folded forms against the separate kernels' references: the add into the 32-bit residual
+    behind a product, and silu(gate) * up behind the product with the stacked gate|up weights."""
     torch.manual_seed(11)
     M, N, K = shape
     if nt == 4 and M <= 16:
         nt = 2
     w = (torch.randn(N, K, device=DEV) * 0.3).bfloat16()
-    # add into the residual (whose rows must be 16-byte aligned), plain and with silu(gate) * up in front
-    N -= N % 4
-    w = w[:N]
+    # add into the residual (whose rows must be 16-byte aligned)
+    n4 = N - N % 4
     a = torch.randn(M, K, device=DEV).bfloat16()
-    stream = torch.randn(M, N, device=DEV)
-    want = stream.cpu() + a.float().cpu() @ w.float().cpu().T
-    ops.gemm_skinny_add(a, w, stream, nt=nt)
+    stream = torch.randn(M, n4, device=DEV)
+    want = stream.cpu() + a.float().cpu() @ w[:n4].float().cpu().T
+    ops.gemm_skinny_add(a, w[:n4], stream, nt=nt)
     assert (stream.cpu() - want).abs().max() <= 1e-4 * want.abs().max() + 1e-4
-    gu = torch.randn(M, 2 * K, device=DEV).bfloat16()
-    stream = torch.randn(M, N, device=DEV)
-    act = plain.silu_and_mul(gu.float().cpu()).bfloat16().float()
-    want = stream.cpu() + act @ w.float().cpu().T
-    ops.gemm_skinny_add(gu, w, stream, silu=True, nt=nt)
-    assert (stream.cpu() - want).abs().max() <= 2e-2 * want.abs().max()
+    # gate|up: any I, also one that is no multiple of 16 (N odd: drop a row so that the halves are equal)
+    inter = N // 2
+    if inter:
+        wgu = torch.cat([w[:inter], w[N - inter:]]).contiguous()
+        gate_up = a.float().cpu() @ wgu.float().cpu().T
+        want = plain.silu_and_mul(gate_up)
+        got = ops.gemm_skinny_silu(a, wgu, nt=nt if nt != 1 else 0)
+        assert got.shape == (M, inter) and got.dtype == torch.bfloat16
+        assert (got.float().cpu() - want).abs().max() <= 1e-2 * want.abs().max()

@@ -4,14 +4,13 @@
 // surround a projection in a decoder layer are folded into it so that they cost no launch and no
 // pass over memory of their own:
 //
-//   how X is produced (PRO)
-//     PLAIN : X is a bfloat16 matrix
-//     SILU  : X = silu(G[:, :K]) * G[:, K:] with G the bfloat16 [M, 2K] gate|up matrix
-//             (ullm/layers/activation.py:16-18 followed by down_proj, ullm/models/qwen3.py:44-45)
 //   what happens to the result (EPI)
 //     STORE : C = result (+ bias), bfloat16 or float32
 //     RESADD: R[M, N] += result, the 32-bit residual stream (the add the reference leaves to the next
 //             norm, ullm/layers/layernorm.py:24-26)
+//     SILU  : W is the stacked gate|up matrix [2 I, K]; a block takes rows n of the gate half and the same
+//             rows of the up half and stores C[M, I] = silu(gate) * up, computed on the 32-bit sums
+//             (ullm/layers/activation.py:16-18 after gate_up_proj, ullm/models/qwen3.py:43-45)
 //
 // A block owns NT x 16 consecutive rows of W; its waves split K between them.  Per 32 values of K a
 // wave issues one 16-byte load per lane and W tile straight from global memory (A operand of
@@ -31,34 +30,14 @@ union Pack8 {
   bf16_t h[8];
 };
 
-enum { PRO_PLAIN = 0, PRO_SILU = 2 };
-enum { EPI_STORE = 0, EPI_RESADD = 1 };
+enum { EPI_STORE = 0, EPI_RESADD = 1, EPI_SILU = 2 };
 
 // most waves per block for a tile shape: bounded by the shared memory that holds the waves' partials
 __host__ __device__ constexpr int sk_max_waves(int mt, int nt) { return mt * nt >= 8 ? 4 : (mt * nt >= 4 ? 8 : 16); }
 
-template <int PRO>
-__device__ __forceinline__ Pack8 load_x(const bf16_t* __restrict__ X, size_t row_off, int k, int silu_off) {
-  Pack8 x;
-  if (PRO == PRO_PLAIN) {
-    x.u4 = *reinterpret_cast<const uint4*>(X + row_off + k);
-  } else {
-    Pack8 gt, up;
-    gt.u4 = *reinterpret_cast<const uint4*>(X + row_off + k);
-    up.u4 = *reinterpret_cast<const uint4*>(X + row_off + silu_off + k);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      // low and high halves of a 32-bit word are two bfloat16 values
-      const float g0 = __uint_as_float(gt.w[j] << 16), g1 = __uint_as_float(gt.w[j] & 0xffff0000u);
-      const float u0 = __uint_as_float(up.w[j] << 16), u1 = __uint_as_float(up.w[j] & 0xffff0000u);
-      x.w[j] = pack2_bf16(fast_silu(g0) * u0, fast_silu(g1) * u1);
-    }
-  }
-  return x;
-}
-
 // MT = 16-row tiles of X (M <= 16 MT); NT = 16-row tiles of W per block.
-template <int MT, int NT, int PRO, int EPI, typename TC>
+// With EPI_SILU the NT tiles of W are NT / 2 of the gate half followed by the same rows of the up half.
+template <int MT, int NT, int EPI, typename TC>
 __global__ void __launch_bounds__(64 * sk_max_waves(MT, NT))
 gemm_skinny_kernel(const bf16_t* __restrict__ X, int ldx, const bf16_t* __restrict__ W, int ldw,
                    const float* __restrict__ bias, TC* __restrict__ C, float* __restrict__ R, int ldc, int M,
@@ -67,11 +46,14 @@ gemm_skinny_kernel(const bf16_t* __restrict__ X, int ldx, const bf16_t* __restri
   __shared__ float red[MAXW - 1][NT * MT][64 * 4];   // wave 0 adds the others' partials to its own
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
   const int g = lane >> 4, r = lane & 15;
-  const int n0 = blockIdx.x * (16 * NT);
+  // N counts the columns of the result; with EPI_SILU W has 2 N rows
+  constexpr int OT = EPI == EPI_SILU ? NT / 2 : NT;      // 16-column tiles of the result per block
+  const int n0 = blockIdx.x * (16 * OT);
   const bf16_t* wp[NT];
 #pragma unroll
   for (int i = 0; i < NT; ++i) {
-    const int n = n0 + 16 * i + r < N ? n0 + 16 * i + r : N - 1;   // rows past N repeat the last row; never stored
+    const int col = n0 + 16 * (i % OT) + r;
+    const int n = (col < N ? col : N - 1) + (i / OT) * N;   // rows past N repeat the last row; never stored
     wp[i] = W + (size_t)n * ldw + 8 * g;
   }
   size_t xo[MT];
@@ -99,7 +81,7 @@ gemm_skinny_kernel(const bf16_t* __restrict__ X, int ldx, const bf16_t* __restri
 #pragma unroll
     for (int u = 0; u < U; ++u)
 #pragma unroll
-      for (int t = 0; t < MT; ++t) x[u][t] = load_x<PRO>(X, xo[t], k + 32 * u, K);
+      for (int t = 0; t < MT; ++t) x[u][t].u4 = *reinterpret_cast<const uint4*>(X + xo[t] + k + 32 * u);
 #pragma unroll
     for (int u = 0; u < U; ++u)
 #pragma unroll
@@ -116,8 +98,7 @@ gemm_skinny_kernel(const bf16_t* __restrict__ X, int ldx, const bf16_t* __restri
     for (int i = 0; i < NT; ++i) w[i].u4 = in ? *reinterpret_cast<const uint4*>(wp[i] + k) : make_uint4(0, 0, 0, 0);
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
-      if (in) x[t] = load_x<PRO>(X, xo[t], k, K);
-      else x[t].u4 = make_uint4(0, 0, 0, 0);
+      x[t].u4 = in ? *reinterpret_cast<const uint4*>(X + xo[t] + k) : make_uint4(0, 0, 0, 0);
     }
 #pragma unroll
     for (int i = 0; i < NT; ++i)
@@ -151,9 +132,13 @@ gemm_skinny_kernel(const bf16_t* __restrict__ X, int ldx, const bf16_t* __restri
     const int m = 16 * t + r;
     if (m >= M) continue;
 #pragma unroll
-    for (int i = 0; i < NT; ++i) {
+    for (int i = 0; i < OT; ++i) {
       const int nn = n0 + 16 * i + 4 * g;
-      if (EPI == EPI_RESADD) {
+      if (EPI == EPI_SILU) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          if (nn + j < N) st_f32(C + (size_t)m * ldc + nn + j, fast_silu(acc[i][t][j]) * acc[i + OT][t][j]);
+      } else if (EPI == EPI_RESADD) {
         float* rp = R + (size_t)m * ldc + nn;
         if (nn + 3 < N) {
           float4 o = *reinterpret_cast<float4*>(rp);
@@ -177,17 +162,18 @@ extern "C" int ullm_gemm_skinny_supports(int M, int N, int K, int ldx, int ldw) 
   return M >= 1 && M <= 64 && N >= 1 && K >= 8 && K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0;
 }
 
-// pro: 0 plain (X bfloat16 [M, K]), 2 silu (X bfloat16 [M, 2K]).  epi: 0 store to C (c_dtype, bias
-// optional), 1 add into R (float32 [M, N], row stride ldc).  force_nt / force_waves: 0 = chosen here.
+// X bfloat16 [M, K]; W bfloat16 [N, K] (with epi 2: [2 N, K]).  epi: 0 store to C (c_dtype, bias optional),
+// 1 add into R (float32 [M, N], row stride ldc), 2 silu(gate) * up to C (bfloat16 [M, N]).
+// force_nt / force_waves: 0 = chosen here.
 extern "C" int ullm_gemm_skinny(const void* X, int ldx, const void* W, int ldw, const float* bias, void* C,
-                                int ldc, int M, int N, int K, int pro, int epi, int c_dtype, int force_nt,
+                                int ldc, int M, int N, int K, int epi, int c_dtype, int force_nt,
                                 int force_waves, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (!ullm_gemm_skinny_supports(M, N, K, ldx, ldw) || ldc < N) return ULLM_ERR_SHAPE;
   if (((uintptr_t)X & 15) || ((uintptr_t)W & 15)) return ULLM_ERR_SHAPE;
-  if ((pro != PRO_PLAIN && pro != PRO_SILU) || epi < 0 || epi > 1) return ULLM_ERR_UNSUPPORTED;
-  if (pro == PRO_SILU && ldx < 2 * K) return ULLM_ERR_SHAPE;
+  if (epi < 0 || epi > 2) return ULLM_ERR_UNSUPPORTED;
   if (epi == EPI_RESADD && (((uintptr_t)C & 15) || ldc % 4 != 0 || bias)) return ULLM_ERR_SHAPE;
+  if (epi == EPI_SILU && (bias || c_dtype != ULLM_BF16)) return ULLM_ERR_UNSUPPORTED;
   int mt = (M + 15) / 16;
   if (mt == 3) mt = 4;                                  // instantiated for 1, 2 and 4 tiles of rows
   const int tiles16 = (N + 15) / 16;
@@ -195,9 +181,11 @@ extern "C" int ullm_gemm_skinny(const void* X, int ldx, const void* W, int ldw, 
   if (force_nt > 0) nt = force_nt;
   else if (tiles16 >= 4096) nt = mt >= 2 ? 4 : 2;
   else if (tiles16 >= 1024 && mt >= 2) nt = 2;
+  if (epi == EPI_SILU) nt = (force_nt == 4 || mt >= 4) ? 4 : 2;   // gate and up tiles come in pairs
   if (nt != 1 && nt != 2 && nt != 4) return ULLM_ERR_UNSUPPORTED;
   if (nt == 4 && mt == 1) nt = 2;                       // not instantiated
-  const int tiles = (tiles16 + nt - 1) / nt;
+  const int out_tiles = epi == EPI_SILU ? nt / 2 : nt;  // 16-column tiles of the result per block
+  const int tiles = (tiles16 + out_tiles - 1) / out_tiles;
   // waves per block: enough blocks x waves to fill the chip, each wave with at least 128 values of K
   const int max_waves = sk_max_waves(mt, nt);
   int waves = 1;
@@ -207,33 +195,38 @@ extern "C" int ullm_gemm_skinny(const void* X, int ldx, const void* W, int ldw, 
   k_per_wave = (k_per_wave + 31) / 32 * 32;
   dim3 grid(tiles), block(64 * waves);
   float* R = (float*)C;
-#define GO(MT, NT, PRO, EPI, TC) hipLaunchKernelGGL((gemm_skinny_kernel<MT, NT, PRO, EPI, TC>), grid, block, 0, stream, \
+#define GO(MT, NT, EPI, TC) hipLaunchKernelGGL((gemm_skinny_kernel<MT, NT, EPI, TC>), grid, block, 0, stream, \
     (const bf16_t*)X, ldx, (const bf16_t*)W, ldw, bias, (TC*)C, R, ldc, M, N, K, k_per_wave)
-#define GO_SHAPE(PRO, EPI, TC)                                              \
-  switch (mt * 8 + nt) {                                                    \
-    case 1 * 8 + 1: GO(1, 1, PRO, EPI, TC); break;                          \
-    case 1 * 8 + 2: GO(1, 2, PRO, EPI, TC); break;                          \
-    case 2 * 8 + 1: GO(2, 1, PRO, EPI, TC); break;                          \
-    case 2 * 8 + 2: GO(2, 2, PRO, EPI, TC); break;                          \
-    case 2 * 8 + 4: GO(2, 4, PRO, EPI, TC); break;                          \
-    case 4 * 8 + 1: GO(4, 1, PRO, EPI, TC); break;                          \
-    case 4 * 8 + 2: GO(4, 2, PRO, EPI, TC); break;                          \
-    case 4 * 8 + 4: GO(4, 4, PRO, EPI, TC); break;                          \
-    default: return ULLM_ERR_UNSUPPORTED;                                   \
+#define GO_SHAPE(EPI, TC)                                              \
+  switch (mt * 8 + nt) {                                               \
+    case 1 * 8 + 1: GO(1, 1, EPI, TC); break;                          \
+    case 1 * 8 + 2: GO(1, 2, EPI, TC); break;                          \
+    case 2 * 8 + 1: GO(2, 1, EPI, TC); break;                          \
+    case 2 * 8 + 2: GO(2, 2, EPI, TC); break;                          \
+    case 2 * 8 + 4: GO(2, 4, EPI, TC); break;                          \
+    case 4 * 8 + 1: GO(4, 1, EPI, TC); break;                          \
+    case 4 * 8 + 2: GO(4, 2, EPI, TC); break;                          \
+    case 4 * 8 + 4: GO(4, 4, EPI, TC); break;                          \
+    default: return ULLM_ERR_UNSUPPORTED;                              \
+  }
+#define GO_PAIRS(EPI, TC)                                              \
+  switch (mt * 8 + nt) {                                               \
+    case 1 * 8 + 2: GO(1, 2, EPI, TC); break;                          \
+    case 2 * 8 + 2: GO(2, 2, EPI, TC); break;                          \
+    case 2 * 8 + 4: GO(2, 4, EPI, TC); break;                          \
+    case 4 * 8 + 4: GO(4, 4, EPI, TC); break;                          \
+    default: return ULLM_ERR_UNSUPPORTED;                              \
   }
   if (epi == EPI_STORE) {
-    if (pro == PRO_PLAIN) {
-      if (c_dtype == ULLM_BF16) { GO_SHAPE(PRO_PLAIN, EPI_STORE, bf16_t) }
-      else if (c_dtype == ULLM_F32) { GO_SHAPE(PRO_PLAIN, EPI_STORE, float) }
-      else return ULLM_ERR_DTYPE;
-    } else {
-      return ULLM_ERR_UNSUPPORTED;
-    }
+    if (c_dtype == ULLM_BF16) { GO_SHAPE(EPI_STORE, bf16_t) }
+    else if (c_dtype == ULLM_F32) { GO_SHAPE(EPI_STORE, float) }
+    else return ULLM_ERR_DTYPE;
+  } else if (epi == EPI_RESADD) {
+    GO_SHAPE(EPI_RESADD, float)
   } else {
-    if (pro == PRO_PLAIN) { GO_SHAPE(PRO_PLAIN, EPI_RESADD, float) }
-    else if (pro == PRO_SILU) { GO_SHAPE(PRO_SILU, EPI_RESADD, float) }
-    else return ULLM_ERR_UNSUPPORTED;
+    GO_PAIRS(EPI_SILU, bf16_t)
   }
+#undef GO_PAIRS
 #undef GO_SHAPE
 #undef GO
   ULLM_LAUNCH_CHECK();

@@ -37,5 +37,5 @@ class SwiGLU(FeedForward):
         return can_fuse(residual, ctx.dtype, self.w_gate_up, self.w_down)
 
     def forward_fused(self, x, residual, ctx: StepContext) -> None:
-        gate_up = linear(x, self.w_gate_up)
-        ops.gemm_skinny_add(gate_up, self.w_down, residual, silu=True)                  # silu*up in front, add behind
+        act = ops.gemm_skinny_silu(x, self.w_gate_up)          # silu(gate) * up behind the first product
+        ops.gemm_skinny_add(act, self.w_down, residual)        # residual add behind the second
