@@ -35,6 +35,9 @@ QWEN3_0P6B = dict(architectures=["Qwen3ForCausalLM"], hidden_size=1024, num_hidd
                   tie_word_embeddings=True, attention_bias=False, use_sliding_window=False,
                   initializer_range=0.02, torch_dtype="bfloat16")
 REFERENCE_MIXED_TOK_S = 9032.37
+QWEN3_14B = dict(QWEN3_8B, hidden_size=5120, num_hidden_layers=40, num_attention_heads=40, intermediate_size=17408)
+QWEN3_32B = dict(QWEN3_8B, hidden_size=5120, num_hidden_layers=64, num_attention_heads=64, intermediate_size=25600)
+SIZES = {"0.6b": QWEN3_0P6B, "8b": QWEN3_8B, "14b": QWEN3_14B, "32b": QWEN3_32B}
 
 
 def parse_args():
@@ -49,8 +52,11 @@ def parse_args():
     ap.add_argument("--dtype", default="bfloat16")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
     ap.add_argument("--eager", action="store_true", help="no HIP graphs")
+    ap.add_argument("--size", choices=sorted(SIZES), default=None,
+                    help="layer sizes of this Qwen3 model (default 8b; 0.6b for --mixed-only)")
     ap.add_argument("--mixed-only", action="store_true",
-                    help="only the reference's own workload: 256 requests of mixed lengths, Qwen3-0.6B sizes")
+                    help="only the reference's own workload: 256 requests of mixed lengths "
+                         "(Qwen3-0.6B sizes unless --size is given)")
     ap.add_argument("--prefill-only", type=int, default=0, metavar="T",
                     help="only time a T-token prompt and print its figures (for profiling)")
     return ap.parse_args()
@@ -78,7 +84,7 @@ def step_flops(cfg, n_tokens, kv_lens_sum_causal, n_logit_rows):
     return L * (per_token * n_tokens + attn) + 2 * H * V * n_logit_rows
 
 
-def run_mixed(dtype, eager):
+def run_mixed(dtype, eager, size="0.6b"):
     """Output tokens per second over 256 requests arriving at once, continuous batching; returns
     (tokens/s, output tokens, seconds, engine steps)."""
     import random
@@ -89,7 +95,7 @@ def run_mixed(dtype, eager):
     from ullm_amd.models import build_model
     from ullm_amd.weights.random_init import bind_random_weights
 
-    cfg, model = build_model(dict(QWEN3_0P6B))
+    cfg, model = build_model(dict(SIZES[size]))
     env = make_env(dtype, "cuda:0", 4096)
     bind_random_weights(model, env, seed=0)
     rng = random.Random(0)
@@ -131,14 +137,16 @@ def main():
     from ullm_amd.weights.random_init import bind_random_weights
 
     if args.mixed_only:
-        tok_s, n_out, secs, steps = run_mixed(args.dtype, args.eager)
-        print(json.dumps({"metric": "output tok/s, 256 requests, lengths 100..1024 in and out, Qwen3-0.6B sizes",
+        size = args.size or "0.6b"
+        tok_s, n_out, secs, steps = run_mixed(args.dtype, args.eager, size)
+        print(json.dumps({"metric": f"output tok/s, 256 requests, lengths 100..1024 in and out, Qwen3-{size} sizes",
                           "value": round(tok_s, 1), "unit": "tokens/s", "output_tokens": n_out,
                           "seconds": round(secs, 3), "engine_steps": steps,
-                          "vs_baseline": round(tok_s / REFERENCE_MIXED_TOK_S, 3),
-                          "baseline": "9032.37 tokens/s, the reference on an A100 40GB"}))
+                          "vs_baseline": round(tok_s / REFERENCE_MIXED_TOK_S, 3) if size == "0.6b" else None,
+                          "baseline": "9032.37 tokens/s, the reference with Qwen3-0.6B on an A100 40GB"}))
         return 0
-    config = dict(QWEN3_8B)
+    args.size = args.size or "8b"
+    config = dict(SIZES[args.size])
     full_layers = config["num_hidden_layers"]
     if args.layers is not None:
         config["num_hidden_layers"] = args.layers
@@ -213,11 +221,11 @@ def main():
     tok_s, ms, bytes_step = run_decode(args.batch, args.steps, args.warmup)
     achieved = bytes_step / (ms * 1e-3) / 1e9
     line = {
-        "metric": "decode tok/s at bs 8 (also bs 1/64, prefill tok/s at 2048; % of roofline), Qwen3-8B",
+        "metric": f"decode tok/s at bs {args.batch} (also bs 1/64, prefill tok/s at 2048; % of roofline), Qwen3-{args.size}",
         "value": round(tok_s, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
-        "config": {"model": "Qwen3-8B sizes, random weights", "layers": config["num_hidden_layers"],
+        "config": {"model": f"Qwen3-{args.size} sizes, random weights", "layers": config["num_hidden_layers"],
                    "layers_of_config": full_layers, "hidden_size": cfg.hidden_size,
                    "num_attention_heads": cfg.num_attention_heads, "num_key_value_heads": cfg.num_key_value_heads,
                    "head_dim": cfg.head_dim, "intermediate_size": cfg.intermediate_size, "vocab_size": cfg.vocab_size,
