@@ -124,6 +124,54 @@ def test_finish_rules_and_abort(model_dirs, plain_models):
         eng.add_request("bad", [503], SamplingParams())
 
 
+def test_scheduling_ahead_changes_no_token(model_dirs, plain_models):
+    """The next step is scheduled and packed while the device still samples the current one; with
+    stop tokens that end requests unannounced, so few pages that requests are preempted, and an
+    abort in between, every request gets the tokens and the ending it gets without that overlap."""
+    from ullm_amd import FinishReason, SamplingParams
+    cfg, w = plain_models["B"]
+    prompts = prompts_of(503, (20, 3, 18, 9, 1, 14), 21)
+    greedy = [plain.greedy_generate(w, cfg, p, 14) for p in prompts]
+    # requests 0 and 3 stop on a token of their own continuation, 1 by max_tokens, the rest by max_new_tokens
+    params = [SamplingParams(temperature=0.0, max_new_tokens=14, eos_token_id=greedy[0][5]),
+              SamplingParams(temperature=0.0, max_tokens=9, ignore_eos=True),
+              SamplingParams(temperature=0.0, max_new_tokens=14, ignore_eos=True),
+              SamplingParams(temperature=0.0, max_new_tokens=14, eos_token_id=greedy[3][0]),
+              SamplingParams(temperature=0.0, max_new_tokens=14, ignore_eos=True),
+              SamplingParams(temperature=0.7, max_new_tokens=14, ignore_eos=True, seed=5)]
+    runs = {}
+    for ahead in (False, True):
+        llm = make_llm(model_dirs["B"], page_size=4, num_pages=12, max_num_batched_tokens=16, max_prefill_chunk=7,
+                       disable_async_scheduling=not ahead)
+        eng = llm.engine
+        for i, (p, sp) in enumerate(zip(prompts, params)):
+            eng.add_request(f"r{i}", p, sp)
+        got, steps = {}, 0
+        while eng.has_unfinished_requests():
+            for r in eng.step():
+                rec = got.setdefault(r.seq_id, [[], None])
+                if r.new_token_id >= 0:
+                    rec[0].append(r.new_token_id)
+                if r.is_finished:
+                    rec[1] = r.finish_reason
+            steps += 1
+            if steps == 6:
+                eng.abort_request("r4")
+        assert eng.runner.cache.num_free_pages() == 12
+        eng.runner.cache.check()
+        runs[ahead] = (got, eng.scheduler.num_preemptions)
+    plain_run, ahead_run = runs[False][0], runs[True][0]
+    aborted = {k: v for k, v in ahead_run.items() if k == "r4"}
+    for k in ("r0", "r1", "r2", "r3", "r5"):
+        assert ahead_run[k] == plain_run[k], k
+    assert ahead_run["r0"][0] == greedy[0][:greedy[0].index(greedy[0][5]) + 1] and ahead_run["r0"][1] is FinishReason.STOP
+    assert ahead_run["r3"][0] == greedy[3][:1] and ahead_run["r3"][1] is FinishReason.STOP
+    assert ahead_run["r1"][0] == greedy[1][:6] and ahead_run["r1"][1] is FinishReason.LENGTH
+    assert ahead_run["r2"][0] == greedy[2] and ahead_run["r2"][1] is FinishReason.LENGTH
+    assert all(v[1] is None for v in aborted.values())            # an aborted request reports no ending
+    assert runs[True][1] > 0 and runs[False][1] > 0               # both runs had to preempt
+
+
 def test_prefix_cache_gives_the_same_tokens(model_dirs, plain_models):
     from ullm_amd import SamplingParams
     cfg, w = plain_models["A"]

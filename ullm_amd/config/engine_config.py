@@ -38,6 +38,7 @@ class EngineConfig:
     pp_size: int = 1
     context_len: int = 2048                     # most tokens (prompt + generated) of a request
     enforce_eager: bool = False                 # True: never replay decode steps from HIP graphs
+    disable_async_scheduling: bool = False      # True: schedule a step only after the one before has ended
     log_level: str = "info"
     # -- beyond the reference ------------------------------------------------------
     dtype: str = "bfloat16"                     # "bfloat16" | "float32" (whole model in true 32-bit)
@@ -78,6 +79,8 @@ class EngineConfig:
                             help="Max context length of the model")
         parser.add_argument("--enforce-eager", action="store_true",
                             help="Enforce eager execution, disable HIP graphs")
+        parser.add_argument("--disable-async-scheduling", action="store_true",
+                            help="Do not schedule the next step while the device runs the current one")
         parser.add_argument("--log-level", type=str, default="info", help="Log level for the engine")
         parser.add_argument("--dtype", type=str, default="bfloat16", help="bfloat16 or float32")
         parser.add_argument("--page-size", type=int, default=16, help="Tokens per cache page")
@@ -101,6 +104,7 @@ class EngineConfig:
             pp_size=args.pp_size,
             context_len=args.context_len,
             enforce_eager=args.enforce_eager,
+            disable_async_scheduling=args.disable_async_scheduling,
             log_level=args.log_level,
             dtype=args.dtype,
             page_size=args.page_size,

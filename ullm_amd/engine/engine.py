@@ -7,6 +7,7 @@ load, cache sizing from free memory).
 from __future__ import annotations
 
 import logging
+from dataclasses import dataclass, field
 from typing import Dict, List, Optional, Sequence
 
 import torch
@@ -15,7 +16,7 @@ from ..config.engine_config import EngineConfig
 from ..sampling import Sampler, SamplingParams
 from .loading import load_model
 from .request import EngineStepResult, FinishReason, Request, RequestStatus, Scheduled
-from .runner import ModelRunner, StepEntry
+from .runner import UNKNOWN_TOKEN, ModelRunner, PreparedStep, StepEntry
 from .scheduler import Scheduler
 
 logger = logging.getLogger("ullm_amd")
@@ -37,6 +38,16 @@ def pages_from_memory(model, env, page_size: int, utilization: float, context_le
     if pages < 1:
         raise RuntimeError("no device memory left for the cache after loading the model")
     return [pages] * len(groups)
+
+
+@dataclass
+class _Plan:
+    """A scheduled step with its host work done."""
+    scheduled: List[Scheduled]
+    early_results: List[EngineStepResult]                 # requests the scheduler itself ended
+    sampling: List[Scheduled] = field(default_factory=list)
+    sample_positions: List[int] = field(default_factory=list)   # index each new token takes in its request
+    prepared: Optional[PreparedStep] = None
 
 
 class Engine:
@@ -61,6 +72,7 @@ class Engine:
                                    config.max_bs)
         self.sampler = Sampler(env.device)
         self._arrivals = 0
+        self._next: Optional[_Plan] = None   # the step after the one that ran last, scheduled and packed ahead
         self.on_logits = None      # optional callable(scheduled that sample, float32 logits): for inspection
         logger.info("cache: %s pages of %d tokens per group, %.2f GiB", num_pages, config.page_size,
                     self.runner.cache_bytes() / 2 ** 30)
@@ -90,42 +102,122 @@ class Engine:
         req = self.scheduler.requests.get(request_id)
         if req is not None:
             self.scheduler.finish(req)
+            self._drop_from_next(req)
 
     def has_unfinished_requests(self) -> bool:
-        return self.scheduler.has_unfinished()
+        """True while a request waits or runs, or a prepared step still has an ending to report."""
+        return self.scheduler.has_unfinished() or (self._next is not None and bool(self._next.early_results))
 
     # ------------------------------------------------------------------ one step
     def step(self) -> List[EngineStepResult]:
-        scheduled = self.scheduler.schedule()
-        results: List[EngineStepResult] = []
-        for req in self.scheduler.finished_by_scheduler:
-            results.append(EngineStepResult(req.request_id, -1, True, req.finish_reason, req.num_prompt_tokens,
-                                            req.num_generated_tokens))
-        self.scheduler.finished_by_scheduler.clear()
-        if not scheduled:
+        """One engine step: the scheduled batch runs, its requests that reached the end of their
+        tokens get one new token each.
+
+        The device works asynchronously, and the host uses that: once this step's kernels are
+        queued, the next step is scheduled and packed while they run (reference: the overlap of
+        scheduling and execution, docs/async_scheduling.md; ``disable_async_scheduling`` switches it
+        off).  What the next step depends on is known without the tokens that are still being
+        sampled: counts decide who continues, and the ids are filled in before its launch.  Only a
+        request that ends on its stop token is a surprise; it is taken out of the prepared step."""
+        plan, self._next = self._next, None
+        if plan is None or not (plan.scheduled or plan.early_results):
+            plan = self._make_plan()          # nothing was prepared (or nothing was there to prepare then)
+        results = plan.early_results
+        if not plan.scheduled:
             return results
-        entries = [StepEntry(s.request.cache, s.request.token_ids[s.start:s.start + s.num_tokens],
-                             [s.num_tokens - 1] if s.samples else []) for s in scheduled]
-        sampling = [s for s in scheduled if s.samples]
-        prepared = None
-        if sampling:                                      # uploaded ahead of the model step
-            prepared = self.sampler.prepare([s.request.params for s in sampling], [s.request.seed for s in sampling],
-                                            [s.request.num_tokens for s in sampling])
-        logits = self.runner.step(entries)
-        if sampling:
-            if self.on_logits is not None:
-                self.on_logits(sampling, logits)
-            ids = self.sampler.sample(logits, prepared=prepared)
-            for s, tok in zip(sampling, ids):
-                req = s.request
+        self._fill_unknown_tokens(plan)
+        sampling = plan.sampling
+        sampler_inputs = None
+        if sampling:                                      # uploaded ahead of the model's kernels
+            sampler_inputs = self.sampler.prepare([s.request.params for s in sampling],
+                                                  [s.request.seed for s in sampling], plan.sample_positions)
+        logits = self.runner.launch(plan.prepared)
+        if not sampling:
+            if not self.config.disable_async_scheduling:
+                self._next = self._make_plan()
+            return results
+        if self.on_logits is not None:
+            self.on_logits(sampling, logits)
+        sampled = self.sampler.launch(logits, sampler_inputs)
+        # while the device works: who ends by length, and the next step
+        ended: Dict[int, FinishReason] = {}
+        if not self.config.disable_async_scheduling:
+            for i, s in enumerate(sampling):
+                self.scheduler.append_token(s.request, UNKNOWN_TOKEN)
+                reason = self._ends_by_length(s.request)
+                if reason is not None:
+                    ended[i] = reason
+                    s.request.finish_reason = reason
+                    self.scheduler.finish(s.request)
+            self._next = self._make_plan()
+        ids = sampled.tolist()                            # waits for the step
+        for i, (s, tok) in enumerate(zip(sampling, ids)):
+            req = s.request
+            if self.config.disable_async_scheduling:
                 self.scheduler.append_token(req, tok)
                 done, reason = self._is_finished(req)
                 if done:
                     req.finish_reason = reason
                     self.scheduler.finish(req)
-                results.append(EngineStepResult(req.request_id, int(tok), done, reason, req.num_prompt_tokens,
-                                                req.num_generated_tokens))
+            else:
+                req.token_ids[plan.sample_positions[i]] = int(tok)
+                stop = tok == req.params.eos_token_id and not req.params.ignore_eos
+                done = stop or i in ended
+                reason = FinishReason.STOP if stop else ended.get(i)
+                if stop:                                  # the stop token wins over a length limit, as in the reference
+                    req.finish_reason = reason
+                    if i not in ended:
+                        self.scheduler.finish(req)
+                        self._drop_from_next(req)
+            results.append(EngineStepResult(req.request_id, int(tok), done, reason, req.num_prompt_tokens,
+                                            req.num_generated_tokens))
         return results
+
+    def _make_plan(self) -> "_Plan":
+        """Schedule a step and do its host work.  Tokens that are still being sampled are packed as
+        unknown and filled in by :meth:`_fill_unknown_tokens`."""
+        scheduled = self.scheduler.schedule()
+        early = [EngineStepResult(req.request_id, -1, True, req.finish_reason, req.num_prompt_tokens,
+                                  req.num_generated_tokens) for req in self.scheduler.finished_by_scheduler]
+        self.scheduler.finished_by_scheduler.clear()
+        plan = _Plan(scheduled, early)
+        self._pack_plan(plan)
+        return plan
+
+    def _pack_plan(self, plan: "_Plan") -> None:
+        scheduled = plan.scheduled
+        plan.sampling = [s for s in scheduled if s.samples]
+        plan.sample_positions = [s.request.num_tokens for s in plan.sampling]
+        plan.prepared = None
+        if scheduled:
+            entries = [StepEntry(s.request.cache, s.request.token_ids[s.start:s.start + s.num_tokens],
+                                 [s.num_tokens - 1] if s.samples else []) for s in scheduled]
+            plan.prepared = self.runner.prepare(entries, allow_unknown=True)
+
+    def _fill_unknown_tokens(self, plan: "_Plan") -> None:
+        for k, (b, j) in enumerate(plan.prepared.unknown_tokens()):
+            s = plan.scheduled[b]
+            token = s.request.token_ids[s.start + j]
+            if token == UNKNOWN_TOKEN:
+                raise RuntimeError(f"request {s.request.request_id!r}: a token of the step is still unknown")
+            plan.prepared.fill_token(k, token)
+        plan.prepared.all_tokens_known()
+
+    def _drop_from_next(self, req: Request) -> None:
+        """A request of the prepared step has ended after all: pack the step again without it."""
+        plan = self._next
+        if plan is not None and any(s.request is req for s in plan.scheduled):
+            plan.scheduled = [s for s in plan.scheduled if s.request is not req]
+            self._pack_plan(plan)
+
+    def _ends_by_length(self, req: Request) -> Optional[FinishReason]:
+        """The length rules of :meth:`_is_finished`; they need no token ids, only counts."""
+        p = req.params
+        if ((p.max_tokens and req.num_tokens >= p.max_tokens)
+                or (p.max_new_tokens and req.num_generated_tokens >= p.max_new_tokens)
+                or req.num_tokens >= self.config.context_len):
+            return FinishReason.LENGTH
+        return None
 
     def _is_finished(self, req: Request):
         """The reference's rules in its order (ullm/core/engine.py:175-200)."""

@@ -33,6 +33,8 @@ class StepError(RuntimeError):
     pass
 
 
+UNKNOWN_TOKEN = -2         # stands for a token that is still being sampled when the step is prepared
+
 from ..kernels.ops import PREFILL_TILE as Q_TILE   # tokens of one request per prompt-portion attention tile
 
 
@@ -81,10 +83,13 @@ class ModelRunner:
                     total += t.numel() * t.element_size()
         return total
 
-    def _pack(self, entries: Sequence[StepEntry], pad_entries: int = 0, table_stride: Optional[int] = None):
+    def _pack(self, entries: Sequence[StepEntry], pad_entries: int = 0, table_stride: Optional[int] = None,
+              allow_unknown: bool = False):
         """Flatten the entries into one int32 host array.  Returns (host array, offsets, facts).
         ``pad_entries`` > len(entries) appends one-token entries that hold no pages (their cache
-        writes are skipped and their outputs ignored), so that a batch fits a captured graph."""
+        writes are skipped and their outputs ignored), so that a batch fits a captured graph.
+        With ``allow_unknown`` a token may be UNKNOWN_TOKEN (its id is filled in before the launch);
+        ``facts["unknown"]`` lists such tokens as (index into the array, entry, index in the entry)."""
         P = self.page_size
         n_real = len(entries)
         lens = [len(e.tokens) for e in entries]
@@ -160,6 +165,13 @@ class ModelRunner:
             for e, n in zip(entries, lens):
                 tok[t:t + n] = e.tokens
                 t += n
+        unknown = []
+        if allow_unknown and int(tok.min()) == UNKNOWN_TOKEN:
+            first_of = q_start[:n_real]
+            for t in np.nonzero(tok == UNKNOWN_TOKEN)[0].tolist():
+                b = int(ent[t])
+                unknown.append((t, b, t - int(first_of[b])))
+            tok[tok == UNKNOWN_TOKEN] = 0
         if int(tok.min()) < 0 or int(tok.max()) >= self.vocab_size:
             bad = next(rc for rc, e in zip(caches, entries) if min(e.tokens) < 0 or max(e.tokens) >= self.vocab_size)
             raise StepError(f"request {bad.request_id!r}: token id outside [0, {self.vocab_size})")
@@ -191,7 +203,7 @@ class ModelRunner:
         facts = dict(T=T, B=B, strides=strides, n_want=n_want, num_decode=len(dec_list), max_dec_kv=max_dec_kv,
                      num_tiles=len(tile_list) // 2, max_q=max(lens), max_kv=max_kv,
                      decode_only=all(n == 1 for n in lens), lens=lens + [1] * n_pad,
-                     starts=starts + [0] * n_pad, slots=slots + [0] * n_pad)
+                     starts=starts + [0] * n_pad, slots=slots + [0] * n_pad, unknown=unknown)
         return host, offs, facts
 
     def _context(self, dev: torch.Tensor, offs, facts) -> tuple:
@@ -213,51 +225,70 @@ class ModelRunner:
             host={"lens": facts["lens"], "starts": facts["starts"], "slots": facts["slots"]})
         return ctx, (view(6) if facts["n_want"] else None)
 
-    def build_context(self, entries: Sequence[StepEntry]):
-        """Flatten the entries into device tensors (one host-to-device copy)."""
-        host, offs, facts = self._pack(entries)
-        return self._context(self._upload(host), offs, facts)
-
     # ------------------------------------------------------------------ the step
     def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
         """Run the entries as one batch.  Pages for the new tokens must have been reserved.
         Returns float32 logits [number of wanted places, vocab] in the order of the entries and of
         their ``want`` lists, or None if nothing is wanted.  On return the requests' caches hold the
         new tokens (``num_computed`` has advanced)."""
+        return self.launch(self.prepare(entries))
+
+    def prepare(self, entries: Sequence[StepEntry], allow_unknown: bool = False) -> "PreparedStep":
+        """The host half of a step: checks and the packed batch description.  Nothing is queued on
+        the device, so this may run while an earlier step is still computing; the requests' caches
+        must already be in the state in which the step will find them."""
+        entries = list(entries)
+        if (self.use_graphs and len(entries) <= self.max_graph_batch and all(len(e.tokens) == 1 for e in entries)):
+            B = len(entries)
+            b_pad = 1
+            while b_pad < B:
+                b_pad *= 2
+            longest = max(e.cache.num_computed + 1 for e in entries)
+            kv_bucket = 256
+            while kv_bucket < longest:
+                kv_bucket *= 2
+            kv_bucket = min(kv_bucket, self.max_table * self.page_size)
+            packed = [StepEntry(e.cache, e.tokens, [0]) for e in entries]
+            host, offs, facts = self._pack(packed, pad_entries=b_pad, table_stride=self.max_table,
+                                           allow_unknown=allow_unknown)
+            return PreparedStep(entries, host, offs, facts, (b_pad, kv_bucket))
+        host, offs, facts = self._pack(entries, allow_unknown=allow_unknown)
+        return PreparedStep(entries, host, offs, facts, None)
+
+    def launch(self, prepared: "PreparedStep") -> Optional[torch.Tensor]:
+        """The device half: upload, the model's kernels (or a graph replay), and the caches' counters."""
+        if prepared.facts["unknown"]:
+            raise StepError("a prepared step still holds tokens without an id")
+        entries = prepared.entries
         fresh = self.cache.take_fresh_slots()
         if fresh:
             for c in self.caches.values():
                 if c.state is not None:
                     c.state[torch.tensor(fresh, device=c.state.device)] = 0
-        if (self.use_graphs and len(entries) <= self.max_graph_batch and all(len(e.tokens) == 1 for e in entries)):
-            logits = self._step_from_graph(entries)
+        if prepared.graph_key is not None:
+            logits = self._launch_graph(prepared)
         else:
-            ctx, rows = self.build_context(entries)
+            ctx, rows = self._context(self._upload(prepared.host), prepared.offs, prepared.facts)
             with torch.no_grad():
                 logits = self.model.forward(ctx, self.caches, rows)
         for e in entries:
             self.cache.commit(e.cache, len(e.tokens))
         return logits
 
+    def build_context(self, entries: Sequence[StepEntry]):
+        """Flatten the entries into device tensors (one host-to-device copy)."""
+        host, offs, facts = self._pack(entries)
+        return self._context(self._upload(host), offs, facts)
+
     # ------------------------------------------------------------------ HIP graphs for decode steps
-    def _step_from_graph(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+    def _launch_graph(self, prepared: "PreparedStep") -> Optional[torch.Tensor]:
+        entries = prepared.entries
         B = len(entries)
-        b_pad = 1
-        while b_pad < B:
-            b_pad *= 2
-        longest = max(e.cache.num_computed + 1 for e in entries)
-        kv_bucket = 256
-        while kv_bucket < longest:
-            kv_bucket *= 2
-        kv_bucket = min(kv_bucket, self.max_table * self.page_size)
-        packed = [StepEntry(e.cache, e.tokens, [0]) for e in entries]
-        host, offs, facts = self._pack(packed, pad_entries=b_pad, table_stride=self.max_table)
-        key = (b_pad, kv_bucket)
-        graph = self._graphs.get(key)
+        graph = self._graphs.get(prepared.graph_key)
         if graph is None:
-            graph = self._capture(key, host, offs, facts)
+            graph = self._capture(prepared.graph_key, prepared.host, prepared.offs, prepared.facts)
         else:
-            self._upload(host, into=graph.static_dev)
+            self._upload(prepared.host, into=graph.static_dev)
         graph.graph.replay()
         wanted = [b for b, e in enumerate(entries) if len(e.want)]
         if not wanted:
@@ -287,6 +318,27 @@ class ModelRunner:
         graph = _DecodeGraph(g, static_dev, logits)
         self._graphs[key] = graph
         return graph
+
+
+@dataclass
+class PreparedStep:
+    """A step whose host work is done (see :meth:`ModelRunner.prepare`)."""
+    entries: List[StepEntry]
+    host: np.ndarray                  # the packed batch description
+    offs: np.ndarray
+    facts: dict
+    graph_key: Optional[tuple]        # (batch bucket, context bucket) if the step replays a graph
+
+    def unknown_tokens(self) -> List[tuple]:
+        """(entry, index among the entry's tokens) of every token that still needs an id."""
+        return [(b, j) for _, b, j in self.facts["unknown"]]
+
+    def fill_token(self, k: int, token: int) -> None:
+        """Give the k-th unknown token its id."""
+        self.host[int(self.offs[0]) + self.facts["unknown"][k][0]] = token
+
+    def all_tokens_known(self) -> None:
+        self.facts["unknown"] = []
 
 
 @dataclass

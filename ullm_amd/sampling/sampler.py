@@ -45,6 +45,15 @@ class Sampler:
         host[6] = positions
         return SamplerInputs(n, self._upload(host.reshape(-1)).view(7, n))
 
+    def launch(self, logits: torch.Tensor, prepared: SamplerInputs) -> torch.Tensor:
+        """Queue the sampling kernel; returns the n token ids as an int32 device tensor (reading it
+        waits for the step)."""
+        if prepared.n != logits.shape[0]:
+            raise ValueError("one parameter set, seed and position per logits row is needed")
+        f = prepared.packed[0:3].view(torch.float32)
+        i = prepared.packed
+        return ops.sample(logits, f[0], i[3], f[1], f[2], i[4], i[5], i[6])
+
     def sample(self, logits: torch.Tensor, params: Optional[Sequence[SamplingParams]] = None,
                seeds: Optional[Sequence[int]] = None, positions: Optional[Sequence[int]] = None,
                prepared: Optional[SamplerInputs] = None) -> List[int]:
@@ -52,9 +61,4 @@ class Sampler:
         :meth:`prepare`.  Returns n token ids."""
         if prepared is None:
             prepared = self.prepare(params, seeds, positions)
-        if prepared.n != logits.shape[0]:
-            raise ValueError("one parameter set, seed and position per logits row is needed")
-        f = prepared.packed[0:3].view(torch.float32)
-        i = prepared.packed
-        out = ops.sample(logits, f[0], i[3], f[1], f[2], i[4], i[5], i[6])
-        return out.tolist()
+        return self.launch(logits, prepared).tolist()
