@@ -1,7 +1,8 @@
 """A test-only architecture, registered from outside the framework: a stack whose layers are chosen
 one by one in the config (attention with any position encoding, window, norm and bias option, or a
-toy mixer with per-request state of fixed size), with an optional run order that names a layer
-twice or lets a layer read another layer's cache.  Beside it, its plain whole-sequence forward.
+toy mixer with per-request state of fixed size; a dense feed-forward or a toy one that routes every
+token to one of several experts; a toy position encoding with angles of its own), with an optional
+run order that names a layer twice or lets a layer read another layer's cache.  Beside it, its plain whole-sequence forward.
 Nothing here is a model of anyone's; it exists to show that the framework's parts, cache manager and
 step function take new parts without a change to the framework's files."""
 from typing import Dict, List
@@ -10,7 +11,7 @@ import torch
 
 import plain_qwen3 as plain
 from ullm_amd.models import Choice, ModelPlan, register_architecture
-from ullm_amd.parts import Mixer, StateNeed, WeightDecl, register_part
+from ullm_amd.parts import FeedForward, Mixer, PositionEncoding, StateNeed, WeightDecl, register_part
 from ullm_amd.parts.linear import linear
 
 
@@ -48,6 +49,61 @@ class RunningMean(Mixer):
         return linear(means.to(x.dtype), self.w)
 
 
+@register_part("ffn", "toy_top1_experts")
+class Top1Experts(FeedForward):
+    """Every token goes to the one expert its router scores highest (scores in float32, first index
+    on ties); y = softmax(scores)[e] * down_e(relu(up_e x)).  Tokens are gathered per expert, run
+    through the framework's linear, and scattered back."""
+
+    def __init__(self, hidden_size: int, expert_size: int, num_experts: int, prefix: str):
+        self.hidden_size, self.expert_size, self.num_experts, self.prefix = hidden_size, expert_size, num_experts, prefix
+
+    def weights(self):
+        p, H, F = self.prefix, self.hidden_size, self.expert_size
+        out = [WeightDecl(f"{p}.router.weight", (self.num_experts, H), keep_fp32=True)]
+        for e in range(self.num_experts):
+            out += [WeightDecl(f"{p}.experts.{e}.up.weight", (F, H)), WeightDecl(f"{p}.experts.{e}.down.weight", (H, F))]
+        return out
+
+    def bind(self, tensors, env):
+        p = self.prefix
+        self.router = tensors[f"{p}.router.weight"]
+        self.up = [tensors[f"{p}.experts.{e}.up.weight"].contiguous() for e in range(self.num_experts)]
+        self.down = [tensors[f"{p}.experts.{e}.down.weight"].contiguous() for e in range(self.num_experts)]
+
+    def forward(self, x, ctx):
+        scores = x.float() @ self.router.float().T
+        choice = scores.argmax(dim=-1)
+        weight = torch.softmax(scores, dim=-1).gather(1, choice[:, None])
+        out = torch.zeros(x.shape, dtype=torch.float32, device=x.device)
+        for e in range(self.num_experts):
+            rows = torch.nonzero(choice == e).flatten()
+            if rows.numel():
+                hidden = torch.relu(linear(x[rows].contiguous(), self.up[e]))
+                out[rows] = linear(hidden, self.down[e]).float()
+        return (out * weight).to(x.dtype)
+
+
+@register_part("position", "toy_linear_angles")
+class LinearAngles(PositionEncoding):
+    """Adjacent pairs rotated by angle[p, i] = p * step * (i + 1): another table for the same kernel."""
+
+    def __init__(self, head_dim: int, step: float):
+        self.head_dim, self.step = head_dim, float(step)
+        self.table = None
+
+    @staticmethod
+    def angles(positions: torch.Tensor, head_dim: int, step: float) -> torch.Tensor:
+        return positions.to(torch.float32)[:, None] * (step * torch.arange(1, head_dim // 2 + 1, dtype=torch.float32))[None, :]
+
+    def bind(self, tensors, env):
+        a = self.angles(torch.arange(env.context_len), self.head_dim, self.step)
+        self.table = torch.cat((a.cos(), a.sin()), dim=-1).contiguous().to(env.device)
+
+    def kernel_args(self):
+        return self.table, self.head_dim, 2
+
+
 def toy_config_from_dict(d):
     return dict(d)
 
@@ -59,8 +115,13 @@ def toy_plan(cfg: dict) -> ModelPlan:
         p = f"stack.{i}"
         if L["mixer"] == "attention":
             rope = L.get("rope", "half")
-            position = None if rope == "none" else Choice("position", "rotary", dict(
-                head_dim=L["head_dim"], theta=cfg["theta"], rotary_dim=L.get("rotary_dim", L["head_dim"]), pairing=rope))
+            if rope == "none":
+                position = None
+            elif rope == "toy_linear":
+                position = Choice("position", "toy_linear_angles", dict(head_dim=L["head_dim"], step=L["angle_step"]))
+            else:
+                position = Choice("position", "rotary", dict(
+                    head_dim=L["head_dim"], theta=cfg["theta"], rotary_dim=L.get("rotary_dim", L["head_dim"]), pairing=rope))
             mixer = Choice("mixer", "gqa_attention", dict(
                 hidden_size=H, num_heads=L["heads"], num_kv_heads=L["kv_heads"], head_dim=L["head_dim"],
                 prefix=f"{p}.attn", position=position, qk_norm_eps=eps if L.get("qk_norm", True) else None,
@@ -68,9 +129,13 @@ def toy_plan(cfg: dict) -> ModelPlan:
         else:
             mixer = Choice("mixer", "toy_running_mean", dict(hidden_size=H, prefix=f"{p}.mix"))
         norm = lambda n: Choice("norm", "rmsnorm", dict(size=H, eps=eps, weight_name=f"{p}.{n}.weight"))  # noqa: E731
+        if L.get("experts"):
+            ffn = Choice("ffn", "toy_top1_experts", dict(hidden_size=H, expert_size=L["ffn_size"],
+                                                         num_experts=L["experts"], prefix=f"{p}.ffn"))
+        else:
+            ffn = Choice("ffn", "swiglu", dict(hidden_size=H, intermediate_size=L["ffn_size"], prefix=f"{p}.ffn"))
         layers.append(Choice("block", "prenorm", dict(
-            mixer_norm=norm("norm1"), mixer=mixer, ffn_norm=norm("norm2"),
-            ffn=Choice("ffn", "swiglu", dict(hidden_size=H, intermediate_size=L["ffn_size"], prefix=f"{p}.ffn")))))
+            mixer_norm=norm("norm1"), mixer=mixer, ffn_norm=norm("norm2"), ffn=ffn)))
     order = [tuple(x) for x in cfg["run_order"]] if cfg.get("run_order") else None
     return ModelPlan(vocab_size=cfg["vocab_size"], hidden_size=H, embedding_weight="tok.weight", layers=layers,
                      final_norm=Choice("norm", "rmsnorm", dict(size=H, eps=eps, weight_name="out_norm.weight")),
@@ -88,7 +153,11 @@ def _rope(x, positions, L, theta):
     if rope == "none":
         return x
     rot = L.get("rotary_dim", L["head_dim"])
-    cos, sin = plain.rope_cos_sin(positions, rot, theta)
+    if rope == "toy_linear":
+        a = LinearAngles.angles(positions, L["head_dim"], L["angle_step"])
+        cos, sin = a.cos(), a.sin()
+    else:
+        cos, sin = plain.rope_cos_sin(positions, rot, theta)
     r, rest = x[..., :rot], x[..., rot:]
     if rope == "half":
         r = plain.apply_rope_concat_layout(r, cos, sin)
@@ -131,7 +200,18 @@ def toy_forward(w: Dict[str, torch.Tensor], cfg: dict, token_ids: List[int]) -> 
             a = plain.linear(means, w[f"{p}.mix.mean_proj.weight"])
         h = h + a
         x = plain.rms_norm(h, w[f"{p}.norm2.weight"], eps)
-        gu = torch.cat((plain.linear(x, w[f"{p}.ffn.gate_proj.weight"]), plain.linear(x, w[f"{p}.ffn.up_proj.weight"])), -1)
-        h = h + plain.linear(plain.silu_and_mul(gu), w[f"{p}.ffn.down_proj.weight"])
+        if L.get("experts"):
+            scores = x @ w[f"{p}.ffn.router.weight"].T
+            probs = torch.softmax(scores, -1)
+            y = torch.zeros_like(x)
+            for t in range(T):
+                e = int(scores[t].argmax())
+                hidden = torch.relu(plain.linear(x[t], w[f"{p}.ffn.experts.{e}.up.weight"]))
+                y[t] = probs[t, e] * plain.linear(hidden, w[f"{p}.ffn.experts.{e}.down.weight"])
+            h = h + y
+        else:
+            gu = torch.cat((plain.linear(x, w[f"{p}.ffn.gate_proj.weight"]),
+                            plain.linear(x, w[f"{p}.ffn.up_proj.weight"])), -1)
+            h = h + plain.linear(plain.silu_and_mul(gu), w[f"{p}.ffn.down_proj.weight"])
     x = plain.rms_norm(h, w["out_norm.weight"], eps)
     return plain.linear(x, w["head.weight"] if "head.weight" in w else w["tok.weight"])
