@@ -771,14 +771,12 @@ extern "C" int ullm_attention_prefill(
   const int chunks = (nq / nkv + PREFILL_WAVES - 1) / PREFILL_WAVES;
   if ((long long)n_tiles * nkv * chunks > 0x7fffffffLL) return ULLM_ERR_SHAPE;
   const float sl = scale * 1.4426950408889634f;
-  const int ks = hd <= 128 ? 2 : 1;                      // keys split over two halves of a block (LDS allows it)
-  dim3 grid(n_tiles * nkv * chunks), block(64 * PREFILL_WAVES * ks);
-#define ARGS (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool, tiles, \
-    positions, token_entry, block_table, bt_stride, page_size, nq, nkv, sl, window, n_tiles
-#define CALL(N) do { if (N <= 4) hipLaunchKernelGGL((attention_prefill_kernel<N, (N <= 4 ? 2 : 1)>), grid, block, 0, stream, ARGS); \
-    else hipLaunchKernelGGL((attention_prefill_kernel<N, 1>), grid, block, 0, stream, ARGS); } while (0)
+  // keys split over two halves of a block where LDS allows it
+#define CALL(N) do { constexpr int KS = N <= 4 ? 2 : 1;                                                        \
+    hipLaunchKernelGGL((attention_prefill_kernel<N, KS>), dim3(n_tiles * nkv * chunks), dim3(64 * PREFILL_WAVES * KS), \
+    0, stream, (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool,  \
+    tiles, positions, token_entry, block_table, bt_stride, page_size, nq, nkv, sl, window, n_tiles); } while (0)
   DISPATCH_NQK(hd, CALL)
-#undef ARGS
 #undef CALL
   ULLM_LAUNCH_CHECK();
 }
