@@ -365,12 +365,21 @@ attention_reduce_kernel(const float* __restrict__ part, bf16_t* __restrict__ out
     const float f = ok ? fast_exp2(pp[sp * row + hd] - M) : 0.f;
     L += wave_sum(ok ? pp[sp * row + hd + 1] * f : 0.f);
     const int n = num_splits - s0 < 64 ? num_splits - s0 : 64;
-    for (int j = 0; j < n; ++j) {
-      const float fj = __shfl(f, j, 64);
-      const float* pj = pp + (size_t)(s0 + j) * row;
+    // eight splits at a time: their loads are all queued before the first is used
+    for (int j0 = 0; j0 < n; j0 += 8) {
+      float v[8][4];
 #pragma unroll
-      for (int r = 0; r < 4; ++r)
-        if (lane + 64 * r < hd) acc[r] += pj[lane + 64 * r] * fj;
+      for (int u = 0; u < 8; ++u) {
+        const float* pj = pp + (size_t)(s0 + (j0 + u < n ? j0 + u : n - 1)) * row;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) v[u][r] = lane + 64 * r < hd ? pj[lane + 64 * r] : 0.f;
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const float fj = j0 + u < n ? __shfl(f, j0 + u, 64) : 0.f;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[r] += v[u][r] * fj;
+      }
     }
   }
   const float inv = L > 0.f ? 1.f / L : 0.f;

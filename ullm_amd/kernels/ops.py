@@ -312,14 +312,16 @@ def attention_mfma_supports(dtype: torch.dtype, hd: int, page_size: int, nq: int
 
 
 def decode_split(n_items: int, nkv: int, groups: int, max_kv: int, hd: int = 128):
-    """(waves, num_splits) of the decode attention launch.  Few (token, kv head) pairs get 8 waves a
-    block; a token's keys are cut evenly over splits * waves waves.  Keys go to several blocks (whose
-    partial results a second kernel adds up) only when a wave would otherwise get more than 512."""
+    """(waves, num_splits) of the decode attention launch.  A wave walks its keys one 32-key tile after
+    the other, each a round trip to memory, so few (token, kv head) pairs are cut further: up to one
+    block per compute unit, down to about one tile per wave; a second small kernel adds the blocks'
+    partial results.  From 256 pairs on there are blocks enough and a token's keys stay in one."""
     pairs = max(1, n_items * nkv * groups)
     waves = 8 if (pairs <= 512 and hd != 256) else 4
     if pairs >= 256:
         return waves, 1
-    return waves, max(1, -(-max_kv // (512 * waves)))
+    tiles = -(-max_kv // 32)
+    return waves, max(1, min(256 // pairs, tiles // waves))
 
 
 def attention_decode_mfma(q, out, k_pool, v_pool, token_list: Optional[torch.Tensor], n_items: int,
