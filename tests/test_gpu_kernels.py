@@ -83,7 +83,13 @@ def test_gemm_simple(ops, shape):
 @pytest.mark.parametrize("cfg", [dict(nq=6, nkv=2, hd=48, P=8, rot=48, style=1, norm=True),
                                  dict(nq=5, nkv=5, hd=64, P=16, rot=32, style=1, norm=True),
                                  dict(nq=4, nkv=1, hd=16, P=4, rot=16, style=2, norm=False),
-                                 dict(nq=2, nkv=2, hd=256, P=32, rot=0, style=0, norm=True)])
+                                 dict(nq=2, nkv=2, hd=256, P=32, rot=0, style=0, norm=True),
+                                 dict(nq=8, nkv=2, hd=128, P=16, rot=128, style=1, norm=True),     # 16 lanes a head
+                                 dict(nq=5, nkv=1, hd=128, P=16, rot=64, style=2, norm=True),
+                                 dict(nq=3, nkv=3, hd=32, P=8, rot=16, style=1, norm=False),       # 4 lanes a head
+                                 dict(nq=70, nkv=2, hd=32, P=8, rot=32, style=2, norm=True),       # heads beyond one block
+                                 dict(nq=2, nkv=1, hd=512, P=16, rot=512, style=1, norm=True),     # a whole wave a head
+                                 dict(nq=4, nkv=2, hd=64, P=16, rot=24, style=1, norm=True)])      # rot no multiple of 16
 def test_qk_norm_rope_write(ops, dtype, cfg):
     torch.manual_seed(4)
     nq, nkv, hd, P, rot, style = (cfg[k] for k in ("nq", "nkv", "hd", "P", "rot", "style"))
