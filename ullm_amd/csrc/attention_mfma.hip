@@ -48,6 +48,7 @@ struct KVTile {
 struct PageWindow {
   int base;               // first sub-block (key / 16) held
   int page;               // lane i: page id of sub-block base + i (or -1)
+  int off;                // lane i: row of that sub-block's first key inside its page
 };
 
 __device__ __forceinline__ PageWindow load_pages(int key_from, int key_end, const int* __restrict__ bt, int page_size) {
@@ -55,6 +56,7 @@ __device__ __forceinline__ PageWindow load_pages(int key_from, int key_end, cons
   w.base = key_from >> 4;
   const int kb = (w.base + (int)(threadIdx.x & 63)) << 4;
   w.page = kb < key_end ? bt[kb / page_size] : -1;
+  w.off = kb % page_size;
   return w;
 }
 
@@ -68,7 +70,7 @@ __device__ __forceinline__ void load_tile(KVTile<NQK>& t, int key0, const PageWi
   for (int sb = 0; sb < 2; ++sb) {
     const int kb = key0 + 16 * sb;
     const int page = __builtin_amdgcn_readlane(pw.page, (kb >> 4) - pw.base);
-    const int off = kb % page_size;
+    const int off = __builtin_amdgcn_readlane(pw.off, (kb >> 4) - pw.base);
     t.ok[sb] = page >= 0;
     if (page >= 0) {
       const bf16_t* kp = k_pool + (((size_t)page * nkv + kvh) * page_size + off + c) * HD + 8 * g;
@@ -398,8 +400,8 @@ attention_reduce_kernel(const float* __restrict__ part, bf16_t* __restrict__ out
 //   values LDS row = one dim, its 32 keys in the order [g][half][4] (the 8 keys lane group g feeds to
 //          one product are 16 adjacent bytes) + 16 bytes of padding
 // With these paddings the 16 lanes that the hardware serves together read 16 different bank groups.
-// Loads run two tiles ahead of the products (two register sets in rotation), the single LDS tile is
-// rewritten between two barriers.
+// Loads run two tiles ahead of the products (two register sets in rotation); two LDS tiles take turns,
+// so a wave writes the next tile right after its own products and one barrier a tile is enough.
 // grid (n_tiles * nkv * head_chunks).  Workgroups go to the 8 XCDs round-robin by their linear id and
 // each XCD has an L2 of its own, so the id is decoded such that all work on one kv head lands on one
 // XCD (kv head = id mod 8 when the kv heads are a multiple of 8): that head's keys and values then
@@ -420,12 +422,42 @@ struct PrefillStage {                     // one 32-key tile on its way from the
   uint4 k[PER_THREAD], v[PER_THREAD];
 };
 
+// What a thread's pieces need that does not change from tile to tile: offsets in the cache relative
+// to the sub-block's first row (elements) and positions in the LDS tile (bytes).
+template <int NQK>
+struct PrefillLanes {
+  int kofs[PrefillStage<NQK>::PER_THREAD], vofs[PrefillStage<NQK>::PER_THREAD];
+  int klds[PrefillStage<NQK>::PER_THREAD], vlds[PrefillStage<NQK>::PER_THREAD];
+};
+
+template <int NQK>
+__device__ __forceinline__ PrefillLanes<NQK> prefill_lanes(int page_size) {
+  using S = PrefillStage<NQK>;
+  constexpr int HD = S::HD;
+  PrefillLanes<NQK> pl;
+  const int tid = threadIdx.x & (S::THREADS - 1);
+#pragma unroll
+  for (int j = 0; j < S::PER_THREAD; ++j) {
+    const int piece = tid + j * S::THREADS;
+    const int sb = piece / (2 * HD), rem = piece % (2 * HD);      // 2 HD pieces per sub-block
+    // keys: row rem / (HD / 8) of the sub-block, 8 values at column 8 (rem % (HD / 8))
+    pl.kofs[j] = (rem / (HD / 8)) * HD + 8 * (rem % (HD / 8));
+    pl.klds[j] = (16 * sb + rem / (HD / 8)) * S::KROW + 16 * (rem % (HD / 8));
+    // values: dim rem / 2, keys 8 (rem % 2) .. +8 of the sub-block; in LDS the first four go to lane
+    // group 2 (rem % 2), the other four to the group after it
+    pl.vofs[j] = (rem / 2) * page_size + 8 * (rem % 2);
+    pl.vlds[j] = (rem / 2) * S::VROW + 8 * sb + 32 * (rem % 2);
+  }
+  return pl;
+}
+
 // Queue the loads of the tile at key0.  A wave's 64 pieces of one round lie in one 16-key sub-block,
-// so its page id is a single lane of the page window.
+// so its page id is a single lane of the page window and the cache address is a base common to the
+// wave plus the thread's own offset.
 template <int NQK>
 __device__ __forceinline__ void stage_load(PrefillStage<NQK>& st, int key0, const PageWindow& pw,
-                                           const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
-                                           int page_size, int nkv, int kvh) {
+                                           const PrefillLanes<NQK>& pl, const bf16_t* __restrict__ k_pool,
+                                           const bf16_t* __restrict__ v_pool, int page_size, int nkv, int kvh) {
   using S = PrefillStage<NQK>;
   constexpr int HD = S::HD;
   const int tid = threadIdx.x & (S::THREADS - 1);
@@ -435,23 +467,21 @@ __device__ __forceinline__ void stage_load(PrefillStage<NQK>& st, int key0, cons
     st.k[j] = make_uint4(0, 0, 0, 0);
     st.v[j] = make_uint4(0, 0, 0, 0);
     if (piece >= S::CHUNKS) continue;
-    const int sb = __builtin_amdgcn_readfirstlane(piece / (2 * HD));      // 2 HD pieces per sub-block
-    const int kb = key0 + 16 * sb;
-    const int page = __builtin_amdgcn_readlane(pw.page, (kb >> 4) - pw.base);
+    const int sub = __builtin_amdgcn_readfirstlane(piece / (2 * HD)) + (key0 >> 4) - pw.base;
+    const int page = __builtin_amdgcn_readlane(pw.page, sub);
     if (page < 0) continue;
-    const int off = kb % page_size, rem = piece % (2 * HD);
+    const int off = __builtin_amdgcn_readlane(pw.off, sub);
     const size_t base = ((size_t)page * nkv + kvh) * page_size * HD;
-    // keys: row rem / (HD / 8) of the sub-block, 8 values at column 8 (rem % (HD / 8))
-    st.k[j] = *reinterpret_cast<const uint4*>(k_pool + base + (size_t)(off + rem / (HD / 8)) * HD + 8 * (rem % (HD / 8)));
-    // values: dim rem / 2, keys off + 8 (rem % 2) .. +8 of the sub-block
-    st.v[j] = *reinterpret_cast<const uint4*>(v_pool + base + (size_t)(rem / 2) * page_size + off + 8 * (rem % 2));
+    st.k[j] = *reinterpret_cast<const uint4*>(k_pool + base + (size_t)off * HD + pl.kofs[j]);
+    st.v[j] = *reinterpret_cast<const uint4*>(v_pool + base + off + pl.vofs[j]);
   }
 }
 
 // Write a loaded tile to LDS; values of keys past max_hi (never written, may hold anything) become 0.
 template <int NQK>
 __device__ __forceinline__ void stage_store(const PrefillStage<NQK>& st, int key0, int max_hi,
-                                            unsigned char* __restrict__ kl, unsigned char* __restrict__ vl) {
+                                            const PrefillLanes<NQK>& pl, unsigned char* __restrict__ kl,
+                                            unsigned char* __restrict__ vl) {
   using S = PrefillStage<NQK>;
   constexpr int HD = S::HD;
   const int tid = threadIdx.x & (S::THREADS - 1);
@@ -460,19 +490,17 @@ __device__ __forceinline__ void stage_store(const PrefillStage<NQK>& st, int key
   for (int j = 0; j < S::PER_THREAD; ++j) {
     const int piece = tid + j * S::THREADS;
     if (piece >= S::CHUNKS) continue;
-    const int sb = piece / (2 * HD), rem = piece % (2 * HD);
-    *reinterpret_cast<uint4*>(kl + (16 * sb + rem / (HD / 8)) * S::KROW + 16 * (rem % (HD / 8))) = st.k[j];
+    *reinterpret_cast<uint4*>(kl + pl.klds[j]) = st.k[j];
     Pack8 v;
     v.u4 = st.v[j];
-    const int half = rem % 2;
     if (edge) {
+      const int sb = piece / (2 * HD), half = piece % 2;
 #pragma unroll
       for (int e = 0; e < 8; ++e)
         if (key0 + 16 * sb + 8 * half + e > max_hi) v.h[e] = 0;
     }
-    unsigned char* row = vl + (rem / 2) * S::VROW + 8 * sb;
-    *reinterpret_cast<uint2*>(row + 16 * (2 * half)) = v.u2[0];         // keys 8 half .. +4 -> lane group 2 half
-    *reinterpret_cast<uint2*>(row + 16 * (2 * half + 1)) = v.u2[1];     // keys 8 half + 4 .. +4 -> group 2 half + 1
+    *reinterpret_cast<uint2*>(vl + pl.vlds[j]) = v.u2[0];          // keys 8 half .. +4
+    *reinterpret_cast<uint2*>(vl + pl.vlds[j] + 16) = v.u2[1];     // keys 8 half + 4 .. +4
   }
 }
 
@@ -503,21 +531,22 @@ __device__ __forceinline__ void process_tile_lds(const unsigned char* __restrict
   bool rescale = false;
 #pragma unroll
   for (int q = 0; q < NG; ++q) {
+    // the maximum is taken over the raw products (the scale is positive) and scaled once; the scale
+    // of the other scores rides along in the multiply-add that subtracts the reference value
     float tile_max = NEG_BIG;
 #pragma unroll
     for (int sb = 0; sb < 2; ++sb)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        float v = s[q][sb][r] * scale_log2e;
         if (masked) {
           const int kk = key0 + 16 * sb + 4 * g + r;
-          v = (kk >= col_lo[q] && kk <= col_hi[q]) ? v : NEG_BIG;
+          if (!(kk >= col_lo[q] && kk <= col_hi[q])) s[q][sb][r] = NEG_BIG;
         }
-        s[q][sb][r] = v;
-        tile_max = fmaxf(tile_max, v);
+        tile_max = fmaxf(tile_max, s[q][sb][r]);
       }
     tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, 64));
     tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, 64));
+    tile_max = (!masked || tile_max > 0.5f * NEG_BIG) ? tile_max * scale_log2e : NEG_BIG;
     const bool moves = tile_max > m[q] + RESCALE_STEP;
     const float m_new = moves ? tile_max : m[q];
     alpha[q] = moves ? fast_exp2(m[q] - m_new) : 1.f;
@@ -529,7 +558,7 @@ __device__ __forceinline__ void process_tile_lds(const unsigned char* __restrict
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         // a masked score stays at NEG_BIG: its weight is zero even while m_new is still NEG_BIG
-        e[r] = (!masked || s[q][sb][r] > 0.5f * NEG_BIG) ? fast_exp2(s[q][sb][r] - m_new) : 0.f;
+        e[r] = (!masked || s[q][sb][r] > 0.5f * NEG_BIG) ? fast_exp2(fmaf(s[q][sb][r], scale_log2e, -m_new)) : 0.f;
         psum += e[r];
       }
       p[q].w[2 * sb] = pack2_bf16(e[0], e[1]);
@@ -542,9 +571,15 @@ __device__ __forceinline__ void process_tile_lds(const unsigned char* __restrict
 #pragma unroll
     for (int q = 0; q < NG; ++q)
 #pragma unroll
-      for (int n = 0; n < 2 * NQK; ++n) {
-        acc[q][n][0] *= alpha[q]; acc[q][n][1] *= alpha[q]; acc[q][n][2] *= alpha[q]; acc[q][n][3] *= alpha[q];
-      }
+      for (int n = 0; n < 2 * NQK; ++n)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          float o = acc[q][n][r] * alpha[q];
+#ifdef __HIP_DEVICE_COMPILE__
+          asm volatile("" : "+v"(o));       // pins the multiply inside the branch: most tiles skip it
+#endif
+          acc[q][n][r] = o;
+        }
   }
 #pragma unroll
   for (int n = 0; n < 2 * NQK; ++n) {
@@ -574,11 +609,10 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __r
   constexpr int TILE_BYTES = S::KBYTES + S::VBYTES;
   constexpr int PER_LANE = NG * (8 * NQK + 2);            // floats a lane hands over in the merge
   static_assert(KS == 1 || 2 * PER_LANE * 64 * 4 <= 2 * TILE_BYTES, "the merge reuses the tiles' memory");
-  __shared__ __attribute__((aligned(16))) unsigned char lds[KS * TILE_BYTES];
+  __shared__ __attribute__((aligned(16))) unsigned char lds[KS * 2 * TILE_BYTES];   // [half][even | odd tile]
   const int lane = threadIdx.x & 63, wave = (threadIdx.x >> 6) % PREFILL_WAVES, half = threadIdx.x / S::THREADS;
   const int g = lane >> 4, c = lane & 15;
-  unsigned char* const k_lds = lds + half * TILE_BYTES;
-  unsigned char* const v_lds = k_lds + S::KBYTES;
+  unsigned char* const tile_lds = lds + half * 2 * TILE_BYTES;
   const int G = nq / nkv, chunks = (G + PREFILL_WAVES - 1) / PREFILL_WAVES, per_kv = n_tiles * chunks;
   int kvh, rest;
   if (nkv % 8 == 0) {
@@ -633,33 +667,46 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __r
   // the page window serves the loads, which run ahead of the products
   PageWindow pw = load_pages(my_begin < key_end ? my_begin : key_begin, key_end, bt, page_size);
   PrefillStage<NQK> st0, st1;
+  const PrefillLanes<NQK> lanes = prefill_lanes<NQK>(page_size);
 #define STAGE_LOAD(ST, K0)                                                         \
   do {                                                                             \
     if ((K0) < my_end) {                                                           \
       if ((K0) >= 16 * (pw.base + 64)) pw = load_pages((K0), key_end, bt, page_size); \
-      stage_load<NQK>(ST, (K0), pw, k_pool, v_pool, page_size, nkv, kvh);          \
+      stage_load<NQK>(ST, (K0), pw, lanes, k_pool, v_pool, page_size, nkv, kvh);   \
     }                                                                              \
   } while (0)
-#define STAGE_WORK(ST, K0)                                                         \
+#define STAGE_STORE(ST, K0, BUF)                                                   \
   do {                                                                             \
-    __syncthreads();                         /* the previous tile has been read by every wave */ \
-    if ((K0) < my_end) stage_store<NQK>(ST, (K0), last_pos, k_lds, v_lds);         \
-    STAGE_LOAD(ST, (K0) + 64);                                                     \
-    __syncthreads();                                                               \
+    if ((K0) < my_end)                                                             \
+      stage_store<NQK>(ST, (K0), last_pos, lanes, tile_lds + (BUF) * TILE_BYTES,      \
+                       tile_lds + (BUF) * TILE_BYTES + S::KBYTES);                 \
+  } while (0)
+  // the tile at K0 is in LDS tile BUF; NEXT holds the tile after it, which goes to the other LDS tile
+  // (last read one step ago, before the barrier) and is then refilled with the tile three further on
+#define STAGE_WORK(K0, BUF, NEXT)                                                  \
+  do {                                                                             \
     if (head_ok && (K0) < my_end) {                                                \
+      const unsigned char* kl = tile_lds + (BUF) * TILE_BYTES;                     \
       if ((K0) + 31 > first_pos || (K0) < open_lo)                                 \
-        process_tile_lds<NQK, NG, true>(k_lds, v_lds, (K0), qreg, clo, chi, scale_log2e, acc, m, l);  \
+        process_tile_lds<NQK, NG, true>(kl, kl + S::KBYTES, (K0), qreg, clo, chi, scale_log2e, acc, m, l);  \
       else                                                                         \
-        process_tile_lds<NQK, NG, false>(k_lds, v_lds, (K0), qreg, clo, chi, scale_log2e, acc, m, l); \
+        process_tile_lds<NQK, NG, false>(kl, kl + S::KBYTES, (K0), qreg, clo, chi, scale_log2e, acc, m, l); \
     }                                                                              \
+    STAGE_STORE(NEXT, (K0) + 32, 1 - (BUF));                                       \
+    STAGE_LOAD(NEXT, (K0) + 96);                                                   \
+    __syncthreads();                                                               \
   } while (0)
   STAGE_LOAD(st0, my_begin);
   STAGE_LOAD(st1, my_begin + 32);
+  STAGE_STORE(st0, my_begin, 0);
+  STAGE_LOAD(st0, my_begin + 64);
+  __syncthreads();
   for (int i = 0; i < steps; i += 2) {                    // the same number of barriers in both halves
-    STAGE_WORK(st0, my_begin + 32 * i);
+    STAGE_WORK(my_begin + 32 * i, 0, st1);
     if (i + 1 >= steps) break;
-    STAGE_WORK(st1, my_begin + 32 * i + 32);
+    STAGE_WORK(my_begin + 32 * i + 32, 1, st0);
   }
+#undef STAGE_STORE
 #undef STAGE_LOAD
 #undef STAGE_WORK
   if (KS == 2) {
