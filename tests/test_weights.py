@@ -31,6 +31,17 @@ def test_random_folder_is_complete_and_deterministic(tmp_path):
     assert abs(wa["model.layers.0.mlp.down_proj.weight"].float().std() - 0.05) < 0.005
 
 
+def test_random_folder_from_the_command_line(tmp_path, capsys):
+    from ullm_amd.weights import random_init
+    cfg_path = tmp_path / "config.json"
+    cfg_path.write_text(json.dumps(TINY_A))
+    assert random_init.main(["--config", str(cfg_path), "--out", str(tmp_path / "m"), "--seed", "3", "--dtype", "float32"]) == 0
+    assert capsys.readouterr().out.strip() == str(tmp_path / "m")
+    same = write_random_model(TINY_A, str(tmp_path / "n"), seed=3, dtype="float32")
+    wa, wb = load_file(str(tmp_path / "m" / "model.safetensors")), load_file(os.path.join(same, "model.safetensors"))
+    assert set(wa) == set(wb) and all(torch.equal(wa[k], wb[k]) and wa[k].dtype == torch.float32 for k in wa)
+
+
 def test_tied_model_stores_no_head_and_binds_the_embedding(tmp_path):
     d = write_random_model(TINY_A, str(tmp_path / "a"), seed=0)
     assert "lm_head.weight" not in checkpoint_index(d)

@@ -71,3 +71,24 @@ def bind_random_weights(model, env: PartEnv, seed: int, std: Optional[float] = N
     for d in pending_alias:
         tensors[d.name] = tensors[d.alias_of]
     model.bind(tensors, env)
+
+
+def main(argv=None) -> int:
+    """``python -m ullm_amd.weights.random_init --config config.json --out DIR --seed 0``"""
+    import argparse
+    ap = argparse.ArgumentParser(prog="ullm_amd.weights.random_init",
+                                 description="Write a model folder with seeded random weights for a config.json")
+    ap.add_argument("--config", required=True, help="config.json of the architecture (its own keys)")
+    ap.add_argument("--out", required=True, help="folder to write config.json and model.safetensors into")
+    ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--std", type=float, default=None, help="standard deviation (default: the config's initializer_range)")
+    ap.add_argument("--dtype", default="bfloat16", choices=sorted(_STORE))
+    args = ap.parse_args(argv)
+    with open(args.config, encoding="utf-8") as f:
+        config = json.load(f)
+    print(write_random_model(config, args.out, args.seed, args.std, args.dtype))
+    return 0
+
+
+if __name__ == "__main__":
+    raise SystemExit(main())
