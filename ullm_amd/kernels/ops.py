@@ -359,7 +359,7 @@ def attention_decode_mfma(q, out, k_pool, v_pool, token_list: Optional[torch.Ten
         _c_int(splits), _c_int(waves), _p(ws), _stream()), "attention_decode")
 
 
-PREFILL_TILE = 32      # tokens of one request per prompt tile (two groups of 16 columns per wave)
+PREFILL_TILE = 32      # tokens of one request per prompt tile (two groups of 16 columns for every wave of a block)
 
 
 def attention_prefill_mfma(q, out, k_pool, v_pool, tiles: torch.Tensor, n_tiles: int, positions, token_entry,

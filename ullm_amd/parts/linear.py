@@ -20,7 +20,7 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
     return ops.gemm_bf16(x, weight, bias, out_dtype=out_dtype)
 
 
-FUSED_MAX_ROWS = 16      # batches up to this many tokens take the projections with folded norm / add
+FUSED_MAX_ROWS = 16      # batches up to this many tokens take the projections with the folded add / activation
 
 
 def can_fuse(residual: torch.Tensor, dtype: torch.dtype, *weights: torch.Tensor) -> bool:
