@@ -89,6 +89,13 @@ def test_engine_config_names_and_checks(tmp_path):
     # the reference's defaults (ullm/entrypoints/api_server.py:133-156)
     base = EngineConfig.from_args(ap.parse_args(["--model", "x"]))
     assert (base.gpu_memory_utilization, base.max_bs, base.context_len, base.tp_size, base.pp_size) == (0.9, 50, 2048, 1, 1)
+    assert (base.nccl_port, base.device_ids, base.profile, base.profile_dir, base.disable_async_scheduling) == \
+        (29500, None, False, "./profiles", False)
+    other = EngineConfig.from_args(ap.parse_args(["--model", "x", "--device-ids", "3", "--profile", "--profile-dir", "/tmp/p",
+                                                  "--disable-async-scheduling", "--nccl-port", "1234"]))
+    assert other.device == "cuda:3" and other.profile and other.profile_dir == "/tmp/p" and other.disable_async_scheduling
+    with pytest.raises(ConfigError, match="exactly one"):
+        EngineConfig(model="x", device_ids=[0, 1])
     with pytest.raises(ConfigError):
         EngineConfig(model="x", tp_size=2)
     with pytest.raises(ConfigError):

@@ -2,6 +2,7 @@
 temperature sampling equals the plain sampler run on the engine's own logits; finish rules;
 preemption and recomputation give the same tokens; the command line."""
 import json
+import os
 
 import pytest
 import torch
@@ -170,6 +171,20 @@ def test_scheduling_ahead_changes_no_token(model_dirs, plain_models):
     assert ahead_run["r2"][0] == greedy[2] and ahead_run["r2"][1] is FinishReason.LENGTH
     assert all(v[1] is None for v in aborted.values())            # an aborted request reports no ending
     assert runs[True][1] > 0 and runs[False][1] > 0               # both runs had to preempt
+
+
+def test_profile_start_stop_writes_a_trace(model_dirs, tmp_path):
+    from ullm_amd import SamplingParams
+    if DEV == "cpu":
+        pytest.skip("the profiler records device activity")
+    llm = make_llm(model_dirs["A"], profile=True, profile_dir=str(tmp_path / "traces"))
+    llm.profile("start")
+    llm.generate([[1, 2, 3]], SamplingParams(temperature=0.0, max_new_tokens=3, ignore_eos=True))
+    llm.profile("stop")
+    llm.profile("stop")                                  # a second stop is ignored
+    assert any(f.endswith(".json.gz") for f in os.listdir(tmp_path / "traces"))
+    with pytest.raises(RuntimeError, match="profiling is off"):
+        make_llm(model_dirs["A"]).profile("start")
 
 
 def test_prefix_cache_gives_the_same_tokens(model_dirs, plain_models):

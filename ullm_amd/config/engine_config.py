@@ -12,7 +12,7 @@ import argparse
 import json
 import os
 from dataclasses import dataclass, field
-from typing import Optional
+from typing import List, Optional
 
 from .model_config import ConfigError
 
@@ -40,6 +40,10 @@ class EngineConfig:
     enforce_eager: bool = False                 # True: never replay decode steps from HIP graphs
     disable_async_scheduling: bool = False      # True: schedule a step only after the one before has ended
     log_level: str = "info"
+    nccl_port: int = 29500                      # the reference's option; one GPU opens no port
+    device_ids: Optional[List[int]] = None      # the reference's option; exactly one id here (sets ``device``)
+    profile: bool = False                       # True: LLM.profile("start" | "stop") records a torch profiler trace
+    profile_dir: str = "./profiles"             # where those traces are written
     # -- beyond the reference ------------------------------------------------------
     dtype: str = "bfloat16"                     # "bfloat16" | "float32" (whole model in true 32-bit)
     page_size: int = 16                         # tokens per cache page
@@ -54,6 +58,10 @@ class EngineConfig:
         self.dtype = normalize_dtype(self.dtype)
         if self.tp_size != 1 or self.pp_size != 1:
             raise ConfigError("this engine runs on one GPU: tp_size and pp_size must be 1")
+        if self.device_ids is not None:
+            if len(self.device_ids) != 1:
+                raise ConfigError(f"this engine runs on one GPU: device_ids={self.device_ids} must name exactly one")
+            self.device = f"cuda:{int(self.device_ids[0])}"
         if self.max_bs < 1:
             raise ConfigError("max_bs must be at least 1")
         if self.context_len < 1:
@@ -79,6 +87,11 @@ class EngineConfig:
                             help="Max context length of the model")
         parser.add_argument("--enforce-eager", action="store_true",
                             help="Enforce eager execution, disable HIP graphs")
+        parser.add_argument("--nccl-port", type=int, default=29500, help="Unused with one GPU (kept for the reference's callers)")
+        parser.add_argument("--device-ids", type=lambda v: [int(x) for x in v.split(",")], default=None,
+                            help="The GPU to use (one id)")
+        parser.add_argument("--profile", action="store_true", help="Enable torch profiler traces (LLM.profile)")
+        parser.add_argument("--profile-dir", type=str, default="./profiles", help="Directory for profiler traces")
         parser.add_argument("--disable-async-scheduling", action="store_true",
                             help="Do not schedule the next step while the device runs the current one")
         parser.add_argument("--log-level", type=str, default="info", help="Log level for the engine")
@@ -105,6 +118,7 @@ class EngineConfig:
             context_len=args.context_len,
             enforce_eager=args.enforce_eager,
             disable_async_scheduling=args.disable_async_scheduling,
+            nccl_port=args.nccl_port, device_ids=args.device_ids, profile=args.profile, profile_dir=args.profile_dir,
             log_level=args.log_level,
             dtype=args.dtype,
             page_size=args.page_size,

@@ -7,6 +7,8 @@ and ``stream`` yields the reference's per-token ``GenerateOutput`` records as th
 """
 from __future__ import annotations
 
+import logging
+import os
 import uuid
 from dataclasses import dataclass, field
 from typing import Dict, Iterator, List, Optional, Sequence, Union
@@ -15,6 +17,8 @@ from .config.engine_config import EngineConfig
 from .engine.engine import Engine
 from .engine.request import EngineStepResult, FinishReason
 from .sampling import SamplingParams
+
+logger = logging.getLogger("ullm_amd")
 
 Prompt = Union[str, Sequence[int]]
 
@@ -64,6 +68,7 @@ class LLM:
         self.config = config
         self.engine = engine if engine is not None else Engine(config)
         self._tokenizer = None
+        self._profiler = None
 
     # ------------------------------------------------------------------ text
     @property
@@ -152,6 +157,32 @@ class LLM:
 
     def abort(self, sequence_id: str) -> None:
         self.engine.abort_request(sequence_id)
+
+    def profile(self, action: str) -> None:
+        """"start" / "stop" a torch profiler trace (host and device activity) into
+        ``config.profile_dir``; needs ``config.profile`` (reference: ullm/core/worker.py:46-64,137-160)."""
+        if not self.config.profile:
+            raise RuntimeError("profiling is off: set EngineConfig.profile (--profile)")
+        if action not in ("start", "stop"):
+            raise ValueError('profile action must be "start" or "stop"')
+        import torch
+        if action == "start":
+            if self._profiler is not None:
+                logger.warning("profiler already started, ignoring")
+                return
+            os.makedirs(self.config.profile_dir, exist_ok=True)
+            self._profiler = torch.profiler.profile(
+                activities=[torch.profiler.ProfilerActivity.CPU, torch.profiler.ProfilerActivity.CUDA],
+                on_trace_ready=torch.profiler.tensorboard_trace_handler(
+                    os.path.abspath(self.config.profile_dir), worker_name=f"ullm_amd_{os.getpid()}", use_gzip=True),
+                record_shapes=True)
+            self._profiler.start()
+        else:
+            if self._profiler is None:
+                logger.warning("profiler already stopped, ignoring")
+                return
+            self._profiler.stop()
+            self._profiler = None
 
     def shutdown(self) -> None:
         """Nothing runs in the background; kept so that callers of the reference's API need no change."""
