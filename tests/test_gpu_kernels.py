@@ -307,7 +307,7 @@ def test_attention_on_the_matrix_cores(ops, case):
             for f in range(0, n, ops.PREFILL_TILE):
                 tiles += [t0 + f, min(ops.PREFILL_TILE, n - f)]
         t0 += n
-    for splits, waves in ((0, 0), (1, 4), (1, 8), (2, 8), (3, 4), (7, 8)):
+    for splits, waves in ((0, 0), (1, 4), (1, 8), (2, 8), (3, 4), (7, 8), (1, 1), (2, 1)):
         out = torch.full((q.shape[0], nq * hd), float("nan"), dtype=dtype, device=DEV)
         if dec:
             ops.attention_decode_mfma(q, out, k_pool, v_pool, torch.tensor(dec, dtype=torch.int32, device=DEV),

@@ -289,7 +289,7 @@ attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __re
                         int num_splits, float* __restrict__ part) {
   constexpr int HD = 32 * NQK;
   constexpr int ROW = HD + 4;                       // output dims, then maximum and sum (rows stay 16-byte aligned)
-  __shared__ float merge[(WAVES / 2) * (8 * NQK + 2) * 64];   // [writer][value][lane]: conflict-free
+  __shared__ float merge[(WAVES > 1 ? WAVES / 2 : 1) * (WAVES > 1 ? (8 * NQK + 2) * 64 : 1)];   // [writer][value][lane]: conflict-free
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g = lane >> 4, c = lane & 15;
   const int split = blockIdx.x;
   const int G = nq / nkv;
@@ -793,23 +793,24 @@ extern "C" int ullm_attention_decode(
     int num_splits, int waves, float* workspace, hipStream_t stream) {
   if (n_items <= 0) return 0;
   if (!ullm_attention_mfma_supports(hd, page_size, nq, nkv)) return ULLM_ERR_UNSUPPORTED;
-  if (waves != 4 && waves != 8) return ULLM_ERR_UNSUPPORTED;
-  if (hd == 256) waves = 4;                              // shared memory of the merge
+  if (waves != 1 && waves != 4 && waves != 8) return ULLM_ERR_UNSUPPORTED;
+  if (hd == 256 && waves == 8) waves = 4;                // shared memory of the merge
   if (num_splits < 1 || num_splits > 65535 || window < 0) return ULLM_ERR_SHAPE;
   if (num_splits > 1 && !workspace) return ULLM_ERR_SHAPE;
   const int G = nq / nkv, groups = (G + 15) / 16;
   if (n_items > 65535 || nkv * groups > 65535) return ULLM_ERR_SHAPE;
   const float sl = scale * 1.4426950408889634f;
   dim3 grid(num_splits, nkv * groups, n_items), block(64 * waves);
-#define CALL(N) do { if (waves == 8) hipLaunchKernelGGL((attention_decode_kernel<N, 8>), grid, block, 0, stream, \
-    (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool, token_list, \
-    positions, token_entry, block_table, bt_stride, page_size, nq, nkv, sl, window, num_splits, workspace); \
-  else hipLaunchKernelGGL((attention_decode_kernel<N, 4>), grid, block, 0, stream, \
-    (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool, token_list, \
-    positions, token_entry, block_table, bt_stride, page_size, nq, nkv, sl, window, num_splits, workspace); \
+#define ARGS (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool, token_list, \
+    positions, token_entry, block_table, bt_stride, page_size, nq, nkv, sl, window, num_splits, workspace
+#define CALL(N) do {                                                                                        \
+    if (waves == 8) hipLaunchKernelGGL((attention_decode_kernel<N, 8>), grid, block, 0, stream, ARGS);      \
+    else if (waves == 4) hipLaunchKernelGGL((attention_decode_kernel<N, 4>), grid, block, 0, stream, ARGS); \
+    else hipLaunchKernelGGL((attention_decode_kernel<N, 1>), grid, block, 0, stream, ARGS);                 \
   } while (0)
   DISPATCH_NQK(hd, CALL)
 #undef CALL
+#undef ARGS
   int rc = (int)hipGetLastError();
   if (rc != 0 || num_splits == 1) return rc;
   hipLaunchKernelGGL(attention_reduce_kernel, dim3(n_items, nq), dim3(64), 0, stream, workspace, (bf16_t*)out,

@@ -109,10 +109,10 @@ class ModelRunner:
             strides.append(widest)
         n_want = sum(len(e.want) for e in entries) + n_pad
         # attention work lists: tokens of one-token entries; tiles of <= Q_TILE tokens of longer entries
-        dec_list, tile_keys, max_dec_kv, t0 = [], [], 0, 0
+        dec_keys, tile_keys, max_dec_kv, t0 = [], [], 0, 0
         for e, n in zip(entries, lens):
             if n == 1:
-                dec_list.append(t0)
+                dec_keys.append((-e.cache.num_computed, t0))
                 max_dec_kv = max(max_dec_kv, e.cache.num_computed + 1)
             else:
                 for first in range(0, n, Q_TILE):
@@ -120,6 +120,8 @@ class ModelRunner:
                     tile_keys.append((e.cache.num_computed + first + count, t0 + first, count))
             t0 += n
         tile_keys.sort()                                  # the attention kernel wants rising numbers of keys
+        dec_keys.sort()                                   # longest contexts first: the short ones fill the tail
+        dec_list = [t for _, t in dec_keys]
         tile_list = [x for _, first, count in tile_keys for x in (first, count)]
         dec_list.extend(range(t0, t0 + n_pad))
         ng = len(groups)
@@ -219,7 +221,7 @@ class ModelRunner:
             q_start=view(3), entry_slot=view(4), entry_start=view(5), groups=gviews,
             max_q_len=facts["max_q"], max_kv_len=facts["max_kv"], decode_only=facts["decode_only"],
             dtype=self.env.dtype,
-            decode_tokens=view(7 + ng) if 0 < facts["num_decode"] < T else None, num_decode=facts["num_decode"],
+            decode_tokens=view(7 + ng) if facts["num_decode"] else None, num_decode=facts["num_decode"],
             max_decode_kv=facts["max_dec_kv"], tiles=view(8 + ng).view(-1, 2) if facts["num_tiles"] else None,
             num_tiles=facts["num_tiles"],
             host={"lens": facts["lens"], "starts": facts["starts"], "slots": facts["slots"]})

@@ -315,8 +315,12 @@ def decode_split(n_items: int, nkv: int, groups: int, max_kv: int, hd: int = 128
     """(waves, num_splits) of the decode attention launch.  A wave walks its keys one 32-key tile after
     the other, each a round trip to memory, so few (token, kv head) pairs are cut further: up to one
     block per compute unit, down to about one tile per wave; a second small kernel adds the blocks'
-    partial results.  From 256 pairs on there are blocks enough and a token's keys stay in one."""
+    partial results.  From 256 pairs on there are blocks enough and a token's keys stay in one block;
+    from 1024 pairs on a block is a single wave that walks all keys of its pair, so that the waves of
+    a compute unit start and end independently and one's start overlaps the others' streaming."""
     pairs = max(1, n_items * nkv * groups)
+    if pairs >= 1024:
+        return 1, 1
     waves = 8 if (pairs <= 512 and hd != 256) else 4
     if pairs >= 256:
         return waves, 1
@@ -345,7 +349,7 @@ def attention_decode_mfma(q, out, k_pool, v_pool, token_list: Optional[torch.Ten
     groups = -(-(nq // nkv) // 16)
     auto_waves, auto_splits = decode_split(n_items, nkv, groups, max_kv, hd)
     waves = waves or auto_waves
-    if hd == 256:
+    if hd == 256 and waves == 8:
         waves = 4
     splits = splits or auto_splits
     lib = build.load("attention_mfma")

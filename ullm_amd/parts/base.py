@@ -87,7 +87,7 @@ class StepContext:
     host: dict = field(default_factory=dict)   # host-side copies for parts that want them
     # how attention kernels split the batch: tokens of one-token entries, and tiles of up to 32
     # consecutive tokens (first token, count) of the longer entries
-    decode_tokens: Optional[torch.Tensor] = None   # int32 [n_decode]; None when every token is one
+    decode_tokens: Optional[torch.Tensor] = None   # int32 [n_decode]: the one-token entries, longest context first
     num_decode: int = 0
     max_decode_kv: int = 0
     tiles: Optional[torch.Tensor] = None           # int32 [n_tiles, 2]
