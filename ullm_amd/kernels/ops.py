@@ -278,6 +278,8 @@ def gemm_skinny_silu(a: torch.Tensor, w_gate_up: torch.Tensor, nt: int = 0, wave
 
 
 SKINNY_MAX_ROWS = 16     # up to here the weight-streaming kernel beats the library product
+# torch.mm(..., out_dtype=float32) stores the 32-bit accumulator of a bfloat16 product; older torch lacks it
+_MM_TAKES_OUT_DTYPE = "out_dtype" in (torch.mm.__doc__ or "")
 
 
 def gemm_bf16(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
@@ -288,7 +290,7 @@ def gemm_bf16(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = N
     out_dtype = out_dtype or a.dtype
     M = a.shape[0]
     library = a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and a.is_cuda
-    if library and out_dtype == torch.float32 and a.is_contiguous() and w.is_contiguous():
+    if library and out_dtype == torch.float32 and a.is_contiguous() and w.is_contiguous() and _MM_TAKES_OUT_DTYPE:
         # the widest product of a step (the vocabulary): the library streams it a little faster at any M
         y = torch.mm(a, w.t(), out_dtype=torch.float32)
         return y if bias is None else y + bias
