@@ -48,6 +48,7 @@ class _Plan:
     sampling: List[Scheduled] = field(default_factory=list)
     sample_positions: List[int] = field(default_factory=list)   # index each new token takes in its request
     prepared: Optional[PreparedStep] = None
+    sampler_staged: Optional[torch.Tensor] = None         # the sampling parameters in pinned memory
 
 
 class Engine:
@@ -73,6 +74,7 @@ class Engine:
         self.sampler = Sampler(env.device)
         self._arrivals = 0
         self._next: Optional[_Plan] = None   # the step after the one that ran last, scheduled and packed ahead
+        self._inflight = None                # (plan, sampled ids on the device) of a step that is running
         self.on_logits = None      # optional callable(scheduled that sample, float32 logits): for inspection
         logger.info("cache: %s pages of %d tokens per group, %.2f GiB", num_pages, config.page_size,
                     self.runner.cache_bytes() / 2 ** 30)
@@ -111,65 +113,111 @@ class Engine:
     # ------------------------------------------------------------------ one step
     def step(self) -> List[EngineStepResult]:
         """One engine step: the scheduled batch runs, its requests that reached the end of their
-        tokens get one new token each.
+        tokens get one new token each; returns what happened to them.
 
-        The device works asynchronously, and the host uses that: once this step's kernels are
-        queued, the next step is scheduled and packed while they run (reference: the overlap of
-        scheduling and execution, docs/async_scheduling.md; ``disable_async_scheduling`` switches it
-        off).  What the next step depends on is known without the tokens that are still being
-        sampled: counts decide who continues, and the ids are filled in before its launch.  Only a
-        request that ends on its stop token is a surprise; it is taken out of the prepared step."""
-        plan, self._next = self._next, None
-        if plan is None or not (plan.scheduled or plan.early_results):
-            plan = self._make_plan()          # nothing was prepared (or nothing was there to prepare then)
+        The device works asynchronously, and the host uses that (reference: the overlap of scheduling
+        and execution, docs/async_scheduling.md; ``disable_async_scheduling`` switches it off).
+        While a step's kernels run, the next step is scheduled and packed: what it depends on is
+        known without the tokens that are still being sampled (counts decide who continues; the ids
+        are filled in before its launch).  When the tokens arrive they are filed, requests that end
+        on their stop token (the one surprise) are taken out of the prepared step, and that step is
+        launched at once; only then are this step's results put together.  So a call returns the
+        results of one step while the next one is already running."""
+        if self.config.disable_async_scheduling:
+            return self._step_in_turn()
+        if self._inflight is None:
+            plan, self._next = self._next, None
+            if plan is None or not (plan.scheduled or plan.early_results):
+                plan = self._make_plan()      # nothing was prepared (or nothing was there to prepare then)
+            if not plan.scheduled:
+                return plan.early_results
+            self._inflight = self._launch(plan)
+        plan, sampled = self._inflight
+        self._inflight = None
         results = plan.early_results
-        if not plan.scheduled:
+        sampling = plan.sampling
+        if sampled is None:                               # prompt portions only: nothing to wait for
+            self._next = self._make_plan()
             return results
+        # while the device works: who ends by length, and the next step
+        ended: Dict[int, FinishReason] = {}
+        filed = []                                        # index of each new token in its request (None: aborted meanwhile)
+        for i, s in enumerate(sampling):
+            req = s.request
+            if req.status is not RequestStatus.RUNNING:
+                filed.append(None)
+                continue
+            filed.append(req.num_tokens)
+            self.scheduler.append_token(req, UNKNOWN_TOKEN)
+            reason = self._ends_by_length(req)
+            if reason is not None:
+                ended[i] = reason
+                req.finish_reason = reason
+                self.scheduler.finish(req)
+        self._next = self._make_plan()
+        ids = sampled.tolist()                            # waits for the step
+        stops = []
+        for i, (s, tok) in enumerate(zip(sampling, ids)):
+            if filed[i] is None:
+                continue
+            req = s.request
+            req.token_ids[filed[i]] = tok
+            if tok == req.params.eos_token_id and not req.params.ignore_eos:
+                stops.append(i)
+                req.finish_reason = FinishReason.STOP    # the stop token wins over a length limit, as in the reference
+                if i not in ended:
+                    self.scheduler.finish(req)
+                    self._drop_from_next(req)
+        nxt, self._next = self._next, None
+        if nxt.scheduled:
+            self._inflight = self._launch(nxt)            # the device is busy again before the results are built
+        elif nxt.early_results:
+            self._next = nxt
+        for i, (s, tok) in enumerate(zip(sampling, ids)):
+            if filed[i] is None:
+                continue
+            req = s.request
+            stop = i in stops
+            results.append(EngineStepResult(req.request_id, tok, stop or i in ended,
+                                            FinishReason.STOP if stop else ended.get(i), req.num_prompt_tokens,
+                                            req.num_generated_tokens))
+        return results
+
+    def _launch(self, plan: "_Plan"):
+        """Queue a prepared step and its sampling on the device; returns (plan, sampled token ids as a
+        device tensor, or None if no request of the step samples)."""
         self._fill_unknown_tokens(plan)
         sampling = plan.sampling
         sampler_inputs = None
         if sampling:                                      # uploaded ahead of the model's kernels
-            sampler_inputs = self.sampler.prepare([s.request.params for s in sampling],
-                                                  [s.request.seed for s in sampling], plan.sample_positions)
+            if plan.sampler_staged is None:
+                self._stage_plan(plan)
+            sampler_inputs = self.sampler.send(plan.sampler_staged)
+            plan.sampler_staged = None
         logits = self.runner.launch(plan.prepared)
         if not sampling:
-            if not self.config.disable_async_scheduling:
-                self._next = self._make_plan()
-            return results
+            return plan, None
         if self.on_logits is not None:
             self.on_logits(sampling, logits)
-        sampled = self.sampler.launch(logits, sampler_inputs)
-        # while the device works: who ends by length, and the next step
-        ended: Dict[int, FinishReason] = {}
-        if not self.config.disable_async_scheduling:
-            for i, s in enumerate(sampling):
-                self.scheduler.append_token(s.request, UNKNOWN_TOKEN)
-                reason = self._ends_by_length(s.request)
-                if reason is not None:
-                    ended[i] = reason
-                    s.request.finish_reason = reason
-                    self.scheduler.finish(s.request)
-            self._next = self._make_plan()
-        ids = sampled.tolist()                            # waits for the step
-        for i, (s, tok) in enumerate(zip(sampling, ids)):
+        return plan, self.sampler.launch(logits, sampler_inputs)
+
+    def _step_in_turn(self) -> List[EngineStepResult]:
+        """Schedule, run, wait, file the tokens: one thing after the other."""
+        plan = self._make_plan()
+        results = plan.early_results
+        if not plan.scheduled:
+            return results
+        _, sampled = self._launch(plan)
+        if sampled is None:
+            return results
+        for s, tok in zip(plan.sampling, sampled.tolist()):
             req = s.request
-            if self.config.disable_async_scheduling:
-                self.scheduler.append_token(req, tok)
-                done, reason = self._is_finished(req)
-                if done:
-                    req.finish_reason = reason
-                    self.scheduler.finish(req)
-            else:
-                req.token_ids[plan.sample_positions[i]] = int(tok)
-                stop = tok == req.params.eos_token_id and not req.params.ignore_eos
-                done = stop or i in ended
-                reason = FinishReason.STOP if stop else ended.get(i)
-                if stop:                                  # the stop token wins over a length limit, as in the reference
-                    req.finish_reason = reason
-                    if i not in ended:
-                        self.scheduler.finish(req)
-                        self._drop_from_next(req)
-            results.append(EngineStepResult(req.request_id, int(tok), done, reason, req.num_prompt_tokens,
+            self.scheduler.append_token(req, tok)
+            done, reason = self._is_finished(req)
+            if done:
+                req.finish_reason = reason
+                self.scheduler.finish(req)
+            results.append(EngineStepResult(req.request_id, tok, done, reason, req.num_prompt_tokens,
                                             req.num_generated_tokens))
         return results
 
@@ -189,10 +237,20 @@ class Engine:
         plan.sampling = [s for s in scheduled if s.samples]
         plan.sample_positions = [s.request.num_tokens for s in plan.sampling]
         plan.prepared = None
+        plan.sampler_staged = None
         if scheduled:
             entries = [StepEntry(s.request.cache, s.request.token_ids[s.start:s.start + s.num_tokens],
                                  [s.num_tokens - 1] if s.samples else []) for s in scheduled]
             plan.prepared = self.runner.prepare(entries, allow_unknown=True)
+            self._stage_plan(plan)
+
+    def _stage_plan(self, plan: "_Plan") -> None:
+        """Put the step's batch description and its sampling parameters into pinned memory, so that
+        its launch only has to fill in late token ids and queue two copies."""
+        self.runner.stage(plan.prepared)
+        if plan.sampling:
+            plan.sampler_staged = self.sampler.stage([s.request.params for s in plan.sampling],
+                                                     [s.request.seed for s in plan.sampling], plan.sample_positions)
 
     def _fill_unknown_tokens(self, plan: "_Plan") -> None:
         for k, (b, j) in enumerate(plan.prepared.unknown_tokens()):

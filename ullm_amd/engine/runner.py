@@ -257,6 +257,16 @@ class ModelRunner:
         host, offs, facts = self._pack(entries, allow_unknown=allow_unknown)
         return PreparedStep(entries, host, offs, facts, None)
 
+    def stage(self, prepared: "PreparedStep") -> None:
+        """Copy a prepared step's description into pinned memory ahead of its launch (optional: the
+        launch does it otherwise).  Only the step that will be launched next may be staged."""
+        prepared.staged = self._upload.stage(prepared.host)
+
+    def _send(self, prepared: "PreparedStep", into: Optional[torch.Tensor] = None) -> torch.Tensor:
+        staged = prepared.staged if prepared.staged is not None else self._upload.stage(prepared.host)
+        prepared.staged = None
+        return self._upload.send(staged, into)
+
     def launch(self, prepared: "PreparedStep") -> Optional[torch.Tensor]:
         """The device half: upload, the model's kernels (or a graph replay), and the caches' counters."""
         if prepared.facts["unknown"]:
@@ -270,7 +280,7 @@ class ModelRunner:
         if prepared.graph_key is not None:
             logits = self._launch_graph(prepared)
         else:
-            ctx, rows = self._context(self._upload(prepared.host), prepared.offs, prepared.facts)
+            ctx, rows = self._context(self._send(prepared), prepared.offs, prepared.facts)
             with torch.no_grad():
                 logits = self.model.forward(ctx, self.caches, rows)
         for e in entries:
@@ -290,7 +300,7 @@ class ModelRunner:
         if graph is None:
             graph = self._capture(prepared.graph_key, prepared.host, prepared.offs, prepared.facts)
         else:
-            self._upload(prepared.host, into=graph.static_dev)
+            self._send(prepared, into=graph.static_dev)
         graph.graph.replay()
         wanted = [b for b, e in enumerate(entries) if len(e.want)]
         if not wanted:
@@ -330,6 +340,7 @@ class PreparedStep:
     offs: np.ndarray
     facts: dict
     graph_key: Optional[tuple]        # (batch bucket, context bucket) if the step replays a graph
+    staged: Optional[torch.Tensor] = None   # the description already in pinned memory (see ModelRunner.stage)
 
     def unknown_tokens(self) -> List[tuple]:
         """(entry, index among the entry's tokens) of every token that still needs an id."""
@@ -337,7 +348,10 @@ class PreparedStep:
 
     def fill_token(self, k: int, token: int) -> None:
         """Give the k-th unknown token its id."""
-        self.host[int(self.offs[0]) + self.facts["unknown"][k][0]] = token
+        at = int(self.offs[0]) + self.facts["unknown"][k][0]
+        self.host[at] = token
+        if self.staged is not None:
+            self.staged[at] = token
 
     def all_tokens_known(self) -> None:
         self.facts["unknown"] = []

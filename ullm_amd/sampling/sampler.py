@@ -27,11 +27,10 @@ class Sampler:
         self.device = device
         self._upload = StagedUpload(device)
 
-    def prepare(self, params: Sequence[SamplingParams], seeds: Sequence[int], positions: Sequence[int]) -> SamplerInputs:
-        """Queue the upload of the rows' parameters.  Called before the model step is launched, the
-        copy does not wait for the step, and sampling can follow it without the host in between.
-        ``positions[i]`` = index the new token of row i will take in its request (the counter of
-        the row's random stream)."""
+    def stage(self, params: Sequence[SamplingParams], seeds: Sequence[int], positions: Sequence[int]) -> torch.Tensor:
+        """Pack the rows' parameters into pinned memory (host work only; may be done while the
+        device runs the step before).  ``positions[i]`` = index the new token of row i will take in
+        its request (the counter of the row's random stream)."""
         n = len(params)
         if not (len(seeds) == len(positions) == n):
             raise ValueError("one parameter set, seed and position per logits row is needed")
@@ -43,7 +42,16 @@ class Sampler:
         host[4] = (s64 & np.uint64(0xFFFFFFFF)).astype(np.uint32).view(np.int32)
         host[5] = (s64 >> np.uint64(32)).astype(np.uint32).view(np.int32)
         host[6] = positions
-        return SamplerInputs(n, self._upload(host.reshape(-1)).view(7, n))
+        return self._upload.stage(host.reshape(-1))
+
+    def send(self, staged: torch.Tensor) -> SamplerInputs:
+        """Queue the upload of staged parameters.  Called before the model step is launched, the copy
+        does not wait for the step, and sampling can follow it without the host in between."""
+        n = staged.numel() // 7
+        return SamplerInputs(n, self._upload.send(staged).view(7, n))
+
+    def prepare(self, params: Sequence[SamplingParams], seeds: Sequence[int], positions: Sequence[int]) -> SamplerInputs:
+        return self.send(self.stage(params, seeds, positions))
 
     def launch(self, logits: torch.Tensor, prepared: SamplerInputs) -> torch.Tensor:
         """Queue the sampling kernel; returns the n token ids as an int32 device tensor (reading it
