@@ -173,6 +173,52 @@ def test_scheduling_ahead_changes_no_token(model_dirs, plain_models):
     assert runs[True][1] > 0 and runs[False][1] > 0               # both runs had to preempt
 
 
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_scheduling_ahead_under_random_arrivals_and_aborts(model_dirs, seed):
+    """Requests arrive while others run, some are aborted, pages are scarce and prefixes are shared:
+    with and without the overlap every request that was not aborted gets the same tokens and the
+    same ending, and all pages come back."""
+    import random
+    from ullm_amd import SamplingParams
+    rng = random.Random(seed)
+    n = 14
+    common = [rng.randrange(503) for _ in range(9)]
+    prompts = [(common if rng.random() < 0.4 else []) + [rng.randrange(503) for _ in range(rng.randint(1, 30))]
+               for _ in range(n)]
+    params = [SamplingParams(temperature=rng.choice([0.0, 0.8]), top_k=rng.choice([-1, 20]), seed=50 + i,
+                             max_new_tokens=rng.randint(1, 12), eos_token_id=rng.randrange(503),
+                             ignore_eos=rng.random() < 0.5) for i in range(n)]
+    arrive = sorted(rng.randint(0, 25) for _ in range(n))              # step at which each request is added
+    aborts = {rng.randrange(n): rng.randint(3, 30) for _ in range(3)}   # request -> step of its abort
+    runs = []
+    for ahead in (False, True):
+        llm = make_llm(model_dirs["B"], page_size=4, num_pages=40, max_num_batched_tokens=20, max_prefill_chunk=9,
+                       max_bs=5, enable_prefix_cache=True, disable_async_scheduling=not ahead)
+        eng = llm.engine
+        got, step, added = {}, 0, 0
+        while added < n or eng.has_unfinished_requests():
+            while added < n and arrive[added] <= step:
+                eng.add_request(f"r{added}", prompts[added], params[added])
+                added += 1
+            for i, when in aborts.items():
+                if when == step:
+                    eng.abort_request(f"r{i}")
+            for r in eng.step():
+                rec = got.setdefault(r.seq_id, [[], None])
+                if r.new_token_id >= 0:
+                    rec[0].append(r.new_token_id)
+                if r.is_finished:
+                    rec[1] = r.finish_reason
+            step += 1
+            assert step < 2000
+        eng.runner.cache.check()
+        runs.append(got)
+    plain_run, ahead_run = runs
+    kept = [f"r{i}" for i in range(n) if i not in aborts]
+    for k in kept:
+        assert ahead_run[k] == plain_run[k] and ahead_run[k][1] is not None, k
+
+
 def test_profile_start_stop_writes_a_trace(model_dirs, tmp_path):
     from ullm_amd import SamplingParams
     if DEV == "cpu":
