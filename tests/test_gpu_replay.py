@@ -184,6 +184,43 @@ def test_other_page_sizes(replayers, plain_models):
         close(np.concatenate(got), want, "float32")
 
 
+@pytest.mark.parametrize("trial", range(8))
+def test_random_configurations(tmp_path, trial):
+    """Configurations drawn at random over what config.json allows (head sizes in steps of 16, heads per
+    kv head from 1 to 8, widths and vocabularies that are no powers of two, windows, tied heads, page
+    sizes): portions of changing size and then single tokens equal the plain model, in both dtypes."""
+    import random
+    from ullm_amd.replay import Replayer
+    from ullm_amd.weights.random_init import write_random_model
+    rng = random.Random(1000 + trial)
+    nkv = rng.choice([1, 2, 3, 4, 8])
+    cfg = dict(architectures=["Qwen3ForCausalLM"], hidden_size=rng.choice([40, 72, 96, 136, 200, 264]),
+               num_hidden_layers=rng.choice([1, 2, 3]), num_attention_heads=nkv * rng.choice([1, 2, 3, 4, 5, 7, 8]),
+               num_key_value_heads=nkv, head_dim=rng.choice([16, 32, 48, 64, 80, 96, 112, 128, 256]),
+               intermediate_size=rng.choice([56, 104, 200, 328]), vocab_size=rng.choice([101, 257, 503, 1000]),
+               rope_theta=rng.choice([1e4, 1e6]), rms_norm_eps=rng.choice([1e-5, 1e-6]), max_position_embeddings=512,
+               tie_word_embeddings=rng.random() < 0.5, initializer_range=0.05, use_sliding_window=rng.random() < 0.4,
+               sliding_window=rng.choice([7, 33, 100]), max_window_layers=rng.choice([0, 1]))
+    page_size, n = rng.choice([4, 8, 16, 32]), rng.choice([40, 97, 150])
+    d = write_random_model(cfg, str(tmp_path / "m"), seed=trial)
+    pc, w = plain.load_model_folder(d)
+    toks = [rng.randrange(cfg["vocab_size"]) for _ in range(n)]
+    want = plain.qwen3_forward(w, pc, toks)
+    cuts, left = [], n - 12
+    while left > 0:
+        cuts.append(min(left, rng.choice([2, 3, 17, 33, 64])))
+        left -= cuts[-1]
+    cuts += [1] * 12
+    for dtype in ("float32", "bfloat16"):
+        rep = Replayer(d, dtype, 512, page_size, DEV)
+        outs, i = [], 0
+        for s, c in enumerate(cuts):
+            outs.append(rep.step({"step": s, "entries": [{"id": "a", "tokens": toks[i:i + c], "want": list(range(c))}],
+                                  "end": []}))
+            i += c
+        close(np.concatenate(outs), want, dtype)
+
+
 def test_pool_too_small_is_an_error_not_a_wrong_result(replayers):
     rep = replayers("A", "float32", max_tokens=64)
     with pytest.raises(RuntimeError, match="pages"):
