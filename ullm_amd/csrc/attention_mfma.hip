@@ -417,16 +417,16 @@ struct PrefillStage {                     // one 32-key tile on its way from the
   static constexpr int THREADS = 64 * PREFILL_WAVES;
   static constexpr int CHUNKS = 4 * HD;   // 16-byte pieces of the key tile, and as many of the value tile
   static constexpr int PER_THREAD = (CHUNKS + THREADS - 1) / THREADS;
-  static constexpr int KROW = 2 * HD + 16, VROW = 64 + 16;     // bytes
+  static constexpr int KROW = 2 * HD + 32, VROW = 64 + 32;     // bytes
   static constexpr int KBYTES = 32 * KROW, VBYTES = HD * VROW;
   uint4 k[PER_THREAD], v[PER_THREAD];
 };
 
-// What a thread's pieces need that does not change from tile to tile: offsets in the cache relative
-// to the sub-block's first row (elements) and positions in the LDS tile (bytes).
+// What a thread's pieces need that does not change from tile to tile: byte offsets in the cache
+// relative to the sub-block's first row and positions in the LDS tile (bytes).
 template <int NQK>
 struct PrefillLanes {
-  int kofs[PrefillStage<NQK>::PER_THREAD], vofs[PrefillStage<NQK>::PER_THREAD];
+  unsigned kofs[PrefillStage<NQK>::PER_THREAD], vofs[PrefillStage<NQK>::PER_THREAD];
   int klds[PrefillStage<NQK>::PER_THREAD], vlds[PrefillStage<NQK>::PER_THREAD];
 };
 
@@ -441,11 +441,11 @@ __device__ __forceinline__ PrefillLanes<NQK> prefill_lanes(int page_size) {
     const int piece = tid + j * S::THREADS;
     const int sb = piece / (2 * HD), rem = piece % (2 * HD);      // 2 HD pieces per sub-block
     // keys: row rem / (HD / 8) of the sub-block, 8 values at column 8 (rem % (HD / 8))
-    pl.kofs[j] = (rem / (HD / 8)) * HD + 8 * (rem % (HD / 8));
+    pl.kofs[j] = 2u * (unsigned)((rem / (HD / 8)) * HD + 8 * (rem % (HD / 8)));
     pl.klds[j] = (16 * sb + rem / (HD / 8)) * S::KROW + 16 * (rem % (HD / 8));
     // values: dim rem / 2, keys 8 (rem % 2) .. +8 of the sub-block; in LDS the first four go to lane
     // group 2 (rem % 2), the other four to the group after it
-    pl.vofs[j] = (rem / 2) * page_size + 8 * (rem % 2);
+    pl.vofs[j] = 2u * (unsigned)((rem / 2) * page_size + 8 * (rem % 2));
     pl.vlds[j] = (rem / 2) * S::VROW + 8 * sb + 32 * (rem % 2);
   }
   return pl;
@@ -453,27 +453,40 @@ __device__ __forceinline__ PrefillLanes<NQK> prefill_lanes(int page_size) {
 
 // Queue the loads of the tile at key0.  A wave's 64 pieces of one round lie in one 16-key sub-block,
 // so its page id is a single lane of the page window and the cache address is a base common to the
-// wave plus the thread's own offset.
+// wave (scalar registers) plus the thread's own 32-bit offset.  `k_head` / `v_head` point at this kv
+// head inside page 0; `page_elems` is the distance between pages.
 template <int NQK>
 __device__ __forceinline__ void stage_load(PrefillStage<NQK>& st, int key0, const PageWindow& pw,
-                                           const PrefillLanes<NQK>& pl, const bf16_t* __restrict__ k_pool,
-                                           const bf16_t* __restrict__ v_pool, int page_size, int nkv, int kvh) {
+                                           const PrefillLanes<NQK>& pl, const bf16_t* __restrict__ k_head,
+                                           const bf16_t* __restrict__ v_head, unsigned page_elems) {
   using S = PrefillStage<NQK>;
   constexpr int HD = S::HD;
   const int tid = threadIdx.x & (S::THREADS - 1);
 #pragma unroll
   for (int j = 0; j < S::PER_THREAD; ++j) {
     const int piece = tid + j * S::THREADS;
+    const int sub = __builtin_amdgcn_readfirstlane(piece / (2 * HD)) + (key0 >> 4) - pw.base;
+    const int page = piece < S::CHUNKS ? __builtin_amdgcn_readlane(pw.page, sub & 63) : -1;
+    if (page < 0) {
+      st.k[j] = make_uint4(0, 0, 0, 0);
+      st.v[j] = make_uint4(0, 0, 0, 0);
+      continue;
+    }
+    const unsigned off = (unsigned)__builtin_amdgcn_readlane(pw.off, sub);
+    const size_t base = (size_t)(unsigned)page * page_elems;
+    const char* kp = reinterpret_cast<const char*>(k_head + base + off * HD);
+    const char* vp = reinterpret_cast<const char*>(v_head + base + off);
+    st.k[j] = *reinterpret_cast<const uint4*>(kp + pl.kofs[j]);
+    st.v[j] = *reinterpret_cast<const uint4*>(vp + pl.vofs[j]);
+  }
+}
+
+template <int NQK>
+__device__ __forceinline__ void stage_zero(PrefillStage<NQK>& st) {
+#pragma unroll
+  for (int j = 0; j < PrefillStage<NQK>::PER_THREAD; ++j) {
     st.k[j] = make_uint4(0, 0, 0, 0);
     st.v[j] = make_uint4(0, 0, 0, 0);
-    if (piece >= S::CHUNKS) continue;
-    const int sub = __builtin_amdgcn_readfirstlane(piece / (2 * HD)) + (key0 >> 4) - pw.base;
-    const int page = __builtin_amdgcn_readlane(pw.page, sub);
-    if (page < 0) continue;
-    const int off = __builtin_amdgcn_readlane(pw.off, sub);
-    const size_t base = ((size_t)page * nkv + kvh) * page_size * HD;
-    st.k[j] = *reinterpret_cast<const uint4*>(k_pool + base + (size_t)off * HD + pl.kofs[j]);
-    st.v[j] = *reinterpret_cast<const uint4*>(v_pool + base + off + pl.vofs[j]);
   }
 }
 
@@ -491,16 +504,19 @@ __device__ __forceinline__ void stage_store(const PrefillStage<NQK>& st, int key
     const int piece = tid + j * S::THREADS;
     if (piece >= S::CHUNKS) continue;
     *reinterpret_cast<uint4*>(kl + pl.klds[j]) = st.k[j];
+    if (!edge) {
+      *reinterpret_cast<uint2*>(vl + pl.vlds[j]) = make_uint2(st.v[j].x, st.v[j].y);       // keys 8 half .. +4
+      *reinterpret_cast<uint2*>(vl + pl.vlds[j] + 16) = make_uint2(st.v[j].z, st.v[j].w);  // keys 8 half + 4 .. +4
+      continue;
+    }
     Pack8 v;
     v.u4 = st.v[j];
-    if (edge) {
-      const int sb = piece / (2 * HD), half = piece % 2;
+    const int sb = piece / (2 * HD), half = piece % 2;
 #pragma unroll
-      for (int e = 0; e < 8; ++e)
-        if (key0 + 16 * sb + 8 * half + e > max_hi) v.h[e] = 0;
-    }
-    *reinterpret_cast<uint2*>(vl + pl.vlds[j]) = v.u2[0];          // keys 8 half .. +4
-    *reinterpret_cast<uint2*>(vl + pl.vlds[j] + 16) = v.u2[1];     // keys 8 half + 4 .. +4
+    for (int e = 0; e < 8; ++e)
+      if (key0 + 16 * sb + 8 * half + e > max_hi) v.h[e] = 0;
+    *reinterpret_cast<uint2*>(vl + pl.vlds[j]) = v.u2[0];
+    *reinterpret_cast<uint2*>(vl + pl.vlds[j] + 16) = v.u2[1];
   }
 }
 
@@ -610,7 +626,8 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __r
   constexpr int PER_LANE = NG * (8 * NQK + 2);            // floats a lane hands over in the merge
   static_assert(KS == 1 || 2 * PER_LANE * 64 * 4 <= 2 * TILE_BYTES, "the merge reuses the tiles' memory");
   __shared__ __attribute__((aligned(16))) unsigned char lds[KS * 2 * TILE_BYTES];   // [half][even | odd tile]
-  const int lane = threadIdx.x & 63, wave = (threadIdx.x >> 6) % PREFILL_WAVES, half = threadIdx.x / S::THREADS;
+  const int wave_id = (int)(threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63, wave = wave_id % PREFILL_WAVES, half = wave_id / PREFILL_WAVES;
   const int g = lane >> 4, c = lane & 15;
   unsigned char* const tile_lds = lds + half * 2 * TILE_BYTES;
   const int G = nq / nkv, chunks = (G + PREFILL_WAVES - 1) / PREFILL_WAVES, per_kv = n_tiles * chunks;
@@ -668,30 +685,33 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __r
   PageWindow pw = load_pages(my_begin < key_end ? my_begin : key_begin, key_end, bt, page_size);
   PrefillStage<NQK> st0, st1;
   const PrefillLanes<NQK> lanes = prefill_lanes<NQK>(page_size);
+  const unsigned page_elems = (unsigned)(nkv * page_size * HD);
+  const bf16_t* const k_head = k_pool + (size_t)kvh * page_size * HD;
+  const bf16_t* const v_head = v_pool + (size_t)kvh * page_size * HD;
 #define STAGE_LOAD(ST, K0)                                                         \
   do {                                                                             \
     if ((K0) < my_end) {                                                           \
       if ((K0) >= 16 * (pw.base + 64)) pw = load_pages((K0), key_end, bt, page_size); \
-      stage_load<NQK>(ST, (K0), pw, lanes, k_pool, v_pool, page_size, nkv, kvh);   \
+      stage_load<NQK>(ST, (K0), pw, lanes, k_head, v_head, page_elems);           \
+    } else {                                                                       \
+      stage_zero<NQK>(ST);                                                         \
     }                                                                              \
   } while (0)
 #define STAGE_STORE(ST, K0, BUF)                                                   \
-  do {                                                                             \
-    if ((K0) < my_end)                                                             \
-      stage_store<NQK>(ST, (K0), last_pos, lanes, tile_lds + (BUF) * TILE_BYTES,      \
-                       tile_lds + (BUF) * TILE_BYTES + S::KBYTES);                 \
-  } while (0)
-  // the tile at K0 is in LDS tile BUF; NEXT holds the tile after it, which goes to the other LDS tile
-  // (last read one step ago, before the barrier) and is then refilled with the tile three further on
+  stage_store<NQK>(ST, (K0), last_pos, lanes, tile_lds + (BUF) * TILE_BYTES,       \
+                   tile_lds + (BUF) * TILE_BYTES + S::KBYTES)
+  // The tile at K0 is in LDS tile BUF; NEXT holds the tile after it, which goes to the other LDS tile
+  // (last read one step ago, before the barrier) and is then refilled with the tile three further on.
+  // Every wave runs every step: a wave without a head has no visible key (its limits are empty), and
+  // a step past the end of this half's keys finds a tile of zeros whose keys no column sees, so
+  // neither changes a sum and the loop needs no test around the products.
 #define STAGE_WORK(K0, BUF, NEXT)                                                  \
   do {                                                                             \
-    if (head_ok && (K0) < my_end) {                                                \
-      const unsigned char* kl = tile_lds + (BUF) * TILE_BYTES;                     \
-      if ((K0) + 31 > first_pos || (K0) < open_lo)                                 \
-        process_tile_lds<NQK, NG, true>(kl, kl + S::KBYTES, (K0), qreg, clo, chi, scale_log2e, acc, m, l);  \
-      else                                                                         \
-        process_tile_lds<NQK, NG, false>(kl, kl + S::KBYTES, (K0), qreg, clo, chi, scale_log2e, acc, m, l); \
-    }                                                                              \
+    const unsigned char* kl = tile_lds + (BUF) * TILE_BYTES;                       \
+    if ((K0) + 31 > first_pos || (K0) < open_lo)                                   \
+      process_tile_lds<NQK, NG, true>(kl, kl + S::KBYTES, (K0), qreg, clo, chi, scale_log2e, acc, m, l);  \
+    else                                                                           \
+      process_tile_lds<NQK, NG, false>(kl, kl + S::KBYTES, (K0), qreg, clo, chi, scale_log2e, acc, m, l); \
     STAGE_STORE(NEXT, (K0) + 32, 1 - (BUF));                                       \
     STAGE_LOAD(NEXT, (K0) + 96);                                                   \
     __syncthreads();                                                               \
@@ -827,6 +847,7 @@ extern "C" int ullm_attention_prefill(
   if (window < 0) return ULLM_ERR_SHAPE;
   const int chunks = (nq / nkv + PREFILL_WAVES - 1) / PREFILL_WAVES;
   if ((long long)n_tiles * nkv * chunks > 0x7fffffffLL) return ULLM_ERR_SHAPE;
+  if ((long long)nkv * page_size * hd > 0x7fffffffLL) return ULLM_ERR_SHAPE;   // 32-bit distance between pages
   const float sl = scale * 1.4426950408889634f;
   // keys split over two halves of a block where LDS allows it
 #define CALL(N) do { constexpr int KS = N <= 4 ? 2 : 1;                                                        \
