@@ -542,14 +542,15 @@ __device__ __forceinline__ void process_tile_lds(const unsigned char* __restrict
       for (int q = 0; q < NG; ++q)
         s[q][sb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qreg[q][ch].v, s[q][sb], 0, 0, 0);
     }
-  Pack8 p[NG];
-  float alpha[NG];
-  bool rescale = false;
+  // Does any score of the tile exceed its column's reference value by more than RESCALE_STEP?  Each
+  // lane looks at its own scores only (the maximum is taken over the raw products, the scale is
+  // positive); the wave votes.  Most tiles pass, and then no value crosses lanes and nothing is
+  // rescaled.
+  float lane_max[NG];
+  bool exceeds = false;
 #pragma unroll
   for (int q = 0; q < NG; ++q) {
-    // the maximum is taken over the raw products (the scale is positive) and scaled once; the scale
-    // of the other scores rides along in the multiply-add that subtracts the reference value
-    float tile_max = NEG_BIG;
+    lane_max[q] = NEG_BIG;
 #pragma unroll
     for (int sb = 0; sb < 2; ++sb)
 #pragma unroll
@@ -558,34 +559,26 @@ __device__ __forceinline__ void process_tile_lds(const unsigned char* __restrict
           const int kk = key0 + 16 * sb + 4 * g + r;
           if (!(kk >= col_lo[q] && kk <= col_hi[q])) s[q][sb][r] = NEG_BIG;
         }
-        tile_max = fmaxf(tile_max, s[q][sb][r]);
+        lane_max[q] = fmaxf(lane_max[q], s[q][sb][r]);
       }
-    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, 64));
-    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, 64));
-    tile_max = (!masked || tile_max > 0.5f * NEG_BIG) ? tile_max * scale_log2e : NEG_BIG;
-    const bool moves = tile_max > m[q] + RESCALE_STEP;
-    const float m_new = moves ? tile_max : m[q];
-    alpha[q] = moves ? fast_exp2(m[q] - m_new) : 1.f;
-    rescale = rescale || moves;
-    float psum = 0.f;
-#pragma unroll
-    for (int sb = 0; sb < 2; ++sb) {
-      float e[4];
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        // a masked score stays at NEG_BIG: its weight is zero even while m_new is still NEG_BIG
-        e[r] = (!masked || s[q][sb][r] > 0.5f * NEG_BIG) ? fast_exp2(fmaf(s[q][sb][r], scale_log2e, -m_new)) : 0.f;
-        psum += e[r];
-      }
-      p[q].w[2 * sb] = pack2_bf16(e[0], e[1]);
-      p[q].w[2 * sb + 1] = pack2_bf16(e[2], e[3]);
-    }
-    l[q] = l[q] * alpha[q] + psum;
-    m[q] = m_new;
+    lane_max[q] = (!masked || lane_max[q] > 0.5f * NEG_BIG) ? lane_max[q] * scale_log2e : NEG_BIG;
+    exceeds = exceeds || lane_max[q] > m[q] + RESCALE_STEP;
   }
-  if (__any(rescale)) {
+  float alpha[NG];
 #pragma unroll
-    for (int q = 0; q < NG; ++q)
+  for (int q = 0; q < NG; ++q) alpha[q] = 1.f;
+  if (__any(exceeds)) {
+    // the columns' maxima (a column's keys lie in four lanes), new reference values where a maximum
+    // is more than RESCALE_STEP above the old one, and the output so far brought to the new values
+#pragma unroll
+    for (int q = 0; q < NG; ++q) {
+      float tile_max = lane_max[q];
+      tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, 64));
+      tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, 64));
+      const bool moves = tile_max > m[q] + RESCALE_STEP;
+      const float m_new = moves ? tile_max : m[q];
+      alpha[q] = moves ? fast_exp2(m[q] - m_new) : 1.f;
+      m[q] = m_new;
 #pragma unroll
       for (int n = 0; n < 2 * NQK; ++n)
 #pragma unroll
@@ -596,6 +589,26 @@ __device__ __forceinline__ void process_tile_lds(const unsigned char* __restrict
 #endif
           acc[q][n][r] = o;
         }
+    }
+  }
+  Pack8 p[NG];
+#pragma unroll
+  for (int q = 0; q < NG; ++q) {
+    // the scale of the scores rides along in the multiply-add that subtracts the reference value
+    float psum = 0.f;
+#pragma unroll
+    for (int sb = 0; sb < 2; ++sb) {
+      float e[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        // a masked score stays at NEG_BIG: its weight is zero even while the reference is still NEG_BIG
+        e[r] = (!masked || s[q][sb][r] > 0.5f * NEG_BIG) ? fast_exp2(fmaf(s[q][sb][r], scale_log2e, -m[q])) : 0.f;
+        psum += e[r];
+      }
+      p[q].w[2 * sb] = pack2_bf16(e[0], e[1]);
+      p[q].w[2 * sb + 1] = pack2_bf16(e[2], e[3]);
+    }
+    l[q] = l[q] * alpha[q] + psum;
   }
 #pragma unroll
   for (int n = 0; n < 2 * NQK; ++n) {
