@@ -35,6 +35,12 @@ union Pack8 {
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// acc + both bfloat16 halves of w (v_dot2c_f32_bf16 with a pair of ones)
+__device__ __forceinline__ float add_pair_bf16(uint32_t w, float acc) {
+  typedef __attribute__((ext_vector_type(2))) __bf16 pair_t;
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(pair_t, w), __builtin_bit_cast(pair_t, 0x3f803f80u), acc, false);
+}
+
 // One 32-key tile of a request's cache in registers: the operands of both products.
 template <int NQK>
 struct KVTile {
@@ -595,7 +601,7 @@ __device__ __forceinline__ void process_tile_lds(const unsigned char* __restrict
 #pragma unroll
   for (int q = 0; q < NG; ++q) {
     // the scale of the scores rides along in the multiply-add that subtracts the reference value
-    float psum = 0.f;
+    float psum = l[q] * alpha[q];
 #pragma unroll
     for (int sb = 0; sb < 2; ++sb) {
       float e[4];
@@ -603,12 +609,14 @@ __device__ __forceinline__ void process_tile_lds(const unsigned char* __restrict
       for (int r = 0; r < 4; ++r) {
         // a masked score stays at NEG_BIG: its weight is zero even while the reference is still NEG_BIG
         e[r] = (!masked || s[q][sb][r] > 0.5f * NEG_BIG) ? fast_exp2(fmaf(s[q][sb][r], scale_log2e, -m[q])) : 0.f;
-        psum += e[r];
       }
       p[q].w[2 * sb] = pack2_bf16(e[0], e[1]);
       p[q].w[2 * sb + 1] = pack2_bf16(e[2], e[3]);
+      // the sum takes the rounded weights, the ones that multiply the values, two per instruction
+      psum = add_pair_bf16(p[q].w[2 * sb], psum);
+      psum = add_pair_bf16(p[q].w[2 * sb + 1], psum);
     }
-    l[q] = l[q] * alpha[q] + psum;
+    l[q] = psum;
   }
 #pragma unroll
   for (int n = 0; n < 2 * NQK; ++n) {
