@@ -307,7 +307,10 @@ def test_attention_on_the_matrix_cores(ops, case):
             for f in range(0, n, ops.PREFILL_TILE):
                 tiles += [t0 + f, min(ops.PREFILL_TILE, n - f)]
         t0 += n
-    for splits, waves in ((0, 0), (1, 4), (1, 8), (2, 8), (3, 4), (7, 8), (1, 1), (2, 1)):
+    # prompt tiles: two halves of a block sharing the keys, one block taking all, and the chooser with
+    # figures that send it either way
+    halves = ((0, {}), (1, {}), (2, {}), (0, dict(keys_total=10 ** 9, keys_max=1)), (0, dict(keys_total=1, keys_max=10 ** 6)))
+    for i, (splits, waves) in enumerate(((0, 0), (1, 4), (1, 8), (2, 8), (3, 4), (7, 8), (1, 1), (2, 1))):
         out = torch.full((q.shape[0], nq * hd), float("nan"), dtype=dtype, device=DEV)
         if dec:
             ops.attention_decode_mfma(q, out, k_pool, v_pool, torch.tensor(dec, dtype=torch.int32, device=DEV),
@@ -315,10 +318,11 @@ def test_attention_on_the_matrix_cores(ops, case):
                                       splits=splits, waves=waves)
         if tiles:
             ops.attention_prefill_mfma(q, out, k_pool, v_pool, torch.tensor(tiles, dtype=torch.int32, device=DEV),
-                                       len(tiles) // 2, positions, entry, bt, P, nq, nkv, hd, scale, window)
+                                       len(tiles) // 2, positions, entry, bt, P, nq, nkv, hd, scale, window,
+                                       halves=halves[i % len(halves)][0], **halves[i % len(halves)][1])
         assert not torch.isnan(out).any()
-        assert (out.float().cpu() - want).abs().max() <= tol(dtype, want), (splits, waves)
-        if not dec:
+        assert (out.float().cpu() - want).abs().max() <= tol(dtype, want), (splits, waves, halves[i % len(halves)])
+        if not dec and i + 1 >= len(halves):
             break
 
 

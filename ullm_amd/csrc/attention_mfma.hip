@@ -859,22 +859,68 @@ extern "C" int ullm_attention_decode(
   ULLM_LAUNCH_CHECK();
 }
 
+template <int N, typename... Args>
+static void prefill_launch(int halves, unsigned blocks, hipStream_t stream, Args... args) {
+  if constexpr (N <= 4) {
+    if (halves == 2) {
+      hipLaunchKernelGGL((attention_prefill_kernel<N, 2>), dim3(blocks), dim3(64 * PREFILL_WAVES * 2), 0, stream, args...);
+      return;
+    }
+  }
+  hipLaunchKernelGGL((attention_prefill_kernel<N, 1>), dim3(blocks), dim3(64 * PREFILL_WAVES), 0, stream, args...);
+}
+
+// Compute units of the current device (asked once per device).
+static int compute_units() {
+  static int units[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (units[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    units[dev] = n;
+  }
+  return units[dev];
+}
+
+// `halves`: 2 = a block's eight waves share the keys of a tile between two halves (blocks last half as
+// long, one block per compute unit: best when a few long tiles would otherwise set the time);
+// 1 = four waves per block take all keys (two independent blocks per compute unit, which drift apart
+// so that one block's products overlap the other's exponentials: best when there is enough work to
+// keep every unit busy to the end); 0 = choose.  The choice compares the work per unit,
+// `keys_total` (sum over the tiles of the keys each sees) spread over two blocks per unit, with the
+// longest tile `keys_max`; without these figures (0) it goes by the number of blocks.
 extern "C" int ullm_attention_prefill(
     const void* q, int q_stride, void* out, int out_stride, const void* k_pool, const void* v_pool,
     const int* tiles, int n_tiles, const int* positions, const int* token_entry, const int* block_table,
-    int bt_stride, int page_size, int nq, int nkv, int hd, float scale, int window, hipStream_t stream) {
+    int bt_stride, int page_size, int nq, int nkv, int hd, float scale, int window, int halves,
+    long long keys_total, int keys_max, hipStream_t stream) {
   if (n_tiles <= 0) return 0;
   if (!ullm_attention_mfma_supports(hd, page_size, nq, nkv)) return ULLM_ERR_UNSUPPORTED;
-  if (window < 0) return ULLM_ERR_SHAPE;
+  if (window < 0 || halves < 0 || halves > 2) return ULLM_ERR_SHAPE;
   const int chunks = (nq / nkv + PREFILL_WAVES - 1) / PREFILL_WAVES;
-  if ((long long)n_tiles * nkv * chunks > 0x7fffffffLL) return ULLM_ERR_SHAPE;
+  const long long blocks = (long long)n_tiles * nkv * chunks;
+  if (blocks > 0x7fffffffLL) return ULLM_ERR_SHAPE;
   if ((long long)nkv * page_size * hd > 0x7fffffffLL) return ULLM_ERR_SHAPE;   // 32-bit distance between pages
+  if (hd > 128) halves = 1;                              // shared memory holds one half's tiles only
+  if (halves == 0) {
+    const long long units = compute_units();
+    bool enough;
+    if (keys_total > 0 && keys_max > 0) {
+      if (window > 0) {
+        if (keys_max > window + 32) keys_max = window + 32;
+        if (keys_total > (long long)n_tiles * (window + 32)) keys_total = (long long)n_tiles * (window + 32);
+      }
+      enough = (double)keys_total * nkv * chunks / (2.0 * units) >= 0.6 * keys_max;
+    } else {
+      enough = blocks >= 3 * units;
+    }
+    halves = (enough && blocks >= 2 * units) ? 1 : 2;
+  }
   const float sl = scale * 1.4426950408889634f;
-  // keys split over two halves of a block where LDS allows it
-#define CALL(N) do { constexpr int KS = N <= 4 ? 2 : 1;                                                        \
-    hipLaunchKernelGGL((attention_prefill_kernel<N, KS>), dim3(n_tiles * nkv * chunks), dim3(64 * PREFILL_WAVES * KS), \
-    0, stream, (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool,  \
-    tiles, positions, token_entry, block_table, bt_stride, page_size, nq, nkv, sl, window, n_tiles); } while (0)
+#define CALL(N) prefill_launch<N>(halves, (unsigned)blocks, stream, (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, \
+    (const bf16_t*)k_pool, (const bf16_t*)v_pool, tiles, positions, token_entry, block_table, bt_stride, page_size,    \
+    nq, nkv, sl, window, n_tiles)
   DISPATCH_NQK(hd, CALL)
 #undef CALL
   ULLM_LAUNCH_CHECK();

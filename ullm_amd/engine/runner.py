@@ -203,7 +203,8 @@ class ModelRunner:
         host[offs[7 + ng]:offs[8 + ng]] = dec_list
         host[offs[8 + ng]:offs[9 + ng]] = tile_list
         facts = dict(T=T, B=B, strides=strides, n_want=n_want, num_decode=len(dec_list), max_dec_kv=max_dec_kv,
-                     num_tiles=len(tile_list) // 2, max_q=max(lens), max_kv=max_kv,
+                     num_tiles=len(tile_list) // 2, tile_keys_total=sum(k for k, _, _ in tile_keys),
+                     tile_keys_max=tile_keys[-1][0] if tile_keys else 0, max_q=max(lens), max_kv=max_kv,
                      decode_only=all(n == 1 for n in lens), lens=lens + [1] * n_pad,
                      starts=starts + [0] * n_pad, slots=slots + [0] * n_pad, unknown=unknown)
         return host, offs, facts
@@ -223,7 +224,8 @@ class ModelRunner:
             dtype=self.env.dtype,
             decode_tokens=view(7 + ng) if facts["num_decode"] else None, num_decode=facts["num_decode"],
             max_decode_kv=facts["max_dec_kv"], tiles=view(8 + ng).view(-1, 2) if facts["num_tiles"] else None,
-            num_tiles=facts["num_tiles"],
+            num_tiles=facts["num_tiles"], tile_keys_total=facts["tile_keys_total"],
+            tile_keys_max=facts["tile_keys_max"],
             host={"lens": facts["lens"], "starts": facts["starts"], "slots": facts["slots"]})
         return ctx, (view(6) if facts["n_want"] else None)
 

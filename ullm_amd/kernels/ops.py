@@ -370,9 +370,12 @@ PREFILL_TILE = 32      # tokens of one request per prompt tile (two groups of 16
 
 def attention_prefill_mfma(q, out, k_pool, v_pool, tiles: torch.Tensor, n_tiles: int, positions, token_entry,
                            block_table, page_size: int, nq: int, nkv: int, hd: int, scale: float,
-                           window: int) -> None:
+                           window: int, halves: int = 0, keys_total: int = 0, keys_max: int = 0) -> None:
     """Tiles (first token, count <= PREFILL_TILE) of consecutive tokens of one request each, every
-    token against the keys up to its own position."""
+    token against the keys up to its own position.  ``halves``: 2 = two halves of a block share a
+    tile's keys, 1 = one block takes them all, 0 = chosen from ``keys_total`` (the sum over the tiles of
+    the keys each sees) and ``keys_max`` (the most any tile sees), or from the number of tiles if
+    these are 0.  Every choice computes the same function."""
     _check_pools(k_pool, v_pool, nkv, page_size, hd, torch.bfloat16)
     _need(q.dtype == torch.bfloat16 and q.stride(1) == 1 and q.shape[1] == nq * hd, "q must be bfloat16 [T, nq*hd]")
     _need(out.dtype == torch.bfloat16 and out.stride(1) == 1 and out.shape == q.shape, "bad attention output")
@@ -385,7 +388,8 @@ def attention_prefill_mfma(q, out, k_pool, v_pool, tiles: torch.Tensor, n_tiles:
     _check(lib.ullm_attention_prefill(
         _p(q), _c_int(q.stride(0)), _p(out), _c_int(out.stride(0)), _p(k_pool), _p(v_pool), _p(tiles),
         _c_int(n_tiles), _p(positions), _p(token_entry), _p(block_table), _c_int(block_table.stride(0)),
-        _c_int(page_size), _c_int(nq), _c_int(nkv), _c_int(hd), _c_float(scale), _c_int(window), _stream()),
+        _c_int(page_size), _c_int(nq), _c_int(nkv), _c_int(hd), _c_float(scale), _c_int(window),
+        _c_int(halves), ctypes.c_longlong(int(keys_total)), _c_int(keys_max), _stream()),
         "attention_prefill")
 
 
@@ -405,7 +409,8 @@ def paged_attention(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
                               ctx.max_decode_kv)
     if ctx.num_tiles:
         attention_prefill_mfma(q, out, k_pool, v_pool, ctx.tiles, ctx.num_tiles, ctx.positions, ctx.token_entry,
-                               group.block_table, group.page_size, nq, nkv, hd, scale, window)
+                               group.block_table, group.page_size, nq, nkv, hd, scale, window,
+                               keys_total=ctx.tile_keys_total, keys_max=ctx.tile_keys_max)
     return out
 
 

@@ -92,6 +92,8 @@ class StepContext:
     max_decode_kv: int = 0
     tiles: Optional[torch.Tensor] = None           # int32 [n_tiles, 2]
     num_tiles: int = 0
+    tile_keys_total: int = 0      # sum over the tiles of the keys each tile's last token sees
+    tile_keys_max: int = 0        # the most keys any tile sees (both: how the tiles' work is spread)
 
 
 # --------------------------------------------------------------------------- parts
