@@ -528,16 +528,19 @@ __device__ __forceinline__ void stage_store(const PrefillStage<NQK>& st, int key
 
 // Scores, softmax update and value product of one wave for the tile in LDS.  `masked` = some key of
 // the tile is hidden from some column (diagonal, window or end of data); otherwise no per-score test.
+// The queries come multiplied by scale * log2(e), and the first product of a score starts from minus
+// the column's reference value (`negm`, the same in all four elements) instead of zero, so the
+// products deliver the exponent itself: exp2 of it is the weight.  A column without a reference
+// value yet (m == NEG_BIG) counts from zero, and the first tile that shows it a key gives it one.
 template <int NQK, int NG, bool masked>
 __device__ __forceinline__ void process_tile_lds(const unsigned char* __restrict__ kl, const unsigned char* __restrict__ vl,
                                                  int key0, const Pack8 (&qreg)[NG][NQK],
-                                                 const int (&col_lo)[NG], const int (&col_hi)[NG], float scale_log2e,
-                                                 f32x4_t (&acc)[NG][2 * NQK], float (&m)[NG], float (&l)[NG]) {
+                                                 const int (&col_lo)[NG], const int (&col_hi)[NG],
+                                                 f32x4_t (&acc)[NG][2 * NQK], float (&m)[NG], f32x4_t (&negm)[NG],
+                                                 float (&l)[NG]) {
   using S = PrefillStage<NQK>;
   const int lane = threadIdx.x & 63, g = lane >> 4, c = lane & 15;
   f32x4_t s[NG][2];
-#pragma unroll
-  for (int q = 0; q < NG; ++q) s[q][0] = s[q][1] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int sb = 0; sb < 2; ++sb)
 #pragma unroll
@@ -546,17 +549,17 @@ __device__ __forceinline__ void process_tile_lds(const unsigned char* __restrict
       kf.u4 = *reinterpret_cast<const uint4*>(kl + (16 * sb + c) * S::KROW + 64 * ch + 16 * g);
 #pragma unroll
       for (int q = 0; q < NG; ++q)
-        s[q][sb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qreg[q][ch].v, s[q][sb], 0, 0, 0);
+        s[q][sb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qreg[q][ch].v, ch == 0 ? negm[q] : s[q][sb], 0, 0, 0);
     }
-  // Does any score of the tile exceed its column's reference value by more than RESCALE_STEP?  Each
-  // lane looks at its own scores only (the maximum is taken over the raw products, the scale is
-  // positive); the wave votes.  Most tiles pass, and then no value crosses lanes and nothing is
-  // rescaled.
-  float lane_max[NG];
+  // Does any exponent exceed RESCALE_STEP, or does a column meet its first key?  Each lane looks at
+  // its own scores only and the wave votes.  Most tiles pass, and then no value crosses lanes and
+  // nothing is rescaled.
+  float lane_max[NG], alpha[NG];
   bool exceeds = false;
 #pragma unroll
   for (int q = 0; q < NG; ++q) {
     lane_max[q] = NEG_BIG;
+    alpha[q] = 1.f;
 #pragma unroll
     for (int sb = 0; sb < 2; ++sb)
 #pragma unroll
@@ -567,24 +570,29 @@ __device__ __forceinline__ void process_tile_lds(const unsigned char* __restrict
         }
         lane_max[q] = fmaxf(lane_max[q], s[q][sb][r]);
       }
-    lane_max[q] = (!masked || lane_max[q] > 0.5f * NEG_BIG) ? lane_max[q] * scale_log2e : NEG_BIG;
-    exceeds = exceeds || lane_max[q] > m[q] + RESCALE_STEP;
+    const bool sees = !masked || lane_max[q] > 0.5f * NEG_BIG;
+    exceeds = exceeds || (sees && (lane_max[q] > RESCALE_STEP || m[q] < 0.5f * NEG_BIG));
   }
-  float alpha[NG];
-#pragma unroll
-  for (int q = 0; q < NG; ++q) alpha[q] = 1.f;
   if (__any(exceeds)) {
-    // the columns' maxima (a column's keys lie in four lanes), new reference values where a maximum
-    // is more than RESCALE_STEP above the old one, and the output so far brought to the new values
+    // the columns' maxima (a column's keys lie in four lanes); where one is more than RESCALE_STEP
+    // above the reference value, or there was none, it becomes the new one: the exponents and the
+    // output so far are brought to it
 #pragma unroll
     for (int q = 0; q < NG; ++q) {
-      float tile_max = lane_max[q];
-      tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, 64));
-      tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, 64));
-      const bool moves = tile_max > m[q] + RESCALE_STEP;
-      const float m_new = moves ? tile_max : m[q];
-      alpha[q] = moves ? fast_exp2(m[q] - m_new) : 1.f;
-      m[q] = m_new;
+      float col_max = lane_max[q];
+      col_max = fmaxf(col_max, __shfl_xor(col_max, 16, 64));
+      col_max = fmaxf(col_max, __shfl_xor(col_max, 32, 64));
+      const bool had = m[q] > 0.5f * NEG_BIG;
+      const bool moves = col_max > 0.5f * NEG_BIG && (!had || col_max > RESCALE_STEP);
+      if (moves) {
+        m[q] = (had ? m[q] : 0.f) + col_max;
+        negm[q] = f32x4_t{-m[q], -m[q], -m[q], -m[q]};
+        if (had) alpha[q] = fast_exp2(-col_max);
+#pragma unroll
+        for (int sb = 0; sb < 2; ++sb)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) s[q][sb][r] -= col_max;     // a hidden score stays far below
+      }
 #pragma unroll
       for (int n = 0; n < 2 * NQK; ++n)
 #pragma unroll
@@ -600,16 +608,13 @@ __device__ __forceinline__ void process_tile_lds(const unsigned char* __restrict
   Pack8 p[NG];
 #pragma unroll
   for (int q = 0; q < NG; ++q) {
-    // the scale of the scores rides along in the multiply-add that subtracts the reference value
     float psum = l[q] * alpha[q];
 #pragma unroll
     for (int sb = 0; sb < 2; ++sb) {
       float e[4];
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        // a masked score stays at NEG_BIG: its weight is zero even while the reference is still NEG_BIG
-        e[r] = (!masked || s[q][sb][r] > 0.5f * NEG_BIG) ? fast_exp2(fmaf(s[q][sb][r], scale_log2e, -m[q])) : 0.f;
-      }
+      for (int r = 0; r < 4; ++r)
+        e[r] = (!masked || s[q][sb][r] > 0.5f * NEG_BIG) ? fast_exp2(s[q][sb][r]) : 0.f;
       p[q].w[2 * sb] = pack2_bf16(e[0], e[1]);
       p[q].w[2 * sb + 1] = pack2_bf16(e[2], e[3]);
       // the sum takes the rounded weights, the ones that multiply the values, two per instruction
@@ -680,6 +685,13 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __r
     for (int ch = 0; ch < NQK; ++ch) {
       if (ok) qreg[qg][ch].u4 = *reinterpret_cast<const uint4*>(qp + 32 * ch);
       else qreg[qg][ch].u4 = make_uint4(0, 0, 0, 0);
+      // scale * log2(e) goes into the queries once, so that a score is its weight's exponent
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        const uint32_t two = qreg[qg][ch].w[w];
+        qreg[qg][ch].w[w] = pack2_bf16(__uint_as_float(two << 16) * scale_log2e,
+                                       __uint_as_float(two & 0xffff0000u) * scale_log2e);
+      }
     }
   }
   const int last_pos = positions[first + count - 1];
@@ -695,11 +707,13 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __r
   const int* bt = block_table + (size_t)token_entry[first] * bt_stride;
   f32x4_t acc[NG][2 * NQK];
   float m[NG], l[NG];
+  f32x4_t negm[NG];                                       // minus the reference value, 0 while there is none
 #pragma unroll
   for (int qg = 0; qg < NG; ++qg) {
 #pragma unroll
     for (int n = 0; n < 2 * NQK; ++n) acc[qg][n] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     m[qg] = NEG_BIG;
+    negm[qg] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     l[qg] = 0.f;
   }
   // the page window serves the loads, which run ahead of the products
@@ -730,9 +744,9 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __r
   do {                                                                             \
     const unsigned char* kl = tile_lds + (BUF) * TILE_BYTES;                       \
     if ((K0) + 31 > first_pos || (K0) < open_lo)                                   \
-      process_tile_lds<NQK, NG, true>(kl, kl + S::KBYTES, (K0), qreg, clo, chi, scale_log2e, acc, m, l);  \
+      process_tile_lds<NQK, NG, true>(kl, kl + S::KBYTES, (K0), qreg, clo, chi, acc, m, negm, l);  \
     else                                                                           \
-      process_tile_lds<NQK, NG, false>(kl, kl + S::KBYTES, (K0), qreg, clo, chi, scale_log2e, acc, m, l); \
+      process_tile_lds<NQK, NG, false>(kl, kl + S::KBYTES, (K0), qreg, clo, chi, acc, m, negm, l); \
     STAGE_STORE(NEXT, (K0) + 32, 1 - (BUF));                                       \
     STAGE_LOAD(NEXT, (K0) + 96);                                                   \
     __syncthreads();                                                               \
