@@ -143,6 +143,59 @@ def test_qk_norm_rope_write(ops, dtype, cfg):
     assert int((k_pool.float().abs().sum(-1) > 0).sum()) == written * nkv       # nothing else was touched
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("cfg", [dict(nq=8, nkv=2, hd=128, P=16), dict(nq=4, nkv=4, hd=64, P=8),
+                                 dict(nq=2, nkv=1, hd=256, P=32), dict(nq=4, nkv=2, hd=32, P=24),
+                                 dict(nq=4, nkv=2, hd=64, P=12),      # pages that do not hold whole groups of 8
+                                 dict(nq=2, nkv=2, hd=512, P=16)])    # too wide for the blocks that write runs
+def test_cache_write_of_many_tokens(ops, dtype, cfg):
+    """With many tokens in the batch the values are written in runs of eight positions: portions that
+    start at odd positions, at 0, single tokens between them, an entry without pages, and a
+    portion that ends in the middle of a group all land where the token-by-token write puts them."""
+    torch.manual_seed(14)
+    nq, nkv, hd, P = (cfg[k] for k in ("nq", "nkv", "hd", "P"))
+    # (entry, first position, tokens); entry 3 has no pages (a padding entry of a captured batch)
+    portions = [(0, 77, 1), (1, 5, 146), (2, 0, 100), (3, 9, 1), (4, 300, 1), (5, 64, 43), (3, 10, 1), (6, 8, 8)]
+    positions = torch.cat([torch.arange(f, f + n) for _, f, n in portions]).int()
+    entry = torch.cat([torch.full((n,), e) for e, _, n in portions]).int()
+    T = positions.numel()
+    assert T >= 128
+    last = {}
+    for e, f, n in portions:
+        last[e] = max(last.get(e, 0), f + n - 1)
+    need = {e: (0 if e == 3 else last[e] // P + 1) for e in last}
+    ids = torch.randperm(sum(need.values()) + 3).tolist()
+    tables, at = [], 0
+    for e in range(7):
+        tables.append(ids[at:at + need[e]])
+        at += need[e]
+    n_pages = len(ids)
+    width = max(len(t) for t in tables)
+    bt = torch.full((7, width), -1, dtype=torch.int32)
+    for e, t in enumerate(tables):
+        bt[e, :len(t)] = torch.tensor(t, dtype=torch.int32)
+    bt = bt.to(DEV)
+    qkv = torch.randn(T, (nq + 2 * nkv) * hd).to(dtype)
+    k_pool = torch.zeros(n_pages, nkv, P, hd, dtype=dtype, device=DEV)
+    v_pool = torch.zeros(n_pages, nkv, hd, P, dtype=dtype, device=DEV)
+    q_out = torch.empty(T, nq * hd, dtype=dtype, device=DEV)
+    ops.qk_norm_rope_write(qkv.to(DEV), q_out, None, None, 1e-6, None, 0, 0, positions.to(DEV), entry.to(DEV), bt,
+                           k_pool, v_pool, P, nq, nkv, hd, write_kv=True)
+    x = qkv.float()
+    k, v = x[:, nq * hd:(nq + nkv) * hd].view(T, nkv, hd), x[:, (nq + nkv) * hd:].view(T, nkv, hd)
+    assert torch.equal(q_out.float().cpu(), x[:, :nq * hd])
+    want_k = torch.zeros(n_pages, nkv, P, hd)
+    want_v = torch.zeros(n_pages, nkv, hd, P)
+    for t in range(T):
+        pos, e = int(positions[t]), int(entry[t])
+        if e == 3:
+            continue
+        want_k[tables[e][pos // P], :, pos % P] = k[t]
+        want_v[tables[e][pos // P], :, :, pos % P] = v[t]
+    assert torch.equal(k_pool.float().cpu(), want_k)
+    assert torch.equal(v_pool.float().cpu(), want_v)
+
+
 def reference_attention(qs, ks, vs, scale, window):
     """qs[b]: [n_b, nq, hd] queries at the last n_b positions of sequence b (ks[b]: [S_b, nkv, hd])."""
     outs = []

@@ -298,6 +298,69 @@ __global__ void qk_norm_rope_write_kernel(
   for (int i = rot + lane; i < hd; i += WAVE) st_f32(dst + i, vals[i]);
 }
 
+// Values of many tokens at once: a block takes VALUE_RUN_TOKENS consecutive tokens of the batch and one
+// kv head, gathers their value rows in LDS and writes them transposed.  Eight tokens of one request at
+// positions 8k .. 8k+7 lie side by side in one row of a page (page sizes that are multiples of 8), so a
+// thread writes them as one 16-byte (bfloat16) or two 16-byte (float) stores per dim instead of eight
+// single elements; tokens that do not fill such a group are written one by one.
+#define VALUE_RUN_TOKENS 16
+#define VALUE_RUN_MAX_HD 256
+template <typename T>
+__device__ __forceinline__ void value_runs_block(
+    const T* __restrict__ qkv, int qkv_stride, const int* __restrict__ positions, const int* __restrict__ token_entry,
+    const int* __restrict__ block_table, int bt_stride, T* __restrict__ v_pool, int page_size, int nq, int nkv,
+    int hd, int n_tokens, int block) {
+  __shared__ __attribute__((aligned(16))) T tile[VALUE_RUN_TOKENS * VALUE_RUN_MAX_HD];
+  __shared__ int s_page[VALUE_RUN_TOKENS], s_off[VALUE_RUN_TOKENS], s_run[VALUE_RUN_TOKENS];
+  const int kvh = block % nkv, tok0 = (block / nkv) * VALUE_RUN_TOKENS;
+  const int n = n_tokens - tok0 < VALUE_RUN_TOKENS ? n_tokens - tok0 : VALUE_RUN_TOKENS;
+  constexpr int PER16 = 16 / (int)sizeof(T);                // elements per 16-byte piece
+  const int pieces = hd / PER16;
+  for (int c = threadIdx.x; c < n * pieces; c += blockDim.x) {
+    const int tok = c / pieces, part = c % pieces;
+    *reinterpret_cast<uint4*>(tile + tok * hd + part * PER16) = *reinterpret_cast<const uint4*>(
+        qkv + (size_t)(tok0 + tok) * qkv_stride + (size_t)(nq + nkv + kvh) * hd + part * PER16);
+  }
+  if ((int)threadIdx.x < n) {
+    // a token leads a run if it is the block's first or does not continue its predecessor's group of 8
+    const int i = threadIdx.x, t = tok0 + i;
+    const int pos = positions[t], ent = token_entry[t];
+    s_page[i] = block_table[(size_t)ent * bt_stride + pos / page_size];
+    s_off[i] = pos % page_size;
+    const bool leads = i == 0 || token_entry[t - 1] != ent || positions[t - 1] != pos - 1 || (pos & 7) == 0;
+    int run = 0;
+    if (leads) {
+      run = 1;
+      while (i + run < n && token_entry[t + run] == ent && positions[t + run] == pos + run && ((pos + run) & 7) != 0) ++run;
+    }
+    s_run[i] = run;
+  }
+  __syncthreads();
+  // item = (dim, half of the block's tokens)
+  for (int item = threadIdx.x; item < 2 * hd; item += blockDim.x) {
+    const int d = item % hd, first = (item / hd) * (VALUE_RUN_TOKENS / 2);
+    for (int i = first; i < first + VALUE_RUN_TOKENS / 2 && i < n; ++i) {
+      const int run = s_run[i];
+      if (run == 0 || s_page[i] < 0) continue;
+      T* dst = v_pool + (((size_t)s_page[i] * nkv + kvh) * hd + d) * page_size + s_off[i];
+      if (run == 8 && (s_off[i] & 7) == 0) {                // one row of one page, aligned
+        __attribute__((aligned(16))) T eight[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) eight[j] = tile[(i + j) * hd + d];
+#pragma unroll
+        for (int j = 0; j < 8 / PER16; ++j)
+          reinterpret_cast<uint4*>(dst)[j] = reinterpret_cast<const uint4*>(eight)[j];
+      } else {
+        // the run's tokens follow each other in the page as long as the page does not end
+        for (int j = 0; j < run; ++j) {
+          if (s_page[i + j] < 0) continue;
+          v_pool[(((size_t)s_page[i + j] * nkv + kvh) * hd + d) * page_size + s_off[i + j]] = tile[(i + j) * hd + d];
+        }
+      }
+    }
+  }
+}
+
 // The same for head sizes of 8 * (a power of two): a head is held by head_dim / 8 neighbouring lanes
 // with 8 consecutive dims each (16-byte loads and stores for bfloat16), a block of 256 threads takes
 // 2048 / head_dim heads of one token.  For half-split pairs the partner dims come from the lane
@@ -310,10 +373,15 @@ qk_norm_rope_write_vec_kernel(
     const float* __restrict__ cos_sin, int table_rows, int rot, int style,
     const int* __restrict__ positions, const int* __restrict__ token_entry,
     const int* __restrict__ block_table, int bt_stride, T* __restrict__ k_pool, T* __restrict__ v_pool,
-    int page_size, int nq, int nkv, int hd, int write_kv) {
+    int page_size, int nq, int nkv, int hd, int write_kv, int n_tokens, int blocks_per_token) {
+  if (blockIdx.x >= (unsigned)(n_tokens * blocks_per_token)) {
+    value_runs_block<T>(qkv, qkv_stride, positions, token_entry, block_table, bt_stride, v_pool, page_size, nq, nkv,
+                        hd, n_tokens, (int)blockIdx.x - n_tokens * blocks_per_token);
+    return;
+  }
   const int lph = hd >> 3;                                  // lanes per head
-  const int t = blockIdx.x;
-  const int head = blockIdx.y * (256 / lph) + threadIdx.x / lph, part = threadIdx.x % lph, d0 = 8 * part;
+  const int t = blockIdx.x / blocks_per_token;
+  const int head = (blockIdx.x % blocks_per_token) * (256 / lph) + threadIdx.x / lph, part = threadIdx.x % lph, d0 = 8 * part;
   const bool live = head < nq + 2 * nkv;
   const int pos = positions[t];
   const bool is_q = head < nq, is_k = !is_q && head < nq + nkv;
@@ -324,7 +392,8 @@ qk_norm_rope_write_vec_kernel(
     x[0] = lo.x; x[1] = lo.y; x[2] = lo.z; x[3] = lo.w; x[4] = hi.x; x[5] = hi.y; x[6] = hi.z; x[7] = hi.w;
   }
   int page = -1;
-  if (live && !is_q && write_kv) page = block_table[(size_t)token_entry[t] * bt_stride + pos / page_size];
+  if (live && !is_q && (write_kv & (is_k ? 1 : 2)))
+    page = block_table[(size_t)token_entry[t] * bt_stride + pos / page_size];
   const int off = pos % page_size;
   if (live && !is_q && !is_k) {                             // v: transposed copy, no arithmetic
     if (page >= 0) {
@@ -411,11 +480,19 @@ extern "C" int ullm_qk_norm_rope_write(
                    (!k_gain || ((uintptr_t)k_gain & 15) == 0) && rot % 8 == 0;
   if (vec) {
     const int heads_per_block = 256 / lph;
-    dim3 vgrid(T_, (nq + 2 * nkv + heads_per_block - 1) / heads_per_block), vblock(256);
+    const int blocks_per_token = (nq + 2 * nkv + heads_per_block - 1) / heads_per_block;
+    // with many tokens the values go through blocks of their own that write runs of eight at once
+    const bool runs = write_kv && T_ >= 128 && page_size % 8 == 0 && hd <= VALUE_RUN_MAX_HD &&
+                      ((uintptr_t)v_pool & 15) == 0;
+    const long long value_blocks = runs ? (long long)((T_ + VALUE_RUN_TOKENS - 1) / VALUE_RUN_TOKENS) * nkv : 0;
+    const long long all_blocks = (long long)T_ * blocks_per_token + value_blocks;
+    if (all_blocks > 0x7fffffffLL) return ULLM_ERR_SHAPE;
+    const int kv_flags = !write_kv ? 0 : (runs ? 1 : 3);   // bit 0: keys, bit 1: values token by token
+    dim3 vgrid((unsigned)all_blocks), vblock(256);
 #define GOV(TT) hipLaunchKernelGGL(qk_norm_rope_write_vec_kernel<TT>, vgrid, vblock, 0, stream, \
     (const TT*)qkv, qkv_stride, (TT*)q_out, q_out_stride, q_gain, k_gain, eps, cos_sin, table_rows, \
     rot, style, positions, token_entry, block_table, bt_stride, (TT*)k_pool, (TT*)v_pool, page_size, \
-    nq, nkv, hd, write_kv)
+    nq, nkv, hd, kv_flags, T_, blocks_per_token)
     if (dtype == ULLM_F32) GOV(float);
     else if (dtype == ULLM_BF16) GOV(bf16_t);
     else return ULLM_ERR_DTYPE;
