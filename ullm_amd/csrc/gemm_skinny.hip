@@ -35,6 +35,65 @@ enum { EPI_STORE = 0, EPI_RESADD = 1, EPI_SILU = 2 };
 // most waves per block for a tile shape: bounded by the shared memory that holds the waves' partials
 __host__ __device__ constexpr int sk_max_waves(int mt, int nt) { return mt * nt >= 8 ? 4 : (mt * nt >= 4 ? 8 : 16); }
 
+// The waves' partial results of a block are added in wave order through `red` and the sum goes where
+// EPI says.  acc[i][t][j] = partial C[m = 16 t + r][n0 + 16 i + 4 g + j].
+template <int MT, int NT, int EPI, typename TC, typename RedT>
+__device__ __forceinline__ void skinny_finish(f32x4_t (&acc)[NT][MT], RedT& red, const float* __restrict__ bias,
+                                              TC* __restrict__ C, float* __restrict__ R, int ldc, int M, int N, int n0) {
+  constexpr int OT = EPI == EPI_SILU ? NT / 2 : NT;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+  const int g = lane >> 4, r = lane & 15;
+  if (nwaves > 1) {
+    if (wave != 0) {
+#pragma unroll
+      for (int i = 0; i < NT; ++i)
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+          *reinterpret_cast<float4*>(&red[wave - 1][i * MT + t][lane * 4]) =
+              make_float4(acc[i][t][0], acc[i][t][1], acc[i][t][2], acc[i][t][3]);
+    }
+    __syncthreads();
+    if (wave != 0) return;
+#pragma unroll
+    for (int i = 0; i < NT; ++i)
+#pragma unroll
+      for (int t = 0; t < MT; ++t)
+        for (int w = 1; w < nwaves; ++w) {
+          const float4 o = *reinterpret_cast<const float4*>(&red[w - 1][i * MT + t][lane * 4]);
+          acc[i][t][0] += o.x; acc[i][t][1] += o.y; acc[i][t][2] += o.z; acc[i][t][3] += o.w;
+        }
+  }
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    const int m = 16 * t + r;
+    if (m >= M) continue;
+#pragma unroll
+    for (int i = 0; i < OT; ++i) {
+      const int nn = n0 + 16 * i + 4 * g;
+      if (EPI == EPI_SILU) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          if (nn + j < N) st_f32(C + (size_t)m * ldc + nn + j, fast_silu(acc[i][t][j]) * acc[i + OT][t][j]);
+      } else if (EPI == EPI_RESADD) {
+        float* rp = R + (size_t)m * ldc + nn;
+        if (nn + 3 < N) {
+          float4 o = *reinterpret_cast<float4*>(rp);
+          o.x += acc[i][t][0]; o.y += acc[i][t][1]; o.z += acc[i][t][2]; o.w += acc[i][t][3];
+          *reinterpret_cast<float4*>(rp) = o;
+        } else {
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            if (nn + j < N) rp[j] += acc[i][t][j];
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          if (nn + j < N) st_f32(C + (size_t)m * ldc + nn + j, acc[i][t][j] + (bias ? bias[nn + j] : 0.f));
+      }
+    }
+  }
+}
+
 // MT = 16-row tiles of X (M <= 16 MT); NT = 16-row tiles of W per block.
 // With EPI_SILU the NT tiles of W are NT / 2 of the gate half followed by the same rows of the up half.
 template <int MT, int NT, int EPI, typename TC>
@@ -106,56 +165,116 @@ gemm_skinny_kernel(const bf16_t* __restrict__ X, int ldx, const bf16_t* __restri
       for (int t = 0; t < MT; ++t)
         acc[i][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[i].v, x[t].v, acc[i][t], 0, 0, 0);
   }
-  // acc[i][t][j] = partial C[m = 16 t + r][n0 + 16 i + 4 g + j]; add the waves' partials in wave order
-  if (nwaves > 1) {
-    if (wave != 0) {
+  skinny_finish<MT, NT, EPI, TC>(acc, red, bias, C, R, ldc, M, N, n0);
+}
+
+// The same product with the operands staged through shared memory.  In the kernel above a load
+// instruction of a wave fetches 64 bytes of each of 16 rows, and of X as many rows as the batch has:
+// half cache lines, and more of them per instruction the more rows X has, which is what its time
+// grows with.  Here a wave fetches whole 128-byte lines, 8 rows per instruction (lane = row l / 8,
+// 16-byte piece l % 8), two stages of 64 values of K ahead in registers, writes a stage to its own
+// part of shared memory and reads the operands from there in the layout the matrix instruction wants
+// (lane (r, g) holds row r, values 8 g .. +8 of a step of 32).  A row takes 128 bytes; piece c of row
+// r lies at piece c ^ ((r >> 1) & 7), which keeps both the 16-byte writes and the 16-byte reads of the
+// hardware's lane groups on different banks.  No barrier in the loop: a wave only reads what it wrote.
+template <int MT, int NT, int EPI, typename TC>
+__global__ void __launch_bounds__(64 * sk_max_waves(MT, NT))
+gemm_skinny_staged_kernel(const bf16_t* __restrict__ X, int ldx, const bf16_t* __restrict__ W, int ldw,
+                          const float* __restrict__ bias, TC* __restrict__ C, float* __restrict__ R, int ldc, int M,
+                          int N, int K, int k_per_wave) {
+  constexpr int MAXW = sk_max_waves(MT, NT);
+  constexpr int TILE_BYTES = 16 * 128, STAGE_BYTES = (NT + MT) * TILE_BYTES;
+  constexpr int RED_BYTES = (MAXW - 1) * NT * MT * 256 * 4;
+  constexpr int LDS_BYTES = MAXW * STAGE_BYTES > RED_BYTES ? MAXW * STAGE_BYTES : RED_BYTES;
+  __shared__ __attribute__((aligned(16))) unsigned char lds[LDS_BYTES];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int g = lane >> 4, r = lane & 15, lrow = lane >> 3, lcol = lane & 7;
+  constexpr int OT = EPI == EPI_SILU ? NT / 2 : NT;
+  const int n0 = blockIdx.x * (16 * OT);
+  const bf16_t* wsrc[NT][2];
+  const bf16_t* xsrc[MT][2];
+  int put[2], get[2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int row = 8 * h + lrow;
+    put[h] = row * 128 + ((lcol ^ ((row >> 1) & 7)) << 4);
+    get[h] = r * 128 + (((4 * h + g) ^ ((r >> 1) & 7)) << 4);      // h here: the step of 32 inside the stage
+#pragma unroll
+    for (int i = 0; i < NT; ++i) {
+      const int col = n0 + 16 * (i % OT) + row;
+      const int n = (col < N ? col : N - 1) + (i / OT) * N;       // rows past N repeat the last row; never stored
+      wsrc[i][h] = W + (size_t)n * ldw + 8 * lcol;
+    }
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      const int m = 16 * t + row < M ? 16 * t + row : M - 1;
+      xsrc[t][h] = X + (size_t)m * ldx + 8 * lcol;
+    }
+  }
+  unsigned char* const mine = lds + wave * STAGE_BYTES;
+  f32x4_t acc[NT][MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t)
+#pragma unroll
+    for (int i = 0; i < NT; ++i) acc[i][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  const int k_begin = wave * k_per_wave;
+  int k_end = k_begin + k_per_wave;
+  if (k_end > K) k_end = K;
+  struct Stage { uint4 w[NT][2], x[MT][2]; };
+  constexpr int DEPTH = 2;                                // stages of 64 values of K on their way (3 and 4 were slower)
+  Stage st[DEPTH];
+  auto fetch = [&](Stage& st, int k0) {
+    const bool in = k0 + 8 * lcol < k_end;                        // K is a multiple of 8
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+#pragma unroll
+      for (int i = 0; i < NT; ++i)
+        st.w[i][h] = in ? *reinterpret_cast<const uint4*>(wsrc[i][h] + k0) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+      for (int t = 0; t < MT; ++t)
+        st.x[t][h] = in ? *reinterpret_cast<const uint4*>(xsrc[t][h] + k0) : make_uint4(0, 0, 0, 0);
+    }
+  };
+  auto work = [&](const Stage& st) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+#pragma unroll
+      for (int i = 0; i < NT; ++i) *reinterpret_cast<uint4*>(mine + i * TILE_BYTES + put[h]) = st.w[i][h];
+#pragma unroll
+      for (int t = 0; t < MT; ++t) *reinterpret_cast<uint4*>(mine + (NT + t) * TILE_BYTES + put[h]) = st.x[t][h];
+    }
+    __builtin_amdgcn_wave_barrier();       // the wave's lanes read each other's pieces: writes stay before reads
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      Pack8 wf[NT], xf[MT];
+#pragma unroll
+      for (int i = 0; i < NT; ++i) wf[i].u4 = *reinterpret_cast<const uint4*>(mine + i * TILE_BYTES + get[j]);
+#pragma unroll
+      for (int t = 0; t < MT; ++t) xf[t].u4 = *reinterpret_cast<const uint4*>(mine + (NT + t) * TILE_BYTES + get[j]);
 #pragma unroll
       for (int i = 0; i < NT; ++i)
 #pragma unroll
         for (int t = 0; t < MT; ++t)
-          *reinterpret_cast<float4*>(&red[wave - 1][i * MT + t][lane * 4]) =
-              make_float4(acc[i][t][0], acc[i][t][1], acc[i][t][2], acc[i][t][3]);
+          acc[i][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[i].v, xf[t].v, acc[i][t], 0, 0, 0);
     }
-    __syncthreads();
-    if (wave != 0) return;
+    __builtin_amdgcn_wave_barrier();       // and the reads before the next stage's writes
+  };
+  if (k_begin < k_end) {
 #pragma unroll
-    for (int i = 0; i < NT; ++i)
+    for (int d = 0; d < DEPTH; ++d) fetch(st[d], k_begin + 64 * d);
+    for (int k = k_begin; k < k_end; k += 64 * DEPTH) {
 #pragma unroll
-      for (int t = 0; t < MT; ++t)
-        for (int w = 1; w < nwaves; ++w) {
-          const float4 o = *reinterpret_cast<const float4*>(&red[w - 1][i * MT + t][lane * 4]);
-          acc[i][t][0] += o.x; acc[i][t][1] += o.y; acc[i][t][2] += o.z; acc[i][t][3] += o.w;
+      for (int d = 0; d < DEPTH; ++d) {
+        if (k + 64 * d < k_end) {
+          work(st[d]);
+          fetch(st[d], k + 64 * (d + DEPTH));
         }
-  }
-#pragma unroll
-  for (int t = 0; t < MT; ++t) {
-    const int m = 16 * t + r;
-    if (m >= M) continue;
-#pragma unroll
-    for (int i = 0; i < OT; ++i) {
-      const int nn = n0 + 16 * i + 4 * g;
-      if (EPI == EPI_SILU) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-          if (nn + j < N) st_f32(C + (size_t)m * ldc + nn + j, fast_silu(acc[i][t][j]) * acc[i + OT][t][j]);
-      } else if (EPI == EPI_RESADD) {
-        float* rp = R + (size_t)m * ldc + nn;
-        if (nn + 3 < N) {
-          float4 o = *reinterpret_cast<float4*>(rp);
-          o.x += acc[i][t][0]; o.y += acc[i][t][1]; o.z += acc[i][t][2]; o.w += acc[i][t][3];
-          *reinterpret_cast<float4*>(rp) = o;
-        } else {
-#pragma unroll
-          for (int j = 0; j < 4; ++j)
-            if (nn + j < N) rp[j] += acc[i][t][j];
-        }
-      } else {
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-          if (nn + j < N) st_f32(C + (size_t)m * ldc + nn + j, acc[i][t][j] + (bias ? bias[nn + j] : 0.f));
       }
     }
   }
+  __syncthreads();                                        // the partial sums take the place of the stages
+  auto& red = *reinterpret_cast<float (*)[MAXW - 1][NT * MT][64 * 4]>(lds);
+  skinny_finish<MT, NT, EPI, TC>(acc, red, bias, C, R, ldc, M, N, n0);
 }
 
 extern "C" int ullm_gemm_skinny_supports(int M, int N, int K, int ldx, int ldw) {
@@ -164,14 +283,17 @@ extern "C" int ullm_gemm_skinny_supports(int M, int N, int K, int ldx, int ldw) 
 
 // X bfloat16 [M, K]; W bfloat16 [N, K] (with epi 2: [2 N, K]).  epi: 0 store to C (c_dtype, bias optional),
 // 1 add into R (float32 [M, N], row stride ldc), 2 silu(gate) * up to C (bfloat16 [M, N]).
-// force_nt / force_waves: 0 = chosen here.
+// force_nt / force_waves: 0 = chosen here.  staged: 1 = operands through shared memory, 0 = straight
+// from memory, -1 = chosen here: staged, except for up to 4 rows against a matrix of 128 MB or more,
+// where the straight kernel is a few percent faster (measured on Qwen3-8B's gate|up matrix).
 extern "C" int ullm_gemm_skinny(const void* X, int ldx, const void* W, int ldw, const float* bias, void* C,
                                 int ldc, int M, int N, int K, int epi, int c_dtype, int force_nt,
-                                int force_waves, hipStream_t stream) {
+                                int force_waves, int staged, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (!ullm_gemm_skinny_supports(M, N, K, ldx, ldw) || ldc < N) return ULLM_ERR_SHAPE;
   if (((uintptr_t)X & 15) || ((uintptr_t)W & 15)) return ULLM_ERR_SHAPE;
-  if (epi < 0 || epi > 2) return ULLM_ERR_UNSUPPORTED;
+  if (epi < 0 || epi > 2 || staged < -1 || staged > 1) return ULLM_ERR_UNSUPPORTED;
+  if (staged < 0) staged = !(M <= 4 && (long long)N * K * (epi == EPI_SILU ? 2 : 1) >= (64LL << 20));
   if (epi == EPI_RESADD && (((uintptr_t)C & 15) || ldc % 4 != 0 || bias)) return ULLM_ERR_SHAPE;
   if (epi == EPI_SILU && (bias || c_dtype != ULLM_BF16)) return ULLM_ERR_UNSUPPORTED;
   int mt = (M + 15) / 16;
@@ -192,11 +314,15 @@ extern "C" int ullm_gemm_skinny(const void* X, int ldx, const void* W, int ldw, 
   while (waves < max_waves && tiles * waves < 4096 && K / (waves * 2) >= 128) waves *= 2;
   if (force_waves > 0) waves = force_waves < max_waves ? force_waves : max_waves;
   int k_per_wave = (K + waves - 1) / waves;
-  k_per_wave = (k_per_wave + 31) / 32 * 32;
+  k_per_wave = staged ? (k_per_wave + 63) / 64 * 64 : (k_per_wave + 31) / 32 * 32;
   dim3 grid(tiles), block(64 * waves);
   float* R = (float*)C;
-#define GO(MT, NT, EPI, TC) hipLaunchKernelGGL((gemm_skinny_kernel<MT, NT, EPI, TC>), grid, block, 0, stream, \
-    (const bf16_t*)X, ldx, (const bf16_t*)W, ldw, bias, (TC*)C, R, ldc, M, N, K, k_per_wave)
+#define GO(MT, NT, EPI, TC) do {                                                                           \
+    if (staged) hipLaunchKernelGGL((gemm_skinny_staged_kernel<MT, NT, EPI, TC>), grid, block, 0, stream,      \
+        (const bf16_t*)X, ldx, (const bf16_t*)W, ldw, bias, (TC*)C, R, ldc, M, N, K, k_per_wave);            \
+    else hipLaunchKernelGGL((gemm_skinny_kernel<MT, NT, EPI, TC>), grid, block, 0, stream,                   \
+        (const bf16_t*)X, ldx, (const bf16_t*)W, ldw, bias, (TC*)C, R, ldc, M, N, K, k_per_wave);            \
+  } while (0)
 #define GO_SHAPE(EPI, TC)                                              \
   switch (mt * 8 + nt) {                                               \
     case 1 * 8 + 1: GO(1, 1, EPI, TC); break;                          \

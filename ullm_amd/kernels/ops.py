@@ -228,11 +228,15 @@ def gemm_skinny_supports(a: torch.Tensor, w: torch.Tensor) -> bool:
     return a.dtype == torch.bfloat16 and _skinny_ok(a.shape[0], a.shape[1], a, w)
 
 
-def _gemm_skinny(x, w, bias, c, M, N, K, epi, c_dtype, nt=0, waves=0) -> None:
+SKINNY_STAGED = -1     # 1: operands through shared memory (whole cache lines per load), 0: straight from memory, -1: the kernel's choice
+
+
+def _gemm_skinny(x, w, bias, c, M, N, K, epi, c_dtype, nt=0, waves=0, staged=None) -> None:
     lib = build.load("gemm_skinny")
     _check(lib.ullm_gemm_skinny(_p(x), _c_int(x.stride(0)), _p(w), _c_int(w.stride(0)), _p(bias),
                                 _p(c), _c_int(c.stride(0)), _c_int(M), _c_int(N), _c_int(K),
-                                _c_int(epi), _c_int(c_dtype), _c_int(nt), _c_int(waves), _stream()),
+                                _c_int(epi), _c_int(c_dtype), _c_int(nt), _c_int(waves),
+                                _c_int(SKINNY_STAGED if staged is None else staged), _stream()),
            "gemm_skinny")
 
 
