@@ -458,17 +458,11 @@ def test_gemm_skinny(ops, shape, out_dtype):
     want = (a.double() @ w.double().T + b.double()).float()
     got = ops.gemm_skinny(a, w, b, out_dtype=out_dtype)
     assert got.dtype == out_dtype
-    # both kernels (operands through shared memory, or straight from memory) in several tilings
-    try:
-        for staged in (0, 1):
-            ops.SKINNY_STAGED = staged
-            for nt, waves in ((0, 0), (1, 1), (2, 2), (2, 16), (4 if M > 16 else 2, 4)):
-                other = ops.gemm_skinny(a, w, b, out_dtype=out_dtype, nt=nt, waves=waves)
-                assert (other.float() - got.float()).abs().max() <= 1e-2 * float(want.abs().max()), (staged, nt, waves)
-                if out_dtype == torch.float32:
-                    assert (other - want).abs().max() <= 2e-5 * float(want.abs().max()), (staged, nt, waves)
-    finally:
-        ops.SKINNY_STAGED = -1
+    for nt, waves in ((1, 1), (2, 2), (2, 16), (4 if M > 16 else 2, 4)):
+        other = ops.gemm_skinny(a, w, b, out_dtype=out_dtype, nt=nt, waves=waves)
+        assert (other.float() - got.float()).abs().max() <= 1e-2 * float(want.abs().max()), (nt, waves)
+        if out_dtype == torch.float32:
+            assert (other - want).abs().max() <= 2e-5 * float(want.abs().max()), (nt, waves)
     bound = (1e-2 if out_dtype == torch.bfloat16 else 2e-5) * float(want.abs().max())
     assert (got.float() - want).abs().max() <= bound
     assert torch.equal(ops.gemm_skinny(a, w, b, out_dtype=out_dtype), got)          # repeatable bit for bit
@@ -492,11 +486,9 @@ def test_gemm_dispatch_refuses_nothing_silently(ops):
 @pytest.mark.parametrize("shape", [(1, 48, 64), (8, 503, 96), (16, 256, 4096), (17, 100, 224), (40, 96, 1032),
                                    (64, 2100, 520), (5, 4096, 128)])
 @pytest.mark.parametrize("nt", [0, 1, 2, 4])
-@pytest.mark.parametrize("staged", [0, 1])
-def test_gemm_skinny_fused_forms(ops, shape, nt, staged, monkeypatch):
+def test_gemm_skinny_fused_forms(ops, shape, nt):
     """The folded forms against the separate kernels' references: the add into the 32-bit residual
     behind a product, and silu(gate) * up behind the product with the stacked gate|up weights."""
-    monkeypatch.setattr(ops, "SKINNY_STAGED", staged)
     torch.manual_seed(11)
     M, N, K = shape
     if nt == 4 and M <= 16:

@@ -12,11 +12,11 @@
 //             rows of the up half and stores C[M, I] = silu(gate) * up, computed on the 32-bit sums
 //             (ullm/layers/activation.py:16-18 after gate_up_proj, ullm/models/qwen3.py:43-45)
 //
-// A block owns NT x 16 consecutive rows of W; its waves split K between them.  Per 32 values of K a
-// wave issues one 16-byte load per lane and W tile straight from global memory (A operand of
-// v_mfma_f32_16x16x32_bf16: lane (r, g) holds W[n0 + r][k + 8g .. +8]) and builds the B operand
-// (lane (m, g) holds X[m][k + 8g .. +8]) per 16 rows of X.  The waves' partial results are added in
-// wave order through shared memory, so the result does not depend on timing.
+// A block owns NT x 16 consecutive rows of W; its waves split K between them.  The A operand of
+// v_mfma_f32_16x16x32_bf16 is a W tile (lane (r, g) holds W[n0 + r][k + 8g .. +8]), the B operand 16
+// rows of X (lane (m, g) holds X[m][k + 8g .. +8]); both reach the registers through the wave's own
+// part of shared memory.  The waves' partial results are added in wave order through shared memory,
+// so the result does not depend on timing.
 // Weights are [out, in] (ullm/layers/linear.py:165).
 #include "common.h"
 
@@ -32,8 +32,10 @@ union Pack8 {
 
 enum { EPI_STORE = 0, EPI_RESADD = 1, EPI_SILU = 2 };
 
-// most waves per block for a tile shape: bounded by the shared memory that holds the waves' partials
-__host__ __device__ constexpr int sk_max_waves(int mt, int nt) { return mt * nt >= 8 ? 4 : (mt * nt >= 4 ? 8 : 16); }
+// Most waves per block for a tile shape,
+// bounded by the shared memory that holds a stage per wave (and later the waves' partials): at most 8
+// waves, so that several blocks fit a compute unit
+__host__ __device__ constexpr int sk_max_waves(int mt, int nt) { return mt * nt >= 8 ? 4 : 8; }
 
 // The waves' partial results of a block are added in wave order through `red` and the sum goes where
 // EPI says.  acc[i][t][j] = partial C[m = 16 t + r][n0 + 16 i + 4 g + j].
@@ -96,90 +98,18 @@ __device__ __forceinline__ void skinny_finish(f32x4_t (&acc)[NT][MT], RedT& red,
 
 // MT = 16-row tiles of X (M <= 16 MT); NT = 16-row tiles of W per block.
 // With EPI_SILU the NT tiles of W are NT / 2 of the gate half followed by the same rows of the up half.
+// A wave fetches whole 128-byte lines, 8 rows per instruction (lane = row l / 8, 16-byte piece l % 8),
+// two stages of 64 values of K ahead in registers, writes a stage to its own part of shared memory and
+// reads the operands from there in the layout the matrix instruction wants (lane (r, g) holds row r,
+// values 8 g .. +8 of a step of 32).  A row takes 128 bytes; piece c of row r lies at piece
+// c ^ ((r >> 1) & 7), which keeps both the 16-byte writes and the 16-byte reads of the hardware's lane
+// groups on different banks.  No barrier in the loop: a wave only reads what it wrote.
+// (Loading the operands straight from memory in the matrix layout, 64 bytes of each of 16 rows per
+// instruction and of X as many rows as the batch has, was slower the more rows X had: 92 against 80 us
+// for the four projections of a Qwen3-8B layer at 8 rows, 105 against 83 us at 16.)
 template <int MT, int NT, int EPI, typename TC>
 __global__ void __launch_bounds__(64 * sk_max_waves(MT, NT))
 gemm_skinny_kernel(const bf16_t* __restrict__ X, int ldx, const bf16_t* __restrict__ W, int ldw,
-                   const float* __restrict__ bias, TC* __restrict__ C, float* __restrict__ R, int ldc, int M,
-                   int N, int K, int k_per_wave) {
-  constexpr int MAXW = sk_max_waves(MT, NT);
-  __shared__ float red[MAXW - 1][NT * MT][64 * 4];   // wave 0 adds the others' partials to its own
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
-  const int g = lane >> 4, r = lane & 15;
-  // N counts the columns of the result; with EPI_SILU W has 2 N rows
-  constexpr int OT = EPI == EPI_SILU ? NT / 2 : NT;      // 16-column tiles of the result per block
-  const int n0 = blockIdx.x * (16 * OT);
-  const bf16_t* wp[NT];
-#pragma unroll
-  for (int i = 0; i < NT; ++i) {
-    const int col = n0 + 16 * (i % OT) + r;
-    const int n = (col < N ? col : N - 1) + (i / OT) * N;   // rows past N repeat the last row; never stored
-    wp[i] = W + (size_t)n * ldw + 8 * g;
-  }
-  size_t xo[MT];
-#pragma unroll
-  for (int t = 0; t < MT; ++t) {
-    const int m = 16 * t + r < M ? 16 * t + r : M - 1;
-    xo[t] = (size_t)m * ldx + 8 * g;
-  }
-  f32x4_t acc[NT][MT];
-#pragma unroll
-  for (int t = 0; t < MT; ++t)
-#pragma unroll
-    for (int i = 0; i < NT; ++i) acc[i][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-  const int k_begin = wave * k_per_wave;
-  int k_end = k_begin + k_per_wave;
-  if (k_end > K) k_end = K;
-  int k = k_begin;
-  constexpr int U = (NT * MT >= 8) ? 1 : ((NT + MT >= 5) ? 2 : 4);       // steps of 32 in flight per wave
-  for (; k + 32 * U <= k_end; k += 32 * U) {
-    Pack8 w[U][NT], x[U][MT];
-#pragma unroll
-    for (int u = 0; u < U; ++u)
-#pragma unroll
-      for (int i = 0; i < NT; ++i) w[u][i].u4 = *reinterpret_cast<const uint4*>(wp[i] + k + 32 * u);
-#pragma unroll
-    for (int u = 0; u < U; ++u)
-#pragma unroll
-      for (int t = 0; t < MT; ++t) x[u][t].u4 = *reinterpret_cast<const uint4*>(X + xo[t] + k + 32 * u);
-#pragma unroll
-    for (int u = 0; u < U; ++u)
-#pragma unroll
-      for (int i = 0; i < NT; ++i)
-#pragma unroll
-        for (int t = 0; t < MT; ++t)
-          acc[i][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[u][i].v, x[u][t].v, acc[i][t], 0, 0, 0);
-  }
-  // remaining steps of 32, the last one possibly short (K is a multiple of 8)
-  for (; k < k_end; k += 32) {
-    const bool in = k + 8 * g < k_end;
-    Pack8 w[NT], x[MT];
-#pragma unroll
-    for (int i = 0; i < NT; ++i) w[i].u4 = in ? *reinterpret_cast<const uint4*>(wp[i] + k) : make_uint4(0, 0, 0, 0);
-#pragma unroll
-    for (int t = 0; t < MT; ++t) {
-      x[t].u4 = in ? *reinterpret_cast<const uint4*>(X + xo[t] + k) : make_uint4(0, 0, 0, 0);
-    }
-#pragma unroll
-    for (int i = 0; i < NT; ++i)
-#pragma unroll
-      for (int t = 0; t < MT; ++t)
-        acc[i][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[i].v, x[t].v, acc[i][t], 0, 0, 0);
-  }
-  skinny_finish<MT, NT, EPI, TC>(acc, red, bias, C, R, ldc, M, N, n0);
-}
-
-// The same product with the operands staged through shared memory.  In the kernel above a load
-// instruction of a wave fetches 64 bytes of each of 16 rows, and of X as many rows as the batch has:
-// half cache lines, and more of them per instruction the more rows X has, which is what its time
-// grows with.  Here a wave fetches whole 128-byte lines, 8 rows per instruction (lane = row l / 8,
-// 16-byte piece l % 8), two stages of 64 values of K ahead in registers, writes a stage to its own
-// part of shared memory and reads the operands from there in the layout the matrix instruction wants
-// (lane (r, g) holds row r, values 8 g .. +8 of a step of 32).  A row takes 128 bytes; piece c of row
-// r lies at piece c ^ ((r >> 1) & 7), which keeps both the 16-byte writes and the 16-byte reads of the
-// hardware's lane groups on different banks.  No barrier in the loop: a wave only reads what it wrote.
-template <int MT, int NT, int EPI, typename TC>
-__global__ void __launch_bounds__(64 * sk_max_waves(MT, NT))
-gemm_skinny_staged_kernel(const bf16_t* __restrict__ X, int ldx, const bf16_t* __restrict__ W, int ldw,
                           const float* __restrict__ bias, TC* __restrict__ C, float* __restrict__ R, int ldc, int M,
                           int N, int K, int k_per_wave) {
   constexpr int MAXW = sk_max_waves(MT, NT);
@@ -283,17 +213,14 @@ extern "C" int ullm_gemm_skinny_supports(int M, int N, int K, int ldx, int ldw) 
 
 // X bfloat16 [M, K]; W bfloat16 [N, K] (with epi 2: [2 N, K]).  epi: 0 store to C (c_dtype, bias optional),
 // 1 add into R (float32 [M, N], row stride ldc), 2 silu(gate) * up to C (bfloat16 [M, N]).
-// force_nt / force_waves: 0 = chosen here.  staged: 1 = operands through shared memory, 0 = straight
-// from memory, -1 = chosen here: staged, except for up to 4 rows against a matrix of 128 MB or more,
-// where the straight kernel is a few percent faster (measured on Qwen3-8B's gate|up matrix).
+// force_nt / force_waves: 0 = chosen here.
 extern "C" int ullm_gemm_skinny(const void* X, int ldx, const void* W, int ldw, const float* bias, void* C,
                                 int ldc, int M, int N, int K, int epi, int c_dtype, int force_nt,
-                                int force_waves, int staged, hipStream_t stream) {
+                                int force_waves, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (!ullm_gemm_skinny_supports(M, N, K, ldx, ldw) || ldc < N) return ULLM_ERR_SHAPE;
   if (((uintptr_t)X & 15) || ((uintptr_t)W & 15)) return ULLM_ERR_SHAPE;
-  if (epi < 0 || epi > 2 || staged < -1 || staged > 1) return ULLM_ERR_UNSUPPORTED;
-  if (staged < 0) staged = !(M <= 4 && (long long)N * K * (epi == EPI_SILU ? 2 : 1) >= (64LL << 20));
+  if (epi < 0 || epi > 2) return ULLM_ERR_UNSUPPORTED;
   if (epi == EPI_RESADD && (((uintptr_t)C & 15) || ldc % 4 != 0 || bias)) return ULLM_ERR_SHAPE;
   if (epi == EPI_SILU && (bias || c_dtype != ULLM_BF16)) return ULLM_ERR_UNSUPPORTED;
   int mt = (M + 15) / 16;
@@ -308,21 +235,18 @@ extern "C" int ullm_gemm_skinny(const void* X, int ldx, const void* W, int ldw, 
   if (nt == 4 && mt == 1) nt = 2;                       // not instantiated
   const int out_tiles = epi == EPI_SILU ? nt / 2 : nt;  // 16-column tiles of the result per block
   const int tiles = (tiles16 + out_tiles - 1) / out_tiles;
-  // waves per block: enough blocks x waves to fill the chip, each wave with at least 128 values of K
+  // waves per block: 8 tiles of W in flight per block (measured: 8 waves with one tile each, 4 with two),
+  // each wave with at least 128 values of K
   const int max_waves = sk_max_waves(mt, nt);
   int waves = 1;
-  while (waves < max_waves && tiles * waves < 4096 && K / (waves * 2) >= 128) waves *= 2;
+  while (waves < max_waves && waves * nt < 8 && K / (waves * 2) >= 128) waves *= 2;
   if (force_waves > 0) waves = force_waves < max_waves ? force_waves : max_waves;
   int k_per_wave = (K + waves - 1) / waves;
-  k_per_wave = staged ? (k_per_wave + 63) / 64 * 64 : (k_per_wave + 31) / 32 * 32;
+  k_per_wave = (k_per_wave + 63) / 64 * 64;
   dim3 grid(tiles), block(64 * waves);
   float* R = (float*)C;
-#define GO(MT, NT, EPI, TC) do {                                                                           \
-    if (staged) hipLaunchKernelGGL((gemm_skinny_staged_kernel<MT, NT, EPI, TC>), grid, block, 0, stream,      \
-        (const bf16_t*)X, ldx, (const bf16_t*)W, ldw, bias, (TC*)C, R, ldc, M, N, K, k_per_wave);            \
-    else hipLaunchKernelGGL((gemm_skinny_kernel<MT, NT, EPI, TC>), grid, block, 0, stream,                   \
-        (const bf16_t*)X, ldx, (const bf16_t*)W, ldw, bias, (TC*)C, R, ldc, M, N, K, k_per_wave);            \
-  } while (0)
+#define GO(MT, NT, EPI, TC) hipLaunchKernelGGL((gemm_skinny_kernel<MT, NT, EPI, TC>), grid, block, 0, stream, \
+    (const bf16_t*)X, ldx, (const bf16_t*)W, ldw, bias, (TC*)C, R, ldc, M, N, K, k_per_wave)
 #define GO_SHAPE(EPI, TC)                                              \
   switch (mt * 8 + nt) {                                               \
     case 1 * 8 + 1: GO(1, 1, EPI, TC); break;                          \

@@ -228,15 +228,11 @@ def gemm_skinny_supports(a: torch.Tensor, w: torch.Tensor) -> bool:
     return a.dtype == torch.bfloat16 and _skinny_ok(a.shape[0], a.shape[1], a, w)
 
 
-SKINNY_STAGED = -1     # 1: operands through shared memory (whole cache lines per load), 0: straight from memory, -1: the kernel's choice
-
-
-def _gemm_skinny(x, w, bias, c, M, N, K, epi, c_dtype, nt=0, waves=0, staged=None) -> None:
+def _gemm_skinny(x, w, bias, c, M, N, K, epi, c_dtype, nt=0, waves=0) -> None:
     lib = build.load("gemm_skinny")
     _check(lib.ullm_gemm_skinny(_p(x), _c_int(x.stride(0)), _p(w), _c_int(w.stride(0)), _p(bias),
                                 _p(c), _c_int(c.stride(0)), _c_int(M), _c_int(N), _c_int(K),
-                                _c_int(epi), _c_int(c_dtype), _c_int(nt), _c_int(waves),
-                                _c_int(SKINNY_STAGED if staged is None else staged), _stream()),
+                                _c_int(epi), _c_int(c_dtype), _c_int(nt), _c_int(waves), _stream()),
            "gemm_skinny")
 
 
@@ -294,12 +290,11 @@ def gemm_bf16(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = N
     out_dtype = out_dtype or a.dtype
     M = a.shape[0]
     library = a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and a.is_cuda
-    if library and out_dtype == torch.float32 and a.is_contiguous() and w.is_contiguous() and _MM_TAKES_OUT_DTYPE:
-        # the widest product of a step (the vocabulary): the library streams it a little faster at any M
-        y = torch.mm(a, w.t(), out_dtype=torch.float32)
-        return y if bias is None else y + bias
     if M <= SKINNY_MAX_ROWS and gemm_skinny_supports(a, w):
         return gemm_skinny(a, w, bias, out_dtype=out_dtype)
+    if library and out_dtype == torch.float32 and a.is_contiguous() and w.is_contiguous() and _MM_TAKES_OUT_DTYPE:
+        y = torch.mm(a, w.t(), out_dtype=torch.float32)
+        return y if bias is None else y + bias
     if library and out_dtype == torch.bfloat16:
         y = torch.nn.functional.linear(a, w)
         return y if bias is None else (y.float() + bias).to(torch.bfloat16)
