@@ -119,8 +119,8 @@ sample_kernel(const float* __restrict__ logits, int V, int ld, const float* __re
   const float inv_t = 1.f / (t < 0.f ? 1.f : t);  // the reference maps T <= 0 to 1 (sampler.py:41)
   const float L2E = 1.4426950408889634f;
   float mloc = -INFINITY;
-  for_range<VEC>(x, wbeg, wend, lane, [&](int, float v) { mloc = fmaxf(mloc, v * inv_t); });
-  const float m = block_max(mloc, fscratch);
+  for_range<VEC>(x, wbeg, wend, lane, [&](int, float v) { mloc = fmaxf(mloc, v); });   // 1 / T is positive
+  const float m = block_max(mloc, fscratch) * inv_t;
   const uint32_t key_max = order_key(m);
   uint32_t kmin = 0;
 #define E_OF(z) __builtin_amdgcn_exp2f(((z) - m) * L2E)
@@ -160,11 +160,15 @@ sample_kernel(const float* __restrict__ logits, int V, int ld, const float* __re
 
   const float mp = min_p[row];
   float s = 0.f;
-  for_range<VEC>(x, wbeg, wend, lane, [&](int, float v) {
-    const float z = v * inv_t;
-    const float e = E_OF(z);
-    if (order_key(z) >= kmin && e >= mp) s += e;
-  });
+  if (kmin == 0 && !(mp > 0.f)) {          // nothing filtered: every value counts (3 instructions a value)
+    for_range<VEC>(x, wbeg, wend, lane, [&](int, float v) { s += E_OF(v * inv_t); });
+  } else {
+    for_range<VEC>(x, wbeg, wend, lane, [&](int, float v) {
+      const float z = v * inv_t;
+      const float e = E_OF(z);
+      if (order_key(z) >= kmin && e >= mp) s += e;
+    });
+  }
   s = wave_sum(s);
   if (tid == 0) chosen = -1;
   if (lane == 0) wave_tot[wave] = s;
