@@ -313,6 +313,36 @@ def test_sampler_kernel_against_the_plain_sampler(ops):
     assert float(((counts - n * probs) ** 2 / (n * probs)).sum()) < 25.0
 
 
+def test_sampler_with_a_small_top_k_over_a_large_vocabulary(ops):
+    """Top-k with a small k gathers the few values that can matter and filters those; rows where that
+    cannot work (many equal values around the k-th largest, the k-th largest far below the maximum)
+    take the pass over the whole vocabulary.  Either way the token is one the plain sampler may draw."""
+    from ullm_amd.sampling import Sampler, SamplingParams
+    torch.manual_seed(17)
+    sampler = Sampler(torch.device(DEV))
+    configs = [(0.6, 20, 0.95, 0.0), (1.0, 5, 1.0, 0.0), (0.8, 50, 0.9, 0.02), (1.0, 1000, 1.0, 0.0), (1.2, 1, 1.0, 0.0),
+               (0.7, 20, 0.5, 0.0), (1.0, 1024, 0.99, 0.0), (1.0, 1025, 1.0, 0.0)]
+    for V in (32000, 151936, 50257):       # 50257: rows not aligned for 16-byte loads
+        kinds = {
+            "spread": torch.randn(len(configs), V) * 3,
+            "flat": torch.randn(len(configs), V) * 0.01,                     # all within a hair of the maximum
+            "ties": (torch.randn(len(configs), V) * 2).round(),              # many equal values: too many candidates
+            "far": torch.cat([torch.tensor([[50.0, 49.25, 48.5]]).expand(len(configs), 3),
+                              torch.randn(len(configs), V - 3)], 1),           # the k-th largest far below the maximum
+        }
+        for name, logits in kinds.items():
+            ps = [SamplingParams(temperature=c[0], top_k=c[1], top_p=c[2], min_p=c[3]) for c in configs]
+            seeds = [7 + i for i in range(len(configs))]
+            pos = [3 * i for i in range(len(configs))]
+            got = sampler.sample(logits.to(DEV), ps, seeds, pos)
+            for i, c in enumerate(configs):
+                if name == "ties" and c[2] < 1.0:
+                    continue       # which of several equal values top-p drops follows the reference's sort; here all or none
+                assert got[i] in plain.sample_token_set(logits[i], *c, seeds[i], pos[i]), (V, name, c, got[i])
+            again = sampler.sample(logits.flip(0).contiguous().to(DEV), ps[::-1], seeds[::-1], pos[::-1])
+            assert again[::-1] == got
+
+
 MFMA_CASES = [dict(nq=8, nkv=2, hd=32, P=16, lens=[(1, 1), (1, 37), (1, 300), (1, 64)], window=0),
               dict(nq=32, nkv=8, hd=128, P=16, lens=[(1, 1153), (1, 31), (1, 32), (1, 33)], window=0),
               dict(nq=8, nkv=1, hd=64, P=32, lens=[(1, 500), (1, 97)], window=0),

@@ -72,6 +72,181 @@ __device__ __forceinline__ void for_range(const float* __restrict__ x, int wbeg,
   }
 }
 
+// ------------------------------------------------------------------------------ small top-k
+// With top-k at work and k small, the values that can matter are few.  Two counting passes find a
+// distance d = 2^(5-j), j = 0..15, such that {z >= max - d} has at least k members but not many
+// more; one more pass gathers these candidates, in index order, into shared memory (each wave its
+// own range and its own segment); every filter and the draw then run over the candidates only, by
+// the same rules as over the whole vocabulary.  Where this does not work out (fewer than k values
+// within 32 of the maximum, or more candidates than a segment holds: many equal values) the caller
+// takes the long way.
+#define SMALL_K_MAX 1024
+#define SEG 256                       // candidates a wave can hold
+#define DELTA_STEPS 16
+
+struct Candidates {
+  float z[16 * SEG];                  // as gathered: a segment per wave
+  int idx[16 * SEG];
+  int n[16];
+  float lz[16 * SEG];                 // side by side
+  int lidx[16 * SEG];
+};
+
+// -1: take the long way.  Otherwise the token.  Every thread of the block returns the same value.
+template <bool VEC>
+__device__ int sample_small_k(const float* __restrict__ x, int wbeg, int wend, float inv_t, float m, int k, float p,
+                              float mp, float uniform, Candidates& cand, int* iscratch) {
+  constexpr int PER = VEC ? 4 : 1;
+  constexpr int STEP = PER * WAVE;
+  const int tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE, nwaves = blockDim.x / WAVE;
+  const float L2E = 1.4426950408889634f;
+  const uint32_t key_max = order_key(m);
+  // 1. the distance: the largest j whose set has at least k members (counts fall as j grows)
+  int j_lo = 0;
+#pragma unroll 1
+  for (int round = 0; round < 2; ++round) {
+    const int stride = round == 0 ? 4 : 1;
+    const uint32_t k1 = order_key(m - exp2f((float)(5 - (j_lo + stride)))), k2 = order_key(m - exp2f((float)(5 - (j_lo + 2 * stride)))),
+                   k3 = order_key(m - exp2f((float)(5 - (j_lo + 3 * stride))));
+    int c1 = 0, c2 = 0, c3 = 0;
+    for_range<VEC>(x, wbeg, wend, lane, [&](int, float v) {
+      const uint32_t key = order_key(v * inv_t);
+      c1 += key >= k1; c2 += key >= k2; c3 += key >= k3;
+    });
+    c1 = block_sum_int(c1, iscratch); c2 = block_sum_int(c2, iscratch); c3 = block_sum_int(c3, iscratch);
+    j_lo += stride * ((c1 >= k) + (c2 >= k) + (c3 >= k));
+  }
+  const uint32_t key_thr = order_key(m - exp2f((float)(5 - j_lo)));
+  // 2. gather, in index order: a wave walks its range and appends what it keeps to its segment
+  int pos = 0;
+  bool overflow = false;
+  constexpr int AHEAD = 4;                                 // steps whose loads are under way together
+  for (int base = wbeg; base < wend && !overflow; base += AHEAD * STEP) {
+    float raw[AHEAD][PER];
+#pragma unroll
+    for (int u = 0; u < AHEAD; ++u) {
+      const int ii = base + u * STEP + PER * lane;
+      if (VEC) {
+        const float4 v = ii < wend ? *reinterpret_cast<const float4*>(x + ii) : make_float4(0.f, 0.f, 0.f, 0.f);
+        raw[u][0] = v.x;
+        if (PER > 1) { raw[u][1] = v.y; raw[u][2] = v.z; raw[u][3] = v.w; }
+      } else {
+        raw[u][0] = ii < wend ? x[ii] : 0.f;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < AHEAD; ++u) {
+      const int ii = base + u * STEP + PER * lane;
+      float z[PER];
+      bool keep[PER];
+      int cnt = 0;
+#pragma unroll
+      for (int c = 0; c < PER; ++c) {
+        z[c] = raw[u][c] * inv_t;
+        keep[c] = ii + c < wend && order_key(z[c]) >= key_thr;
+        cnt += keep[c];
+      }
+      if (overflow || !__any(cnt)) continue;
+      int incl = cnt;
+#pragma unroll
+      for (int d = 1; d < WAVE; d <<= 1) {
+        const int o = __shfl_up(incl, d, WAVE);
+        if (lane >= d) incl += o;
+      }
+      const int total = __shfl(incl, WAVE - 1, WAVE);
+      if (pos + total > SEG) { overflow = true; continue; }
+      int o = wave * SEG + pos + incl - cnt;
+#pragma unroll
+      for (int c = 0; c < PER; ++c)
+        if (keep[c]) { cand.z[o] = z[c]; cand.idx[o] = ii + c; ++o; }
+      pos += total;
+    }
+  }
+  if (lane == 0) cand.n[wave] = overflow ? -1 : pos;
+  __syncthreads();
+  int n_all = 0;
+  bool bad = false;
+  for (int w = 0; w < nwaves; ++w) { bad = bad || cand.n[w] < 0; n_all += cand.n[w] < 0 ? 0 : cand.n[w]; }
+  if (bad || n_all < k) return -1;
+  // the candidates side by side (still in index order): from here on every wave does the same work on
+  // the whole list with reductions inside the wave, so no barrier is needed and all agree
+  {
+    int off = 0;
+    for (int w = 0; w < wave; ++w) off += cand.n[w];
+    for (int j = lane; j < cand.n[wave]; j += WAVE) {
+      cand.lz[off + j] = cand.z[wave * SEG + j];
+      cand.lidx[off + j] = cand.idx[wave * SEG + j];
+    }
+  }
+  __syncthreads();
+#define E_OF(zz) __builtin_amdgcn_exp2f(((zz) - m) * L2E)
+  auto count_if = [&](auto pred) {
+    int c = 0;
+    for (int j = lane; j < n_all; j += WAVE) c += pred(cand.lz[j]);
+#pragma unroll
+    for (int d = WAVE / 2; d > 0; d >>= 1) c += __shfl_xor(c, d, WAVE);
+    return c;
+  };
+  auto mass_if = [&](auto pred) {
+    float a = 0.f;
+    for (int j = lane; j < n_all; j += WAVE) {
+      const float zz = cand.lz[j];
+      if (pred(zz)) a += E_OF(zz);
+    }
+    return wave_sum(a);
+  };
+  // 3. top-k: the largest key v with #{key >= v} >= k; all such keys are candidates
+  uint32_t kmin;
+  {
+    uint32_t lo = key_thr, hi = key_max;
+    while (lo < hi) {
+      const uint32_t mid = lo + (hi - lo + 1) / 2;
+      if (count_if([&](float zz) { return order_key(zz) >= mid; }) >= k) lo = mid; else hi = mid - 1;
+    }
+    kmin = lo;
+  }
+  // 4. top-p on what top-k left
+  if (p > 0.f && p < 1.f) {
+    const float bound = p * mass_if([&](float zz) { return order_key(zz) >= kmin; });
+    uint32_t lo = kmin, hi = key_max;
+    while (lo < hi) {
+      const uint32_t mid = lo + (hi - lo) / 2;
+      if (mass_if([&](float zz) { return order_key(zz) > mid; }) < bound) hi = mid; else lo = mid + 1;
+    }
+    kmin = lo;
+  }
+  // 5. min-p and the draw: a walk along the list, 64 candidates at a time
+  auto weight = [&](int j) {
+    if (j >= n_all) return 0.f;
+    const float zz = cand.lz[j];
+    const float e = E_OF(zz);
+    return (order_key(zz) >= kmin && e >= mp) ? e : 0.f;
+  };
+  float total = 0.f;
+  for (int j = lane; j < n_all; j += WAVE) total += weight(j);
+  total = wave_sum(total);
+  const float target = uniform * total;
+  float run = 0.f;
+  int token = -1, last_kept = -1;
+  for (int j0 = 0; j0 < n_all && token < 0; j0 += WAVE) {
+    const float e = weight(j0 + lane);
+    float incl = e;
+#pragma unroll
+    for (int d = 1; d < WAVE; d <<= 1) {
+      const float o = __shfl_up(incl, d, WAVE);
+      if (lane >= d) incl += o;
+    }
+    const unsigned long long kept = __ballot(e > 0.f);
+    const unsigned long long crossed = __ballot(e > 0.f && run + incl > target);
+    if (crossed) token = cand.lidx[j0 + __ffsll((long long)crossed) - 1];
+    if (kept) last_kept = cand.lidx[j0 + 63 - __clzll((long long)kept)];
+    run += __shfl(incl, WAVE - 1, WAVE);
+  }
+  if (token < 0) token = last_kept < 0 ? 0 : last_kept;   // rounding pushed the target past the total: the last index kept
+#undef E_OF
+  return token;
+}
+
 // Each wave owns a contiguous range of the vocabulary, so sums over a wave's range are sums over
 // consecutive indices and the draw can walk the index order wave by wave.
 template <bool VEC>
@@ -85,6 +260,7 @@ sample_kernel(const float* __restrict__ logits, int V, int ld, const float* __re
   __shared__ int iscratch[16];
   __shared__ float wave_tot[16];
   __shared__ int chosen;
+  __shared__ Candidates cand;
   constexpr int STEP = VEC ? 4 * WAVE : WAVE;        // values a wave reads per access
   const int row = blockIdx.x, tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
   const int nwaves = blockDim.x / WAVE;
@@ -126,6 +302,16 @@ sample_kernel(const float* __restrict__ logits, int V, int ld, const float* __re
 #define E_OF(z) __builtin_amdgcn_exp2f(((z) - m) * L2E)
 
   const int k = top_k[row];
+  if (k > 0 && k < V && k <= SMALL_K_MAX && blockDim.x == SAMPLE_THREADS) {
+    const uint64_t seed = ((uint64_t)seed_hi[row] << 32) | (uint64_t)seed_lo[row];
+    const int token = sample_small_k<VEC>(x, wbeg, wend, inv_t, m, k, top_p[row], min_p[row],
+                                          uniform_from_seed(seed, (uint32_t)position[row]), cand, iscratch);
+    if (token >= 0) {
+      if (tid == 0) out[row] = token;
+      return;
+    }
+    __syncthreads();
+  }
   if (k > 0 && k < V) {  // largest key v with #{key >= v} >= k
     uint32_t lo = 0, hi = key_max;
     while (lo < hi) {
