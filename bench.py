@@ -158,7 +158,7 @@ def main():
     kv_per_token = sum(g.bytes_per_token(itemsize) for g in model.cache_layout()[0])
     gen = torch.Generator().manual_seed(0)
 
-    def run_decode(batch, steps, warmup):
+    def run_decode(batch, steps, warmup, top_k=-1, top_p=1.0):
         """tokens/s, ms per step, bytes read per step (mean over the timed steps)."""
         budget = max(8192, batch)
         # requests that finish their prompt early decode while the others are still in theirs
@@ -169,8 +169,8 @@ def main():
         eng = Engine(ec, model=model, env=env, model_config=cfg)
         for i in range(batch):
             prompt = torch.randint(0, cfg.vocab_size, (args.prompt_len,), generator=gen).tolist()
-            eng.add_request(f"r{i}", prompt, SamplingParams(temperature=0.6, ignore_eos=True, seed=i,
-                                                            max_new_tokens=new_tokens))
+            eng.add_request(f"r{i}", prompt, SamplingParams(temperature=0.6, top_k=top_k, top_p=top_p, ignore_eos=True,
+                                                            seed=i, max_new_tokens=new_tokens))
         while any(r.num_computed < args.prompt_len for r in eng.scheduler.requests.values()) or eng.scheduler.waiting:
             eng.step()                                   # prefill (untimed)
         for _ in range(warmup):
@@ -240,7 +240,10 @@ def main():
         line["prefill"] = {"value": round(p_tok_s, 1), "tokens": 2048, "ms": round(p_ms, 3), "frac": round(p_frac, 4)}
         b1, _, _ = run_decode(1, min(args.steps, 32), min(args.warmup, 4))
         b64, _, _ = run_decode(64, min(args.steps, 32), min(args.warmup, 4))
-        line["points"] = {"decode_b1": round(b1, 2), "decode_b64": round(b64, 2)}
+        # the same batch with the sampling of Qwen3's generation_config.json (top-k 20, top-p 0.95)
+        b8f, _, _ = run_decode(args.batch, min(args.steps, 32), min(args.warmup, 4), top_k=20, top_p=0.95)
+        line["points"] = {"decode_b1": round(b1, 2), "decode_b64": round(b64, 2),
+                          f"decode_b{args.batch}_top_k20_top_p95": round(b8f, 2)}
         del model
         torch.cuda.empty_cache()
         m_tok_s, m_out, m_secs, _ = run_mixed(args.dtype, args.eager)

@@ -314,17 +314,19 @@ def test_sampler_kernel_against_the_plain_sampler(ops):
 
 
 def test_sampler_with_a_small_top_k_over_a_large_vocabulary(ops):
-    """Top-k with a small k gathers the few values that can matter and filters those; rows where that
-    cannot work (many equal values around the k-th largest, the k-th largest far below the maximum)
-    take the pass over the whole vocabulary.  Either way the token is one the plain sampler may draw."""
+    """Top-k with a small k, and top-p alone on a peaked row, gather the few values that can matter and
+    filter those; rows where that cannot work (many equal values around the k-th largest, the k-th largest
+    far below the maximum, a flat row under top-p alone) take the passes over the whole vocabulary.  Either way the token is one the plain sampler may draw."""
     from ullm_amd.sampling import Sampler, SamplingParams
     torch.manual_seed(17)
     sampler = Sampler(torch.device(DEV))
     configs = [(0.6, 20, 0.95, 0.0), (1.0, 5, 1.0, 0.0), (0.8, 50, 0.9, 0.02), (1.0, 1000, 1.0, 0.0), (1.2, 1, 1.0, 0.0),
-               (0.7, 20, 0.5, 0.0), (1.0, 1024, 0.99, 0.0), (1.0, 1025, 1.0, 0.0)]
+               (0.7, 20, 0.5, 0.0), (1.0, 1024, 0.99, 0.0), (1.0, 1025, 1.0, 0.0),
+               (0.7, -1, 0.9, 0.0), (1.0, 0, 0.5, 0.02), (0.5, -1, 0.99, 0.0)]        # top-p alone
     for V in (32000, 151936, 50257):       # 50257: rows not aligned for 16-byte loads
         kinds = {
             "spread": torch.randn(len(configs), V) * 3,
+            "peaked": torch.randn(len(configs), V) * 8,
             "flat": torch.randn(len(configs), V) * 0.01,                     # all within a hair of the maximum
             "ties": (torch.randn(len(configs), V) * 2).round(),              # many equal values: too many candidates
             "far": torch.cat([torch.tensor([[50.0, 49.25, 48.5]]).expand(len(configs), 3),

@@ -72,14 +72,15 @@ __device__ __forceinline__ void for_range(const float* __restrict__ x, int wbeg,
   }
 }
 
-// ------------------------------------------------------------------------------ small top-k
-// With top-k at work and k small, the values that can matter are few.  Two counting passes find a
-// distance d = 2^(5-j), j = 0..15, such that {z >= max - d} has at least k members but not many
+// ------------------------------------------------------------------------------ few candidates
+// With top-k at work and k small, or with top-p alone on a peaked row, the values that can matter
+// are few.  Two passes find a distance d = 2^(5-j), j = 0..15, such that {z >= max - d} has at least
+// k members (top-k) or a little more than the share p of all weight (top-p alone) but not much
 // more; one more pass gathers these candidates, in index order, into shared memory (each wave its
 // own range and its own segment); every filter and the draw then run over the candidates only, by
 // the same rules as over the whole vocabulary.  Where this does not work out (fewer than k values
-// within 32 of the maximum, or more candidates than a segment holds: many equal values) the caller
-// takes the long way.
+// within 32 of the maximum, or more candidates than a segment holds: many equal values, a flat row
+// under top-p alone) the caller takes the long way.
 #define SMALL_K_MAX 1024
 #define SEG 256                       // candidates a wave can hold
 #define DELTA_STEPS 16
@@ -89,32 +90,53 @@ struct Candidates {
   int idx[16 * SEG];
   int n[16];
   float lz[16 * SEG];                 // side by side
+  float le[16 * SEG];                 // their weights exp(z - max)
   int lidx[16 * SEG];
+  int result;
 };
 
 // -1: take the long way.  Otherwise the token.  Every thread of the block returns the same value.
 template <bool VEC>
 __device__ int sample_small_k(const float* __restrict__ x, int wbeg, int wend, float inv_t, float m, int k, float p,
-                              float mp, float uniform, Candidates& cand, int* iscratch) {
+                              float mp, float uniform, Candidates& cand, float* fscratch, int* iscratch) {
   constexpr int PER = VEC ? 4 : 1;
   constexpr int STEP = PER * WAVE;
   const int tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE, nwaves = blockDim.x / WAVE;
   const float L2E = 1.4426950408889634f;
   const uint32_t key_max = order_key(m);
-  // 1. the distance: the largest j whose set has at least k members (counts fall as j grows)
+  // 1. the distance: the largest j whose set still holds what is needed: k members with top-k; without
+  // it (top-p alone) a little more than the share p of all weight, so that the nucleus ends inside
+  const bool by_count = k > 0;
+  float all_weight = 0.f;
   int j_lo = 0;
 #pragma unroll 1
   for (int round = 0; round < 2; ++round) {
     const int stride = round == 0 ? 4 : 1;
     const uint32_t k1 = order_key(m - exp2f((float)(5 - (j_lo + stride)))), k2 = order_key(m - exp2f((float)(5 - (j_lo + 2 * stride)))),
                    k3 = order_key(m - exp2f((float)(5 - (j_lo + 3 * stride))));
-    int c1 = 0, c2 = 0, c3 = 0;
-    for_range<VEC>(x, wbeg, wend, lane, [&](int, float v) {
-      const uint32_t key = order_key(v * inv_t);
-      c1 += key >= k1; c2 += key >= k2; c3 += key >= k3;
-    });
-    c1 = block_sum_int(c1, iscratch); c2 = block_sum_int(c2, iscratch); c3 = block_sum_int(c3, iscratch);
-    j_lo += stride * ((c1 >= k) + (c2 >= k) + (c3 >= k));
+    if (by_count) {
+      int c1 = 0, c2 = 0, c3 = 0;
+      for_range<VEC>(x, wbeg, wend, lane, [&](int, float v) {
+        const uint32_t key = order_key(v * inv_t);
+        c1 += key >= k1; c2 += key >= k2; c3 += key >= k3;
+      });
+      c1 = block_sum_int(c1, iscratch); c2 = block_sum_int(c2, iscratch); c3 = block_sum_int(c3, iscratch);
+      j_lo += stride * ((c1 >= k) + (c2 >= k) + (c3 >= k));
+    } else {
+      float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+      for_range<VEC>(x, wbeg, wend, lane, [&](int, float v) {
+        const float zz = v * inv_t;
+        const uint32_t key = order_key(zz);
+        const float e = __builtin_amdgcn_exp2f((zz - m) * L2E);
+        a0 += e;
+        a1 += key >= k1 ? e : 0.f; a2 += key >= k2 ? e : 0.f; a3 += key >= k3 ? e : 0.f;
+      });
+      // the sum over all values is taken exactly as the pass over the whole vocabulary takes it
+      if (round == 0) all_weight = block_sum(a0, fscratch);
+      a1 = block_sum(a1, fscratch); a2 = block_sum(a2, fscratch); a3 = block_sum(a3, fscratch);
+      const float need = p * all_weight * 1.001f;
+      j_lo += stride * ((a1 >= need) + (a2 >= need) + (a3 >= need));
+    }
   }
   const uint32_t key_thr = order_key(m - exp2f((float)(5 - j_lo)));
   // 2. gather, in index order: a wave walks its range and appends what it keeps to its segment
@@ -167,19 +189,22 @@ __device__ int sample_small_k(const float* __restrict__ x, int wbeg, int wend, f
   int n_all = 0;
   bool bad = false;
   for (int w = 0; w < nwaves; ++w) { bad = bad || cand.n[w] < 0; n_all += cand.n[w] < 0 ? 0 : cand.n[w]; }
-  if (bad || n_all < k) return -1;
-  // the candidates side by side (still in index order): from here on every wave does the same work on
-  // the whole list with reductions inside the wave, so no barrier is needed and all agree
+  if (bad || n_all < (by_count ? k : 1)) return -1;
+  // the candidates side by side (still in index order) with their weights; the rest is the work of
+  // one wave, with reductions inside the wave
+#define E_OF(zz) __builtin_amdgcn_exp2f(((zz) - m) * L2E)
   {
     int off = 0;
     for (int w = 0; w < wave; ++w) off += cand.n[w];
     for (int j = lane; j < cand.n[wave]; j += WAVE) {
-      cand.lz[off + j] = cand.z[wave * SEG + j];
+      const float zz = cand.z[wave * SEG + j];
+      cand.lz[off + j] = zz;
+      cand.le[off + j] = E_OF(zz);
       cand.lidx[off + j] = cand.idx[wave * SEG + j];
     }
   }
   __syncthreads();
-#define E_OF(zz) __builtin_amdgcn_exp2f(((zz) - m) * L2E)
+  auto list_phase = [&]() -> int {
   auto count_if = [&](auto pred) {
     int c = 0;
     for (int j = lane; j < n_all; j += WAVE) c += pred(cand.lz[j]);
@@ -190,14 +215,13 @@ __device__ int sample_small_k(const float* __restrict__ x, int wbeg, int wend, f
   auto mass_if = [&](auto pred) {
     float a = 0.f;
     for (int j = lane; j < n_all; j += WAVE) {
-      const float zz = cand.lz[j];
-      if (pred(zz)) a += E_OF(zz);
+      if (pred(cand.lz[j])) a += cand.le[j];
     }
     return wave_sum(a);
   };
   // 3. top-k: the largest key v with #{key >= v} >= k; all such keys are candidates
-  uint32_t kmin;
-  {
+  uint32_t kmin = key_thr;
+  if (by_count) {
     uint32_t lo = key_thr, hi = key_max;
     while (lo < hi) {
       const uint32_t mid = lo + (hi - lo + 1) / 2;
@@ -205,9 +229,11 @@ __device__ int sample_small_k(const float* __restrict__ x, int wbeg, int wend, f
     }
     kmin = lo;
   }
-  // 4. top-p on what top-k left
+  // 4. top-p on what top-k left (without top-k: on everything, and the candidates must hold the nucleus)
   if (p > 0.f && p < 1.f) {
-    const float bound = p * mass_if([&](float zz) { return order_key(zz) >= kmin; });
+    const float listed = mass_if([&](float zz) { return order_key(zz) >= kmin; });
+    const float bound = p * (by_count ? listed : all_weight);
+    if (!by_count && listed < bound) return -1;
     uint32_t lo = kmin, hi = key_max;
     while (lo < hi) {
       const uint32_t mid = lo + (hi - lo) / 2;
@@ -218,9 +244,8 @@ __device__ int sample_small_k(const float* __restrict__ x, int wbeg, int wend, f
   // 5. min-p and the draw: a walk along the list, 64 candidates at a time
   auto weight = [&](int j) {
     if (j >= n_all) return 0.f;
-    const float zz = cand.lz[j];
-    const float e = E_OF(zz);
-    return (order_key(zz) >= kmin && e >= mp) ? e : 0.f;
+    const float e = cand.le[j];
+    return (order_key(cand.lz[j]) >= kmin && e >= mp) ? e : 0.f;
   };
   float total = 0.f;
   for (int j = lane; j < n_all; j += WAVE) total += weight(j);
@@ -243,8 +268,15 @@ __device__ int sample_small_k(const float* __restrict__ x, int wbeg, int wend, f
     run += __shfl(incl, WAVE - 1, WAVE);
   }
   if (token < 0) token = last_kept < 0 ? 0 : last_kept;   // rounding pushed the target past the total: the last index kept
-#undef E_OF
   return token;
+  };
+  if (wave == 0) {
+    const int token = list_phase();
+    if (lane == 0) cand.result = token;
+  }
+  __syncthreads();
+#undef E_OF
+  return cand.result;
 }
 
 // Each wave owns a contiguous range of the vocabulary, so sums over a wave's range are sums over
@@ -302,10 +334,11 @@ sample_kernel(const float* __restrict__ logits, int V, int ld, const float* __re
 #define E_OF(z) __builtin_amdgcn_exp2f(((z) - m) * L2E)
 
   const int k = top_k[row];
-  if (k > 0 && k < V && k <= SMALL_K_MAX && blockDim.x == SAMPLE_THREADS) {
+  const bool top_k_on = k > 0 && k < V, top_p_on = top_p[row] > 0.f && top_p[row] < 1.f;
+  if (((top_k_on && k <= SMALL_K_MAX) || (!top_k_on && top_p_on)) && blockDim.x == SAMPLE_THREADS) {
     const uint64_t seed = ((uint64_t)seed_hi[row] << 32) | (uint64_t)seed_lo[row];
-    const int token = sample_small_k<VEC>(x, wbeg, wend, inv_t, m, k, top_p[row], min_p[row],
-                                          uniform_from_seed(seed, (uint32_t)position[row]), cand, iscratch);
+    const int token = sample_small_k<VEC>(x, wbeg, wend, inv_t, m, top_k_on ? k : 0, top_p[row], min_p[row],
+                                          uniform_from_seed(seed, (uint32_t)position[row]), cand, fscratch, iscratch);
     if (token >= 0) {
       if (tid == 0) out[row] = token;
       return;
