@@ -50,6 +50,8 @@ def parse_args():
     ap.add_argument("--prompt-len", type=int, default=1024)
     ap.add_argument("--context-len", type=int, default=4096)
     ap.add_argument("--dtype", default="bfloat16")
+    ap.add_argument("--top-k", type=int, default=-1, help="top-k of the decode requests (default: off)")
+    ap.add_argument("--top-p", type=float, default=1.0, help="top-p of the decode requests (default: off)")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 points and the prefill")
     ap.add_argument("--eager", action="store_true", help="no HIP graphs")
     ap.add_argument("--size", choices=sorted(SIZES), default=None,
@@ -218,7 +220,7 @@ def main():
         print(json.dumps({"prefill": {"value": round(p_tok_s, 1), "tokens": args.prefill_only, "ms": round(p_ms, 3),
                                       "frac": round(p_frac, 4)}}))
         return 0
-    tok_s, ms, bytes_step = run_decode(args.batch, args.steps, args.warmup)
+    tok_s, ms, bytes_step = run_decode(args.batch, args.steps, args.warmup, args.top_k, args.top_p)
     achieved = bytes_step / (ms * 1e-3) / 1e9
     line = {
         "metric": f"decode tok/s at bs {args.batch} (also bs 1/64, prefill tok/s at 2048; % of roofline), Qwen3-{args.size}",
@@ -230,7 +232,7 @@ def main():
                    "num_attention_heads": cfg.num_attention_heads, "num_key_value_heads": cfg.num_key_value_heads,
                    "head_dim": cfg.head_dim, "intermediate_size": cfg.intermediate_size, "vocab_size": cfg.vocab_size,
                    "global_batch": args.batch, "prompt_len": args.prompt_len, "seq_len": args.context_len,
-                   "page_size": 16, "sampling": "temperature 0.6, seeded", "parallelism": "single GPU",
+                   "page_size": 16, "sampling": "temperature 0.6, seeded" + (f", top-k {args.top_k}" if args.top_k > 0 else "") + (f", top-p {args.top_p}" if args.top_p < 1 else ""), "parallelism": "single GPU",
                    "hip_graphs": not args.eager},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4)},
@@ -241,7 +243,7 @@ def main():
         b1, _, _ = run_decode(1, min(args.steps, 32), min(args.warmup, 4))
         b64, _, _ = run_decode(64, min(args.steps, 32), min(args.warmup, 4))
         # the same batch with the sampling of Qwen3's generation_config.json (top-k 20, top-p 0.95)
-        b8f, _, _ = run_decode(args.batch, min(args.steps, 32), min(args.warmup, 4), top_k=20, top_p=0.95)
+        b8f, _, _ = run_decode(args.batch, args.steps, args.warmup, top_k=20, top_p=0.95)
         line["points"] = {"decode_b1": round(b1, 2), "decode_b64": round(b64, 2),
                           f"decode_b{args.batch}_top_k20_top_p95": round(b8f, 2)}
         del model
