@@ -650,7 +650,7 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __r
   constexpr int NG = PREFILL_GROUPS;
   constexpr int TILE_BYTES = S::KBYTES + S::VBYTES;
   constexpr int PER_LANE = NG * (8 * NQK + 2);            // floats a lane hands over in the merge
-  static_assert(KS == 1 || 2 * PER_LANE * 64 * 4 <= 2 * TILE_BYTES, "the merge reuses the tiles' memory");
+  static_assert(KS == 1 || PREFILL_WAVES * PER_LANE * 64 * 4 <= KS * 2 * TILE_BYTES, "the merge reuses the tiles' memory");
   __shared__ __attribute__((aligned(16))) unsigned char lds[KS * 2 * TILE_BYTES];   // [half][even | odd tile]
   const int wave_id = (int)(threadIdx.x >> 6);
   const int lane = threadIdx.x & 63, wave = wave_id % PREFILL_WAVES, half = wave_id / PREFILL_WAVES;
@@ -765,38 +765,34 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __r
 #undef STAGE_LOAD
 #undef STAGE_WORK
   if (KS == 2) {
-    // waves 4..7 hand over to waves 0..3, two at a time through the tiles' memory, lane by lane
-    float* buf = reinterpret_cast<float*>(lds);
+    // waves 4..7 hand over to waves 0..3 through the tiles' memory (free since the loop's last barrier),
+    // lane by lane
+    float* w = reinterpret_cast<float*>(lds) + (size_t)wave * PER_LANE * 64 + lane;
+    if (half == 1) {
 #pragma unroll
-    for (int r = 0; r < PREFILL_WAVES / 2; ++r) {
-      __syncthreads();
-      float* w = buf + (size_t)(wave & 1) * PER_LANE * 64 + lane;
-      if (half == 1 && (wave >> 1) == r) {
+      for (int qg = 0; qg < NG; ++qg) {
 #pragma unroll
-        for (int qg = 0; qg < NG; ++qg) {
+        for (int n = 0; n < 2 * NQK; ++n)
 #pragma unroll
-          for (int n = 0; n < 2 * NQK; ++n)
-#pragma unroll
-            for (int e = 0; e < 4; ++e) w[(qg * (8 * NQK + 2) + 4 * n + e) * 64] = acc[qg][n][e];
-          w[(qg * (8 * NQK + 2) + 8 * NQK) * 64] = m[qg];
-          w[(qg * (8 * NQK + 2) + 8 * NQK + 1) * 64] = l[qg];
-        }
+          for (int e = 0; e < 4; ++e) w[(qg * (8 * NQK + 2) + 4 * n + e) * 64] = acc[qg][n][e];
+        w[(qg * (8 * NQK + 2) + 8 * NQK) * 64] = m[qg];
+        w[(qg * (8 * NQK + 2) + 8 * NQK + 1) * 64] = l[qg];
       }
-      __syncthreads();
-      if (half == 0 && (wave >> 1) == r) {
+    }
+    __syncthreads();
+    if (half == 0) {
 #pragma unroll
-        for (int qg = 0; qg < NG; ++qg) {
-          const float m_b = w[(qg * (8 * NQK + 2) + 8 * NQK) * 64], l_b = w[(qg * (8 * NQK + 2) + 8 * NQK + 1) * 64];
-          const float M = fmaxf(m[qg], m_b);
-          const float fa = fast_exp2(m[qg] - M), fb = fast_exp2(m_b - M);
+      for (int qg = 0; qg < NG; ++qg) {
+        const float m_b = w[(qg * (8 * NQK + 2) + 8 * NQK) * 64], l_b = w[(qg * (8 * NQK + 2) + 8 * NQK + 1) * 64];
+        const float M = fmaxf(m[qg], m_b);
+        const float fa = fast_exp2(m[qg] - M), fb = fast_exp2(m_b - M);
 #pragma unroll
-          for (int n = 0; n < 2 * NQK; ++n)
+        for (int n = 0; n < 2 * NQK; ++n)
 #pragma unroll
-            for (int e = 0; e < 4; ++e)
-              acc[qg][n][e] = acc[qg][n][e] * fa + w[(qg * (8 * NQK + 2) + 4 * n + e) * 64] * fb;
-          l[qg] = l[qg] * fa + l_b * fb;
-          m[qg] = M;
-        }
+          for (int e = 0; e < 4; ++e)
+            acc[qg][n][e] = acc[qg][n][e] * fa + w[(qg * (8 * NQK + 2) + 4 * n + e) * 64] * fb;
+        l[qg] = l[qg] * fa + l_b * fb;
+        m[qg] = M;
       }
     }
     if (half == 1) return;
