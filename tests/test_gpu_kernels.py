@@ -505,6 +505,43 @@ def test_gemm_skinny(ops, shape, out_dtype):
     assert torch.equal(got2, got)
 
 
+@pytest.mark.parametrize("shape", [(17, 256, 512), (33, 100, 4104), (48, 4100, 72), (64, 640, 2048), (5, 128, 8),
+                                   (64, 4096, 1032), (40, 24, 12288)])
+def test_gemm_partial_sums(ops, shape):
+    """The product for 17 to 64 rows as a stack of partial sums over slices of K, and the add + norm
+    kernel that adds the stack."""
+    torch.manual_seed(12)
+    M, N, K = shape
+    a = torch.randn(M, K, device=DEV).bfloat16()
+    w = (torch.randn(N, K, device=DEV) * 0.2).bfloat16()
+    want = a.double().cpu() @ w.double().cpu().T
+    stack = ops.gemm_partial_sums(a, w)
+    assert stack.dtype == torch.float32 and stack.shape[1:] == (M, N) and stack.shape[0] >= 1
+    assert (stack.sum(0).double().cpu() - want).abs().max() <= 2e-5 * float(want.abs().max()) + 1e-6
+    assert torch.equal(ops.gemm_partial_sums(a, w), stack)                     # repeatable bit for bit
+    fewer = ops.gemm_partial_sums(a[:M // 2 + 1], w)                             # the slices follow the matrix, not the batch
+    assert fewer.shape[0] == stack.shape[0] and torch.equal(fewer, stack[:, :M // 2 + 1])
+    # strided activations (a column slice of a wider buffer)
+    wide = torch.randn(M, K + 64, device=DEV).bfloat16()
+    wide[:, 32:32 + K] = a
+    assert torch.equal(ops.gemm_partial_sums(wide[:, 32:32 + K], w), stack)
+    # the norm adds the stack, in order, into the 32-bit stream
+    for out_dtype in (torch.bfloat16, torch.float32):
+        stream = torch.randn(M, N, device=DEV)
+        gain = (1 + 0.2 * torch.randn(N)).to(DEV)
+        total = stream.clone()
+        for part in stack:
+            total += part
+        y = ops.add_rmsnorm(stack, stream, gain, 1e-5, out_dtype)
+        assert torch.equal(stream, total)
+        ref = plain.rms_norm(total.cpu(), gain.cpu(), 1e-5)
+        assert (y.float().cpu() - ref).abs().max() <= tol(out_dtype, ref)
+        rows = torch.tensor([M - 1, 0], dtype=torch.int32, device=DEV)          # selected rows: the stream stays
+        y2 = ops.add_rmsnorm(stack, stream, gain, 1e-5, out_dtype, rows=rows)
+        ref2 = plain.rms_norm((total + stack.sum(0)).cpu()[[M - 1, 0]], gain.cpu(), 1e-5)
+        assert torch.equal(stream, total) and (y2.float().cpu() - ref2).abs().max() <= tol(out_dtype, ref2)
+
+
 def test_gemm_dispatch_refuses_nothing_silently(ops):
     a = torch.randn(4, 20, device=DEV).bfloat16()          # K not a multiple of 8: the general kernel takes it
     w = torch.randn(6, 20, device=DEV).bfloat16()

@@ -57,7 +57,8 @@ extern "C" int ullm_embedding(const int* ids, const void* table, float* residual
 
 // ------------------------------------------------------------------ add + RMS norm
 // For output row r (input row i = rows ? rows[r] : r):
-//   s = residual[i] + float(branch[i])      (branch may be null: s = residual[i])
+//   s = residual[i] + float(branch[i])      (branch may be null: s = residual[i]; it may also be a stack
+//                                            of n_branch arrays branch_stride apart, added in order)
 //   if write_res: residual[i] = s           (the stream stays 32-bit, never rounded)
 //   y[r] = s * rsqrt(mean(s^2) + eps) * gain
 // One block per row.  The general kernel walks the row twice with scalar loads; the fast one
@@ -66,7 +67,8 @@ extern "C" int ullm_embedding(const int* ids, const void* table, float* residual
 template <typename TB, typename TY>
 __global__ void add_rmsnorm_kernel(const TB* __restrict__ branch, float* __restrict__ residual,
                                    const float* __restrict__ gain, float eps, TY* __restrict__ y,
-                                   const int* __restrict__ rows, int H, int write_res) {
+                                   const int* __restrict__ rows, int H, int write_res, int n_branch,
+                                   long long branch_stride) {
   __shared__ float scratch[16];
   const int r = blockIdx.x;
   const int i = rows ? rows[r] : r;
@@ -75,7 +77,8 @@ __global__ void add_rmsnorm_kernel(const TB* __restrict__ branch, float* __restr
   float ss = 0.f;
   for (int c = threadIdx.x; c < H; c += blockDim.x) {
     float s = res[c];
-    if (br) s += ld_f32(br + c);
+    if (br)
+      for (int p = 0; p < n_branch; ++p) s += ld_f32(br + (size_t)p * branch_stride + c);
     if (write_res && br) res[c] = s;
     ss += s * s;
   }
@@ -84,7 +87,8 @@ __global__ void add_rmsnorm_kernel(const TB* __restrict__ branch, float* __restr
   TY* out = y + (size_t)r * H;
   for (int c = threadIdx.x; c < H; c += blockDim.x) {
     float s = res[c];
-    if (br && !write_res) s += ld_f32(br + c);
+    if (br && !write_res)
+      for (int p = 0; p < n_branch; ++p) s += ld_f32(br + (size_t)p * branch_stride + c);
     st_f32(out + c, (s * rs) * gain[c]);
   }
 }
@@ -93,7 +97,8 @@ __global__ void add_rmsnorm_kernel(const TB* __restrict__ branch, float* __restr
 template <typename TB, typename TY>
 __global__ void add_rmsnorm_vec_kernel(const TB* __restrict__ branch, float* __restrict__ residual,
                                        const float* __restrict__ gain, float eps, TY* __restrict__ y,
-                                       const int* __restrict__ rows, int H, int write_res) {
+                                       const int* __restrict__ rows, int H, int write_res, int n_branch,
+                                       long long branch_stride) {
   __shared__ float scratch[16];
   const int r = blockIdx.x;
   const int i = rows ? rows[r] : r;
@@ -107,8 +112,10 @@ __global__ void add_rmsnorm_vec_kernel(const TB* __restrict__ branch, float* __r
     if (c < H) {
       float4 s = ld4_f32(res + c);
       if (br) {
-        const float4 b = ld4_f32(br + c);
-        s.x += b.x; s.y += b.y; s.z += b.z; s.w += b.w;
+        for (int p = 0; p < n_branch; ++p) {
+          const float4 b = ld4_f32(br + (size_t)p * branch_stride + c);
+          s.x += b.x; s.y += b.y; s.z += b.z; s.w += b.w;
+        }
         if (write_res) st4_f32(res + c, s);
       }
       v[j] = s;
@@ -129,18 +136,19 @@ __global__ void add_rmsnorm_vec_kernel(const TB* __restrict__ branch, float* __r
 
 extern "C" int ullm_add_rmsnorm(const void* branch, float* residual, const float* gain, float eps,
                                 void* y, const int* rows, int n_rows, int H, int branch_dtype,
-                                int y_dtype, int write_res, hipStream_t stream) {
+                                int y_dtype, int write_res, int n_branch, long long branch_stride,
+                                hipStream_t stream) {
   if (n_rows <= 0) return 0;
-  if (H <= 0) return ULLM_ERR_SHAPE;
+  if (H <= 0 || n_branch < 1 || (n_branch > 1 && branch_stride % 4 != 0)) return ULLM_ERR_SHAPE;
   if (rows && write_res) return ULLM_ERR_UNSUPPORTED;  // a gathered row could be updated twice
   const int threads = H >= 4096 ? 512 : 256;
   const bool vec = H % 4 == 0 && H <= 4 * NORM_VEC_MAX * threads && !(((uintptr_t)residual | (uintptr_t)gain |
                    (uintptr_t)y | (uintptr_t)branch) & 15);
   dim3 grid(n_rows), block(threads);
 #define GO(TB, TY) do { if (vec) hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TB, TY>), grid, block, 0, stream, \
-    (const TB*)branch, residual, gain, eps, (TY*)y, rows, H, write_res); \
+    (const TB*)branch, residual, gain, eps, (TY*)y, rows, H, write_res, n_branch, branch_stride); \
   else hipLaunchKernelGGL((add_rmsnorm_kernel<TB, TY>), grid, block, 0, stream, \
-    (const TB*)branch, residual, gain, eps, (TY*)y, rows, H, write_res); } while (0)
+    (const TB*)branch, residual, gain, eps, (TY*)y, rows, H, write_res, n_branch, branch_stride); } while (0)
   if (branch_dtype == ULLM_F32 && y_dtype == ULLM_F32) GO(float, float);
   else if (branch_dtype == ULLM_BF16 && y_dtype == ULLM_BF16) GO(bf16_t, bf16_t);
   else if (branch_dtype == ULLM_BF16 && y_dtype == ULLM_F32) GO(bf16_t, float);

@@ -44,6 +44,8 @@ class ModelRunner:
         if model.env is None:
             raise StepError("the model has no weights bound")
         self.model, self.env = model, env
+        # may mixers and feed-forwards hand the next norm a stack of partial sums?  Only if every norm adds one up
+        self._stacked_branches = all(getattr(part, "adds_stacks", False) for part in model.parts() if part.kind == "norm")
         self.page_size = page_size
         self.max_requests = max_requests
         groups, cache_group, states = model.cache_layout()
@@ -225,7 +227,7 @@ class ModelRunner:
             decode_tokens=view(7 + ng) if facts["num_decode"] else None, num_decode=facts["num_decode"],
             max_decode_kv=facts["max_dec_kv"], tiles=view(8 + ng).view(-1, 2) if facts["num_tiles"] else None,
             num_tiles=facts["num_tiles"], tile_keys_total=facts["tile_keys_total"],
-            tile_keys_max=facts["tile_keys_max"],
+            tile_keys_max=facts["tile_keys_max"], stacked_branches=self._stacked_branches,
             host={"lens": facts["lens"], "starts": facts["starts"], "slots": facts["slots"]})
         return ctx, (view(6) if facts["n_want"] else None)
 

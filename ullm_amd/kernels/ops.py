@@ -90,12 +90,17 @@ def add_rmsnorm(branch: Optional[torch.Tensor], residual: torch.Tensor, gain: to
                 out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """residual (float32 [T, H], updated in place unless ``rows``) += branch; returns the RMS-normed
     sum times ``gain`` (float32 [H]) in ``out_dtype``.  With ``rows`` (int32 [n]) only those rows are
-    produced and the residual stays untouched."""
+    produced and the residual stays untouched.  ``branch`` may be a stack [S, T, H] of partial sums
+    (see :func:`gemm_partial_sums`): they are added in order."""
     T, H = residual.shape
     _need(residual.dtype == torch.float32 and residual.is_contiguous(), "residual must be contiguous float32")
     _need(gain.dtype == torch.float32 and gain.numel() == H and gain.is_contiguous(), "gain must be float32 [H]")
+    n_branch, branch_stride = 1, 0
     if branch is not None:
-        _need(branch.shape == (T, H) and branch.is_contiguous(), "branch must be contiguous [T, H]")
+        _need(branch.shape[-2:] == (T, H) and branch.dim() in (2, 3) and branch.is_contiguous(),
+              "branch must be contiguous [T, H] or a stack [S, T, H]")
+        if branch.dim() == 3:
+            n_branch, branch_stride = branch.shape[0], T * H
     n = T
     if rows is not None:
         _i32(rows, "rows")
@@ -107,7 +112,8 @@ def add_rmsnorm(branch: Optional[torch.Tensor], residual: torch.Tensor, gain: to
     bdt = _dt(branch) if branch is not None else _dt(out)
     _check(lib.ullm_add_rmsnorm(_p(branch), _p(residual), _p(gain), _c_float(eps), _p(out), _p(rows),
                                 _c_int(n), _c_int(H), _c_int(bdt), _c_int(_dt(out)),
-                                _c_int(0 if rows is not None else 1), _stream()), "add_rmsnorm")
+                                _c_int(0 if rows is not None else 1), _c_int(n_branch),
+                                ctypes.c_longlong(branch_stride), _stream()), "add_rmsnorm")
     return out
 
 
@@ -274,6 +280,33 @@ def gemm_skinny_silu(a: torch.Tensor, w_gate_up: torch.Tensor, nt: int = 0, wave
     _need(a.dtype == torch.bfloat16 and _skinny_ok(M, K, a, w_gate_up), "gemm_skinny_silu takes bfloat16 [M <= 64, K]")
     out = torch.empty((M, two_i // 2), dtype=torch.bfloat16, device=a.device)
     _gemm_skinny(a, w_gate_up, None, out, M, two_i // 2, K, 2, BF16, nt, waves)
+    return out
+
+
+PARTIAL_SUMS_MAX_ROWS = 64
+
+
+def gemm_partial_sums_supports(a: torch.Tensor, w: torch.Tensor) -> bool:
+    M, K = a.shape
+    return (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and a.stride(1) == 1 and w.stride(1) == 1
+            and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0 and w.shape[1] == K
+            and bool(build.load("gemm_mid").ullm_gemm_partial_sums_supports(
+                _c_int(M), _c_int(w.shape[0]), _c_int(K), _c_int(a.stride(0)), _c_int(w.stride(0)))))
+
+
+def gemm_partial_sums(a: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """a (bfloat16 [M <= 64, K]) times w (bfloat16 [N, K]) transposed as a stack [S, M, N] of float32
+    partial sums over S slices of K; the product is their sum.  S depends on the matrix alone.  For
+    17 to 64 rows of the projections that end in the residual stream: the add + norm kernel adds the
+    stack (:func:`add_rmsnorm`), so the slices cost no kernel of their own."""
+    M, K = a.shape
+    N = w.shape[0]
+    _need(gemm_partial_sums_supports(a, w), "gemm_partial_sums takes bfloat16, M <= 64, K a multiple of 8, N of 4")
+    lib = build.load("gemm_mid")
+    slices = int(lib.ullm_gemm_partial_sums_slices(_c_int(N), _c_int(K)))
+    out = torch.empty((slices, M, N), dtype=torch.float32, device=a.device)
+    _check(lib.ullm_gemm_partial_sums(_p(a), _c_int(a.stride(0)), _p(w), _c_int(w.stride(0)), _p(out), _c_int(M),
+                                      _c_int(N), _c_int(K), _stream()), "gemm_partial_sums")
     return out
 
 

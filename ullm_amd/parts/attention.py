@@ -14,7 +14,7 @@ import torch
 
 from ..kernels import ops
 from .base import KVNeed, LayerCache, Mixer, PartEnv, PositionEncoding, StepContext, WeightDecl, register_part
-from .linear import can_fuse, linear
+from .linear import can_fuse, linear, linear_into_stream
 
 
 @register_part("mixer", "gqa_attention")
@@ -68,7 +68,7 @@ class GQAttention(Mixer):
             self.k_gain = tensors[f"{p}.k_norm.weight"].contiguous()
 
     def forward(self, x: torch.Tensor, ctx: StepContext, cache: LayerCache) -> torch.Tensor:
-        return linear(self._attend(linear(x, self.w_qkv, self.b_qkv), ctx, cache), self.w_o)
+        return linear_into_stream(self._attend(linear(x, self.w_qkv, self.b_qkv), ctx, cache), self.w_o, ctx)
 
     def fusable(self, residual, ctx: StepContext) -> bool:
         return can_fuse(residual, ctx.dtype, self.w_qkv, self.w_o)

@@ -94,6 +94,9 @@ class StepContext:
     num_tiles: int = 0
     tile_keys_total: int = 0      # sum over the tiles of the keys each tile's last token sees
     tile_keys_max: int = 0        # the most keys any tile sees (both: how the tiles' work is spread)
+    # every norm of the model takes a stack [S, T, hidden] of float32 partial sums as its branch and
+    # adds them up (Norm.adds_stacks): a mixer or feed-forward may then return such a stack
+    stacked_branches: bool = False
 
 
 # --------------------------------------------------------------------------- parts
@@ -158,8 +161,11 @@ class FeedForward(Part):
 
 class Norm(Part):
     """``add_norm(branch, residual, rows) -> normed``: adds the branch output (if any) into
-    the 32-bit residual stream, then normalises the sum; ``rows`` selects output rows."""
+    the 32-bit residual stream, then normalises the sum; ``rows`` selects output rows.
+    ``adds_stacks``: the branch may also be a stack [S, T, hidden] of float32 partial sums, which
+    the norm adds in order."""
     kind = "norm"
+    adds_stacks = False
 
     def add_norm(self, branch: Optional[torch.Tensor], residual: torch.Tensor,
                  rows: Optional[torch.Tensor] = None, out_dtype: torch.dtype = None) -> torch.Tensor:

@@ -10,7 +10,7 @@ import torch
 
 from ..kernels import ops
 from .base import FeedForward, PartEnv, StepContext, WeightDecl, register_part
-from .linear import can_fuse, linear
+from .linear import can_fuse, linear, linear_into_stream
 
 
 @register_part("ffn", "swiglu")
@@ -31,7 +31,7 @@ class SwiGLU(FeedForward):
         self.w_down = tensors[f"{p}.down_proj.weight"].contiguous()
 
     def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
-        return linear(ops.silu_mul(linear(x, self.w_gate_up)), self.w_down)
+        return linear_into_stream(ops.silu_mul(linear(x, self.w_gate_up)), self.w_down, ctx)
 
     def fusable(self, residual, ctx: StepContext) -> bool:
         return can_fuse(residual, ctx.dtype, self.w_gate_up, self.w_down)

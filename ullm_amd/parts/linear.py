@@ -31,3 +31,17 @@ def can_fuse(residual: torch.Tensor, dtype: torch.dtype, *weights: torch.Tensor)
         return False
     return all(w.dtype == torch.bfloat16 and w.shape[1] % 8 == 0 and w.shape[0] % 4 == 0 and w.data_ptr() % 16 == 0
                for w in weights)
+
+
+STACKED_MIN_ROWS, STACKED_MAX_ROWS = 17, 64
+
+
+def linear_into_stream(x: torch.Tensor, weight: torch.Tensor, ctx) -> torch.Tensor:
+    """The last projection of a mixer or feed-forward, whose result the next norm adds to the residual
+    stream.  For 17 to 64 rows in bfloat16, where the model's norms add stacks, it is a stack of
+    float32 partial sums over slices of the inner dimension (the slices fill the chip, the norm adds
+    them in order); otherwise the plain product."""
+    if (ctx.stacked_branches and x.dtype == torch.bfloat16 and STACKED_MIN_ROWS <= x.shape[0] <= STACKED_MAX_ROWS
+            and ops.gemm_partial_sums_supports(x, weight)):
+        return ops.gemm_partial_sums(x, weight)
+    return linear(x, weight)

@@ -16,6 +16,8 @@ from .base import Norm, PartEnv, WeightDecl, register_part
 
 @register_part("norm", "rmsnorm")
 class RMSNorm(Norm):
+    adds_stacks = True
+
     def __init__(self, size: int, eps: float, weight_name: str):
         self.size = size
         self.eps = float(eps)
@@ -29,5 +31,6 @@ class RMSNorm(Norm):
         self.gain = tensors[self.weight_name].contiguous()
 
     def add_norm(self, branch, residual, rows=None, out_dtype=None):
-        return ops.add_rmsnorm(branch, residual, self.gain, self.eps,
-                               out_dtype or (branch.dtype if branch is not None else torch.float32), rows=rows)
+        if out_dtype is None:
+            out_dtype = branch.dtype if branch is not None and branch.dim() == 2 else torch.float32
+        return ops.add_rmsnorm(branch, residual, self.gain, self.eps, out_dtype, rows=rows)
