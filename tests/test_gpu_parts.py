@@ -161,6 +161,33 @@ def test_norm_part_and_block_wiring(dtype):
     assert (y.float().cpu() - want).abs().max() <= tol(dtype, want)
 
 
+def test_feed_forward_hands_the_norm_a_stack_of_partial_sums():
+    """For 17 to 64 rows in bfloat16 the last projection of a feed-forward comes as a stack of float32
+    partial sums if every norm of the model adds stacks; the norm's sum is the plain result."""
+    from types import SimpleNamespace
+    from ullm_amd.parts import PartEnv, build_part
+    torch.manual_seed(5)
+    H, I = 96, 224
+    env = PartEnv(torch.device(DEV), torch.bfloat16, 16)
+    ffn = build_part("ffn", "swiglu", hidden_size=H, intermediate_size=I, prefix="f")
+    w = {f"f.{n}.weight": (torch.randn(*shape) * 0.1).bfloat16().to(DEV)
+         for n, shape in (("gate_proj", (I, H)), ("up_proj", (I, H)), ("down_proj", (H, I)))}
+    ffn.bind(w, env)
+    norm = build_part("norm", "rmsnorm", size=H, eps=1e-5, weight_name="g")
+    norm.bind({"g": torch.ones(H, device=DEV)}, env)
+    assert norm.adds_stacks
+    for T, stacked in ((40, True), (16, False), (65, False)):
+        x = torch.randn(T, H).bfloat16().to(DEV)
+        plain_out = ffn.forward(x, SimpleNamespace(stacked_branches=False, dtype=torch.bfloat16))
+        out = ffn.forward(x, SimpleNamespace(stacked_branches=True, dtype=torch.bfloat16))
+        assert (out.dim() == 3) == stacked and plain_out.dim() == 2
+        a, b = torch.zeros(T, H, device=DEV), torch.zeros(T, H, device=DEV)
+        ya = norm.add_norm(out, a, out_dtype=torch.bfloat16)
+        yb = norm.add_norm(plain_out, b, out_dtype=torch.bfloat16)
+        assert (a - b).abs().max() <= 1e-2 * b.abs().max()        # the plain result is rounded to bfloat16, the stack is not
+        assert (ya.float() - yb.float()).abs().max() <= 3e-2 * yb.float().abs().max()
+
+
 def test_rotary_part_table_matches_the_plain_angles():
     from ullm_amd.parts import PartEnv, build_part
     rot = build_part("position", "rotary", head_dim=24, theta=777.0, rotary_dim=12, pairing="half")
