@@ -13,6 +13,9 @@ from .base import FeedForward, PartEnv, StepContext, WeightDecl, register_part
 from .linear import can_fuse, linear, linear_into_stream
 
 
+GATE_UP_SKINNY_MAX_ROWS = 32     # measured on Qwen3-8B's matrix; from 33 rows on the library product is faster
+
+
 @register_part("ffn", "swiglu")
 class SwiGLU(FeedForward):
     def __init__(self, hidden_size: int, intermediate_size: int, prefix: str):
@@ -31,7 +34,12 @@ class SwiGLU(FeedForward):
         self.w_down = tensors[f"{p}.down_proj.weight"].contiguous()
 
     def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
-        return linear_into_stream(ops.silu_mul(linear(x, self.w_gate_up)), self.w_down, ctx)
+        if (x.dtype == torch.bfloat16 and x.shape[0] <= GATE_UP_SKINNY_MAX_ROWS
+                and ops.gemm_skinny_supports(x, self.w_gate_up)):
+            act = ops.gemm_skinny_silu(x, self.w_gate_up)        # up to 32 rows: 43 us against the library's 45 + the activation's 5
+        else:
+            act = ops.silu_mul(linear(x, self.w_gate_up))
+        return linear_into_stream(act, self.w_down, ctx)
 
     def fusable(self, residual, ctx: StepContext) -> bool:
         return can_fuse(residual, ctx.dtype, self.w_gate_up, self.w_down)
