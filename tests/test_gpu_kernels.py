@@ -506,9 +506,10 @@ def test_gemm_skinny(ops, shape, out_dtype):
 
 
 @pytest.mark.parametrize("shape", [(17, 256, 512), (33, 100, 4104), (48, 4100, 72), (64, 640, 2048), (5, 128, 8),
-                                   (64, 4096, 1032), (40, 24, 12288)])
+                                   (64, 4096, 1032), (40, 24, 12288), (65, 260, 520), (100, 128, 1096), (129, 512, 264),
+                                   (200, 96, 4096), (256, 1032, 776)])
 def test_gemm_partial_sums(ops, shape):
-    """The product for 17 to 64 rows as a stack of partial sums over slices of K, and the add + norm
+    """The product for 17 to 256 rows as a stack of partial sums over slices of K, and the add + norm
     kernel that adds the stack."""
     torch.manual_seed(12)
     M, N, K = shape

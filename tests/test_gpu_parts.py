@@ -162,7 +162,7 @@ def test_norm_part_and_block_wiring(dtype):
 
 
 def test_feed_forward_hands_the_norm_a_stack_of_partial_sums():
-    """For 17 to 64 rows in bfloat16 the last projection of a feed-forward comes as a stack of float32
+    """For 17 to 256 rows in bfloat16 (its down projection has few long rows) the last projection of a feed-forward comes as a stack of float32
     partial sums if every norm of the model adds stacks; the norm's sum is the plain result."""
     from types import SimpleNamespace
     from ullm_amd.parts import PartEnv, build_part
@@ -176,7 +176,7 @@ def test_feed_forward_hands_the_norm_a_stack_of_partial_sums():
     norm = build_part("norm", "rmsnorm", size=H, eps=1e-5, weight_name="g")
     norm.bind({"g": torch.ones(H, device=DEV)}, env)
     assert norm.adds_stacks
-    for T, stacked in ((40, True), (16, False), (65, False)):
+    for T, stacked in ((40, True), (16, False), (200, True), (257, False)):
         x = torch.randn(T, H).bfloat16().to(DEV)
         plain_out = ffn.forward(x, SimpleNamespace(stacked_branches=False, dtype=torch.bfloat16))
         out = ffn.forward(x, SimpleNamespace(stacked_branches=True, dtype=torch.bfloat16))

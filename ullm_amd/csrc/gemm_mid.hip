@@ -1,4 +1,4 @@
-// P[s][M, N] = X[M, K(s)] * W[N, K(s)]^T for 17 to 64 rows: partial sums over S slices of K, 32-bit.
+// P[s][M, N] = X[M, K(s)] * W[N, K(s)]^T for 17 to 256 rows: partial sums over S slices of K, 32-bit.
 //
 // With this many rows a block that reads all of X for 16 rows of W (the few-rows kernel's shape)
 // fetches more of X than of W.  Here the 8 waves of a block take 16 rows of W each and share the
@@ -9,7 +9,8 @@
 // projections, 4096 to 8192 rows) then give 32 to 64 blocks, too few for the chip; K is therefore
 // cut into S slices, one per blockIdx.y, and every slice stores its own partial sum.  Who adds the
 // partial sums is the caller's business (the add + norm kernel takes a stack of them, in order, so
-// the result does not depend on timing).
+// the result does not depend on timing).  From 128 rows on the time is set by the shared-memory reads of X
+// (one matrix instruction per 16-byte read), still well ahead of what the library picks for these shapes.
 //
 // A operand of v_mfma_f32_16x16x32_bf16 = a W tile (lane (r, g) holds W[n0 + r][k + 8g .. +8]), B
 // operand = 16 rows of X.  Shared-memory rows are 128 bytes; piece c of row r lies at piece
@@ -137,7 +138,7 @@ extern "C" int ullm_gemm_partial_sums_slices(int N, int K) {
 }
 
 extern "C" int ullm_gemm_partial_sums_supports(int M, int N, int K, int ldx, int ldw) {
-  return M >= 1 && M <= 64 && N >= 4 && N % 4 == 0 && K >= 8 && K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0;
+  return M >= 1 && M <= 256 && N >= 4 && N % 4 == 0 && K >= 8 && K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0;
 }
 
 // X bfloat16 [M, K]; W bfloat16 [N, K]; P float32 [slices, M, N] with slices = ullm_gemm_partial_sums_slices(N, K).
@@ -155,7 +156,11 @@ extern "C" int ullm_gemm_partial_sums(const void* X, int ldx, const void* W, int
   if (M <= 16) GO(1);
   else if (M <= 32) GO(2);
   else if (M <= 48) GO(3);
-  else GO(4);
+  else if (M <= 64) GO(4);
+  else if (M <= 96) GO(6);
+  else if (M <= 128) GO(8);
+  else if (M <= 192) GO(12);
+  else GO(16);
 #undef GO
   ULLM_LAUNCH_CHECK();
 }

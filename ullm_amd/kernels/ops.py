@@ -283,7 +283,7 @@ def gemm_skinny_silu(a: torch.Tensor, w_gate_up: torch.Tensor, nt: int = 0, wave
     return out
 
 
-PARTIAL_SUMS_MAX_ROWS = 64
+PARTIAL_SUMS_MAX_ROWS = 256
 
 
 def gemm_partial_sums_supports(a: torch.Tensor, w: torch.Tensor) -> bool:
@@ -295,13 +295,13 @@ def gemm_partial_sums_supports(a: torch.Tensor, w: torch.Tensor) -> bool:
 
 
 def gemm_partial_sums(a: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
-    """a (bfloat16 [M <= 64, K]) times w (bfloat16 [N, K]) transposed as a stack [S, M, N] of float32
+    """a (bfloat16 [M <= 256, K]) times w (bfloat16 [N, K]) transposed as a stack [S, M, N] of float32
     partial sums over S slices of K; the product is their sum.  S depends on the matrix alone.  For
-    17 to 64 rows of the projections that end in the residual stream: the add + norm kernel adds the
+    17 to 256 rows of the projections that end in the residual stream: the add + norm kernel adds the
     stack (:func:`add_rmsnorm`), so the slices cost no kernel of their own."""
     M, K = a.shape
     N = w.shape[0]
-    _need(gemm_partial_sums_supports(a, w), "gemm_partial_sums takes bfloat16, M <= 64, K a multiple of 8, N of 4")
+    _need(gemm_partial_sums_supports(a, w), "gemm_partial_sums takes bfloat16, M <= 256, K a multiple of 8, N of 4")
     lib = build.load("gemm_mid")
     slices = int(lib.ullm_gemm_partial_sums_slices(_c_int(N), _c_int(K)))
     out = torch.empty((slices, M, N), dtype=torch.float32, device=a.device)
