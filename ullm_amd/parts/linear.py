@@ -43,8 +43,8 @@ def linear_into_stream(x: torch.Tensor, weight: torch.Tensor, ctx) -> torch.Tens
     stream.  For 17 to 128 rows in bfloat16 (to 256 for a matrix with few long rows), where the model's
     norms add stacks, it is a stack of float32 partial sums over slices of the inner dimension (the
     slices fill the chip, the norm adds them in order); otherwise the plain product.  Measured against
-    the library product at these shapes: down projection of Qwen3-8B / 14B / 32B at 128 rows 30 / 64 /
-    93 us against 63 / 147 / 180 us, output projection 14 / 21 / 29 us against 21 / 26 / 37 us."""
+    the library product at these shapes: down projection of Qwen3-8B / 14B / 32B at 128 rows 28 / 46 /
+    68 us against 63 / 147 / 180 us, output projection 14 / 18 / 24 us against 21 / 26 / 37 us."""
     T = x.shape[0]
     most = STACKED_MAX_ROWS_DEEP if weight.shape[1] >= 2 * weight.shape[0] else STACKED_MAX_ROWS
     if (ctx.stacked_branches and x.dtype == torch.bfloat16 and STACKED_MIN_ROWS <= T <= most
