@@ -33,21 +33,18 @@ def can_fuse(residual: torch.Tensor, dtype: torch.dtype, *weights: torch.Tensor)
                for w in weights)
 
 
-STACKED_MIN_ROWS = 17
-STACKED_MAX_ROWS = 128           # any matrix up to here
-STACKED_MAX_ROWS_DEEP = 256      # a matrix whose rows are at least twice as long as it has rows (the down projection)
+STACKED_MIN_ROWS, STACKED_MAX_ROWS = 17, 256
 
 
 def linear_into_stream(x: torch.Tensor, weight: torch.Tensor, ctx) -> torch.Tensor:
     """The last projection of a mixer or feed-forward, whose result the next norm adds to the residual
-    stream.  For 17 to 128 rows in bfloat16 (to 256 for a matrix with few long rows), where the model's
-    norms add stacks, it is a stack of float32 partial sums over slices of the inner dimension (the
-    slices fill the chip, the norm adds them in order); otherwise the plain product.  Measured against
-    the library product at these shapes: down projection of Qwen3-8B / 14B / 32B at 128 rows 28 / 46 /
-    68 us against 63 / 147 / 180 us, output projection 14 / 18 / 24 us against 21 / 26 / 37 us."""
-    T = x.shape[0]
-    most = STACKED_MAX_ROWS_DEEP if weight.shape[1] >= 2 * weight.shape[0] else STACKED_MAX_ROWS
-    if (ctx.stacked_branches and x.dtype == torch.bfloat16 and STACKED_MIN_ROWS <= T <= most
+    stream.  For 17 to 256 rows in bfloat16, where the model's norms add stacks, it is a stack of
+    float32 partial sums over slices of the inner dimension (the slices fill the chip, the norm adds
+    them in order); otherwise the plain product.  Measured against the library product at these
+    shapes: down projection of Qwen3-8B / 14B / 32B at 128 rows 28 / 46 / 68 us against 63 / 147 /
+    180 us, at 256 rows 41 / 72 / 103 us against 51 / 223 / 262 us; output projection at 128 rows
+    14 / 18 / 24 us against 21 / 26 / 37 us, at 256 rows 20 / 27 / 36 us against 20 / 45 / 69 us."""
+    if (ctx.stacked_branches and x.dtype == torch.bfloat16 and STACKED_MIN_ROWS <= x.shape[0] <= STACKED_MAX_ROWS
             and ops.gemm_partial_sums_supports(x, weight)):
         return ops.gemm_partial_sums(x, weight)
     return linear(x, weight)
