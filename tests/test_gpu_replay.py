@@ -146,6 +146,31 @@ def test_mixed_with_page_reuse(replayers, plain_models, name, dtype):
     assert reused                                                   # a later request got a page an ended one had used
 
 
+@pytest.mark.parametrize("name", ["B", "C"])
+def test_portions_whose_projections_come_as_stacks_of_partial_sums(model_dirs, plain_models, name, monkeypatch):
+    """Steps of 17 to 256 tokens hand the output and down projections to the next norm as stacks of
+    partial sums where the matrices are large; here the size limit is lifted so that the tiny model
+    takes that way too, beside steps that do not."""
+    from ullm_amd.parts import linear
+    from ullm_amd.replay import Replayer
+    monkeypatch.setattr(linear, "STACKED_MIN_WEIGHT", 0)
+    calls, inner = [], linear.ops.gemm_partial_sums
+    monkeypatch.setattr(linear.ops, "gemm_partial_sums", lambda x, w: calls.append(x.shape[0]) or inner(x, w))
+    rep = Replayer(model_dirs[name], "bfloat16", 512, 16, DEV)
+    vocab = plain_models[name][0]["vocab_size"]
+    toks = make_tokens(vocab, 250, 31)
+    want = oracle(plain_models, name, toks)
+    sizes = [17, 3, 64, 40, 1, 60, 16, 25, 24]
+    assert sum(sizes) == 250
+    got, i = [], 0
+    for s, n in enumerate(sizes):
+        got.append(rep.step({"step": s, "entries": [{"id": "r", "tokens": toks[i:i + n], "want": list(range(n))}],
+                             "end": ["r"] if i + n == 250 else []}))
+        i += n
+    assert set(calls) == {n for n in sizes if n >= 17}
+    close(np.concatenate(got), want, "bfloat16")
+
+
 @pytest.mark.parametrize("name,dtype", [("B", "float32"), ("C", "bfloat16"), ("C", "float32")])
 def test_long_decoding(replayers, plain_models, name, dtype):
     rep = replayers(name, dtype)

@@ -34,6 +34,9 @@ def can_fuse(residual: torch.Tensor, dtype: torch.dtype, *weights: torch.Tensor)
 
 
 STACKED_MIN_ROWS, STACKED_MAX_ROWS = 17, 256
+# smallest matrix (elements) that goes this way: below, the stack the norm has to read outweighs the matrix
+# (Qwen3-0.6B's projections, 2-3 M elements: its 256-request workload ran 2% slower with stacks)
+STACKED_MIN_WEIGHT = 8 << 20
 
 
 def linear_into_stream(x: torch.Tensor, weight: torch.Tensor, ctx) -> torch.Tensor:
@@ -45,6 +48,6 @@ def linear_into_stream(x: torch.Tensor, weight: torch.Tensor, ctx) -> torch.Tens
     180 us, at 256 rows 41 / 72 / 103 us against 51 / 223 / 262 us; output projection at 128 rows
     14 / 18 / 24 us against 21 / 26 / 37 us, at 256 rows 20 / 27 / 36 us against 20 / 45 / 69 us."""
     if (ctx.stacked_branches and x.dtype == torch.bfloat16 and STACKED_MIN_ROWS <= x.shape[0] <= STACKED_MAX_ROWS
-            and ops.gemm_partial_sums_supports(x, weight)):
+            and weight.numel() >= STACKED_MIN_WEIGHT and ops.gemm_partial_sums_supports(x, weight)):
         return ops.gemm_partial_sums(x, weight)
     return linear(x, weight)
