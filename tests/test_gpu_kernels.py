@@ -505,6 +505,51 @@ def test_gemm_skinny(ops, shape, out_dtype):
     assert torch.equal(got2, got)
 
 
+@pytest.mark.parametrize("shape", [(1, 64, 128), (8, 6144, 4096), (5, 100, 1032), (16, 328, 72), (3, 70000, 264),
+                                   (13, 24, 5128)])
+def test_gemm_skinny_with_the_norm_folded_in(ops, shape):
+    """rmsnorm(stream) W^T, and silu(gate) * up of it, straight from the 32-bit residual stream: against the plain
+    norm followed by the plain product.  The rows' scales differ by orders of magnitude, so that a
+    sum of squares that leaks from one row into another, or a missing scale, shows."""
+    torch.manual_seed(14)
+    M, N, K = shape
+    stream = torch.randn(M, K, device=DEV) * torch.logspace(-2, 2, M, device=DEV)[:, None]
+    gain = 1.0 + 0.5 * torch.randn(K, device=DEV)
+    w = (torch.randn(N, K, device=DEV) * 0.3).bfloat16()
+    b = torch.randn(N, device=DEV)
+    eps = 1e-3
+    normed = plain.rms_norm(stream.cpu(), gain.cpu(), eps)
+    want = normed @ w.float().cpu().T + b.cpu()
+    for out_dtype in (torch.bfloat16, torch.float32):
+        got = ops.gemm_skinny_normed(stream, gain, eps, w, b, out_dtype=out_dtype)
+        assert got.dtype == out_dtype and got.shape == (M, N)
+        # the inputs of the matrix cores are rounded to bfloat16 (2^-9 each way) as after a norm kernel of its own
+        assert (got.float().cpu() - want).abs().max() <= 1e-2 * float(want.abs().max())
+        assert torch.equal(ops.gemm_skinny_normed(stream, gain, eps, w, b, out_dtype=out_dtype), got)
+        for nt, waves in ((1, 1), (2, 2), (1, 8), (2, 4)):
+            other = ops.gemm_skinny_normed(stream, gain, eps, w, b, out_dtype=out_dtype, nt=nt, waves=waves)
+            assert (other.float().cpu() - want).abs().max() <= 1e-2 * float(want.abs().max()), (nt, waves)
+    # against the two kernels it replaces: the same but for where the rounding to bfloat16 falls
+    two = ops.gemm_skinny(ops.add_rmsnorm(None, stream.clone(), gain, eps, torch.bfloat16), w, b, out_dtype=torch.float32)
+    one = ops.gemm_skinny_normed(stream, gain, eps, w, b, out_dtype=torch.float32)
+    assert (one - two).abs().max() <= 4e-3 * float(want.abs().max())
+    # fewer rows of the same stream: every row as before, bit for bit
+    if M > 1:
+        fewer = ops.gemm_skinny_normed(stream[:M // 2], gain, eps, w, b, out_dtype=torch.float32)
+        assert torch.equal(fewer, one[:M // 2])
+    # a row of zeros: eps alone under the root, no NaN
+    zeros = torch.zeros(2, K, device=DEV)
+    assert torch.equal(ops.gemm_skinny_normed(zeros, gain, eps, w, out_dtype=torch.float32),
+                       torch.zeros(2, N, device=DEV))
+    inter = N // 2
+    if inter:
+        wgu = torch.cat([w[:inter], w[N - inter:]]).contiguous()
+        want = plain.silu_and_mul(normed @ wgu.float().cpu().T)
+        got = ops.gemm_skinny_normed(stream, gain, eps, wgu, silu=True)
+        assert got.shape == (M, inter) and got.dtype == torch.bfloat16
+        assert (got.float().cpu() - want).abs().max() <= 1e-2 * float(want.abs().max())
+
+
 @pytest.mark.parametrize("shape", [(17, 256, 512), (33, 100, 4104), (48, 4100, 72), (64, 640, 2048), (5, 128, 8),
                                    (64, 4096, 1032), (40, 24, 12288), (65, 260, 520), (100, 128, 1096), (129, 512, 264),
                                    (200, 96, 4096), (256, 1032, 776)])

@@ -189,6 +189,44 @@ def test_feed_forward_hands_the_norm_a_stack_of_partial_sums(monkeypatch):
         assert (ya.float() - yb.float()).abs().max() <= 3e-2 * yb.float().abs().max()
 
 
+def test_norm_left_to_the_feed_forwards_first_projection(monkeypatch):
+    """With few rows and nothing left to add, the block hands a part that folds norms the norm as a
+    record; the feed-forward then adds ffn(norm(stream)) into the stream, as the plain functions do.
+    The rows' sizes differ by orders of magnitude, so that a scale from the wrong row shows."""
+    from types import SimpleNamespace
+    from ullm_amd.parts import PartEnv, PendingNorm, build_part
+    from ullm_amd.parts.block import PreNormBlock
+    torch.manual_seed(6)
+    H, I, eps = 96, 224, 1e-3
+    env = PartEnv(torch.device(DEV), torch.bfloat16, 16)
+    ffn = build_part("ffn", "swiglu", hidden_size=H, intermediate_size=I, prefix="f")
+    w = {f"f.{n}.weight": (torch.randn(*shape) * 0.1).bfloat16() for n, shape in
+         (("gate_proj", (I, H)), ("up_proj", (I, H)), ("down_proj", (H, I)))}
+    ffn.bind({k: v.to(DEV) for k, v in w.items()}, env)
+    gain = 1 + 0.3 * torch.randn(H)
+    norm = build_part("norm", "rmsnorm", size=H, eps=eps, weight_name="g")
+    norm.bind({"g": gain.to(DEV)}, env)
+    ctx = SimpleNamespace(stacked_branches=False, dtype=torch.bfloat16)
+    assert ffn.folds_norm
+    from ullm_amd.kernels import ops
+    seen, inner = [], ops.gemm_skinny_normed
+    monkeypatch.setattr(ops, "gemm_skinny_normed", lambda *a, **k: seen.append(1) or inner(*a, **k))
+    for T, folded in ((1, True), (7, True), (8, True), (9, False), (16, False)):
+        stream = torch.randn(T, H) * torch.logspace(-2, 2, T)[:, None]
+        want = stream + plain.qwen3_mlp(plain.rms_norm(stream, gain, eps), {k: v.float() for k, v in w.items()}, "f")
+        got = stream.clone().to(DEV)
+        assert ffn.fusable(got, ctx)
+        x = PreNormBlock._normed(norm, ffn, None, got, ctx)
+        assert isinstance(x, PendingNorm)
+        seen.clear()
+        ffn.forward_fused(x, got, ctx)
+        assert bool(seen) == folded
+        assert (got.cpu() - want).abs().max() <= 2e-2 * (want - stream).abs().max()
+    # something left to add: the norm runs as a kernel of its own
+    x = PreNormBlock._normed(norm, ffn, torch.zeros(4, H, device=DEV, dtype=torch.bfloat16), torch.randn(4, H, device=DEV), ctx)
+    assert isinstance(x, torch.Tensor)
+
+
 def test_rotary_part_table_matches_the_plain_angles():
     from ullm_amd.parts import PartEnv, build_part
     rot = build_part("position", "rotary", head_dim=24, theta=777.0, rotary_dim=12, pairing="half")

@@ -18,7 +18,15 @@
 // part of shared memory.  The waves' partial results are added in wave order through shared memory,
 // so the result does not depend on timing.
 // Weights are [out, in] (ullm/layers/linear.py:165).
+//
+//   what comes before it (NORMX)
+//     the RMS norm of the 32-bit residual stream (ullm/layers/layernorm.py:28-33): X is then the stream
+//     itself, float32 [M, K].  The kernel reads every row of X in full anyway, so it multiplies by the
+//     gain and rounds to bfloat16 on the way into shared memory, adds up the squares beside that, and
+//     multiplies the finished sums by rsqrt(mean of squares + eps): y = rs * ((x * gain) W^T).  Against
+//     a norm kernel of its own this saves a launch and a pass, which at these sizes is all latency.
 #include "common.h"
+#include <type_traits>
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
@@ -39,9 +47,12 @@ __host__ __device__ constexpr int sk_max_waves(int mt, int nt) { return mt * nt 
 
 // The waves' partial results of a block are added in wave order through `red` and the sum goes where
 // EPI says.  acc[i][t][j] = partial C[m = 16 t + r][n0 + 16 i + 4 g + j].
-template <int MT, int NT, int EPI, typename TC, typename RedT>
+// With NORMX, sq[w][m] holds wave w's sum of squares of row m of X and the sums are scaled by
+// rsqrt(their total / K + eps) first.
+template <int MT, int NT, int EPI, typename TC, bool NORMX, typename RedT>
 __device__ __forceinline__ void skinny_finish(f32x4_t (&acc)[NT][MT], RedT& red, const float* __restrict__ bias,
-                                              TC* __restrict__ C, float* __restrict__ R, int ldc, int M, int N, int n0) {
+                                              TC* __restrict__ C, float* __restrict__ R, int ldc, int M, int N, int n0,
+                                              const float (*sq)[16 * MT], int K, float eps) {
   constexpr int OT = EPI == EPI_SILU ? NT / 2 : NT;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
   const int g = lane >> 4, r = lane & 15;
@@ -64,6 +75,18 @@ __device__ __forceinline__ void skinny_finish(f32x4_t (&acc)[NT][MT], RedT& red,
           const float4 o = *reinterpret_cast<const float4*>(&red[w - 1][i * MT + t][lane * 4]);
           acc[i][t][0] += o.x; acc[i][t][1] += o.y; acc[i][t][2] += o.z; acc[i][t][3] += o.w;
         }
+  }
+  if (NORMX) {
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      float total = 0.f;
+      for (int w = 0; w < nwaves; ++w) total += sq[w][16 * t + r];
+      const float rs = rsqrtf(total / (float)K + eps);
+#pragma unroll
+      for (int i = 0; i < NT; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][t][j] *= rs;
+    }
   }
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
@@ -107,22 +130,32 @@ __device__ __forceinline__ void skinny_finish(f32x4_t (&acc)[NT][MT], RedT& red,
 // (Loading the operands straight from memory in the matrix layout, 64 bytes of each of 16 rows per
 // instruction and of X as many rows as the batch has, was slower the more rows X had: 92 against 80 us
 // for the four projections of a Qwen3-8B layer at 8 rows, 105 against 83 us at 16.)
-template <int MT, int NT, int EPI, typename TC>
+// NORMX: X is float32 and gain [K] float32, see above; else X is bfloat16.
+// XH: 8-row halves of a tile of X that are fetched: 1 for M <= 8 (then MT = 1), where the other half
+// stays zero in shared memory and costs neither loads nor the registers that hold them in flight
+// (with NORMX 75 against 116 registers, that is 6 against 4 waves per SIMD).
+template <int MT, int NT, int EPI, typename TC, bool NORMX, int XH>
 __global__ void __launch_bounds__(64 * sk_max_waves(MT, NT))
-gemm_skinny_kernel(const bf16_t* __restrict__ X, int ldx, const bf16_t* __restrict__ W, int ldw,
-                          const float* __restrict__ bias, TC* __restrict__ C, float* __restrict__ R, int ldc, int M,
-                          int N, int K, int k_per_wave) {
+gemm_skinny_kernel(const void* __restrict__ Xv, int ldx, const bf16_t* __restrict__ W, int ldw,
+                   const float* __restrict__ bias, const float* __restrict__ gain, float eps, TC* __restrict__ C,
+                   float* __restrict__ R, int ldc, int M, int N, int K, int k_per_wave) {
   constexpr int MAXW = sk_max_waves(MT, NT);
   constexpr int TILE_BYTES = 16 * 128, STAGE_BYTES = (NT + MT) * TILE_BYTES;
   constexpr int RED_BYTES = (MAXW - 1) * NT * MT * 256 * 4;
   constexpr int LDS_BYTES = MAXW * STAGE_BYTES > RED_BYTES ? MAXW * STAGE_BYTES : RED_BYTES;
   __shared__ __attribute__((aligned(16))) unsigned char lds[LDS_BYTES];
+  __shared__ float sq[NORMX ? MAXW : 1][16 * MT];
+  using XT = typename std::conditional<NORMX, float, bf16_t>::type;
+  constexpr int XV = NORMX ? 2 : 1;                       // 16-byte loads per 8 values of X
+  const XT* const X = reinterpret_cast<const XT*>(Xv);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int g = lane >> 4, r = lane & 15, lrow = lane >> 3, lcol = lane & 7;
   constexpr int OT = EPI == EPI_SILU ? NT / 2 : NT;
   const int n0 = blockIdx.x * (16 * OT);
   const bf16_t* wsrc[NT][2];
-  const bf16_t* xsrc[MT][2];
+  static_assert(XH == 2 || MT == 1, "half a tile of X only where it is the only tile");
+  const XT* xsrc[MT][XH];
+  bool xrow[MT][XH];                                      // rows of X past M are zeros and cost no load
   int put[2], get[2];
 #pragma unroll
   for (int h = 0; h < 2; ++h) {
@@ -135,13 +168,16 @@ gemm_skinny_kernel(const bf16_t* __restrict__ X, int ldx, const bf16_t* __restri
       const int n = (col < N ? col : N - 1) + (i / OT) * N;       // rows past N repeat the last row; never stored
       wsrc[i][h] = W + (size_t)n * ldw + 8 * lcol;
     }
+    if (h < XH) {
 #pragma unroll
-    for (int t = 0; t < MT; ++t) {
-      const int m = 16 * t + row < M ? 16 * t + row : M - 1;
-      xsrc[t][h] = X + (size_t)m * ldx + 8 * lcol;
+      for (int t = 0; t < MT; ++t) {
+        xrow[t][h] = 16 * t + row < M;
+        xsrc[t][h] = X + (size_t)(xrow[t][h] ? 16 * t + row : M - 1) * ldx + 8 * lcol;
+      }
     }
   }
   unsigned char* const mine = lds + wave * STAGE_BYTES;
+  if (XH == 1) *reinterpret_cast<uint4*>(mine + NT * TILE_BYTES + put[1]) = make_uint4(0, 0, 0, 0);
   f32x4_t acc[NT][MT];
 #pragma unroll
   for (int t = 0; t < MT; ++t)
@@ -150,7 +186,10 @@ gemm_skinny_kernel(const bf16_t* __restrict__ X, int ldx, const bf16_t* __restri
   const int k_begin = wave * k_per_wave;
   int k_end = k_begin + k_per_wave;
   if (k_end > K) k_end = K;
-  struct Stage { uint4 w[NT][2], x[MT][2]; };
+  struct Stage { uint4 w[NT][2], x[MT][XH][XV], gm[XV]; };
+  float ss[MT][XH];                                        // squares of rows 16 t + 8 h + lrow, this lane's pieces
+#pragma unroll
+  for (int t = 0; t < MT; ++t) ss[t][0] = ss[t][XH - 1] = 0.f;
   constexpr int DEPTH = 2;                                // stages of 64 values of K on their way (3 and 4 were slower)
   Stage st[DEPTH];
   auto fetch = [&](Stage& st, int k0) {
@@ -160,9 +199,19 @@ gemm_skinny_kernel(const bf16_t* __restrict__ X, int ldx, const bf16_t* __restri
 #pragma unroll
       for (int i = 0; i < NT; ++i)
         st.w[i][h] = in ? *reinterpret_cast<const uint4*>(wsrc[i][h] + k0) : make_uint4(0, 0, 0, 0);
+      if (h < XH) {
 #pragma unroll
-      for (int t = 0; t < MT; ++t)
-        st.x[t][h] = in ? *reinterpret_cast<const uint4*>(xsrc[t][h] + k0) : make_uint4(0, 0, 0, 0);
+        for (int t = 0; t < MT; ++t)
+#pragma unroll
+          for (int v = 0; v < XV; ++v)
+            st.x[t][h][v] = in && xrow[t][h] ? *reinterpret_cast<const uint4*>(xsrc[t][h] + k0 + 4 * v)
+                                             : make_uint4(0, 0, 0, 0);
+      }
+    }
+    if (NORMX) {
+#pragma unroll
+      for (int v = 0; v < XV; ++v)
+        st.gm[v] = in ? *reinterpret_cast<const uint4*>(gain + k0 + 8 * lcol + 4 * v) : make_uint4(0, 0, 0, 0);
     }
   };
   auto work = [&](const Stage& st) {
@@ -170,8 +219,24 @@ gemm_skinny_kernel(const bf16_t* __restrict__ X, int ldx, const bf16_t* __restri
     for (int h = 0; h < 2; ++h) {
 #pragma unroll
       for (int i = 0; i < NT; ++i) *reinterpret_cast<uint4*>(mine + i * TILE_BYTES + put[h]) = st.w[i][h];
+      if (h >= XH) continue;
 #pragma unroll
-      for (int t = 0; t < MT; ++t) *reinterpret_cast<uint4*>(mine + (NT + t) * TILE_BYTES + put[h]) = st.x[t][h];
+      for (int t = 0; t < MT; ++t) {
+        uint4 piece;
+        if constexpr (NORMX) {
+          const float4 a = __builtin_bit_cast(float4, st.x[t][h][0]), b = __builtin_bit_cast(float4, st.x[t][h][XV - 1]);
+          const float4 ga = __builtin_bit_cast(float4, st.gm[0]), gb = __builtin_bit_cast(float4, st.gm[XV - 1]);
+          float q = ss[t][h];
+          q = fmaf(a.x, a.x, q); q = fmaf(a.y, a.y, q); q = fmaf(a.z, a.z, q); q = fmaf(a.w, a.w, q);
+          q = fmaf(b.x, b.x, q); q = fmaf(b.y, b.y, q); q = fmaf(b.z, b.z, q); q = fmaf(b.w, b.w, q);
+          ss[t][h] = q;
+          piece = make_uint4(pack2_bf16(a.x * ga.x, a.y * ga.y), pack2_bf16(a.z * ga.z, a.w * ga.w),
+                             pack2_bf16(b.x * gb.x, b.y * gb.y), pack2_bf16(b.z * gb.z, b.w * gb.w));
+        } else {
+          piece = st.x[t][h][0];
+        }
+        *reinterpret_cast<uint4*>(mine + (NT + t) * TILE_BYTES + put[h]) = piece;
+      }
     }
     __builtin_amdgcn_wave_barrier();       // the wave's lanes read each other's pieces: writes stay before reads
 #pragma unroll
@@ -202,9 +267,38 @@ gemm_skinny_kernel(const bf16_t* __restrict__ X, int ldx, const bf16_t* __restri
       }
     }
   }
+  if (NORMX) {
+    // the 8 lanes of a row hold its pieces: add them, one lane of each row stores the wave's sum
+#pragma unroll
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+      for (int h = 0; h < XH; ++h) {
+        float q = ss[t][h];
+        q += __shfl_xor(q, 1);
+        q += __shfl_xor(q, 2);
+        q += __shfl_xor(q, 4);
+        if (lcol == 0) sq[wave][16 * t + 8 * h + lrow] = q;
+      }
+    if (XH == 1 && lcol == 0) sq[wave][8 + lrow] = 0.f;
+  }
   __syncthreads();                                        // the partial sums take the place of the stages
   auto& red = *reinterpret_cast<float (*)[MAXW - 1][NT * MT][64 * 4]>(lds);
-  skinny_finish<MT, NT, EPI, TC>(acc, red, bias, C, R, ldc, M, N, n0);
+  skinny_finish<MT, NT, EPI, TC, NORMX>(acc, red, bias, C, R, ldc, M, N, n0, sq, K, eps);
+}
+
+template <int MT, int NT, int EPI, typename TC, bool NORMX, typename... Args>
+static void skinny_launch(dim3 grid, dim3 block, hipStream_t stream, const void* X, int ldx, const bf16_t* W, int ldw,
+                          const float* bias, const float* gain, float eps, TC* C, float* R, int ldc, int M,
+                          Args... rest) {
+  if constexpr (MT == 1) {
+    if (M <= 8) {
+      hipLaunchKernelGGL((gemm_skinny_kernel<1, NT, EPI, TC, NORMX, 1>), grid, block, 0, stream, X, ldx, W, ldw, bias,
+                         gain, eps, C, R, ldc, M, rest...);
+      return;
+    }
+  }
+  hipLaunchKernelGGL((gemm_skinny_kernel<MT, NT, EPI, TC, NORMX, 2>), grid, block, 0, stream, X, ldx, W, ldw, bias,
+                     gain, eps, C, R, ldc, M, rest...);
 }
 
 extern "C" int ullm_gemm_skinny_supports(int M, int N, int K, int ldx, int ldw) {
@@ -213,14 +307,16 @@ extern "C" int ullm_gemm_skinny_supports(int M, int N, int K, int ldx, int ldw) 
 
 // X bfloat16 [M, K]; W bfloat16 [N, K] (with epi 2: [2 N, K]).  epi: 0 store to C (c_dtype, bias optional),
 // 1 add into R (float32 [M, N], row stride ldc), 2 silu(gate) * up to C (bfloat16 [M, N]).
-// force_nt / force_waves: 0 = chosen here.
+// With gain (float32 [K]): X is float32 [M <= 16, K] and its RMS norm with this gain and eps is what
+// is multiplied (epi 0 and 2).  force_nt / force_waves: 0 = chosen here.
 extern "C" int ullm_gemm_skinny(const void* X, int ldx, const void* W, int ldw, const float* bias, void* C,
                                 int ldc, int M, int N, int K, int epi, int c_dtype, int force_nt,
-                                int force_waves, hipStream_t stream) {
+                                int force_waves, const float* gain, float eps, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (!ullm_gemm_skinny_supports(M, N, K, ldx, ldw) || ldc < N) return ULLM_ERR_SHAPE;
   if (((uintptr_t)X & 15) || ((uintptr_t)W & 15)) return ULLM_ERR_SHAPE;
   if (epi < 0 || epi > 2) return ULLM_ERR_UNSUPPORTED;
+  if (gain && (M > 16 || epi == EPI_RESADD || ((uintptr_t)gain & 15))) return ULLM_ERR_UNSUPPORTED;
   if (epi == EPI_RESADD && (((uintptr_t)C & 15) || ldc % 4 != 0 || bias)) return ULLM_ERR_SHAPE;
   if (epi == EPI_SILU && (bias || c_dtype != ULLM_BF16)) return ULLM_ERR_UNSUPPORTED;
   int mt = (M + 15) / 16;
@@ -230,6 +326,9 @@ extern "C" int ullm_gemm_skinny(const void* X, int ldx, const void* W, int ldw, 
   if (force_nt > 0) nt = force_nt;
   else if (tiles16 >= 4096) nt = mt >= 2 ? 4 : 2;
   else if (tiles16 >= 1024 && mt >= 2) nt = 2;
+  // with the norm folded in, a tile of X costs a wave as much as a tile of W: two tiles of W per tile of X
+  // (projection to q|k|v of Qwen3-8B at 8 rows: 15.6 us against 16.5)
+  if (gain && force_nt <= 0) nt = 2;
   if (epi == EPI_SILU) nt = (force_nt == 4 || mt >= 4) ? 4 : 2;   // gate and up tiles come in pairs
   if (nt != 1 && nt != 2 && nt != 4) return ULLM_ERR_UNSUPPORTED;
   if (nt == 4 && mt == 1) nt = 2;                       // not instantiated
@@ -239,14 +338,16 @@ extern "C" int ullm_gemm_skinny(const void* X, int ldx, const void* W, int ldw, 
   // each wave with at least 128 values of K
   const int max_waves = sk_max_waves(mt, nt);
   int waves = 1;
-  while (waves < max_waves && waves * nt < 8 && K / (waves * 2) >= 128) waves *= 2;
+  const int in_flight = gain && epi == EPI_STORE ? 16 : 8;
+  while (waves < max_waves && waves * nt < in_flight && K / (waves * 2) >= 128) waves *= 2;
   if (force_waves > 0) waves = force_waves < max_waves ? force_waves : max_waves;
   int k_per_wave = (K + waves - 1) / waves;
   k_per_wave = (k_per_wave + 63) / 64 * 64;
   dim3 grid(tiles), block(64 * waves);
   float* R = (float*)C;
-#define GO(MT, NT, EPI, TC) hipLaunchKernelGGL((gemm_skinny_kernel<MT, NT, EPI, TC>), grid, block, 0, stream, \
-    (const bf16_t*)X, ldx, (const bf16_t*)W, ldw, bias, (TC*)C, R, ldc, M, N, K, k_per_wave)
+#define GO_(MT, NT, EPI, TC, NORMX) skinny_launch<MT, NT, EPI, TC, NORMX>(grid, block, stream, X, ldx, \
+    (const bf16_t*)W, ldw, bias, gain, eps, (TC*)C, R, ldc, M, N, K, k_per_wave)
+#define GO(MT, NT, EPI, TC) GO_(MT, NT, EPI, TC, false)
 #define GO_SHAPE(EPI, TC)                                              \
   switch (mt * 8 + nt) {                                               \
     case 1 * 8 + 1: GO(1, 1, EPI, TC); break;                          \
@@ -267,7 +368,16 @@ extern "C" int ullm_gemm_skinny(const void* X, int ldx, const void* W, int ldw, 
     case 4 * 8 + 4: GO(4, 4, EPI, TC); break;                          \
     default: return ULLM_ERR_UNSUPPORTED;                              \
   }
-  if (epi == EPI_STORE) {
+  if (gain) {                                            // one tile of rows
+    if (epi == EPI_SILU) {
+      if (nt != 2) return ULLM_ERR_UNSUPPORTED;
+      GO_(1, 2, EPI_SILU, bf16_t, true);
+    } else if (c_dtype == ULLM_BF16) {
+      if (nt == 1) GO_(1, 1, EPI_STORE, bf16_t, true); else GO_(1, 2, EPI_STORE, bf16_t, true);
+    } else if (c_dtype == ULLM_F32) {
+      if (nt == 1) GO_(1, 1, EPI_STORE, float, true); else GO_(1, 2, EPI_STORE, float, true);
+    } else return ULLM_ERR_DTYPE;
+  } else if (epi == EPI_STORE) {
     if (c_dtype == ULLM_BF16) { GO_SHAPE(EPI_STORE, bf16_t) }
     else if (c_dtype == ULLM_F32) { GO_SHAPE(EPI_STORE, float) }
     else return ULLM_ERR_DTYPE;
@@ -279,5 +389,6 @@ extern "C" int ullm_gemm_skinny(const void* X, int ldx, const void* W, int ldw, 
 #undef GO_PAIRS
 #undef GO_SHAPE
 #undef GO
+#undef GO_
   ULLM_LAUNCH_CHECK();
 }

@@ -234,11 +234,12 @@ def gemm_skinny_supports(a: torch.Tensor, w: torch.Tensor) -> bool:
     return a.dtype == torch.bfloat16 and _skinny_ok(a.shape[0], a.shape[1], a, w)
 
 
-def _gemm_skinny(x, w, bias, c, M, N, K, epi, c_dtype, nt=0, waves=0) -> None:
+def _gemm_skinny(x, w, bias, c, M, N, K, epi, c_dtype, nt=0, waves=0, gain=None, eps=0.0) -> None:
     lib = build.load("gemm_skinny")
     _check(lib.ullm_gemm_skinny(_p(x), _c_int(x.stride(0)), _p(w), _c_int(w.stride(0)), _p(bias),
                                 _p(c), _c_int(c.stride(0)), _c_int(M), _c_int(N), _c_int(K),
-                                _c_int(epi), _c_int(c_dtype), _c_int(nt), _c_int(waves), _stream()),
+                                _c_int(epi), _c_int(c_dtype), _c_int(nt), _c_int(waves), _p(gain),
+                                ctypes.c_float(eps), _stream()),
            "gemm_skinny")
 
 
@@ -280,6 +281,38 @@ def gemm_skinny_silu(a: torch.Tensor, w_gate_up: torch.Tensor, nt: int = 0, wave
     _need(a.dtype == torch.bfloat16 and _skinny_ok(M, K, a, w_gate_up), "gemm_skinny_silu takes bfloat16 [M <= 64, K]")
     out = torch.empty((M, two_i // 2), dtype=torch.bfloat16, device=a.device)
     _gemm_skinny(a, w_gate_up, None, out, M, two_i // 2, K, 2, BF16, nt, waves)
+    return out
+
+
+NORMED_MAX_ROWS = 16
+
+
+def gemm_skinny_normed_supports(stream: torch.Tensor, gain: torch.Tensor, w: torch.Tensor) -> bool:
+    M, K = stream.shape
+    return (stream.dtype == torch.float32 and gain.dtype == torch.float32 and w.dtype == torch.bfloat16
+            and M <= NORMED_MAX_ROWS and gain.numel() == K and gain.is_contiguous() and gain.data_ptr() % 16 == 0
+            and _skinny_ok(M, K, stream, w))
+
+
+def gemm_skinny_normed(stream: torch.Tensor, gain: torch.Tensor, eps: float, w: torch.Tensor,
+                       bias: Optional[torch.Tensor] = None, out_dtype: torch.dtype = torch.bfloat16,
+                       silu: bool = False, nt: int = 0, waves: int = 0) -> torch.Tensor:
+    """rmsnorm(stream) times w transposed for the float32 residual stream [M <= 16, K], the norm
+    (gain float32 [K], eps) folded into the product: the kernel rounds stream * gain to bfloat16 for
+    the matrix cores, sums the squares of the rows it reads anyway and scales the 32-bit sums by
+    rsqrt(mean + eps).  With silu, w is gate | up [2 I, K] and the result silu(gate) * up [M, I]."""
+    M, K = stream.shape
+    N, K2 = w.shape
+    _need(K == K2, f"inner sizes differ: the stream is [{M}, {K}], w is [{N}, {K2}]")
+    _need(gemm_skinny_normed_supports(stream, gain, w),
+          "gemm_skinny_normed takes a float32 stream [M <= 16, K], a float32 gain [K] and bfloat16 weights")
+    if silu:
+        _need(N % 2 == 0 and bias is None and out_dtype == torch.bfloat16, "gate|up weights must be [2 I, K], no bias")
+        N //= 2
+    if bias is not None:
+        _need(bias.dtype == torch.float32 and bias.numel() == N and bias.is_contiguous(), "bias must be float32 [N]")
+    out = torch.empty((M, N), dtype=out_dtype, device=stream.device)
+    _gemm_skinny(stream, w, bias, out, M, N, K, 2 if silu else 0, _dt(out), nt, waves, gain, float(eps))
     return out
 
 

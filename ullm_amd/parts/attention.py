@@ -14,11 +14,13 @@ import torch
 
 from ..kernels import ops
 from .base import KVNeed, LayerCache, Mixer, PartEnv, PositionEncoding, StepContext, WeightDecl, register_part
-from .linear import can_fuse, linear, linear_into_stream
+from .linear import can_fuse, linear, linear_into_stream, linear_of_norm
 
 
 @register_part("mixer", "gqa_attention")
 class GQAttention(Mixer):
+    folds_norm = True
+
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, prefix: str,
                  position: Optional[PositionEncoding] = None, qk_norm_eps: Optional[float] = None,
                  bias: bool = False, window: int = 0, scale: Optional[float] = None):
@@ -74,7 +76,7 @@ class GQAttention(Mixer):
         return can_fuse(residual, ctx.dtype, self.w_qkv, self.w_o)
 
     def forward_fused(self, x, residual, ctx: StepContext, cache: LayerCache) -> None:
-        qkv = linear(x, self.w_qkv, self.b_qkv)
+        qkv = linear_of_norm(x, self.w_qkv, self.b_qkv)                               # the norm before folded in
         ops.gemm_skinny_add(self._attend(qkv, ctx, cache), self.w_o, residual)        # residual add folded behind
 
     def _attend(self, qkv: torch.Tensor, ctx: StepContext, cache: LayerCache) -> torch.Tensor:

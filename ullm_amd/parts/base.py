@@ -128,8 +128,10 @@ class Mixer(Part):
 
     A mixer may also offer ``forward_fused(x, residual, ctx, cache)``: add mixer(x) into the 32-bit
     residual in place, with the add folded into its last kernel.  It is called only when
-    ``fusable(residual, ctx)`` says so."""
+    ``fusable(residual, ctx)`` says so.  With ``folds_norm`` its ``forward_fused`` also takes a
+    :class:`PendingNorm` for x: the norm before it, left to the mixer's first projection."""
     kind = "mixer"
+    folds_norm = False
 
     def cache_need(self) -> CacheNeed:
         return None
@@ -146,8 +148,9 @@ class Mixer(Part):
 
 class FeedForward(Part):
     """``forward(x [T, hidden], ctx) -> [T, hidden]``; keeps nothing between steps.
-    ``fusable`` and ``forward_fused(x, residual, ctx)`` as for mixers."""
+    ``fusable``, ``forward_fused(x, residual, ctx)`` and ``folds_norm`` as for mixers."""
     kind = "ffn"
+    folds_norm = False
 
     def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
         raise NotImplementedError
@@ -159,13 +162,30 @@ class FeedForward(Part):
         raise NotImplementedError
 
 
+class PendingNorm:
+    """A norm of the residual stream that has not been computed: what a consumer needs to fold it
+    into its first projection (``stream`` float32 [T, hidden], ``gain`` float32 [hidden], ``eps``;
+    the scale is rsqrt(mean of squares + eps)), and ``apply()`` for a consumer that cannot after all."""
+
+    def __init__(self, norm: "Norm", stream: torch.Tensor, gain: torch.Tensor, eps: float, out_dtype: torch.dtype):
+        self.norm, self.stream, self.gain, self.eps, self.out_dtype = norm, stream, gain, eps, out_dtype
+
+    def apply(self) -> torch.Tensor:
+        return self.norm.add_norm(None, self.stream, out_dtype=self.out_dtype)
+
+
 class Norm(Part):
     """``add_norm(branch, residual, rows) -> normed``: adds the branch output (if any) into
     the 32-bit residual stream, then normalises the sum; ``rows`` selects output rows.
     ``adds_stacks``: the branch may also be a stack [S, T, hidden] of float32 partial sums, which
-    the norm adds in order."""
+    the norm adds in order.
+    ``pending(residual, out_dtype)``: a :class:`PendingNorm` of a stream with nothing left to add, for
+    a consumer with ``folds_norm``, or None if this norm has no such form."""
     kind = "norm"
     adds_stacks = False
+
+    def pending(self, residual: torch.Tensor, out_dtype: torch.dtype) -> Optional["PendingNorm"]:
+        return None
 
     def add_norm(self, branch: Optional[torch.Tensor], residual: torch.Tensor,
                  rows: Optional[torch.Tensor] = None, out_dtype: torch.dtype = None) -> torch.Tensor:

@@ -25,14 +25,23 @@ class PreNormBlock(Block):
         # Each half: the norm kernel adds the pending branch into the stream and normalises; the
         # part then either adds its result into the stream itself (folded into its last kernel,
         # where it offers that for this batch) or returns it as the next pending branch.
-        x = self.mixer_norm.add_norm(pending, residual, out_dtype=ctx.dtype)
+        # Where nothing is left to add, a part that folds the norm into its first projection gets
+        # the norm as a record instead of its result: then a half is two or three kernels.
         if self.mixer.fusable(residual, ctx):
-            self.mixer.forward_fused(x, residual, ctx, cache)
+            self.mixer.forward_fused(self._normed(self.mixer_norm, self.mixer, pending, residual, ctx), residual, ctx,
+                                     cache)
             pending = None
         else:
-            pending = self.mixer.forward(x, ctx, cache)
-        x = self.ffn_norm.add_norm(pending, residual, out_dtype=ctx.dtype)
+            pending = self.mixer.forward(self.mixer_norm.add_norm(pending, residual, out_dtype=ctx.dtype), ctx, cache)
         if self.ffn.fusable(residual, ctx):
-            self.ffn.forward_fused(x, residual, ctx)
+            self.ffn.forward_fused(self._normed(self.ffn_norm, self.ffn, pending, residual, ctx), residual, ctx)
             return residual, None
-        return residual, self.ffn.forward(x, ctx)
+        return residual, self.ffn.forward(self.ffn_norm.add_norm(pending, residual, out_dtype=ctx.dtype), ctx)
+
+    @staticmethod
+    def _normed(norm: Norm, part, pending, residual, ctx: StepContext):
+        if pending is None and part.folds_norm:
+            record = norm.pending(residual, ctx.dtype)
+            if record is not None:
+                return record
+        return norm.add_norm(pending, residual, out_dtype=ctx.dtype)

@@ -10,7 +10,7 @@ import torch
 
 from ..kernels import ops
 from .base import FeedForward, PartEnv, StepContext, WeightDecl, register_part
-from .linear import can_fuse, linear, linear_into_stream
+from .linear import can_fuse, linear, linear_into_stream, linear_of_norm
 
 
 GATE_UP_SKINNY_MAX_ROWS = 32     # measured on Qwen3-8B's matrix; from 33 rows on the library product is faster
@@ -18,6 +18,8 @@ GATE_UP_SKINNY_MAX_ROWS = 32     # measured on Qwen3-8B's matrix; from 33 rows o
 
 @register_part("ffn", "swiglu")
 class SwiGLU(FeedForward):
+    folds_norm = True
+
     def __init__(self, hidden_size: int, intermediate_size: int, prefix: str):
         self.hidden_size, self.intermediate_size, self.prefix = hidden_size, intermediate_size, prefix
         self.w_gate_up = self.w_down = None
@@ -45,5 +47,5 @@ class SwiGLU(FeedForward):
         return can_fuse(residual, ctx.dtype, self.w_gate_up, self.w_down)
 
     def forward_fused(self, x, residual, ctx: StepContext) -> None:
-        act = ops.gemm_skinny_silu(x, self.w_gate_up)          # silu(gate) * up behind the first product
+        act = linear_of_norm(x, self.w_gate_up, silu=True)     # the norm before, silu(gate) * up behind the first product
         ops.gemm_skinny_add(act, self.w_down, residual)        # residual add behind the second

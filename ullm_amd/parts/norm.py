@@ -11,7 +11,7 @@ from typing import Dict, List, Optional
 import torch
 
 from ..kernels import ops
-from .base import Norm, PartEnv, WeightDecl, register_part
+from .base import Norm, PartEnv, PendingNorm, WeightDecl, register_part
 
 
 @register_part("norm", "rmsnorm")
@@ -34,3 +34,6 @@ class RMSNorm(Norm):
         if out_dtype is None:
             out_dtype = branch.dtype if branch is not None and branch.dim() == 2 else torch.float32
         return ops.add_rmsnorm(branch, residual, self.gain, self.eps, out_dtype, rows=rows)
+
+    def pending(self, residual, out_dtype):
+        return PendingNorm(self, residual, self.gain, self.eps, out_dtype)
