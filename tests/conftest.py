@@ -35,7 +35,14 @@ TINY_C = dict(architectures=["Qwen3ForCausalLM"], hidden_size=80, num_hidden_lay
               use_sliding_window=True, sliding_window=24, max_window_layers=1, initializer_range=0.06,
               torch_dtype="bfloat16")
 
-CONFIGS = {"A": (TINY_A, 0), "B": (TINY_B, 2), "C": (TINY_C, 5)}
+# Tiny D: head_dim 64 (two 32-dim chunks per head in the matrix-core attention kernels), pairs of query
+# heads, three kv heads, theta 5e3, eps 1e-4, tied head.
+TINY_D = dict(architectures=["Qwen3ForCausalLM"], hidden_size=72, num_hidden_layers=2, num_attention_heads=6,
+              num_key_value_heads=3, head_dim=64, intermediate_size=136, vocab_size=300, rope_theta=5000.0,
+              rms_norm_eps=1e-4, max_position_embeddings=320, tie_word_embeddings=True, attention_bias=False,
+              use_sliding_window=False, initializer_range=0.04, torch_dtype="bfloat16")
+
+CONFIGS = {"A": (TINY_A, 0), "B": (TINY_B, 2), "C": (TINY_C, 5), "D": (TINY_D, 7)}
 
 
 @pytest.fixture(scope="session")

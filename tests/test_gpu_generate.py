@@ -26,7 +26,7 @@ def prompts_of(vocab, lens, seed):
 
 
 @pytest.mark.parametrize("name,page_size,budget,chunk", [("A", 16, 64, 64), ("A", 16, 9, 4), ("B", 4, 16, 7),
-                                                          ("C", 8, 12, 5)])
+                                                          ("C", 8, 12, 5), ("D", 16, 20, 9)])
 def test_greedy_generation_equals_the_plain_implementation(model_dirs, plain_models, name, page_size, budget, chunk):
     from ullm_amd import SamplingParams
     cfg, w = plain_models[name]

@@ -46,7 +46,7 @@ def oracle(plain_models, name, toks):
     return plain.qwen3_forward(w, cfg, toks)
 
 
-CASES = [(n, d) for n in ("A", "B", "C") for d in ("float32", "bfloat16")]
+CASES = [(n, d) for n in ("A", "B", "C", "D") for d in ("float32", "bfloat16")]
 
 
 @pytest.mark.parametrize("name,dtype", CASES)
@@ -171,7 +171,7 @@ def test_portions_whose_projections_come_as_stacks_of_partial_sums(model_dirs, p
     close(np.concatenate(got), want, "bfloat16")
 
 
-@pytest.mark.parametrize("name,dtype", [("B", "float32"), ("C", "bfloat16"), ("C", "float32")])
+@pytest.mark.parametrize("name,dtype", [("B", "float32"), ("C", "bfloat16"), ("C", "float32"), ("D", "bfloat16")])
 def test_long_decoding(replayers, plain_models, name, dtype):
     rep = replayers(name, dtype)
     vocab = plain_models[name][0]["vocab_size"]
