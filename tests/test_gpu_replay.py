@@ -197,6 +197,36 @@ def test_first_tokens_and_skipped_logits(replayers, plain_models, name, dtype):
     close(b, want[[19, 9]], dtype)                                   # order of `want` is kept
 
 
+ODD_SIZES = [dict(hidden_size=90, num_attention_heads=3, num_key_value_heads=1, head_dim=16, intermediate_size=100,
+                  vocab_size=301),                                  # a width that is no multiple of 4
+             dict(hidden_size=36, num_attention_heads=2, num_key_value_heads=2, head_dim=80, intermediate_size=44,
+                  vocab_size=77),                                   # heads wider than the model
+             dict(hidden_size=100, num_attention_heads=4, num_key_value_heads=2, head_dim=112, intermediate_size=108,
+                  vocab_size=130)]
+
+
+@pytest.mark.parametrize("sizes", ODD_SIZES)
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_sizes_the_vector_kernels_do_not_take(tmp_path, sizes, dtype):
+    """Widths, head sizes and vocabularies that are no multiples of 8 (or of 4): the kernels with 16-byte
+    accesses must step aside for the general ones, in a prompt portion and in one-token steps."""
+    from ullm_amd.replay import Replayer
+    from ullm_amd.weights.random_init import write_random_model
+    cfg = dict(architectures=["Qwen3ForCausalLM"], num_hidden_layers=2, rope_theta=10000.0, rms_norm_eps=1e-5,
+               max_position_embeddings=128, tie_word_embeddings=False, attention_bias=True, use_sliding_window=False,
+               initializer_range=0.05, torch_dtype="bfloat16", **sizes)
+    write_random_model(cfg, str(tmp_path), seed=3)
+    pcfg, w = plain.load_model_folder(str(tmp_path))
+    rep = Replayer(str(tmp_path), dtype, 256, 16, DEV)
+    toks = make_tokens(cfg["vocab_size"], 60, 1)
+    want = plain.qwen3_forward(w, pcfg, toks)
+    got = [rep.step({"step": 0, "entries": [{"id": "r", "tokens": toks[:37], "want": list(range(37))}], "end": []})]
+    for i in range(37, 60):
+        got.append(rep.step({"step": i, "entries": [{"id": "r", "tokens": [toks[i]], "want": [0]}],
+                             "end": ["r"] if i == 59 else []}))
+    close(np.concatenate(got), want, dtype)
+
+
 def test_other_page_sizes(replayers, plain_models):
     for page_size in (4, 64):
         rep = replayers("B", "float32", max_tokens=128, page_size=page_size)
