@@ -227,6 +227,33 @@ def test_sizes_the_vector_kernels_do_not_take(tmp_path, sizes, dtype):
     close(np.concatenate(got), want, dtype)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_long_context_beside_a_short_one(tmp_path, dtype):
+    """2,600 tokens of one request (two long portions, then one token a step) beside a short request
+    that decodes meanwhile: block tables of more than 1,024 keys, prompt tiles with many keys, decode
+    steps whose keys are cut over many blocks."""
+    from conftest import TINY_D
+    from ullm_amd.replay import Replayer
+    from ullm_amd.weights.random_init import write_random_model
+    cfg = dict(TINY_D, max_position_embeddings=4096)
+    write_random_model(cfg, str(tmp_path), seed=9)
+    pcfg, w = plain.load_model_folder(str(tmp_path))
+    rep = Replayer(str(tmp_path), dtype, 2816, 16, DEV)
+    long, short = make_tokens(cfg["vocab_size"], 2600, 60), make_tokens(cfg["vocab_size"], 51, 61)
+    wl, ws = plain.qwen3_forward(w, pcfg, long), plain.qwen3_forward(w, pcfg, short)
+    got = rep.step({"step": 0, "entries": [{"id": "l", "tokens": long[:1500], "want": [0, 1499]},
+                                           {"id": "s", "tokens": short[:20], "want": [19]}], "end": []})
+    close(got, torch.stack([wl[0], wl[1499], ws[19]]), dtype)
+    got = rep.step({"step": 1, "entries": [{"id": "s", "tokens": [short[20]], "want": [0]},
+                                           {"id": "l", "tokens": long[1500:2570], "want": [0, 523, 524, 1069]}], "end": []})
+    close(got, torch.stack([ws[20], wl[1500], wl[2023], wl[2024], wl[2569]]), dtype)
+    for i in range(30):
+        last = i == 29
+        got = rep.step({"step": 2 + i, "entries": [{"id": "l", "tokens": [long[2570 + i]], "want": [0]},
+                                                   {"id": "s", "tokens": [short[21 + i]], "want": [0]}], "end": ["l", "s"] if last else []})
+        close(got, torch.stack([wl[2570 + i], ws[21 + i]]), dtype)
+
+
 def test_other_page_sizes(replayers, plain_models):
     for page_size in (4, 64):
         rep = replayers("B", "float32", max_tokens=128, page_size=page_size)
