@@ -76,7 +76,7 @@ gemm_partial_sums_kernel(const bf16_t* __restrict__ X, int ldx, const bf16_t* __
   auto fetch = [&](Stage& s, int k0) {
     const bool in = k0 + 8 * lcol < k_end;                          // K is a multiple of 8
 #pragma unroll
-    for (int h = 0; h < 2; ++h) s.w[h] = in ? *reinterpret_cast<const uint4*>(wsrc[h] + k0) : make_uint4(0, 0, 0, 0);
+    for (int h = 0; h < 2; ++h) s.w[h] = in ? ld_stream16(wsrc[h] + k0) : make_uint4(0, 0, 0, 0);
 #pragma unroll
     for (int q = 0; q < XQ; ++q) {
       const bool xin = xok[q] && k0 + 8 * ((tid + 64 * MID_WAVES * q) & 7) < k_end;

@@ -198,7 +198,7 @@ gemm_skinny_kernel(const void* __restrict__ Xv, int ldx, const bf16_t* __restric
     for (int h = 0; h < 2; ++h) {
 #pragma unroll
       for (int i = 0; i < NT; ++i)
-        st.w[i][h] = in ? *reinterpret_cast<const uint4*>(wsrc[i][h] + k0) : make_uint4(0, 0, 0, 0);
+        st.w[i][h] = in ? ld_stream16(wsrc[i][h] + k0) : make_uint4(0, 0, 0, 0);
       if (h < XH) {
 #pragma unroll
         for (int t = 0; t < MT; ++t)
