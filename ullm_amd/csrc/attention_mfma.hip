@@ -81,10 +81,10 @@ __device__ __forceinline__ void load_tile(KVTile<NQK>& t, int key0, const PageWi
     if (page >= 0) {
       const bf16_t* kp = k_pool + (((size_t)page * nkv + kvh) * page_size + off + c) * HD + 8 * g;
 #pragma unroll
-      for (int ch = 0; ch < NQK; ++ch) t.k[sb][ch].u4 = *reinterpret_cast<const uint4*>(kp + 32 * ch);
+      for (int ch = 0; ch < NQK; ++ch) t.k[sb][ch].u4 = ld_stream16(kp + 32 * ch);   // a decode step reads a key once
       const bf16_t* vp = v_pool + (((size_t)page * nkv + kvh) * HD + c) * page_size + off + 4 * g;
 #pragma unroll
-      for (int n = 0; n < 2 * NQK; ++n) t.v[n][sb] = *reinterpret_cast<const uint2*>(vp + (size_t)16 * n * page_size);
+      for (int n = 0; n < 2 * NQK; ++n) t.v[n][sb] = ld_stream8(vp + (size_t)16 * n * page_size);
     } else {
 #pragma unroll
       for (int ch = 0; ch < NQK; ++ch) t.k[sb][ch].u4 = make_uint4(0, 0, 0, 0);

@@ -48,6 +48,12 @@ __device__ __forceinline__ uint4 ld_stream16(const void* p) {
   return make_uint4(v.x, v.y, v.z, v.w);
 }
 
+__device__ __forceinline__ uint2 ld_stream8(const void* p) {
+  typedef __attribute__((ext_vector_type(2))) unsigned int u32x2;
+  const u32x2 v = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(p));
+  return make_uint2(v.x, v.y);
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int m = WAVE / 2; m > 0; m >>= 1) v += __shfl_xor(v, m, WAVE);
