@@ -14,6 +14,16 @@ __device__ __forceinline__ float4 ld4_f32(const bf16_t* p) {
   return make_float4(__uint_as_float(u.x << 16), __uint_as_float(u.x & 0xffff0000u),
                      __uint_as_float(u.y << 16), __uint_as_float(u.y & 0xffff0000u));
 }
+// the same for values that are read once (a branch result, the gate|up product): non-temporal loads
+__device__ __forceinline__ float4 ld4_f32_stream(const float* p) {
+  const uint4 u = ld_stream16(p);
+  return make_float4(__uint_as_float(u.x), __uint_as_float(u.y), __uint_as_float(u.z), __uint_as_float(u.w));
+}
+__device__ __forceinline__ float4 ld4_f32_stream(const bf16_t* p) {
+  const uint2 u = ld_stream8(p);
+  return make_float4(__uint_as_float(u.x << 16), __uint_as_float(u.x & 0xffff0000u),
+                     __uint_as_float(u.y << 16), __uint_as_float(u.y & 0xffff0000u));
+}
 __device__ __forceinline__ void st4_f32(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
 __device__ __forceinline__ void st4_f32(bf16_t* p, float4 v) {
   *reinterpret_cast<uint2*>(p) = make_uint2(pack2_bf16(v.x, v.y), pack2_bf16(v.z, v.w));
@@ -113,7 +123,7 @@ __global__ void add_rmsnorm_vec_kernel(const TB* __restrict__ branch, float* __r
       float4 s = ld4_f32(res + c);
       if (br) {
         for (int p = 0; p < n_branch; ++p) {
-          const float4 b = ld4_f32(br + (size_t)p * branch_stride + c);
+          const float4 b = ld4_f32_stream(br + (size_t)p * branch_stride + c);
           s.x += b.x; s.y += b.y; s.z += b.z; s.w += b.w;
         }
         if (write_res) st4_f32(res + c, s);
@@ -199,7 +209,7 @@ __global__ void silu_mul_vec_kernel(const T* __restrict__ gu, T* __restrict__ ou
   const size_t t = idx / per_row;
   const int i = 4 * (int)(idx - t * per_row);
   const T* row = gu + t * (size_t)(2 * I);
-  const float4 g = ld4_f32(row + i), u = ld4_f32(row + I + i);
+  const float4 g = ld4_f32_stream(row + i), u = ld4_f32_stream(row + I + i);
   float4 o;
   if (sizeof(T) == 4) {
     o = make_float4(g.x / (1.f + expf(-g.x)) * u.x, g.y / (1.f + expf(-g.y)) * u.y,
