@@ -151,7 +151,9 @@ extern "C" int ullm_add_rmsnorm(const void* branch, float* residual, const float
   if (n_rows <= 0) return 0;
   if (H <= 0 || n_branch < 1 || (n_branch > 1 && branch_stride % 4 != 0)) return ULLM_ERR_SHAPE;
   if (rows && write_res) return ULLM_ERR_UNSUPPORTED;  // a gathered row could be updated twice
-  const int threads = H >= 4096 ? 512 : 256;
+  // a block a row; with few rows the chip is far from full, so wide rows get as many threads as they have
+  // groups of four values (up to 1024), which puts all of a row's loads on their way at once
+  const int threads = H >= 4096 ? (n_rows <= 1024 ? 1024 : 512) : (H >= 2048 && n_rows <= 1024 ? 512 : 256);
   const bool vec = H % 4 == 0 && H <= 4 * NORM_VEC_MAX * threads && !(((uintptr_t)residual | (uintptr_t)gain |
                    (uintptr_t)y | (uintptr_t)branch) & 15);
   dim3 grid(n_rows), block(threads);
