@@ -408,7 +408,7 @@ qk_norm_rope_write_vec_kernel(
   float x[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   if (live) {
     const T* src = qkv + (size_t)t * qkv_stride + (size_t)head * hd + d0;
-    const float4 lo = ld4_f32(src), hi = ld4_f32(src + 4);
+    const float4 lo = ld4_f32_stream(src), hi = ld4_f32_stream(src + 4);     // the projection row is read once
     x[0] = lo.x; x[1] = lo.y; x[2] = lo.z; x[3] = lo.w; x[4] = hi.x; x[5] = hi.y; x[6] = hi.z; x[7] = hi.w;
   }
   int page = -1;
