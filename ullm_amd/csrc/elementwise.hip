@@ -65,6 +65,26 @@ extern "C" int ullm_embedding(const int* ids, const void* table, float* residual
   ULLM_LAUNCH_CHECK();
 }
 
+// ------------------------------------------------------------------ token ids that are still on the device
+// ids[t] = source[feed[t]] where feed[t] >= 0: the token a request sampled in the step before is taken
+// from that step's output, so the next step can be queued before the host has seen the token
+// (reference: the device-resident last sampled token, ullm/core/input_batch.py:184-186,
+// ullm/core/model_runner.py:277-280).
+__global__ void feed_tokens_kernel(int* __restrict__ ids, const int* __restrict__ feed, const int* __restrict__ source,
+                                   int n, int n_source) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= n) return;
+  const int f = feed[t];
+  if (f >= 0 && f < n_source) ids[t] = source[f];
+}
+
+extern "C" int ullm_feed_tokens(int* ids, const int* feed, const int* source, int n, int n_source, hipStream_t stream) {
+  if (n <= 0) return 0;
+  if (n_source <= 0) return ULLM_ERR_SHAPE;
+  hipLaunchKernelGGL(feed_tokens_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, ids, feed, source, n, n_source);
+  ULLM_LAUNCH_CHECK();
+}
+
 // ------------------------------------------------------------------ add + RMS norm
 // For output row r (input row i = rows ? rows[r] : r):
 //   s = residual[i] + float(branch[i])      (branch may be null: s = residual[i]; it may also be a stack

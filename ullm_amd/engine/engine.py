@@ -72,6 +72,13 @@ class Engine:
         self.scheduler = Scheduler(self.runner.cache, config.max_num_batched_tokens, config.max_prefill_chunk,
                                    config.max_bs)
         self.sampler = Sampler(env.device)
+        # the sampled ids of the step that ran last, on the device: the next step takes late token ids from
+        # here; each step's ids also go to pinned host memory (two buffers in turn) right behind its sampling
+        self._sampled_dev = torch.zeros(max(1, config.max_bs), dtype=torch.int32, device=env.device)
+        self.runner.feed_source = self._sampled_dev
+        pin = env.device.type == "cuda"
+        self._sampled_host = [torch.zeros(max(1, config.max_bs), dtype=torch.int32, pin_memory=pin) for _ in range(2)]
+        self._sampled_turn = 0
         self._arrivals = 0
         self._next: Optional[_Plan] = None   # the step after the one that ran last, scheduled and packed ahead
         self._inflight = None                # (plan, sampled ids on the device) of a step that is running
@@ -117,12 +124,14 @@ class Engine:
 
         The device works asynchronously, and the host uses that (reference: the overlap of scheduling
         and execution, docs/async_scheduling.md; ``disable_async_scheduling`` switches it off).
-        While a step's kernels run, the next step is scheduled and packed: what it depends on is
-        known without the tokens that are still being sampled (counts decide who continues; the ids
-        are filled in before its launch).  When the tokens arrive they are filed, requests that end
-        on their stop token (the one surprise) are taken out of the prepared step, and that step is
-        launched at once; only then are this step's results put together.  So a call returns the
-        results of one step while the next one is already running."""
+        While a step's kernels run, the next step is scheduled, packed and queued behind it: what it
+        depends on is known without the tokens that are still being sampled (counts decide who
+        continues; the ids stay on the device, where the next step picks them up from the sampler's
+        output, as the reference's device-resident last token does, docs/async_scheduling.md:13).
+        Only then does the host wait for this step's tokens and file them.  A request that ends on
+        its stop token (the one surprise) has one more token computed in the step already queued;
+        that step's result for it is dropped.  So a call returns the results of one step while the
+        next one is already running, and the device never waits for the host."""
         if self.config.disable_async_scheduling:
             return self._step_in_turn()
         if self._inflight is None:
@@ -137,7 +146,11 @@ class Engine:
         results = plan.early_results
         sampling = plan.sampling
         if sampled is None:                               # prompt portions only: nothing to wait for
-            self._next = self._make_plan()
+            nxt = self._make_plan()
+            if nxt.scheduled:
+                self._inflight = self._launch(nxt)
+            elif nxt.early_results:
+                self._next = nxt
             return results
         # while the device works: who ends by length, and the next step
         ended: Dict[int, FinishReason] = {}
@@ -154,8 +167,13 @@ class Engine:
                 ended[i] = reason
                 req.finish_reason = reason
                 self.scheduler.finish(req)
-        self._next = self._make_plan()
-        ids = sampled.tolist()                            # waits for the step
+        nxt = self._make_plan()
+        if nxt.scheduled:
+            # queued behind the running step at once: ids still unknown come from that step's output on the device
+            self._inflight = self._launch(nxt, {id(s.request): i for i, s in enumerate(sampling)})
+        elif nxt.early_results:
+            self._next = nxt
+        ids = self._read_sampled(sampled)                 # waits for the step
         stops = []
         for i, (s, tok) in enumerate(zip(sampling, ids)):
             if filed[i] is None:
@@ -165,14 +183,8 @@ class Engine:
             if tok == req.params.eos_token_id and not req.params.ignore_eos:
                 stops.append(i)
                 req.finish_reason = FinishReason.STOP    # the stop token wins over a length limit, as in the reference
-                if i not in ended:
-                    self.scheduler.finish(req)
-                    self._drop_from_next(req)
-        nxt, self._next = self._next, None
-        if nxt.scheduled:
-            self._inflight = self._launch(nxt)            # the device is busy again before the results are built
-        elif nxt.early_results:
-            self._next = nxt
+                if i not in ended and req.status is RequestStatus.RUNNING:
+                    self.scheduler.finish(req)            # the queued step still computes a token for it: dropped there
         for i, (s, tok) in enumerate(zip(sampling, ids)):
             if filed[i] is None:
                 continue
@@ -183,10 +195,12 @@ class Engine:
                                             req.num_generated_tokens))
         return results
 
-    def _launch(self, plan: "_Plan"):
-        """Queue a prepared step and its sampling on the device; returns (plan, sampled token ids as a
-        device tensor, or None if no request of the step samples)."""
-        self._fill_unknown_tokens(plan)
+    def _launch(self, plan: "_Plan", sampled_before: Optional[Dict[int, int]] = None):
+        """Queue a prepared step and its sampling on the device; returns (plan, handle of the sampled
+        token ids for :meth:`_read_sampled`, or None if no request of the step samples).
+        ``sampled_before``: id(request) -> row of the running step's sampler output, for the
+        requests whose newest token is still being sampled."""
+        self._fill_unknown_tokens(plan, sampled_before)
         sampling = plan.sampling
         sampler_inputs = None
         if sampling:                                      # uploaded ahead of the model's kernels
@@ -199,7 +213,24 @@ class Engine:
             return plan, None
         if self.on_logits is not None:
             self.on_logits(sampling, logits)
-        return plan, self.sampler.launch(logits, sampler_inputs)
+        n = len(sampling)
+        sampled = self.sampler.launch(logits, sampler_inputs, out=self._sampled_dev)
+        host = self._sampled_host[self._sampled_turn]
+        self._sampled_turn ^= 1
+        host[:n].copy_(sampled, non_blocking=True)        # in stream order: before the next step's sampling overwrites it
+        if host.is_pinned():
+            done = torch.cuda.Event()
+            done.record()
+        else:
+            done = None
+        return plan, (host, n, done)
+
+    @staticmethod
+    def _read_sampled(handle) -> List[int]:
+        host, n, done = handle
+        if done is not None:
+            done.synchronize()
+        return host[:n].tolist()
 
     def _step_in_turn(self) -> List[EngineStepResult]:
         """Schedule, run, wait, file the tokens: one thing after the other."""
@@ -210,7 +241,7 @@ class Engine:
         _, sampled = self._launch(plan)
         if sampled is None:
             return results
-        for s, tok in zip(plan.sampling, sampled.tolist()):
+        for s, tok in zip(plan.sampling, self._read_sampled(sampled)):
             req = s.request
             self.scheduler.append_token(req, tok)
             done, reason = self._is_finished(req)
@@ -252,13 +283,20 @@ class Engine:
             plan.sampler_staged = self.sampler.stage([s.request.params for s in plan.sampling],
                                                      [s.request.seed for s in plan.sampling], plan.sample_positions)
 
-    def _fill_unknown_tokens(self, plan: "_Plan") -> None:
+    def _fill_unknown_tokens(self, plan: "_Plan", sampled_before: Optional[Dict[int, int]] = None) -> None:
+        """Ids the host has learnt since the step was packed are written in; one that is still being
+        sampled (the newest token of a request of the running step) is left to the device."""
         for k, (b, j) in enumerate(plan.prepared.unknown_tokens()):
             s = plan.scheduled[b]
-            token = s.request.token_ids[s.start + j]
-            if token == UNKNOWN_TOKEN:
-                raise RuntimeError(f"request {s.request.request_id!r}: a token of the step is still unknown")
-            plan.prepared.fill_token(k, token)
+            req = s.request
+            token = req.token_ids[s.start + j]
+            if token != UNKNOWN_TOKEN:
+                plan.prepared.fill_token(k, token)
+                continue
+            row = None if sampled_before is None else sampled_before.get(id(req))
+            if row is None or s.start + j != req.num_tokens - 1:
+                raise RuntimeError(f"request {req.request_id!r}: a token of the step is still unknown")
+            plan.prepared.feed_token(k, row)
         plan.prepared.all_tokens_known()
 
     def _drop_from_next(self, req: Request) -> None:

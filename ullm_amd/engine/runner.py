@@ -35,6 +35,7 @@ class StepError(RuntimeError):
 
 UNKNOWN_TOKEN = -2         # stands for a token that is still being sampled when the step is prepared
 
+from ..kernels import ops
 from ..kernels.ops import PREFILL_TILE as Q_TILE   # tokens of one request per prompt-portion attention tile
 
 
@@ -67,6 +68,8 @@ class ModelRunner:
             self.caches[cache_id] = LayerCache(
                 state=torch.zeros((max_requests,) + tuple(need.shape), dtype=need.dtype, device=env.device))
         self._upload = StagedUpload(env.device)
+        # int32 device tensor the steps take late token ids from (the sampler's output of the step before), or None
+        self.feed_source: Optional[torch.Tensor] = None
         self.vocab_size = model.plan.vocab_size
         # Steps in which every entry brings one token are replayed from HIP graphs, one graph per
         # (batch size bucket, context length bucket).  Padding entries would disturb per-request state,
@@ -127,12 +130,13 @@ class ModelRunner:
         tile_list = [x for _, first, count in tile_keys for x in (first, count)]
         dec_list.extend(range(t0, t0 + n_pad))
         ng = len(groups)
-        sizes = [T, T, T, B + 1, B, B, n_want] + [B * s for s in strides] + [len(dec_list), len(tile_list)]
+        sizes = [T, T, T, B + 1, B, B, n_want] + [B * s for s in strides] + [len(dec_list), len(tile_list), T]
         offs = np.concatenate(([0], np.cumsum(sizes)))
         host = np.zeros(int(offs[-1]), dtype=np.int32)
         ids, pos, ent = host[offs[0]:offs[1]], host[offs[1]:offs[2]], host[offs[2]:offs[3]]
         q_start, slot, start = host[offs[3]:offs[4]], host[offs[4]:offs[5]], host[offs[5]:offs[6]]
         rows = host[offs[6]:offs[7]]
+        host[offs[9 + ng]:offs[10 + ng]] = -1             # per token: where the device takes its id from (-1: from ids)
         caches = [e.cache for e in entries]
         starts = [rc.num_computed for rc in caches]
         slots = [rc.slot for rc in caches]
@@ -284,12 +288,21 @@ class ModelRunner:
         if prepared.graph_key is not None:
             logits = self._launch_graph(prepared)
         else:
-            ctx, rows = self._context(self._send(prepared), prepared.offs, prepared.facts)
+            dev = self._send(prepared)
+            self._feed(dev, prepared.offs)
+            ctx, rows = self._context(dev, prepared.offs, prepared.facts)
             with torch.no_grad():
                 logits = self.model.forward(ctx, self.caches, rows)
         for e in entries:
             self.cache.commit(e.cache, len(e.tokens))
         return logits
+
+    def _feed(self, dev: torch.Tensor, offs) -> None:
+        """Token ids that the step before has sampled and the host has not seen (see
+        :meth:`PreparedStep.feed_token`) are taken from ``feed_source`` on the device."""
+        if self.feed_source is not None:
+            last = len(offs) - 1
+            ops.feed_tokens(dev[int(offs[0]):int(offs[1])], dev[int(offs[last - 1]):int(offs[last])], self.feed_source)
 
     def build_context(self, entries: Sequence[StepEntry]):
         """Flatten the entries into device tensors (one host-to-device copy)."""
@@ -324,12 +337,14 @@ class ModelRunner:
             side = torch.cuda.Stream()
             side.wait_stream(torch.cuda.current_stream())
             with torch.cuda.stream(side):
+                self._feed(static_dev, offs)
                 self.model.forward(ctx, self.caches, rows)
             torch.cuda.current_stream().wait_stream(side)
             if self._graph_pool is None:
                 self._graph_pool = torch.cuda.graph_pool_handle()
             g = torch.cuda.CUDAGraph()
             with torch.cuda.graph(g, pool=self._graph_pool):
+                self._feed(static_dev, offs)
                 logits = self.model.forward(ctx, self.caches, rows)
         graph = _DecodeGraph(g, static_dev, logits)
         self._graphs[key] = graph
@@ -356,6 +371,14 @@ class PreparedStep:
         self.host[at] = token
         if self.staged is not None:
             self.staged[at] = token
+
+    def feed_token(self, k: int, index: int) -> None:
+        """The k-th unknown token is entry ``index`` of the runner's ``feed_source`` when the step runs."""
+        t = self.facts["unknown"][k][0]
+        at = int(self.offs[len(self.offs) - 2]) + t
+        self.host[at] = index
+        if self.staged is not None:
+            self.staged[at] = index
 
     def all_tokens_known(self) -> None:
         self.facts["unknown"] = []

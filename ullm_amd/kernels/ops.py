@@ -85,6 +85,17 @@ def embedding(ids: torch.Tensor, table: torch.Tensor, out: Optional[torch.Tensor
     return out
 
 
+def feed_tokens(ids: torch.Tensor, feed: torch.Tensor, source: torch.Tensor) -> None:
+    """ids[t] = source[feed[t]] wherever feed[t] >= 0 (all int32): token ids that the step before has
+    sampled and the host has not yet seen are taken from that step's output on the device."""
+    n = ids.numel()
+    _i32(ids, "ids")
+    _i32(feed, "feed", n)
+    _i32(source, "source")
+    _check(build.load("elementwise").ullm_feed_tokens(_p(ids), _p(feed), _p(source), _c_int(n),
+                                                      _c_int(source.numel()), _stream()), "feed_tokens")
+
+
 def add_rmsnorm(branch: Optional[torch.Tensor], residual: torch.Tensor, gain: torch.Tensor, eps: float,
                 out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None,
                 out: Optional[torch.Tensor] = None) -> torch.Tensor:

@@ -53,14 +53,14 @@ class Sampler:
     def prepare(self, params: Sequence[SamplingParams], seeds: Sequence[int], positions: Sequence[int]) -> SamplerInputs:
         return self.send(self.stage(params, seeds, positions))
 
-    def launch(self, logits: torch.Tensor, prepared: SamplerInputs) -> torch.Tensor:
+    def launch(self, logits: torch.Tensor, prepared: SamplerInputs, out: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Queue the sampling kernel; returns the n token ids as an int32 device tensor (reading it
-        waits for the step)."""
+        waits for the step), the first n entries of ``out`` if that is given."""
         if prepared.n != logits.shape[0]:
             raise ValueError("one parameter set, seed and position per logits row is needed")
         f = prepared.packed[0:3].view(torch.float32)
         i = prepared.packed
-        return ops.sample(logits, f[0], i[3], f[1], f[2], i[4], i[5], i[6])
+        return ops.sample(logits, f[0], i[3], f[1], f[2], i[4], i[5], i[6], out=out)[:prepared.n]
 
     def sample(self, logits: torch.Tensor, params: Optional[Sequence[SamplingParams]] = None,
                seeds: Optional[Sequence[int]] = None, positions: Optional[Sequence[int]] = None,
