@@ -505,6 +505,43 @@ def test_gemm_skinny(ops, shape, out_dtype):
     assert torch.equal(got2, got)
 
 
+@pytest.mark.parametrize("shape", [(8, 200, 256), (3, 6144, 512), (16, 1000, 264), (20, 520, 128)])
+def test_gemm_skinny_with_fewer_columns_a_block(ops, shape):
+    """A block may own fewer columns of the result than its tiles hold (so that the blocks spread
+    evenly over the compute units): every such split gives the same product, the folded forms too."""
+    torch.manual_seed(16)
+    M, N, K = shape
+    a = torch.randn(M, K, device=DEV).bfloat16()
+    w = (torch.randn(N, K, device=DEV) * 0.3).bfloat16()
+    b = torch.randn(N, device=DEV)
+    want = ops.gemm_skinny(a, w, b, out_dtype=torch.float32)
+    ref = a.double().cpu() @ w.double().cpu().T + b.double().cpu()
+    assert (want.double().cpu() - ref).abs().max() <= 2e-5 * float(ref.abs().max())
+    stream0 = torch.randn(M, N, device=DEV)
+    gain = 1.0 + 0.5 * torch.randn(K, device=DEV)
+    hstream = torch.randn(M, K, device=DEV)
+    for nt, rows in ((1, 4), (1, 12), (2, 20), (2, 24), (2, 28), (1, 16), (2, 32)):
+        got = ops.gemm_skinny(a, w, b, out_dtype=torch.float32, nt=nt, rows=rows)
+        assert torch.equal(got, want) or (got - want).abs().max() <= 2e-6 * float(want.abs().max()), (nt, rows)
+        s1, s2 = stream0.clone(), stream0.clone()
+        ops.gemm_skinny_add(a, w, s1, nt=nt)
+        ops.gemm_skinny_add(a, w, s2, nt=nt, rows=rows)
+        assert (s1 - s2).abs().max() <= 2e-6 * float(s1.abs().max()), (nt, rows)
+        if M <= 16:
+            n1 = ops.gemm_skinny_normed(hstream, gain, 1e-5, w, b, out_dtype=torch.float32, nt=nt)
+            n2 = ops.gemm_skinny_normed(hstream, gain, 1e-5, w, b, out_dtype=torch.float32, nt=nt, rows=rows)
+            assert (n1 - n2).abs().max() <= 2e-6 * float(n1.abs().max()), (nt, rows)
+    inter = N // 2
+    wgu = torch.cat([w[:inter], w[N - inter:]]).contiguous()
+    g1 = ops.gemm_skinny_silu(a, wgu)
+    for rows in (4, 12, 16):
+        assert torch.equal(ops.gemm_skinny_silu(a, wgu, rows=rows), g1), rows
+    with pytest.raises(Exception):
+        ops.gemm_skinny(a, w, b, nt=1, rows=20)            # more than a tile holds
+    with pytest.raises(Exception):
+        ops.gemm_skinny(a, w, b, nt=2, rows=10)            # no multiple of 4
+
+
 @pytest.mark.parametrize("shape", [(1, 64, 128), (8, 6144, 4096), (5, 100, 1032), (16, 328, 72), (3, 70000, 264),
                                    (13, 24, 5128)])
 def test_gemm_skinny_with_the_norm_folded_in(ops, shape):

@@ -138,7 +138,7 @@ template <int MT, int NT, int EPI, typename TC, bool NORMX, int XH>
 __global__ void __launch_bounds__(64 * sk_max_waves(MT, NT))
 gemm_skinny_kernel(const void* __restrict__ Xv, int ldx, const bf16_t* __restrict__ W, int ldw,
                    const float* __restrict__ bias, const float* __restrict__ gain, float eps, TC* __restrict__ C,
-                   float* __restrict__ R, int ldc, int M, int N, int K, int k_per_wave) {
+                   float* __restrict__ R, int ldc, int M, int N, int K, int k_per_wave, int rows_per_block) {
   constexpr int MAXW = sk_max_waves(MT, NT);
   constexpr int TILE_BYTES = 16 * 128, STAGE_BYTES = (NT + MT) * TILE_BYTES;
   constexpr int RED_BYTES = (MAXW - 1) * NT * MT * 256 * 4;
@@ -151,8 +151,12 @@ gemm_skinny_kernel(const void* __restrict__ Xv, int ldx, const bf16_t* __restric
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int g = lane >> 4, r = lane & 15, lrow = lane >> 3, lcol = lane & 7;
   constexpr int OT = EPI == EPI_SILU ? NT / 2 : NT;
-  const int n0 = blockIdx.x * (16 * OT);
+  // a block's columns of the result: rows_per_block <= 16 OT of them (the host picks the number that spreads
+  // the matrix evenly over the compute units); rows of W past them are neither fetched nor stored
+  const int n0 = blockIdx.x * rows_per_block;
+  const int n_end = n0 + rows_per_block < N ? n0 + rows_per_block : N;
   const bf16_t* wsrc[NT][2];
+  bool wrow[NT][2];
   static_assert(XH == 2 || MT == 1, "half a tile of X only where it is the only tile");
   const XT* xsrc[MT][XH];
   bool xrow[MT][XH];                                      // rows of X past M are zeros and cost no load
@@ -165,7 +169,8 @@ gemm_skinny_kernel(const void* __restrict__ Xv, int ldx, const bf16_t* __restric
 #pragma unroll
     for (int i = 0; i < NT; ++i) {
       const int col = n0 + 16 * (i % OT) + row;
-      const int n = (col < N ? col : N - 1) + (i / OT) * N;       // rows past N repeat the last row; never stored
+      wrow[i][h] = col < n_end;
+      const int n = (wrow[i][h] ? col : n_end - 1) + (i / OT) * N;
       wsrc[i][h] = W + (size_t)n * ldw + 8 * lcol;
     }
     if (h < XH) {
@@ -198,7 +203,7 @@ gemm_skinny_kernel(const void* __restrict__ Xv, int ldx, const bf16_t* __restric
     for (int h = 0; h < 2; ++h) {
 #pragma unroll
       for (int i = 0; i < NT; ++i)
-        st.w[i][h] = in ? ld_stream16(wsrc[i][h] + k0) : make_uint4(0, 0, 0, 0);
+        st.w[i][h] = in && wrow[i][h] ? ld_stream16(wsrc[i][h] + k0) : make_uint4(0, 0, 0, 0);
       if (h < XH) {
 #pragma unroll
         for (int t = 0; t < MT; ++t)
@@ -283,7 +288,7 @@ gemm_skinny_kernel(const void* __restrict__ Xv, int ldx, const bf16_t* __restric
   }
   __syncthreads();                                        // the partial sums take the place of the stages
   auto& red = *reinterpret_cast<float (*)[MAXW - 1][NT * MT][64 * 4]>(lds);
-  skinny_finish<MT, NT, EPI, TC, NORMX>(acc, red, bias, C, R, ldc, M, N, n0, sq, K, eps);
+  skinny_finish<MT, NT, EPI, TC, NORMX>(acc, red, bias, C, R, ldc, M, n_end, n0, sq, K, eps);
 }
 
 template <int MT, int NT, int EPI, typename TC, bool NORMX, typename... Args>
@@ -301,6 +306,33 @@ static void skinny_launch(dim3 grid, dim3 block, hipStream_t stream, const void*
                      gain, eps, C, R, ldc, M, rest...);
 }
 
+static int skinny_compute_units() {
+  static int units[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (units[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    units[dev] = n;
+  }
+  return units[dev];
+}
+
+// Columns of the result per block for a block shape that holds up to `cap` of them: the matrix is cut into a
+// whole multiple of the compute units' number of blocks (a matrix whose 16-column tiles are 1.25 or 1.5 times
+// that number otherwise leaves most units idle for the last part of the run), in steps of 4 columns.
+// Returns the share of block slots that do work, in 1/1024.
+static int skinny_rows(int N, int cap, int units, int* rows) {
+  const int bmin = (N + cap - 1) / cap;
+  const int rounds = (bmin + units - 1) / units;
+  int r = (N + rounds * units - 1) / (rounds * units);
+  r = (r + 3) / 4 * 4;
+  if (r > cap) r = cap;
+  *rows = r;
+  const int blocks = (N + r - 1) / r;
+  return (int)(1024LL * blocks / ((long long)((blocks + units - 1) / units) * units));
+}
+
 extern "C" int ullm_gemm_skinny_supports(int M, int N, int K, int ldx, int ldw) {
   return M >= 1 && M <= 64 && N >= 1 && K >= 8 && K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0;
 }
@@ -311,7 +343,7 @@ extern "C" int ullm_gemm_skinny_supports(int M, int N, int K, int ldx, int ldw) 
 // is multiplied (epi 0 and 2).  force_nt / force_waves: 0 = chosen here.
 extern "C" int ullm_gemm_skinny(const void* X, int ldx, const void* W, int ldw, const float* bias, void* C,
                                 int ldc, int M, int N, int K, int epi, int c_dtype, int force_nt,
-                                int force_waves, const float* gain, float eps, hipStream_t stream) {
+                                int force_waves, const float* gain, float eps, int force_rows, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (!ullm_gemm_skinny_supports(M, N, K, ldx, ldw) || ldc < N) return ULLM_ERR_SHAPE;
   if (((uintptr_t)X & 15) || ((uintptr_t)W & 15)) return ULLM_ERR_SHAPE;
@@ -332,21 +364,41 @@ extern "C" int ullm_gemm_skinny(const void* X, int ldx, const void* W, int ldw, 
   if (epi == EPI_SILU) nt = (force_nt == 4 || mt >= 4) ? 4 : 2;   // gate and up tiles come in pairs
   if (nt != 1 && nt != 2 && nt != 4) return ULLM_ERR_UNSUPPORTED;
   if (nt == 4 && mt == 1) nt = 2;                       // not instantiated
+  // Columns of the result per block.  Up to 16 rows of X, a matrix that fills the chip is spread evenly over
+  // the compute units; for store and add that may take two tiles of W a block of which only a part is used
+  // (5120 columns: 256 blocks of 20 instead of 320 of 16; down projection of Qwen3-32B at 8 rows 63.9 -> 50.4 us,
+  // of Qwen3-14B 44.1 -> 34.6 us; q|k|v of Qwen3-8B, 6144 columns in 256 blocks of 24, 14.8 -> 14.0 us).
+  int rows = 16 * (epi == EPI_SILU ? nt / 2 : nt);
+  const int units = skinny_compute_units();
+  if (force_rows <= 0 && mt == 1 && N >= 16 * units) {
+    if (epi == EPI_SILU || force_nt > 0 || nt == 2) {
+      skinny_rows(N, rows, units, &rows);
+    } else {
+      int r1 = 16, r2 = 32;
+      const int e1 = skinny_rows(N, 16, units, &r1), e2 = skinny_rows(N, 32, units, &r2);
+      if (e2 > e1) { nt = 2; rows = r2; } else { nt = 1; rows = r1; }
+    }
+  }
   const int out_tiles = epi == EPI_SILU ? nt / 2 : nt;  // 16-column tiles of the result per block
-  const int tiles = (tiles16 + out_tiles - 1) / out_tiles;
+  if (force_rows > 0) {
+    if (force_rows > 16 * out_tiles || force_rows % 4) return ULLM_ERR_UNSUPPORTED;
+    rows = force_rows;
+  }
+  const int tiles = (N + rows - 1) / rows;
   // waves per block: 8 tiles of W in flight per block (measured: 8 waves with one tile each, 4 with two),
   // each wave with at least 128 values of K
   const int max_waves = sk_max_waves(mt, nt);
   int waves = 1;
-  const int in_flight = gain && epi == EPI_STORE ? 16 : 8;
-  while (waves < max_waves && waves * nt < in_flight && K / (waves * 2) >= 128) waves *= 2;
+  const int in_flight = (gain && epi == EPI_STORE) || epi == EPI_SILU ? 16 : 8;   // in 16-row tiles of W
+  const int w_rows = rows * (nt / out_tiles);           // rows of W a block fetches
+  while (waves < max_waves && waves * w_rows < 16 * in_flight && K / (waves * 2) >= 128) waves *= 2;
   if (force_waves > 0) waves = force_waves < max_waves ? force_waves : max_waves;
   int k_per_wave = (K + waves - 1) / waves;
   k_per_wave = (k_per_wave + 63) / 64 * 64;
   dim3 grid(tiles), block(64 * waves);
   float* R = (float*)C;
 #define GO_(MT, NT, EPI, TC, NORMX) skinny_launch<MT, NT, EPI, TC, NORMX>(grid, block, stream, X, ldx, \
-    (const bf16_t*)W, ldw, bias, gain, eps, (TC*)C, R, ldc, M, N, K, k_per_wave)
+    (const bf16_t*)W, ldw, bias, gain, eps, (TC*)C, R, ldc, M, N, K, k_per_wave, rows)
 #define GO(MT, NT, EPI, TC) GO_(MT, NT, EPI, TC, false)
 #define GO_SHAPE(EPI, TC)                                              \
   switch (mt * 8 + nt) {                                               \

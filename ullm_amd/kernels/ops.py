@@ -245,18 +245,18 @@ def gemm_skinny_supports(a: torch.Tensor, w: torch.Tensor) -> bool:
     return a.dtype == torch.bfloat16 and _skinny_ok(a.shape[0], a.shape[1], a, w)
 
 
-def _gemm_skinny(x, w, bias, c, M, N, K, epi, c_dtype, nt=0, waves=0, gain=None, eps=0.0) -> None:
+def _gemm_skinny(x, w, bias, c, M, N, K, epi, c_dtype, nt=0, waves=0, gain=None, eps=0.0, rows=0) -> None:
     lib = build.load("gemm_skinny")
     _check(lib.ullm_gemm_skinny(_p(x), _c_int(x.stride(0)), _p(w), _c_int(w.stride(0)), _p(bias),
                                 _p(c), _c_int(c.stride(0)), _c_int(M), _c_int(N), _c_int(K),
                                 _c_int(epi), _c_int(c_dtype), _c_int(nt), _c_int(waves), _p(gain),
-                                ctypes.c_float(eps), _stream()),
+                                ctypes.c_float(eps), _c_int(rows), _stream()),
            "gemm_skinny")
 
 
 def gemm_skinny(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
                 out_dtype: Optional[torch.dtype] = None, out: Optional[torch.Tensor] = None,
-                nt: int = 0, waves: int = 0) -> torch.Tensor:
+                nt: int = 0, waves: int = 0, rows: int = 0) -> torch.Tensor:
     """a [M <= 64, K] times w [N, K] transposed, bfloat16 operands streamed once through the matrix
     cores, 32-bit accumulation; output bfloat16 or float32."""
     M, K = a.shape
@@ -268,11 +268,12 @@ def gemm_skinny(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] =
     _need(out.shape == (M, N) and out.stride(1) == 1, "bad gemm output")
     if bias is not None:
         _need(bias.dtype == torch.float32 and bias.numel() == N and bias.is_contiguous(), "bias must be float32 [N]")
-    _gemm_skinny(a, w, bias, out, M, N, K, 0, _dt(out), nt, waves)
+    _gemm_skinny(a, w, bias, out, M, N, K, 0, _dt(out), nt, waves, rows=rows)
     return out
 
 
-def gemm_skinny_add(a: torch.Tensor, w: torch.Tensor, residual: torch.Tensor, nt: int = 0, waves: int = 0) -> None:
+def gemm_skinny_add(a: torch.Tensor, w: torch.Tensor, residual: torch.Tensor, nt: int = 0, waves: int = 0,
+                    rows: int = 0) -> None:
     """residual (float32 [M, N]) += a (bfloat16 [M, K]) times w transposed."""
     M = a.shape[0]
     N, K = w.shape
@@ -280,10 +281,10 @@ def gemm_skinny_add(a: torch.Tensor, w: torch.Tensor, residual: torch.Tensor, nt
           "gemm_skinny_add takes bfloat16 activations [M <= 64, K]")
     _need(residual.dtype == torch.float32 and residual.shape == (M, N) and residual.stride(1) == 1
           and residual.stride(0) % 4 == 0 and residual.data_ptr() % 16 == 0, "residual must be float32 [M, N]")
-    _gemm_skinny(a, w, None, residual, M, N, K, 1, F32, nt, waves)
+    _gemm_skinny(a, w, None, residual, M, N, K, 1, F32, nt, waves, rows=rows)
 
 
-def gemm_skinny_silu(a: torch.Tensor, w_gate_up: torch.Tensor, nt: int = 0, waves: int = 0) -> torch.Tensor:
+def gemm_skinny_silu(a: torch.Tensor, w_gate_up: torch.Tensor, nt: int = 0, waves: int = 0, rows: int = 0) -> torch.Tensor:
     """silu(a g^T) * (a u^T) as bfloat16 [M, I] for a (bfloat16 [M, K]) and the stacked weights
     g | u (bfloat16 [2 I, K]); the activation is applied to the 32-bit sums."""
     M, K = a.shape
@@ -291,7 +292,7 @@ def gemm_skinny_silu(a: torch.Tensor, w_gate_up: torch.Tensor, nt: int = 0, wave
     _need(K == K2 and two_i % 2 == 0, f"gate|up weights must be [2 I, {K}]")
     _need(a.dtype == torch.bfloat16 and _skinny_ok(M, K, a, w_gate_up), "gemm_skinny_silu takes bfloat16 [M <= 64, K]")
     out = torch.empty((M, two_i // 2), dtype=torch.bfloat16, device=a.device)
-    _gemm_skinny(a, w_gate_up, None, out, M, two_i // 2, K, 2, BF16, nt, waves)
+    _gemm_skinny(a, w_gate_up, None, out, M, two_i // 2, K, 2, BF16, nt, waves, rows=rows)
     return out
 
 
@@ -307,7 +308,7 @@ def gemm_skinny_normed_supports(stream: torch.Tensor, gain: torch.Tensor, w: tor
 
 def gemm_skinny_normed(stream: torch.Tensor, gain: torch.Tensor, eps: float, w: torch.Tensor,
                        bias: Optional[torch.Tensor] = None, out_dtype: torch.dtype = torch.bfloat16,
-                       silu: bool = False, nt: int = 0, waves: int = 0) -> torch.Tensor:
+                       silu: bool = False, nt: int = 0, waves: int = 0, rows: int = 0) -> torch.Tensor:
     """rmsnorm(stream) times w transposed for the float32 residual stream [M <= 16, K], the norm
     (gain float32 [K], eps) folded into the product: the kernel rounds stream * gain to bfloat16 for
     the matrix cores, sums the squares of the rows it reads anyway and scales the 32-bit sums by
@@ -323,7 +324,7 @@ def gemm_skinny_normed(stream: torch.Tensor, gain: torch.Tensor, eps: float, w: 
     if bias is not None:
         _need(bias.dtype == torch.float32 and bias.numel() == N and bias.is_contiguous(), "bias must be float32 [N]")
     out = torch.empty((M, N), dtype=out_dtype, device=stream.device)
-    _gemm_skinny(stream, w, bias, out, M, N, K, 2 if silu else 0, _dt(out), nt, waves, gain, float(eps))
+    _gemm_skinny(stream, w, bias, out, M, N, K, 2 if silu else 0, _dt(out), nt, waves, gain, float(eps), rows)
     return out
 
 
