@@ -318,7 +318,7 @@ attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __re
   {
     const bf16_t* const cq[1] = {col_ok ? q + (size_t)t * q_stride + (size_t)head * HD : nullptr};
     const int clo[1] = {lo}, chi[1] = {col_ok ? pos : -1};
-    attend_range<NQK, 1, (WAVES > 4 ? 1 : 2)>(cq, clo, chi, begin, end, pos, k_pool, v_pool,
+    attend_range<NQK, 1, (WAVES > 4 || NQK >= 8 ? 1 : 2)>(cq, clo, chi, begin, end, pos, k_pool, v_pool,
                                               block_table + (size_t)token_entry[t] * bt_stride, page_size, nkv, kvh,
                                               scale_log2e, accs, ms, ls);
   }
