@@ -113,6 +113,16 @@ class Engine:
             self.scheduler.finish(req)
             self._drop_from_next(req)
 
+    def drain(self) -> None:
+        """Wait for a step that is still running on the device (its results are dropped)."""
+        if self._inflight is not None:
+            _, handle = self._inflight
+            self._inflight = None
+            if handle is not None:
+                self._read_sampled(handle)
+        if self.env.device.type == "cuda":
+            torch.cuda.synchronize(self.env.device)
+
     def has_unfinished_requests(self) -> bool:
         """True while a request waits or runs, or a prepared step still has an ending to report."""
         return self.scheduler.has_unfinished() or (self._next is not None and bool(self._next.early_results))
@@ -214,6 +224,8 @@ class Engine:
         if self.on_logits is not None:
             self.on_logits(sampling, logits)
         n = len(sampling)
+        if n > self._sampled_dev.numel():
+            raise RuntimeError(f"{n} requests sample in one step, more than max_bs={self.config.max_bs}")
         sampled = self.sampler.launch(logits, sampler_inputs, out=self._sampled_dev)
         host = self._sampled_host[self._sampled_turn]
         self._sampled_turn ^= 1

@@ -185,5 +185,8 @@ class LLM:
             self._profiler = None
 
     def shutdown(self) -> None:
-        """Nothing runs in the background; kept so that callers of the reference's API need no change."""
+        """Nothing runs in the background; a step that was queued ahead for requests which have ended
+        meanwhile is waited for, then the engine is let go (the reference's callers need no change)."""
+        if self.engine is not None:
+            self.engine.drain()
         self.engine = None
