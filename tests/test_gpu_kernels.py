@@ -18,6 +18,26 @@ def ops():
     return o
 
 
+def test_feed_tokens(ops):
+    """Token ids a step takes from the sampler's output of the step before: only where the map says so."""
+    ids = torch.tensor([5, 0, 9, 0, 0, 7], dtype=torch.int32, device=DEV)
+    feed = torch.tensor([-1, 2, -1, 0, 3, -1], dtype=torch.int32, device=DEV)
+    source = torch.tensor([40, 41, 42, 43], dtype=torch.int32, device=DEV)
+    ops.feed_tokens(ids, feed, source)
+    assert ids.tolist() == [5, 42, 9, 40, 43, 7]
+    big = torch.arange(1000, dtype=torch.int32, device=DEV)
+    feed = torch.full((1000,), -1, dtype=torch.int32, device=DEV)
+    feed[::3] = torch.arange(334, dtype=torch.int32, device=DEV) % 4
+    want = big.clone()
+    want[::3] = source[(torch.arange(334, device=DEV) % 4).long()]
+    ops.feed_tokens(big, feed, source)
+    assert torch.equal(big, want)
+    # an index past the source leaves the id alone (the host never packs one)
+    ids = torch.tensor([1, 2], dtype=torch.int32, device=DEV)
+    ops.feed_tokens(ids, torch.tensor([9, -1], dtype=torch.int32, device=DEV), source)
+    assert ids.tolist() == [1, 2]
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_embedding(ops, dtype):
     torch.manual_seed(0)
