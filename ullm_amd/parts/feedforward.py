@@ -14,9 +14,11 @@ from .linear import can_fuse, linear, linear_into_stream, linear_of_norm
 
 
 # Rows up to which the weight-streaming kernel with the activation folded in beats the library product plus the
-# activation kernel: at 16 rows 32.9 against 46.3 us on Qwen3-8B's matrix and 68.3 against 77.5 us on Qwen3-14B's;
-# at 24 rows 45.9 against 46.6 and 84.2 against 78.8 us.
-GATE_UP_SKINNY_MAX_ROWS = 16
+# activation kernel (in a graph, gate|up of Qwen3-8B / 14B / 32B): at 16 rows 33 / 68 / 95 us against 46 / 87 / 97 us;
+# at 17 to 32 rows 36-40 / 71-83 / 98-115 us against 48-52 / 85-89 / 96-99 us; from 33 rows on the library is ahead
+# everywhere.  So up to 32 rows, but only up to 16 for matrices beyond Qwen3-14B's 178 M elements.
+GATE_UP_SKINNY_MAX_ROWS = 32
+GATE_UP_SKINNY_WIDE_MAX_WEIGHT = 200_000_000     # elements of gate|up up to which 17 to 32 rows take that kernel too
 
 
 @register_part("ffn", "swiglu")
@@ -39,7 +41,9 @@ class SwiGLU(FeedForward):
         self.w_down = tensors[f"{p}.down_proj.weight"].contiguous()
 
     def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
-        if (x.dtype == torch.bfloat16 and x.shape[0] <= GATE_UP_SKINNY_MAX_ROWS
+        rows = x.shape[0]
+        if (x.dtype == torch.bfloat16 and rows <= GATE_UP_SKINNY_MAX_ROWS
+                and (rows <= 16 or self.w_gate_up.numel() <= GATE_UP_SKINNY_WIDE_MAX_WEIGHT)
                 and ops.gemm_skinny_supports(x, self.w_gate_up)):
             act = ops.gemm_skinny_silu(x, self.w_gate_up)
         else:
