@@ -173,6 +173,79 @@ def test_scheduling_ahead_changes_no_token(model_dirs, plain_models):
     assert runs[True][1] > 0 and runs[False][1] > 0               # both runs had to preempt
 
 
+@pytest.mark.parametrize("pages", [9, 11, 13])
+def test_stop_tokens_while_requests_are_preempted(model_dirs, plain_models, pages):
+    """Every request stops on a token of its own continuation while pages are so scarce that the
+    youngest requests are preempted again and again (also in the very step that samples their stop
+    token, and while the step after it is already queued): each ends where the plain continuation
+    first shows its stop token, with and without the overlap, and all pages come back."""
+    from ullm_amd import FinishReason, SamplingParams
+    cfg, w = plain_models["B"]
+    prompts = prompts_of(503, (13, 6, 9, 3, 11, 5, 8), 33)
+    greedy = [plain.greedy_generate(w, cfg, p, 12) for p in prompts]
+    stops = [g[k] for g, k in zip(greedy, (9, 3, 6, 11, 4, 8, 2))]
+    want = [g[:g.index(t) + 1] for g, t in zip(greedy, stops)]
+    preempted = 0
+    for ahead in (False, True):
+        llm = make_llm(model_dirs["B"], page_size=4, num_pages=pages, max_num_batched_tokens=12, max_prefill_chunk=5,
+                       disable_async_scheduling=not ahead)
+        eng = llm.engine
+        for i, (p, t) in enumerate(zip(prompts, stops)):
+            eng.add_request(f"r{i}", p, SamplingParams(temperature=0.0, max_new_tokens=12, eos_token_id=t))
+        got, steps = {}, 0
+        while eng.has_unfinished_requests():
+            for r in eng.step():
+                rec = got.setdefault(r.seq_id, [[], None])
+                if r.new_token_id >= 0:
+                    rec[0].append(r.new_token_id)
+                if r.is_finished:
+                    rec[1] = r.finish_reason
+            steps += 1
+            assert steps < 3000
+        for i in range(len(prompts)):
+            assert got[f"r{i}"] == [want[i], FinishReason.STOP], (ahead, i)
+        assert eng.runner.cache.num_free_pages() == pages
+        eng.runner.cache.check()
+        preempted += eng.scheduler.num_preemptions
+    assert preempted > 0
+
+
+@pytest.mark.parametrize("ahead", [False, True])
+def test_a_request_preempted_while_its_stop_token_is_sampled_ends_there(model_dirs, plain_models, ahead):
+    """Three requests need a new page in the same step and none is free: the youngest loses its pages to
+    the two older ones, in the planning round in which its third token, its stop token as it turns
+    out, is still on the device.  When the token arrives the request ends; it is not run again."""
+    from ullm_amd import FinishReason, SamplingParams
+    cfg, w = plain_models["B"]
+    for seed in range(40, 60):                       # a youngest request whose third token is new to its continuation
+        prompts = prompts_of(503, (14, 14, 6), seed)
+        third = plain.greedy_generate(w, cfg, prompts[2], 3)
+        if third[2] not in third[:2]:
+            break
+    greedy = [plain.greedy_generate(w, cfg, p, 6) for p in prompts[:2]]
+    llm = make_llm(model_dirs["B"], page_size=4, num_pages=10, max_num_batched_tokens=64, max_prefill_chunk=64,
+                   disable_async_scheduling=not ahead)
+    eng = llm.engine
+    for i in range(2):
+        eng.add_request(f"r{i}", prompts[i], SamplingParams(temperature=0.0, max_new_tokens=6, ignore_eos=True))
+    eng.add_request("r2", prompts[2], SamplingParams(temperature=0.0, max_new_tokens=10, eos_token_id=third[2]))
+    got, steps = {}, 0
+    while eng.has_unfinished_requests():
+        for r in eng.step():
+            rec = got.setdefault(r.seq_id, [[], None])
+            if r.new_token_id >= 0:
+                rec[0].append(r.new_token_id)
+            if r.is_finished:
+                rec[1] = r.finish_reason
+        steps += 1
+        assert steps < 200
+    assert eng.scheduler.num_preemptions == (1 if ahead else 0)     # in turn, the stop token is known before the pages run out
+    assert got["r2"] == [third, FinishReason.STOP]
+    assert got["r0"] == [greedy[0], FinishReason.LENGTH] and got["r1"] == [greedy[1], FinishReason.LENGTH]
+    assert eng.runner.cache.num_free_pages() == 10
+    eng.runner.cache.check()
+
+
 @pytest.mark.parametrize("seed", [0, 1, 2])
 def test_scheduling_ahead_under_random_arrivals_and_aborts(model_dirs, seed):
     """Requests arrive while others run, some are aborted, pages are scarce and prefixes are shared:

@@ -193,8 +193,10 @@ class Engine:
             if tok == req.params.eos_token_id and not req.params.ignore_eos:
                 stops.append(i)
                 req.finish_reason = FinishReason.STOP    # the stop token wins over a length limit, as in the reference
-                if i not in ended and req.status is RequestStatus.RUNNING:
-                    self.scheduler.finish(req)            # the queued step still computes a token for it: dropped there
+                if i not in ended:
+                    # whatever its state (it may have lost its pages in this very round); if the queued step
+                    # computes one more token for it, that is dropped there
+                    self.scheduler.finish(req)
         for i, (s, tok) in enumerate(zip(sampling, ids)):
             if filed[i] is None:
                 continue
