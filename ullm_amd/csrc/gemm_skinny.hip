@@ -389,7 +389,7 @@ extern "C" int ullm_gemm_skinny(const void* X, int ldx, const void* W, int ldw, 
   // each wave with at least 128 values of K
   const int max_waves = sk_max_waves(mt, nt);
   int waves = 1;
-  const int in_flight = (gain && epi == EPI_STORE) || epi == EPI_SILU ? 16 : 8;   // in 16-row tiles of W
+  const int in_flight = (gain && epi == EPI_STORE) || epi == EPI_SILU || nt == 4 ? 16 : 8;   // in 16-row tiles of W
   const int w_rows = rows * (nt / out_tiles);           // rows of W a block fetches
   while (waves < max_waves && waves * w_rows < 16 * in_flight && K / (waves * 2) >= 128) waves *= 2;
   if (force_waves > 0) waves = force_waves < max_waves ? force_waves : max_waves;
