@@ -653,6 +653,14 @@ def test_gemm_dispatch_refuses_nothing_silently(ops):
     assert (got - a.float() @ w.float().T).abs().max() < 1e-4
     with pytest.raises(ops.KernelError):
         ops.gemm_skinny(a, w)
+    # 32-bit results over very many columns (a logits head) at 17 to 32 rows, and just past them
+    torch.manual_seed(18)
+    w = (torch.randn(70001, 264, device=DEV) * 0.2).bfloat16()
+    for M in (17, 32, 33):
+        a = torch.randn(M, 264, device=DEV).bfloat16()
+        got = ops.gemm_bf16(a, w, out_dtype=torch.float32)
+        want = a.double().cpu() @ w.double().cpu().T
+        assert got.dtype == torch.float32 and (got.double().cpu() - want).abs().max() <= 2e-5 * float(want.abs().max())
 
 
 @pytest.mark.parametrize("shape", [(1, 48, 64), (8, 503, 96), (16, 256, 4096), (17, 100, 224), (40, 96, 1032),
