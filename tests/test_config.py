@@ -111,3 +111,25 @@ def test_cli_parser_has_sampling_options():
     a = build_parser().parse_args(["--model", "m", "--prompt-ids", "1,2,3", "--temperature", "0", "--top-k", "5",
                                    "--top-p", "0.9", "--min-p", "0.1", "--max-new-tokens", "4", "--ignore-eos"])
     assert a.prompt_ids == ["1,2,3"] and a.temperature == 0 and a.top_k == 5 and a.ignore_eos
+
+
+def test_scaled_rotation_is_refused_not_ignored():
+    """The engine builds its angles from rope_theta alone (as ullm/models/qwen3.py:97-102 does): a config that
+    asks for anything else must not load."""
+    for ok in (None, {"rope_type": "default"}, {"type": "default"}):
+        assert Qwen3Config.from_dict(dict(TINY_A, rope_scaling=ok)).rope_theta == TINY_A["rope_theta"]
+    for bad in ({"rope_type": "yarn", "factor": 4.0, "original_max_position_embeddings": 32768},
+                {"type": "linear", "factor": 2.0}, {"rope_type": "dynamic", "factor": 2.0}, "yarn"):
+        with pytest.raises(ConfigError, match="rope_scaling"):
+            Qwen3Config.from_dict(dict(TINY_A, rope_scaling=bad))
+
+
+def test_every_stop_id_of_the_config_is_kept():
+    c = Qwen3Config.from_dict(dict(TINY_A, eos_token_id=[7, 9, 200]))
+    assert c.eos_token_id == 7 and c.eos_token_ids == (7, 9, 200)
+    c = Qwen3Config.from_dict(dict(TINY_A, eos_token_id=5))
+    assert c.eos_token_id == 5 and c.eos_token_ids == (5,)
+    c = Qwen3Config.from_dict(TINY_A)
+    assert c.eos_token_id == -1 and c.eos_token_ids == ()
+    with pytest.raises(ConfigError, match="eos_token_id"):
+        Qwen3Config.from_dict(dict(TINY_A, eos_token_id="7"))

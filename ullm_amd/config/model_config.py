@@ -77,7 +77,8 @@ class Qwen3Config:
     sliding_window: int
     max_window_layers: int
     torch_dtype: str
-    eos_token_id: int
+    eos_token_id: int             # the first stop id config.json names (-1: none)
+    eos_token_ids: tuple          # all of them: config.json may hold a list
     initializer_range: float
 
     @classmethod
@@ -113,9 +114,20 @@ class Qwen3Config:
         dtype = d.get("dtype") or d.get("torch_dtype") or "bfloat16"
         if not isinstance(dtype, str):
             raise ConfigError(f"config.json: dtype={dtype!r} is not a string")
-        eos = d.get("eos_token_id", -1)
-        if isinstance(eos, (list, tuple)):
-            eos = eos[0] if eos else -1
+        eos = d.get("eos_token_id")
+        eos_ids = tuple(eos) if isinstance(eos, (list, tuple)) else (() if eos is None else (eos,))
+        for e in eos_ids:
+            if isinstance(e, bool) or not isinstance(e, int) or e < 0:
+                raise ConfigError(f"config.json: eos_token_id={eos!r} must be a token id or a list of token ids")
+        # The reference builds its rotation angles from rope_theta alone (ullm/models/qwen3.py:97-102,
+        # ullm/layers/rotary_embedding.py:52-75) and so does this engine: a config that asks for scaled
+        # angles would run with wrong ones, so it is refused rather than served quietly.
+        scaling = d.get("rope_scaling")
+        if scaling is not None:
+            kind = scaling.get("rope_type", scaling.get("type")) if isinstance(scaling, Mapping) else scaling
+            if kind not in (None, "default"):
+                raise ConfigError(f"config.json: rope_scaling={scaling!r} is not supported (only absent, null or "
+                                  "type 'default': the rotation angles come from rope_theta alone)")
         cfg = cls(
             architectures=tuple(str(a) for a in archs),
             vocab_size=_take(d, "vocab_size", int),
@@ -135,7 +147,8 @@ class Qwen3Config:
             sliding_window=window,
             max_window_layers=max_window_layers,
             torch_dtype=dtype,
-            eos_token_id=-1 if eos is None else int(eos),
+            eos_token_id=int(eos_ids[0]) if eos_ids else -1,
+            eos_token_ids=tuple(int(e) for e in eos_ids),
             initializer_range=_take(d, "initializer_range", float, 0.02),
         )
         for name in ("vocab_size", "hidden_size", "num_hidden_layers", "head_dim",

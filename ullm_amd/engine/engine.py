@@ -98,8 +98,13 @@ class Engine:
         for t in prompt:
             if not (0 <= t < self.runner.vocab_size):
                 raise ValueError(f"prompt token id {t} outside [0, {self.runner.vocab_size})")
-        if params.eos_token_id == -1 and getattr(self.model_config, "eos_token_id", -1) is not None:
-            params.eos_token_id = getattr(self.model_config, "eos_token_id", -1)
+        if params.eos_token_id == -1:
+            # config.json may name several stop ids: the first becomes the request's eos_token_id (the
+            # reference knows one, ullm/llm.py:93-94), the others join its stop_token_ids
+            ids = tuple(getattr(self.model_config, "eos_token_ids", ()) or ())
+            if ids:
+                params.eos_token_id = ids[0]
+                params.stop_token_ids = list(params.stop_token_ids) + [t for t in ids[1:] if t not in params.stop_token_ids]
         order = self._arrivals
         self._arrivals += 1
         seed = params.seed if params.seed is not None else (self.config.seed * 1000003 + order)
@@ -190,7 +195,7 @@ class Engine:
                 continue
             req = s.request
             req.token_ids[filed[i]] = tok
-            if tok == req.params.eos_token_id and not req.params.ignore_eos:
+            if _is_stop_token(req.params, tok):
                 stops.append(i)
                 req.finish_reason = FinishReason.STOP    # the stop token wins over a length limit, as in the reference
                 if i not in ended:
@@ -332,7 +337,7 @@ class Engine:
     def _is_finished(self, req: Request):
         """The reference's rules in its order (ullm/core/engine.py:175-200)."""
         p = req.params
-        if req.token_ids[-1] == p.eos_token_id and not p.ignore_eos:
+        if _is_stop_token(p, req.token_ids[-1]):
             return True, FinishReason.STOP
         if p.max_tokens and req.num_tokens >= p.max_tokens:
             return True, FinishReason.LENGTH
@@ -341,3 +346,10 @@ class Engine:
         if req.num_tokens >= self.config.context_len:
             return True, FinishReason.LENGTH
         return False, None
+
+
+def _is_stop_token(params: SamplingParams, token: int) -> bool:
+    """The request's eos_token_id or one of its stop_token_ids, unless it ignores them."""
+    if params.ignore_eos:
+        return False
+    return token == params.eos_token_id or token in params.stop_token_ids

@@ -19,6 +19,7 @@ class SamplingParams:
     stop: List[str] = field(default_factory=list)   # carried, not used (as in the reference)
     ignore_eos: bool = False
     eos_token_id: int = -1                  # -1: filled from the model's config when it names one
+    stop_token_ids: List[int] = field(default_factory=list)   # further ids that end the request like eos_token_id
 
     seed: Optional[int] = None              # None: the engine's seed mixed with the request's order
 
