@@ -18,6 +18,7 @@
 // Semantics as in the general kernel: causal with the queries at the end of the keys, optional
 // window, query head h reads kv head h / (nq / nkv) (ullm/layers/attention.py:76-104,271,298-309).
 #include "common.h"
+#include "no_alloc.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
@@ -837,7 +838,7 @@ extern "C" int ullm_attention_mfma_supports(int hd, int page_size, int nq, int n
 extern "C" long long ullm_attention_decode_workspace(int n_items, int nq, int hd, int num_splits) {
   return num_splits <= 1 ? 0 : (long long)n_items * nq * num_splits * (hd + 4);
 }
-extern "C" int ullm_attention_decode(
+static int decode_launch(
     const void* q, int q_stride, void* out, int out_stride, const void* k_pool, const void* v_pool,
     const int* token_list, int n_items, const int* positions, const int* token_entry,
     const int* block_table, int bt_stride, int page_size, int nq, int nkv, int hd, float scale, int window,
@@ -867,6 +868,52 @@ extern "C" int ullm_attention_decode(
   hipLaunchKernelGGL(attention_reduce_kernel, dim3(n_items, nq), dim3(64), 0, stream, workspace, (bf16_t*)out,
                      out_stride, token_list, nq, hd, num_splits);
   ULLM_LAUNCH_CHECK();
+}
+
+extern "C" int ullm_attention_decode(
+    const void* q, int q_stride, void* out, int out_stride, const void* k_pool, const void* v_pool,
+    const int* token_list, int n_items, const int* positions, const int* token_entry,
+    const int* block_table, int bt_stride, int page_size, int nq, int nkv, int hd, float scale, int window,
+    int num_splits, int waves, float* workspace, hipStream_t stream) {
+  return decode_launch(q, q_stride, out, out_stride, k_pool, v_pool, token_list, n_items, positions, token_entry,
+                       block_table, bt_stride, page_size, nq, nkv, hd, scale, window, num_splits, waves, workspace,
+                       stream);
+}
+
+// ------------------------------------------------------------------------------- no allocation
+// The splits' partial results of ullm_attention_decode_static (see no_alloc.h).  In host code this
+// name is only a stand-in for the symbol: the address kernels can use is looked up per device.
+static __device__ __align__(256) float scratch[ULLM_DECODE_SCRATCH_FLOATS];
+
+#define ULLM_MAX_DEVICES 64
+static float* scratch_ptr[ULLM_MAX_DEVICES];      // per device: that GPU's copy of the array
+
+extern "C" long long ullm_attention_decode_static_capacity(void) { return ULLM_DECODE_SCRATCH_FLOATS; }
+
+extern "C" int ullm_attention_decode_static(
+    const void* q, int q_stride, void* out, int out_stride, const void* k_pool, const void* v_pool,
+    const int* token_list, int n_items, const int* positions, const int* token_entry,
+    const int* block_table, int bt_stride, int page_size, int nq, int nkv, int hd, float scale, int window,
+    int num_splits, int waves, hipStream_t stream) {
+  if (n_items <= 0) return 0;
+  if (num_splits < 1 || nq < 1 || hd < 1) return ULLM_ERR_SHAPE;
+  if (ullm_attention_decode_workspace(n_items, nq, hd, num_splits) > (long long)ULLM_DECODE_SCRATCH_FLOATS)
+    return ULLM_ERR_SCRATCH;
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= ULLM_MAX_DEVICES) return ULLM_ERR_UNSUPPORTED;
+  float* ws = __atomic_load_n(&scratch_ptr[dev], __ATOMIC_ACQUIRE);
+  if (!ws) {                                      // first call on this device, which is current
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return (int)e;
+    if (!p) return (int)hipErrorInvalidSymbol;
+    ws = static_cast<float*>(p);
+    __atomic_store_n(&scratch_ptr[dev], ws, __ATOMIC_RELEASE);   // two first callers store the same address
+  }
+  return decode_launch(q, q_stride, out, out_stride, k_pool, v_pool, token_list, n_items, positions, token_entry,
+                       block_table, bt_stride, page_size, nq, nkv, hd, scale, window, num_splits, waves, ws, stream);
 }
 
 template <int N, typename... Args>

@@ -31,6 +31,7 @@ HIPCC_FLAGS = [
     "-Wno-unused-command-line-argument",
 ]
 HEADERS = ["common.h"]
+FAMILY_HEADERS = {"attention_mfma": ["no_alloc.h"]}     # headers only this family includes
 
 _lock = threading.Lock()
 _loaded: Dict[str, ctypes.CDLL] = {}
@@ -55,7 +56,7 @@ def _find_hipcc() -> str:
 def _source_hash(family: str) -> str:
     h = hashlib.sha256()
     h.update(" ".join(HIPCC_FLAGS).encode())
-    for name in [family + ".hip"] + HEADERS:
+    for name in [family + ".hip"] + HEADERS + FAMILY_HEADERS.get(family, []):
         with open(os.path.join(CSRC_DIR, name), "rb") as f:
             h.update(name.encode())
             h.update(f.read())

@@ -19,7 +19,7 @@ class KernelError(RuntimeError):
 
 
 _ERR_NAMES = {-1: "unsupported dtype combination", -2: "operand shape outside what the kernel takes",
-              -3: "unsupported argument combination"}
+              -3: "unsupported argument combination", -4: "partial results exceed the fixed scratch array"}
 
 
 def _check(rc: int, what: str) -> None:
