@@ -466,6 +466,74 @@ def test_matrix_core_attention_finds_one_far_key_at_every_edge(ops):
                     assert (got[h] - v[target, h // 4]).abs().max() < 3e-2, (window, target, n, h)
 
 
+def _dominant_key_problem(hd, S, n, target, nq=8, nkv=2, P=16, seed=0):
+    """A cache of S keys in which key ``target`` is the only one the last of n queries looks at."""
+    g = torch.Generator().manual_seed(1000 * seed + target)
+    dtype = torch.bfloat16
+    k = torch.randn(S, nkv, hd, generator=g) * 0.1
+    v = torch.randn(S, nkv, hd, generator=g).to(dtype).float()
+    q = torch.randn(n, nq, hd, generator=g) * 0.1
+    direction = torch.randn(hd, generator=g)
+    direction /= direction.norm()
+    k[target] = 30.0 * direction
+    q[-1] = 30.0 * direction
+    k, q = k.to(dtype).float(), q.to(dtype).float()
+    k_pool, v_pool, tables = paged_cache([k], [v], P, dtype, DEV, seed=target)
+    positions = torch.arange(S - n, S).int().to(DEV)
+    entry = torch.zeros(n, dtype=torch.int32, device=DEV)
+    return q.reshape(n, -1).to(DEV, dtype), k_pool, v_pool, positions, entry, table_tensor(tables, DEV), v
+
+
+@pytest.mark.parametrize("hd", [64, 128])
+def test_matrix_core_attention_finds_one_far_key_beyond_a_thousand_keys(ops, hd):
+    """The kernels fetch page ids 1024 keys at a time, cut a token's keys over waves and blocks, and (prompt
+    tiles) over two halves of a block: one dominant key at every such seam must be found, by every shape of
+    launch, and a dominant key one place before the window must not be seen.  Random data cannot show a
+    dropped or doubled 16-key sub-block among two thousand keys; this can."""
+    nq, nkv, P, S = 8, 2, 16, 2203
+    decode_shapes = ((1, 1), (1, 4), (1, 8), (2, 8), (7, 8), (3, 1), (5, 4))          # (splits, waves)
+    for window in (0, S - 1024, S - 1008, S - 2047, 300):
+        lo = 0 if window == 0 else S - window
+        seams = {lo, lo + 1, 1007, 1008, 1022, 1023, 1024, 1025, 1039, 1040, 2047, 2048, 2049, S - 33, S - 32, S - 2, S - 1}
+        for target in sorted(t for t in seams if lo <= t < S):
+            qd, k_pool, v_pool, positions, entry, bt, v = _dominant_key_problem(hd, S, 1, target, nq, nkv, P)
+            for splits, waves in decode_shapes:
+                out = torch.zeros(1, nq * hd, dtype=torch.bfloat16, device=DEV)
+                ops.attention_decode_mfma(qd, out, k_pool, v_pool, None, 1, positions, entry, bt, P, nq, nkv, hd,
+                                          1.0, window, S, splits=splits, waves=waves)
+                got = out.float().cpu().view(nq, hd)
+                for h in range(nq):
+                    assert (got[h] - v[target, h // 4]).abs().max() < 3e-2, ("decode", window, target, splits, waves, h)
+            for n in (5, 40):                     # one tile, and two tiles (the last query in the second)
+                qd, k_pool, v_pool, positions, entry, bt, v = _dominant_key_problem(hd, S, n, target, nq, nkv, P, seed=1)
+                tiles = [x for f in range(0, n, ops.PREFILL_TILE) for x in (f, min(ops.PREFILL_TILE, n - f))]
+                for halves in (1, 2):
+                    out = torch.zeros(n, nq * hd, dtype=torch.bfloat16, device=DEV)
+                    ops.attention_prefill_mfma(qd, out, k_pool, v_pool, torch.tensor(tiles, dtype=torch.int32, device=DEV),
+                                               len(tiles) // 2, positions, entry, bt, P, nq, nkv, hd, 1.0, window,
+                                               halves=halves)
+                    got = out.float().cpu().view(n, nq, hd)[-1]
+                    for h in range(nq):
+                        assert (got[h] - v[target, h // 4]).abs().max() < 3e-2, ("prompt", window, target, n, halves, h)
+        if window:
+            # the key one place before the window dominates every key inside it, and must not be seen
+            target = lo - 1
+            qd, k_pool, v_pool, positions, entry, bt, v = _dominant_key_problem(hd, S, 1, target, nq, nkv, P, seed=2)
+            for splits, waves in decode_shapes:
+                out = torch.zeros(1, nq * hd, dtype=torch.bfloat16, device=DEV)
+                ops.attention_decode_mfma(qd, out, k_pool, v_pool, None, 1, positions, entry, bt, P, nq, nkv, hd,
+                                          1.0, window, S, splits=splits, waves=waves)
+                got = out.float().cpu().view(nq, hd)
+                assert (got[0] - v[target, 0]).abs().max() > 0.1, ("decode sees past its window", window, splits, waves)
+            qd, k_pool, v_pool, positions, entry, bt, v = _dominant_key_problem(hd, S, 5, target, nq, nkv, P, seed=3)
+            for halves in (1, 2):
+                out = torch.zeros(5, nq * hd, dtype=torch.bfloat16, device=DEV)
+                ops.attention_prefill_mfma(qd, out, k_pool, v_pool, torch.tensor([0, 5], dtype=torch.int32, device=DEV), 1,
+                                           positions, entry, bt, P, nq, nkv, hd, 1.0, window, halves=halves)
+                got = out.float().cpu().view(5, nq, hd)[-1]
+                assert (got[0] - v[target, 0]).abs().max() > 0.1, ("a prompt tile sees past its window", window, halves)
+
+
 def test_matrix_core_attention_with_scores_that_climb(ops):
     """The reference value of the exponentials follows the running maximum only in steps: scores that
     rise a little with every tile (so it lags, then jumps) and scores that fall must both come out right."""
