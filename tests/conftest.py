@@ -42,7 +42,16 @@ TINY_D = dict(architectures=["Qwen3ForCausalLM"], hidden_size=72, num_hidden_lay
               rms_norm_eps=1e-4, max_position_embeddings=320, tie_word_embeddings=True, attention_bias=False,
               use_sliding_window=False, initializer_range=0.04, torch_dtype="bfloat16")
 
-CONFIGS = {"A": (TINY_A, 0), "B": (TINY_B, 2), "C": (TINY_C, 5), "D": (TINY_D, 7)}
+# Tiny E: a window on head_dim 128 (four 32-dim chunks), shorter than the test prompts, on layers >= 1: with
+# pages of 16 the bfloat16 engine runs the matrix-core attention kernels over block tables whose first
+# pages have been given back.
+TINY_E = dict(architectures=["Qwen3ForCausalLM"], hidden_size=88, num_hidden_layers=3, num_attention_heads=4,
+              num_key_value_heads=2, head_dim=128, intermediate_size=152, vocab_size=211, rope_theta=20000.0,
+              rms_norm_eps=2e-5, max_position_embeddings=640, tie_word_embeddings=False, attention_bias=False,
+              use_sliding_window=True, sliding_window=40, max_window_layers=1, initializer_range=0.05,
+              torch_dtype="bfloat16")
+
+CONFIGS = {"A": (TINY_A, 0), "B": (TINY_B, 2), "C": (TINY_C, 5), "D": (TINY_D, 7), "E": (TINY_E, 11)}
 
 
 @pytest.fixture(scope="session")

@@ -55,7 +55,7 @@ def test_window_is_chosen_layer_by_layer():
     groups, cache_group, states = model.cache_layout()
     assert len(groups) == 2 and not states
     by_window = {g.window: g for g in groups}
-    assert by_window[0].layers == (0,) and by_window[24].layers == (1, 2)
+    assert by_window[0].layers == ((0, 0),) and by_window[24].layers == ((1, 0), (2, 0))    # (cache id, need index)
 
 
 def test_registry_maps_the_architecture_name():

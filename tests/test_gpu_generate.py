@@ -292,6 +292,128 @@ def test_scheduling_ahead_under_random_arrivals_and_aborts(model_dirs, seed):
         assert ahead_run[k] == plain_run[k] and ahead_run[k][1] is not None, k
 
 
+def untied(tmp_path, name, seed):
+    """The tiny configuration with an output matrix of its own (a tied one mostly predicts the token it was
+    given, so greedy continuations would repeat one token and every stop token would come first)."""
+    from conftest import CONFIGS
+    from ullm_amd.weights.random_init import write_random_model
+    d = write_random_model(dict(CONFIGS[name][0], tie_word_embeddings=False), str(tmp_path / f"untied{name}"), seed=seed)
+    return d, plain.load_model_folder(d)
+
+
+def run_and_check_own_path(llm, cfg, w, prompts, params, abort=None, rel=3e-2):
+    """Run the requests to the end and check every request along the path it took itself: the logits the
+    engine sampled from are the plain implementation's for the request's own tokens so far, every greedy token
+    is the first largest of those logits, and the request ended where its rules say.  (In bfloat16 a near-tie
+    may go the other way than in 32-bit, so tokens are not compared with a 32-bit run.)"""
+    from ullm_amd import FinishReason
+    eng = llm.engine
+    seen = {}
+
+    def hook(sampling, logits):
+        for s_, row in zip(sampling, logits.float().cpu()):
+            seen.setdefault(s_.request.request_id, []).append((s_.request.num_tokens, row))
+    eng.on_logits = hook
+    for i, (p, sp) in enumerate(zip(prompts, params)):
+        eng.add_request(f"r{i}", p, sp)
+    got, steps = {}, 0
+    while eng.has_unfinished_requests():
+        for r in eng.step():
+            rec = got.setdefault(r.seq_id, [[], None])
+            if r.new_token_id >= 0:
+                rec[0].append(r.new_token_id)
+            if r.is_finished:
+                rec[1] = r.finish_reason
+        steps += 1
+        if abort is not None and steps == abort[1]:
+            eng.abort_request(abort[0])
+        assert steps < 3000
+    checked = 0
+    for i, (p, sp) in enumerate(zip(prompts, params)):
+        rid = f"r{i}"
+        tokens, reason = got.get(rid, [[], None])
+        if abort is not None and rid == abort[0]:
+            assert reason is None
+            continue
+        seq = p + tokens
+        full = plain.qwen3_forward(w, cfg, seq)
+        bound = rel * float(full.abs().max()) + 1e-6
+        for pos, row in seen[rid]:
+            if pos >= len(seq):
+                continue                     # a token computed for a request that had already met its stop token
+            assert float((row - full[pos - 1]).abs().max()) <= bound, (rid, pos)
+            assert seq[pos] == int(row.argmax()), (rid, pos)
+            checked += 1
+        assert len(tokens) >= 1
+        stops = {sp.eos_token_id} | set(sp.stop_token_ids) if not sp.ignore_eos else set()
+        hit = [k for k, t_ in enumerate(tokens) if t_ in stops]
+        if hit:
+            assert hit[0] == len(tokens) - 1 and reason is FinishReason.STOP, (rid, tokens)
+        else:
+            assert reason is FinishReason.LENGTH, rid
+            limits = [sp.max_new_tokens or 10 ** 9, (sp.max_tokens or 10 ** 9) - len(p)]
+            assert len(tokens) == min(limits), (rid, tokens)
+    return got, checked
+
+
+@pytest.mark.parametrize("name,pages", [("D", 8), ("D", 9), ("E", 5)])
+def test_bfloat16_generation_under_preemption_with_stop_tokens(tmp_path, name, pages):
+    """The bfloat16 product path as generation runs it: matrix-core attention (head sizes 64 and 128, pages
+    of 16, in E with a window whose pages are given back), decode steps replayed from graphs, token ids fed
+    from the sampler's output on the device, so few pages that the youngest requests are preempted and
+    recomputed, and stop tokens that end requests unannounced; with and without steps queued ahead."""
+    from ullm_amd import SamplingParams
+    d, (cfg, w) = untied(tmp_path, name, 21)
+    prompts = prompts_of(cfg["vocab_size"], (13, 14, 15, 12, 11, 15, 14), 33)        # all but one cross a page's edge
+    greedy = [plain.greedy_generate(w, cfg, p, 12) for p in prompts]
+    # each request's stop token: the last token of its 32-bit continuation that had not occurred before
+    stops = [g[max(k for k in range(12) if g.index(g[k]) == k)] for g in greedy]
+    preempted = graphs = stopped = 0
+    for ahead in (False, True):
+        # a budget that admits all seven at once (a page each), portions of five: they then grow together
+        llm = make_llm(d, dtype="bfloat16", page_size=16, num_pages=pages, max_num_batched_tokens=128,
+                       max_prefill_chunk=5, disable_async_scheduling=not ahead)
+        params = [SamplingParams(temperature=0.0, max_new_tokens=12, eos_token_id=t) for t in stops]
+        got, checked = run_and_check_own_path(llm, cfg, w, prompts, params)
+        eng = llm.engine
+        assert checked >= 20
+        stopped += sum(1 for v in got.values() if v[1].name == "STOP")
+        for g in range(len(eng.runner.cache.groups)):
+            assert eng.runner.cache.allocators[g].num_free == pages
+        eng.runner.cache.check()
+        preempted += eng.scheduler.num_preemptions
+        graphs += len(eng.runner._graphs)
+    assert preempted > 0
+    assert graphs > 0
+    assert stopped >= 4               # the bfloat16 runs met stop tokens too
+
+
+def test_bfloat16_scheduling_ahead(tmp_path):
+    """As the 32-bit test of scheduling ahead, on the bfloat16 path (config D with an output matrix of its
+    own, pages of 16: matrix-core attention, graphs, ids fed on the device): stop tokens, length limits,
+    scarce pages, an abort in between."""
+    from ullm_amd import SamplingParams
+    d, (cfg, w) = untied(tmp_path, "D", 22)
+    prompts = prompts_of(cfg["vocab_size"], (20, 3, 18, 9, 1, 14), 21)
+    greedy = [plain.greedy_generate(w, cfg, p, 14) for p in prompts]
+    preempted = 0
+    for ahead in (False, True):
+        params = [SamplingParams(temperature=0.0, max_new_tokens=14, eos_token_id=greedy[0][5]),
+                  SamplingParams(temperature=0.0, max_tokens=9, ignore_eos=True),
+                  SamplingParams(temperature=0.0, max_new_tokens=14, ignore_eos=True),
+                  SamplingParams(temperature=0.0, max_new_tokens=14, eos_token_id=greedy[3][0]),
+                  SamplingParams(temperature=0.0, max_new_tokens=14, ignore_eos=True),
+                  SamplingParams(temperature=0.0, max_new_tokens=14, ignore_eos=True)]
+        llm = make_llm(d, dtype="bfloat16", page_size=16, num_pages=7, max_num_batched_tokens=64,
+                       max_prefill_chunk=7, disable_async_scheduling=not ahead)
+        got, checked = run_and_check_own_path(llm, cfg, w, prompts, params, abort=("r4", 6))
+        assert checked >= 30
+        assert llm.engine.runner.cache.num_free_pages() == 7
+        llm.engine.runner.cache.check()
+        preempted += llm.engine.scheduler.num_preemptions
+    assert preempted > 0
+
+
 def test_profile_start_stop_writes_a_trace(model_dirs, tmp_path):
     from ullm_amd import SamplingParams
     if DEV == "cpu":

@@ -129,13 +129,29 @@ def test_run_order_names_a_layer_twice_and_shares_a_cache(tmp_path, dtype):
     assert sorted(rep.runner.caches) == [0, 1, 7]
     _, model = __import__("ullm_amd.models", fromlist=["build_model"]).build_model(cfg)
     groups, cache_group, _ = model.cache_layout()
-    assert {g.window: g.layers for g in groups} == {0: (0,), 13: (1, 7)}
+    assert {g.window: g.layers for g in groups} == {0: ((0, 0),), 13: ((1, 0), (7, 0))}
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_block_that_keeps_keys_and_values_and_state(tmp_path, dtype):
+    """One block with two mixers, one with a paged cache (windowed) and one with fixed-size state: the
+    block declares a list of needs and gets one view per need; an ordinary attention layer runs beside it."""
+    cfg = base_cfg([dict(ATT, mixer="both", window=19), ATT, dict(TOY)])
+    rep, _ = run_and_compare(tmp_path, cfg, dtype, CUTS[2], seed=17)
+    model = rep.model
+    groups, cache_group, states = model.cache_layout()
+    assert {g.window: g.layers for g in groups} == {19: ((0, 0),), 0: ((1, 0),)}
+    assert sorted(states) == [(0, 1), (2, 0)]
+    both = rep.runner.caches[0]
+    assert len(both.parts) == 2 and both.parts[0].k_pool is not None and both.parts[1].state is not None
+    assert both.k_pool is both.parts[0].k_pool and both.state is both.parts[1].state
+    assert rep.runner.caches[1].parts == [] and rep.runner.caches[2].state is not None
 
 
 def test_parts_are_found_by_name_and_unknown_names_fail():
     from ullm_amd.parts import build_part, registered_parts
     assert "toy_running_mean" in registered_parts("mixer") and "gqa_attention" in registered_parts("mixer")
-    assert "swiglu" in registered_parts("ffn") and registered_parts("block") == ["prenorm"]
+    assert "swiglu" in registered_parts("ffn") and registered_parts("block") == ["prenorm", "toy_two_mixers"]
     with pytest.raises(KeyError, match="no mixer part named"):
         build_part("mixer", "does_not_exist")
     with pytest.raises(ValueError, match="needs differ"):
@@ -166,6 +182,7 @@ def test_feed_forward_hands_the_norm_a_stack_of_partial_sums(monkeypatch):
     partial sums if every norm of the model adds stacks; the norm's sum is the plain result."""
     from types import SimpleNamespace
     from ullm_amd.parts import PartEnv, build_part, linear
+    from ullm_amd.weights.loader import bind_tensors
     monkeypatch.setattr(linear, "STACKED_MIN_WEIGHT", 0)      # the test's matrices are small
     torch.manual_seed(5)
     H, I = 96, 224
@@ -173,7 +190,7 @@ def test_feed_forward_hands_the_norm_a_stack_of_partial_sums(monkeypatch):
     ffn = build_part("ffn", "swiglu", hidden_size=H, intermediate_size=I, prefix="f")
     w = {f"f.{n}.weight": (torch.randn(*shape) * 0.1).bfloat16().to(DEV)
          for n, shape in (("gate_proj", (I, H)), ("up_proj", (I, H)), ("down_proj", (H, I)))}
-    ffn.bind(w, env)
+    bind_tensors(ffn, w, env)
     norm = build_part("norm", "rmsnorm", size=H, eps=1e-5, weight_name="g")
     norm.bind({"g": torch.ones(H, device=DEV)}, env)
     assert norm.adds_stacks
@@ -196,13 +213,14 @@ def test_norm_left_to_the_feed_forwards_first_projection(monkeypatch):
     from types import SimpleNamespace
     from ullm_amd.parts import PartEnv, PendingNorm, build_part
     from ullm_amd.parts.block import PreNormBlock
+    from ullm_amd.weights.loader import bind_tensors
     torch.manual_seed(6)
     H, I, eps = 96, 224, 1e-3
     env = PartEnv(torch.device(DEV), torch.bfloat16, 16)
     ffn = build_part("ffn", "swiglu", hidden_size=H, intermediate_size=I, prefix="f")
     w = {f"f.{n}.weight": (torch.randn(*shape) * 0.1).bfloat16() for n, shape in
          (("gate_proj", (I, H)), ("up_proj", (I, H)), ("down_proj", (H, I)))}
-    ffn.bind({k: v.to(DEV) for k, v in w.items()}, env)
+    bind_tensors(ffn, w, env)
     gain = 1 + 0.3 * torch.randn(H)
     norm = build_part("norm", "rmsnorm", size=H, eps=eps, weight_name="g")
     norm.bind({"g": gain.to(DEV)}, env)

@@ -46,7 +46,7 @@ def oracle(plain_models, name, toks):
     return plain.qwen3_forward(w, cfg, toks)
 
 
-CASES = [(n, d) for n in ("A", "B", "C", "D") for d in ("float32", "bfloat16")]
+CASES = [(n, d) for n in ("A", "B", "C", "D", "E") for d in ("float32", "bfloat16")]
 
 
 @pytest.mark.parametrize("name,dtype", CASES)
@@ -171,7 +171,8 @@ def test_portions_whose_projections_come_as_stacks_of_partial_sums(model_dirs, p
     close(np.concatenate(got), want, "bfloat16")
 
 
-@pytest.mark.parametrize("name,dtype", [("B", "float32"), ("C", "bfloat16"), ("C", "float32"), ("D", "bfloat16")])
+@pytest.mark.parametrize("name,dtype", [("B", "float32"), ("C", "bfloat16"), ("C", "float32"), ("D", "bfloat16"),
+                                        ("E", "bfloat16")])
 def test_long_decoding(replayers, plain_models, name, dtype):
     rep = replayers(name, dtype)
     vocab = plain_models[name][0]["vocab_size"]
@@ -266,12 +267,15 @@ def test_other_page_sizes(replayers, plain_models):
         close(np.concatenate(got), want, "float32")
 
 
-@pytest.mark.parametrize("trial", range(8))
-def test_random_configurations(tmp_path, trial):
+@pytest.mark.parametrize("trial,matrix_cores", [(t, False) for t in range(8)] + [(t, True) for t in range(8, 13)])
+def test_random_configurations(tmp_path, trial, matrix_cores):
     """Configurations drawn at random over what config.json allows (head sizes in steps of 16, heads per
     kv head from 1 to 8, widths and vocabularies that are no powers of two, windows, tied heads, page
-    sizes): portions of changing size and then single tokens equal the plain model, in both dtypes."""
+    sizes): portions of changing size and then single tokens equal the plain model, in both dtypes.
+    With ``matrix_cores`` the head size and the page size are drawn among those the matrix-core attention
+    kernels take, so that the bfloat16 run goes through them (the other trials mostly take the general kernel)."""
     import random
+    from ullm_amd.kernels import ops
     from ullm_amd.replay import Replayer
     from ullm_amd.weights.random_init import write_random_model
     rng = random.Random(1000 + trial)
@@ -284,6 +288,12 @@ def test_random_configurations(tmp_path, trial):
                tie_word_embeddings=rng.random() < 0.5, initializer_range=0.05, use_sliding_window=rng.random() < 0.4,
                sliding_window=rng.choice([7, 33, 100]), max_window_layers=rng.choice([0, 1]))
     page_size, n = rng.choice([4, 8, 16, 32]), rng.choice([40, 97, 150])
+    if matrix_cores:
+        cfg["head_dim"] = rng.choice([32, 64, 96, 128, 256])
+        cfg["use_sliding_window"] = trial % 2 == 0
+        page_size, n = rng.choice([16, 32, 64]), rng.choice([97, 150, 230])
+    assert ops.attention_mfma_supports(torch.bfloat16, cfg["head_dim"], page_size, cfg["num_attention_heads"], nkv) == matrix_cores \
+        or not matrix_cores
     d = write_random_model(cfg, str(tmp_path / "m"), seed=trial)
     pc, w = plain.load_model_folder(d)
     toks = [rng.randrange(cfg["vocab_size"]) for _ in range(n)]

@@ -183,3 +183,133 @@ def test_uniform_is_reproducible_and_spread():
     assert us == [plain.uniform_from_seed(7, p) for p in range(2000)]
     assert all(0.0 <= u < 1.0 for u in us) and abs(sum(us) / 2000 - 0.5) < 0.03
     assert us[:5] != [plain.uniform_from_seed(8, p) for p in range(5)]
+
+
+# ------------------------------------------------------------------------------------------------
+# Pins of the formulas that the reference's text alone fixed before: each is a property of the
+# operation itself (an invariant or a special case that is a library routine) that the plausible
+# wrong reading does not have.  The reference ships no vectors, and model code of installed packages
+# is not a source for this build, so a run of another implementation does not stand here: what these
+# cannot reach (the sliding window, which the reference never applies) stays "parity unpinned".
+
+def _attention_weights(cfg, seed, gain_spread=0.0):
+    g = torch.Generator().manual_seed(seed)
+    nq, nkv, d, H = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"], cfg["hidden_size"]
+    rnd = lambda *s: torch.randn(*s, generator=g) * 0.3   # noqa: E731
+    w = {"a.q_proj.weight": rnd(nq * d, H), "a.k_proj.weight": rnd(nkv * d, H), "a.v_proj.weight": rnd(nkv * d, H),
+         "a.o_proj.weight": rnd(H, nq * d),
+         "a.q_norm.weight": 1.0 + gain_spread * torch.rand(d, generator=g),
+         "a.k_norm.weight": 1.0 + gain_spread * torch.rand(d, generator=g)}
+    return w, rnd
+
+
+def test_qk_norm_comes_before_the_rotation():
+    """Rotary scores depend on the distance of two positions only.  That survives a per-dimension gain
+    applied *before* the rotation (it is part of the vectors that are rotated) and not one applied after
+    it, unless both halves of every rotated pair have the same gain.  With gains that differ within the
+    pairs, shifting all positions must leave the layer's output unchanged: a rotation before the norm's
+    gain fails this (checked below on a deliberately swapped copy)."""
+    cfg = dict(TINY_B, attention_bias=False)
+    w, rnd = _attention_weights(cfg, 11, gain_spread=3.0)
+    x = rnd(7, cfg["hidden_size"])
+    base = plain.qwen3_attention(x, torch.arange(7), w, "a", cfg, 0)
+    shifted = plain.qwen3_attention(x, torch.arange(7) + 40, w, "a", cfg, 0)
+    assert torch.allclose(base, shifted, atol=2e-4 * float(base.abs().max()))
+
+    def swapped(x, positions):                      # rotation first, then the per-head norm: the wrong order
+        nq, nkv, d, T = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"], x.shape[0]
+        q = plain.linear(x, w["a.q_proj.weight"]).view(T, nq, d)
+        k = plain.linear(x, w["a.k_proj.weight"]).view(T, nkv, d)
+        v = plain.linear(x, w["a.v_proj.weight"]).view(T, nkv, d)
+        cos, sin = plain.rope_cos_sin(positions, d, cfg["rope_theta"])
+        q = plain.rms_norm(plain.apply_rope_concat_layout(q, cos, sin), w["a.q_norm.weight"], cfg["rms_norm_eps"])
+        k = plain.rms_norm(plain.apply_rope_concat_layout(k, cos, sin), w["a.k_norm.weight"], cfg["rms_norm_eps"])
+        return plain.linear(plain.causal_gqa_attention(q, k, v, d ** -0.5).reshape(T, nq * d), w["a.o_proj.weight"])
+    a, b = swapped(x, torch.arange(7)), swapped(x, torch.arange(7) + 40)
+    assert float((a - b).abs().max()) > 1e-2 * float(a.abs().max())     # the invariant tells the two orders apart
+
+
+def test_attention_layer_without_rotation_is_the_library_routine_with_its_default_scale():
+    """With a rotation base so large that every pair but the first stands still, and the first pair's
+    gain zero, the layer is projection, per-head RMS norm, plain causal attention, projection.  The
+    library routine's default scale is 1/sqrt(size of a query vector) = head_dim^-0.5; here head_dim
+    (32) is not hidden_size / heads (12), so a scale taken from the width fails."""
+    cfg = dict(TINY_B, attention_bias=False, rope_theta=1e300)
+    nq, nkv, d, H = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"], cfg["hidden_size"]
+    assert d != H // nq
+    w, rnd = _attention_weights(cfg, 12, gain_spread=1.0)
+    for n in ("a.q_norm.weight", "a.k_norm.weight"):
+        w[n][0] = 0.0
+        w[n][d // 2] = 0.0                           # the only pair that still turns (its frequency is 1)
+    T = 9
+    x = rnd(T, H)
+    got = plain.qwen3_attention(x, torch.arange(T) + 5, w, "a", cfg, 0)
+    q = F.rms_norm((x @ w["a.q_proj.weight"].T).view(T, nq, d), (d,), w["a.q_norm.weight"], cfg["rms_norm_eps"])
+    k = F.rms_norm((x @ w["a.k_proj.weight"].T).view(T, nkv, d), (d,), w["a.k_norm.weight"], cfg["rms_norm_eps"])
+    v = (x @ w["a.v_proj.weight"].T).view(T, nkv, d)
+    o = F.scaled_dot_product_attention(q.transpose(0, 1)[None], k.transpose(0, 1)[None], v.transpose(0, 1)[None],
+                                       is_causal=True, enable_gqa=True)[0].transpose(0, 1)
+    want = o.reshape(T, nq * d) @ w["a.o_proj.weight"].T
+    assert torch.allclose(got, want, atol=1e-5 * float(want.abs().max()) + 1e-6)
+    wrong = F.scaled_dot_product_attention(q.transpose(0, 1)[None], k.transpose(0, 1)[None], v.transpose(0, 1)[None],
+                                           is_causal=True, enable_gqa=True, scale=(H // nq) ** -0.5)[0].transpose(0, 1)
+    assert not torch.allclose(wrong.reshape(T, nq * d) @ w["a.o_proj.weight"].T, want, atol=1e-3 * float(want.abs().max()))
+
+
+def test_the_gate_is_the_half_that_goes_through_the_activation():
+    """silu(gate) * up is linear in up and not in gate: doubling up_proj doubles the output, doubling
+    gate_proj does not.  A feed-forward that activated the other half fails both."""
+    g = torch.Generator().manual_seed(13)
+    H, I = 24, 40
+    w = {"m.gate_proj.weight": torch.randn(I, H, generator=g), "m.up_proj.weight": torch.randn(I, H, generator=g),
+         "m.down_proj.weight": torch.randn(H, I, generator=g)}
+    x = torch.randn(5, H, generator=g)
+    y = plain.qwen3_mlp(x, w, "m")
+    y_up = plain.qwen3_mlp(x, dict(w, **{"m.up_proj.weight": 2 * w["m.up_proj.weight"]}), "m")
+    y_gate = plain.qwen3_mlp(x, dict(w, **{"m.gate_proj.weight": 2 * w["m.gate_proj.weight"]}), "m")
+    assert torch.allclose(y_up, 2 * y, atol=1e-4 * float(y.abs().max()))
+    assert float((y_gate - 2 * y).abs().max()) > 1e-2 * float(y.abs().max())
+    # and it is the library's activation on that half: one hidden unit, up = 1
+    one = {"m.gate_proj.weight": torch.tensor([[1.0]]), "m.up_proj.weight": torch.tensor([[0.0]]),
+           "m.down_proj.weight": torch.tensor([[1.0]])}
+    t = torch.linspace(-4, 4, 9)[:, None]
+    assert torch.all(plain.qwen3_mlp(t, one, "m") == 0)                                          # up = 0 kills it
+    one["m.up_proj.weight"] = torch.tensor([[1.0]])
+    assert torch.allclose(plain.qwen3_mlp(t, one, "m"), F.silu(t) * t, atol=1e-6)
+
+
+def test_each_norm_feeds_its_own_branch_and_nothing_else(plain_models):
+    """input_layernorm is what attention reads, post_attention_layernorm what the feed-forward reads,
+    and neither touches the residual stream: a zero gain on one silences exactly that branch (there are
+    no biases), so the model equals the one whose branch output matrix is zero.  A norm placed on a
+    branch's output, or on the stream, fails."""
+    cfg, w = plain_models["B"]
+    toks = [9, 400, 1, 33, 250, 7, 100]
+    for layer in range(cfg["num_hidden_layers"]):
+        p = f"model.layers.{layer}"
+        for norm, out_matrix in ((f"{p}.input_layernorm.weight", f"{p}.self_attn.o_proj.weight"),
+                                 (f"{p}.post_attention_layernorm.weight", f"{p}.mlp.down_proj.weight")):
+            silenced = plain.qwen3_forward(dict(w, **{norm: torch.zeros_like(w[norm])}), cfg, toks)
+            removed = plain.qwen3_forward(dict(w, **{out_matrix: torch.zeros_like(w[out_matrix])}), cfg, toks)
+            full = plain.qwen3_forward(w, cfg, toks)
+            assert torch.allclose(silenced, removed, atol=1e-5 * float(full.abs().max()))
+            assert float((silenced - full).abs().max()) > 1e-3 * float(full.abs().max())
+    # pre-norm: the stream itself is never normalised, so scaling the embedding by 1000 makes the branches
+    # (whose inputs are normalised) negligible beside it: logits approach norm(embedding) @ head
+    big = dict(w, **{"model.embed_tokens.weight": w["model.embed_tokens.weight"].float() * 1000.0})
+    expect = plain.rms_norm(w["model.embed_tokens.weight"].float()[toks], w["model.norm.weight"], 0.0) @ w["lm_head.weight"].float().T
+    got = plain.qwen3_forward(big, cfg, toks)
+    assert float((got - expect).abs().max()) < 2e-2 * float(expect.abs().max())
+
+
+def test_window_special_cases(plain_models):
+    """What can be said of the window without the reference (which has none): a window that reaches the
+    start changes nothing, and with a window of one a layer's attention is its own value row."""
+    cfg, w = plain_models["C"]
+    toks = list(range(30, 60))
+    wide = plain.qwen3_forward(w, dict(cfg, sliding_window=len(toks)), toks)
+    none = plain.qwen3_forward(w, dict(cfg, use_sliding_window=False), toks)
+    assert torch.allclose(wide, none, atol=1e-6)
+    torch.manual_seed(14)
+    q, k, v = torch.randn(6, 2, 8), torch.randn(6, 2, 8), torch.randn(6, 2, 8)
+    assert torch.allclose(plain.causal_gqa_attention(q, k, v, 1.0, window=1), v, atol=1e-6)

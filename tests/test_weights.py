@@ -111,3 +111,88 @@ def test_tensors_may_be_spread_over_files_and_stored_in_32_bit(tmp_path):
     load_weights(model16, d, CPU16)
     assert model16.embedding.dtype == torch.bfloat16 and model16.final_norm.gain.dtype == torch.float32
     assert torch.equal(model16.final_norm.gain, w["model.norm.weight"])     # a 32-bit gain stays as stored
+
+
+def test_a_checkpoint_may_hold_the_merged_matrices_whole(tmp_path):
+    """q | k | v and gate | up already put together in the file, under the reference's own names
+    (ullm/models/qwen3.py:300-310, split again by ullm/layers/linear.py:359-379,473-485): the same model."""
+    d = write_random_model(TINY_B, str(tmp_path / "b"), seed=4)
+    path = os.path.join(d, "model.safetensors")
+    w = load_file(path)
+    _, pieces = build_model(TINY_B)
+    load_weights(pieces, d, CPU32)
+    for i in range(TINY_B["num_hidden_layers"]):
+        a, m = f"model.layers.{i}.self_attn", f"model.layers.{i}.mlp"
+        w[f"{a}.qkv_proj.weight"] = torch.cat([w.pop(f"{a}.{n}_proj.weight") for n in "qkv"])
+        if i != 1:                                               # layer 1 keeps gate and up apart: both forms in one file
+            w[f"{m}.gate_up_proj.weight"] = torch.cat([w.pop(f"{m}.gate_proj.weight"), w.pop(f"{m}.up_proj.weight")])
+    save_file(w, path)
+    _, whole = build_model(TINY_B)
+    load_weights(whole, d, CPU32)
+    for b0, b1 in zip(pieces.blocks, whole.blocks):
+        assert torch.equal(b0.mixer.w_qkv, b1.mixer.w_qkv) and torch.equal(b0.ffn.w_gate_up, b1.ffn.w_gate_up)
+    # a merged matrix of the wrong height, and a merged matrix beside one of its pieces, are named in the error
+    w["model.layers.0.self_attn.qkv_proj.weight"] = w["model.layers.0.self_attn.qkv_proj.weight"][:-1].contiguous()
+    w["model.layers.2.mlp.up_proj.weight"] = torch.zeros(224, 96, dtype=torch.bfloat16)
+    save_file(w, path)
+    with pytest.raises(WeightError) as e:
+        load_weights(build_model(TINY_B)[1], d, CPU32)
+    msg = str(e.value)
+    assert "wrong shapes (1)" in msg and "qkv_proj.weight" in msg and "[383, 96]" in msg and "[384, 96]" in msg
+    assert "unexpected tensors (1)" in msg and "model.layers.2.mlp.gate_up_proj.weight" in msg and "up_proj.weight" in msg
+
+
+def test_a_missing_piece_of_a_merged_matrix_is_named(tmp_path):
+    d = write_random_model(TINY_A, str(tmp_path / "a"), seed=4)
+    path = os.path.join(d, "model.safetensors")
+    w = load_file(path)
+    del w["model.layers.1.self_attn.k_proj.weight"]
+    save_file(w, path)
+    with pytest.raises(WeightError, match=r"missing tensors \(1\):\n  model.layers.1.self_attn.k_proj.weight  expected shape \[32, 64\]"):
+        load_weights(build_model(TINY_A)[1], d, CPU32)
+
+
+def test_random_weights_bound_in_place(tmp_path):
+    """The mode every benchmark runs on: every declared tensor is there with its shape and dtype, a tied
+    head is the embedding itself, the same seed gives the same tensors, and the 32-bit engine holds
+    exactly the bfloat16 engine's weights."""
+    from conftest import TINY_C
+    from ullm_amd.weights.loader import merged_tensors, unique_decls
+    from ullm_amd.weights.random_init import bind_random_weights
+
+    def bound(cfg, env, seed):
+        _, model = build_model(cfg)
+        seen = {}
+        inner = model.bind
+        model.bind = lambda tensors, e: (seen.update(tensors), inner(tensors, e))
+        bind_random_weights(model, env, seed)
+        return model, seen
+
+    for cfg in (TINY_A, TINY_C):                                  # tied head; biases and an untied head
+        m16, t16 = bound(cfg, CPU16, 5)
+        m32, t32 = bound(cfg, CPU32, 5)
+        again, t16b = bound(cfg, CPU16, 5)
+        other, t16c = bound(cfg, CPU16, 6)
+        decls = unique_decls(m16.weight_decls())
+        merged = merged_tensors(m16.weight_decls())
+        want = {n: (d.shape, d.keep_fp32) for n, d in decls.items() if d.merged_into is None}
+        want.update({n: (m.shape, m.pieces[0].keep_fp32) for n, m in merged.items()})
+        assert set(t16) == set(want) == set(t32)
+        for n, (shape, keep) in want.items():
+            assert tuple(t16[n].shape) == tuple(shape) == tuple(t32[n].shape), n
+            assert t16[n].dtype == (torch.float32 if keep else torch.bfloat16) and t32[n].dtype == torch.float32, n
+            assert torch.equal(t16[n].float(), t32[n]), n             # widened exactly
+            assert torch.equal(t16[n], t16b[n]), n
+        assert any(not torch.equal(t16[n], t16c[n]) for n in want)
+        if cfg["tie_word_embeddings"]:
+            assert m16.head.data_ptr() == m16.embedding.data_ptr()
+        else:
+            assert m16.head.data_ptr() != m16.embedding.data_ptr()
+        std = cfg["initializer_range"]
+        assert abs(float(m32.blocks[0].ffn.w_gate_up.std()) - std) < 0.1 * std
+        assert abs(float(m32.final_norm.gain.mean()) - 1.0) < 3 * std
+        # the pieces of a merged matrix are different draws, not one draw repeated
+        w = m32.blocks[0].mixer.w_qkv
+        nq_rows = cfg["num_attention_heads"] * cfg["head_dim"]
+        kv_rows = cfg["num_key_value_heads"] * cfg["head_dim"]
+        assert not torch.equal(w[nq_rows:nq_rows + kv_rows], w[nq_rows + kv_rows:])

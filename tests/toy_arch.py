@@ -11,7 +11,8 @@ import torch
 
 import plain_qwen3 as plain
 from ullm_amd.models import Choice, ModelPlan, register_architecture
-from ullm_amd.parts import FeedForward, Mixer, PositionEncoding, StateNeed, WeightDecl, register_part
+from ullm_amd.kernels import ops
+from ullm_amd.parts import Block, FeedForward, Mixer, PositionEncoding, StateNeed, WeightDecl, register_part
 from ullm_amd.parts.linear import linear
 
 
@@ -104,6 +105,31 @@ class LinearAngles(PositionEncoding):
         return self.table, self.head_dim, 2
 
 
+@register_part("block", "toy_two_mixers")
+class TwoMixers(Block):
+    """h += attention(norm1 h) + running_mean(norm1 h); h += ffn(norm2 h).  One block that keeps keys
+    and values *and* fixed-size state: it declares both needs and hands each mixer its own view."""
+
+    def __init__(self, mixer_norm, attention, mean, ffn_norm, ffn):
+        self.mixer_norm, self.attention, self.mean, self.ffn_norm, self.ffn = mixer_norm, attention, mean, ffn_norm, ffn
+
+    def children(self):
+        return [self.mixer_norm, self.attention, self.mean, self.ffn_norm, self.ffn]
+
+    def cache_need(self):
+        return [self.attention.cache_need(), self.mean.cache_need()]
+
+    def forward(self, residual, pending, ctx, cache):
+        x = self.mixer_norm.add_norm(pending, residual, out_dtype=ctx.dtype)
+        kv_view, state_view = cache.parts
+        a = self.attention.forward(x, ctx, kv_view)
+        if a.dim() == 3:                       # a stack of partial sums: this block adds them itself
+            a = a.sum(0)
+        ops.residual_add(a.contiguous(), residual)
+        pending = self.mean.forward(x, ctx, state_view)
+        return residual, self.ffn.forward(self.ffn_norm.add_norm(pending, residual, out_dtype=ctx.dtype), ctx)
+
+
 def toy_config_from_dict(d):
     return dict(d)
 
@@ -113,7 +139,7 @@ def toy_plan(cfg: dict) -> ModelPlan:
     layers = []
     for i, L in enumerate(cfg["layers"]):
         p = f"stack.{i}"
-        if L["mixer"] == "attention":
+        if L["mixer"] in ("attention", "both"):
             rope = L.get("rope", "half")
             if rope == "none":
                 position = None
@@ -134,6 +160,11 @@ def toy_plan(cfg: dict) -> ModelPlan:
                                                          num_experts=L["experts"], prefix=f"{p}.ffn"))
         else:
             ffn = Choice("ffn", "swiglu", dict(hidden_size=H, intermediate_size=L["ffn_size"], prefix=f"{p}.ffn"))
+        if L["mixer"] == "both":
+            mean = Choice("mixer", "toy_running_mean", dict(hidden_size=H, prefix=f"{p}.mix"))
+            layers.append(Choice("block", "toy_two_mixers", dict(
+                mixer_norm=norm("norm1"), attention=mixer, mean=mean, ffn_norm=norm("norm2"), ffn=ffn)))
+            continue
         layers.append(Choice("block", "prenorm", dict(
             mixer_norm=norm("norm1"), mixer=mixer, ffn_norm=norm("norm2"), ffn=ffn)))
     order = [tuple(x) for x in cfg["run_order"]] if cfg.get("run_order") else None
@@ -178,7 +209,8 @@ def toy_forward(w: Dict[str, torch.Tensor], cfg: dict, token_ids: List[int]) -> 
     for layer, cache_id in order:
         L, p = cfg["layers"][layer], f"stack.{layer}"
         x = plain.rms_norm(h, w[f"{p}.norm1.weight"], eps)
-        if L["mixer"] == "attention":
+        a = 0.0
+        if L["mixer"] in ("attention", "both"):
             nq, nkv, d = L["heads"], L["kv_heads"], L["head_dim"]
             b = (lambda n: w[f"{p}.attn.{n}_proj.bias"]) if L.get("bias", False) else (lambda n: None)
             q = plain.linear(x, w[f"{p}.attn.q_proj.weight"], b("q")).view(T, nq, d)
@@ -195,9 +227,9 @@ def toy_forward(w: Dict[str, torch.Tensor], cfg: dict, token_ids: List[int]) -> 
             scale = L.get("scale") or d ** -0.5
             o = plain.causal_gqa_attention(q, k, v, scale, L.get("window", 0))
             a = plain.linear(o.reshape(T, nq * d), w[f"{p}.attn.o_proj.weight"])
-        else:
+        if L["mixer"] != "attention":
             means = torch.cumsum(x, 0) / torch.arange(1, T + 1, dtype=torch.float32)[:, None]
-            a = plain.linear(means, w[f"{p}.mix.mean_proj.weight"])
+            a = a + plain.linear(means, w[f"{p}.mix.mean_proj.weight"])
         h = h + a
         x = plain.rms_norm(h, w[f"{p}.norm2.weight"], eps)
         if L.get("experts"):

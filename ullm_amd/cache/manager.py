@@ -30,7 +30,7 @@ class CacheGroupSpec:
     num_kv_heads: int
     head_dim: int
     window: int                   # 0 = every earlier key
-    layers: tuple                 # model layers that own a cache in this group
+    layers: tuple                 # the caches of this group, one set of pools each (any hashable names)
 
     def bytes_per_token(self, itemsize: int) -> int:
         return 2 * self.num_kv_heads * self.head_dim * itemsize * len(self.layers)

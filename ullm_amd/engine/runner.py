@@ -15,6 +15,8 @@ import numpy as np
 import torch
 
 from ..cache.manager import CacheManager, RequestCache
+from ..kernels import ops
+from ..kernels.ops import PREFILL_TILE as Q_TILE   # tokens of one request per prompt-portion attention tile
 from ..models.model import Model
 from ..parts import GroupView, LayerCache, PartEnv, StepContext
 from ..staging import StagedUpload
@@ -35,9 +37,6 @@ class StepError(RuntimeError):
 
 UNKNOWN_TOKEN = -2         # stands for a token that is still being sampled when the step is prepared
 
-from ..kernels import ops
-from ..kernels.ops import PREFILL_TILE as Q_TILE   # tokens of one request per prompt-portion attention tile
-
 
 class ModelRunner:
     def __init__(self, model: Model, env: PartEnv, page_size: int, num_pages, max_requests: int,
@@ -55,18 +54,23 @@ class ModelRunner:
         self.cache = CacheManager(groups, list(num_pages), page_size, max_requests,
                                   enable_prefix_cache=enable_prefix_cache and not states)
         self.max_table = -(-env.context_len // page_size)
-        self.caches: Dict[int, LayerCache] = {}
+        views: Dict[tuple, LayerCache] = {}      # (cache id, index of the need in its block) -> view
         for g, spec in enumerate(groups):
             k_shape = (num_pages[g], spec.num_kv_heads, page_size, spec.head_dim)
             v_shape = (num_pages[g], spec.num_kv_heads, spec.head_dim, page_size)   # transposed inside a page
-            for cache_id in spec.layers:
+            for key in spec.layers:
                 # zeroed once so that no row ever holds a non-finite bit pattern before it is written
-                self.caches[cache_id] = LayerCache(
+                views[key] = LayerCache(
                     group=g, k_pool=torch.zeros(k_shape, dtype=env.dtype, device=env.device),
                     v_pool=torch.zeros(v_shape, dtype=env.dtype, device=env.device))
-        for cache_id, need in states.items():
-            self.caches[cache_id] = LayerCache(
+        for key, need in states.items():
+            views[key] = LayerCache(
                 state=torch.zeros((max_requests,) + tuple(need.shape), dtype=need.dtype, device=env.device))
+        self._views = views
+        # per cache id what its block sees: the one view, or one view per declared need
+        self.caches: Dict[int, LayerCache] = {}
+        for cache_id in sorted({c for c, _ in views}):
+            self.caches[cache_id] = LayerCache.of_parts([views[(cache_id, i)] for i in range(model.num_needs(cache_id))])
         self._upload = StagedUpload(env.device)
         # int32 device tensor the steps take late token ids from (the sampler's output of the step before), or None
         self.feed_source: Optional[torch.Tensor] = None
@@ -82,7 +86,7 @@ class ModelRunner:
     # ------------------------------------------------------------------ helpers
     def cache_bytes(self) -> int:
         total = 0
-        for c in self.caches.values():
+        for c in self._views.values():
             for t in (c.k_pool, c.v_pool, c.state):
                 if t is not None:
                     total += t.numel() * t.element_size()
@@ -282,7 +286,7 @@ class ModelRunner:
         entries = prepared.entries
         fresh = self.cache.take_fresh_slots()
         if fresh:
-            for c in self.caches.values():
+            for c in self._views.values():
                 if c.state is not None:
                     c.state[torch.tensor(fresh, device=c.state.device)] = 0
         if prepared.graph_key is not None:

@@ -15,7 +15,7 @@ import torch
 from ..cache.manager import CacheGroupSpec
 from ..kernels import ops
 from ..parts import (Block, KVNeed, LayerCache, Norm, Part, PartEnv, StateNeed, StepContext, WeightDecl,
-                     build_part, walk)
+                     build_part, cache_needs_of, walk)
 from ..parts.linear import linear
 
 
@@ -90,28 +90,33 @@ class Model:
 
     # ------------------------------------------------------------------ cache layout
     def cache_layout(self):
-        """Groups of caches with equal needs, and the per-request state needs.
-        Returns (groups, {cache id: group index}, {cache id: StateNeed})."""
-        keyed: Dict[Tuple[int, int, int], List[int]] = {}
-        states: Dict[int, StateNeed] = {}
+        """Groups of caches with equal needs, and the per-request state needs.  A cache is named by
+        (cache id, index of the need among those its block declares).
+        Returns (groups, {(cache id, need index): group index}, {(cache id, need index): StateNeed})."""
+        keyed: Dict[Tuple[int, int, int], List[Tuple[int, int]]] = {}
+        states: Dict[Tuple[int, int], StateNeed] = {}
         for cache_id, idx in self.cache_owner.items():
-            need = self.blocks[self.run_order[idx][0]].cache_need()
-            if isinstance(need, KVNeed):
-                keyed.setdefault((need.num_kv_heads, need.head_dim, need.window), []).append(cache_id)
-            elif isinstance(need, StateNeed):
-                states[cache_id] = need
-        groups, layer_group = [], {}
-        for (nkv, hd, window), ids in keyed.items():
-            for c in ids:
-                layer_group[c] = len(groups)
-            groups.append(CacheGroupSpec(nkv, hd, window, tuple(ids)))
+            for i, need in enumerate(cache_needs_of(self.blocks[self.run_order[idx][0]])):
+                if isinstance(need, KVNeed):
+                    keyed.setdefault((need.num_kv_heads, need.head_dim, need.window), []).append((cache_id, i))
+                else:
+                    states[(cache_id, i)] = need
+        groups, cache_group = [], {}
+        for (nkv, hd, window), keys in keyed.items():
+            for c in keys:
+                cache_group[c] = len(groups)
+            groups.append(CacheGroupSpec(nkv, hd, window, tuple(keys)))
         for idx, (layer, cache_id) in enumerate(self.run_order):
             owner_layer = self.run_order[self.cache_owner[cache_id]][0]
-            a, b = self.blocks[layer].cache_need(), self.blocks[owner_layer].cache_need()
+            a, b = cache_needs_of(self.blocks[layer]), cache_needs_of(self.blocks[owner_layer])
             if a != b:
                 raise ValueError(f"layer {layer} reads cache {cache_id} written by layer {owner_layer} "
                                  f"but their needs differ: {a} vs {b}")
-        return groups, layer_group, states
+        return groups, cache_group, states
+
+    def num_needs(self, cache_id: int) -> int:
+        """How many needs the block that owns this cache declares."""
+        return len(cache_needs_of(self.blocks[self.run_order[self.cache_owner[cache_id]][0]]))
 
     # ------------------------------------------------------------------ forward
     def forward(self, ctx: StepContext, caches: Dict[int, LayerCache], logit_rows: Optional[torch.Tensor]):
@@ -124,7 +129,7 @@ class Model:
             if cache is None:
                 cache = LayerCache()
             elif self.cache_owner[cache_id] != idx:
-                cache = LayerCache(cache.group, cache.k_pool, cache.v_pool, cache.state, owner=False)
+                cache = cache.reader()
             residual, pending = self.blocks[layer].forward(residual, pending, ctx, cache)
         if logit_rows is None or logit_rows.numel() == 0:
             return None

@@ -45,14 +45,15 @@ class GQAttention(Mixer):
 
     def weights(self) -> List[WeightDecl]:
         p, H, hd = self.prefix, self.hidden_size, self.hd
-        out = [WeightDecl(f"{p}.q_proj.weight", (self.nq * hd, H)),
-               WeightDecl(f"{p}.k_proj.weight", (self.nkv * hd, H)),
-               WeightDecl(f"{p}.v_proj.weight", (self.nkv * hd, H)),
-               WeightDecl(f"{p}.o_proj.weight", (H, self.nq * hd))]
+        # q, k and v are used as one matrix with rows q | k | v, as the reference merges them
+        # (ullm/layers/linear.py:381-389); the loader puts the three tensors into its rows
+        rows = (("q", self.nq * hd, 0), ("k", self.nkv * hd, self.nq * hd), ("v", self.nkv * hd, (self.nq + self.nkv) * hd))
+        out = [WeightDecl(f"{p}.{n}_proj.weight", (r, H), merged_into=f"{p}.qkv_proj.weight", row_offset=off)
+               for n, r, off in rows]
+        out.append(WeightDecl(f"{p}.o_proj.weight", (H, self.nq * hd)))
         if self.bias:   # qwen3.py:146 (attention_bias): on q, k, v only; o_proj never has one (qwen3.py:94)
-            out += [WeightDecl(f"{p}.q_proj.bias", (self.nq * hd,), keep_fp32=True),
-                    WeightDecl(f"{p}.k_proj.bias", (self.nkv * hd,), keep_fp32=True),
-                    WeightDecl(f"{p}.v_proj.bias", (self.nkv * hd,), keep_fp32=True)]
+            out += [WeightDecl(f"{p}.{n}_proj.bias", (r,), keep_fp32=True, merged_into=f"{p}.qkv_proj.bias", row_offset=off)
+                    for n, r, off in rows]
         if self.qk_norm_eps is not None:
             out += [WeightDecl(f"{p}.q_norm.weight", (hd,), init="gain", keep_fp32=True),
                     WeightDecl(f"{p}.k_norm.weight", (hd,), init="gain", keep_fp32=True)]
@@ -60,11 +61,10 @@ class GQAttention(Mixer):
 
     def bind(self, tensors: Dict[str, torch.Tensor], env: PartEnv) -> None:
         p = self.prefix
-        # one fused projection with rows q | k | v, as the reference merges them (linear.py:381-389)
-        self.w_qkv = torch.cat([tensors[f"{p}.{n}_proj.weight"] for n in "qkv"], dim=0).contiguous()
+        self.w_qkv = tensors[f"{p}.qkv_proj.weight"].contiguous()
         self.w_o = tensors[f"{p}.o_proj.weight"].contiguous()
         if self.bias:
-            self.b_qkv = torch.cat([tensors[f"{p}.{n}_proj.bias"] for n in "qkv"], dim=0).contiguous()
+            self.b_qkv = tensors[f"{p}.qkv_proj.bias"].contiguous()
         if self.qk_norm_eps is not None:
             self.q_gain = tensors[f"{p}.q_norm.weight"].contiguous()
             self.k_gain = tensors[f"{p}.k_norm.weight"].contiguous()

@@ -25,6 +25,12 @@ class WeightDecl:
     init: str = "normal"          # random mode: "normal" N(0,s) | "gain" 1+N(0,s)
     keep_fp32: bool = False       # held in 32-bit whatever the compute dtype (norm gains)
     alias_of: Optional[str] = None  # if absent from the checkpoint, bind this tensor instead
+    # A tensor that is used only as rows ``row_offset ..`` of a larger matrix (q | k | v, gate | up)
+    # names that matrix here.  The loader allocates the matrix once, copies every such tensor into its
+    # rows, and hands ``bind`` the matrix under the name ``merged_into`` (not the pieces); a checkpoint
+    # that already holds the whole matrix under that name is taken as it is.
+    merged_into: Optional[str] = None
+    row_offset: int = 0
 
 
 # --------------------------------------------------------------------------- cache needs
@@ -47,6 +53,22 @@ class StateNeed:
 CacheNeed = Union[KVNeed, StateNeed, None]
 
 
+def cache_needs_of(block) -> Tuple[Union[KVNeed, StateNeed], ...]:
+    """What a block keeps between steps as a tuple: ``Block.cache_need()`` may return nothing, one
+    need, or a list of needs (a block with keys and values and fixed-size state, or with two shapes
+    of keys)."""
+    need = block.cache_need()
+    if need is None:
+        return ()
+    if isinstance(need, (KVNeed, StateNeed)):
+        return (need,)
+    needs = tuple(need)
+    for n in needs:
+        if not isinstance(n, (KVNeed, StateNeed)):
+            raise TypeError(f"{type(block).__name__}.cache_need() returned {n!r}: not a KVNeed or StateNeed")
+    return needs
+
+
 # --------------------------------------------------------------------------- step context
 
 @dataclass
@@ -60,12 +82,32 @@ class GroupView:
 
 @dataclass
 class LayerCache:
-    """What a mixer sees of the cache: its layer's pools or its layer's state rows."""
+    """What a mixer sees of the cache: its layer's pools or its layer's state rows.
+
+    A block that declares several needs gets one view per need, in the order declared, as ``parts``
+    and hands each of its mixers the one that is its own (``cache.parts[i]``); the outer view's own
+    fields then show the first need of each kind, so a block with one need never looks at ``parts``."""
     group: int = -1                        # index into StepContext.groups for KV mixers
     k_pool: Optional[torch.Tensor] = None  # [num_pages, kv_heads, page_size, head_dim]
     v_pool: Optional[torch.Tensor] = None  # [num_pages, kv_heads, head_dim, page_size]
     state: Optional[torch.Tensor] = None   # [num_slots, *StateNeed.shape]
     owner: bool = True                     # False: reads another layer's cache, writes nothing
+    parts: List["LayerCache"] = field(default_factory=list)
+
+    @staticmethod
+    def of_parts(parts: List["LayerCache"]) -> "LayerCache":
+        """The view of a block from the views of its needs."""
+        if len(parts) == 1:
+            return parts[0]
+        kv = next((p for p in parts if p.k_pool is not None), None)
+        st = next((p for p in parts if p.state is not None), None)
+        return LayerCache(group=kv.group if kv else -1, k_pool=kv.k_pool if kv else None,
+                          v_pool=kv.v_pool if kv else None, state=st.state if st else None, parts=list(parts))
+
+    def reader(self) -> "LayerCache":
+        """The same cache for a layer that only reads it."""
+        return LayerCache(self.group, self.k_pool, self.v_pool, self.state, owner=False,
+                          parts=[p.reader() for p in self.parts])
 
 
 @dataclass
@@ -107,6 +149,17 @@ class PartEnv:
     device: torch.device
     dtype: torch.dtype            # compute dtype: torch.bfloat16 or torch.float32
     context_len: int              # most positions any request reaches
+    # tensors that parts of many layers would otherwise each build for themselves (position tables):
+    # built once per key and shared, see ``shared``
+    _shared: Dict[tuple, torch.Tensor] = field(default_factory=dict, compare=False, repr=False)
+
+    def shared(self, key: tuple, build: Callable[[], torch.Tensor]) -> torch.Tensor:
+        """The tensor of this key, built by ``build()`` the first time it is asked for.  The key must
+        name everything the tensor depends on (kind, sizes, constants, rows)."""
+        t = self._shared.get(key)
+        if t is None:
+            t = self._shared[key] = build()
+        return t
 
 
 class Part:
@@ -209,7 +262,9 @@ class Block(Part):
     32-bit stream [T, hidden] and ``pending`` a branch output not yet added to it."""
     kind = "block"
 
-    def cache_need(self) -> CacheNeed:
+    def cache_need(self):
+        """Nothing, one need (``KVNeed`` / ``StateNeed``) or a list of needs; with a list the block
+        gets ``cache.parts`` in the same order."""
         return None
 
     def forward(self, residual, pending, ctx: StepContext, cache: LayerCache):

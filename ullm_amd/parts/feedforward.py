@@ -31,13 +31,14 @@ class SwiGLU(FeedForward):
 
     def weights(self) -> List[WeightDecl]:
         p, H, I = self.prefix, self.hidden_size, self.intermediate_size
-        return [WeightDecl(f"{p}.gate_proj.weight", (I, H)), WeightDecl(f"{p}.up_proj.weight", (I, H)),
+        merged = f"{p}.gate_up_proj.weight"          # rows gate | up, put together by the loader
+        return [WeightDecl(f"{p}.gate_proj.weight", (I, H), merged_into=merged, row_offset=0),
+                WeightDecl(f"{p}.up_proj.weight", (I, H), merged_into=merged, row_offset=I),
                 WeightDecl(f"{p}.down_proj.weight", (H, I))]
 
     def bind(self, tensors: Dict[str, torch.Tensor], env: PartEnv) -> None:
         p = self.prefix
-        self.w_gate_up = torch.cat([tensors[f"{p}.gate_proj.weight"], tensors[f"{p}.up_proj.weight"]],
-                                   dim=0).contiguous()
+        self.w_gate_up = tensors[f"{p}.gate_up_proj.weight"].contiguous()
         self.w_down = tensors[f"{p}.down_proj.weight"].contiguous()
 
     def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:

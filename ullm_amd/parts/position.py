@@ -48,7 +48,9 @@ class Rotary(PositionEncoding):
 
     def bind(self, tensors: Dict[str, torch.Tensor], env: PartEnv) -> None:
         rows = env.context_len if self.max_positions is None else min(env.context_len, self.max_positions)
-        self.table = self.make_table(self.rotary_dim, self.theta, rows).to(env.device)
+        # every layer with the same rotation shares one table: built once, read by all their kernels
+        self.table = env.shared(("rotary", self.rotary_dim, self.theta, rows),
+                                lambda: self.make_table(self.rotary_dim, self.theta, rows).to(env.device))
 
     def kernel_args(self):
         return self.table, self.rotary_dim, self.style

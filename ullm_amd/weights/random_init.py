@@ -50,24 +50,42 @@ def write_random_model(config: Mapping, out_dir: str, seed: int, std: Optional[f
     return out_dir
 
 
-def bind_random_weights(model, env: PartEnv, seed: int, std: Optional[float] = None) -> None:
-    """Draw every declared tensor on ``env.device`` (own seeded generator) and bind the model."""
+def bind_random_weights(model, env: PartEnv, seed: int, std: Optional[float] = None,
+                        store_dtype: str = "bfloat16") -> None:
+    """Draw every declared tensor on ``env.device`` (own seeded generator) and bind the model.
+    Matrices are drawn in ``store_dtype`` and then brought to the compute dtype, as a checkpoint
+    stored in that dtype would be: the same seed gives the bfloat16 and the float32 engine the same
+    weights (the float32 one holds them widened exactly).  Tensors a part keeps in 32-bit are drawn
+    in 32-bit.  Pieces of a merged matrix are drawn straight into its rows."""
+    from .loader import merged_tensors, unique_decls
+    if store_dtype not in _STORE:
+        raise ValueError(f"storage dtype {store_dtype!r}: choose bfloat16 or float32")
     sigma = model.plan.init_std if std is None else float(std)
     gen = torch.Generator(device=env.device).manual_seed(int(seed))
+    decls = model.weight_decls()
+    merged = merged_tensors(decls)
     tensors: Dict[str, torch.Tensor] = {}
     pending_alias = []
-    for d in model.weight_decls():
-        if d.name in tensors:
-            continue
+    for d in unique_decls(decls).values():
         if d.alias_of is not None:
             pending_alias.append(d)
             continue
         final = torch.float32 if d.keep_fp32 else env.dtype
-        if final == torch.float32:
-            tensors[d.name] = _draw(d, sigma, gen, env.device)
-        else:   # large matrices: draw in the final dtype, no 32-bit copy
-            t = torch.empty(d.shape, dtype=final, device=env.device).normal_(0.0, sigma, generator=gen)
-            tensors[d.name] = t + 1.0 if d.init == "gain" else t
+        drawn = torch.float32 if d.keep_fp32 else _STORE[store_dtype]
+        if d.merged_into is not None:
+            m = merged[d.merged_into]
+            buf = tensors.get(m.name)
+            if buf is None:
+                buf = tensors[m.name] = torch.empty(m.shape, dtype=final, device=env.device)
+            target = buf[d.row_offset:d.row_offset + d.shape[0]]
+        else:
+            target = tensors[d.name] = torch.empty(d.shape, dtype=final, device=env.device)
+        if drawn == final:
+            target.normal_(0.0, sigma, generator=gen)          # in place: no second copy of a large matrix
+        else:
+            target.copy_(torch.empty(d.shape, dtype=drawn, device=env.device).normal_(0.0, sigma, generator=gen))
+        if d.init == "gain":
+            target += 1.0
     for d in pending_alias:
         tensors[d.name] = tensors[d.alias_of]
     model.bind(tensors, env)
