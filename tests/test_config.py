@@ -133,3 +133,29 @@ def test_every_stop_id_of_the_config_is_kept():
     assert c.eos_token_id == -1 and c.eos_token_ids == ()
     with pytest.raises(ConfigError, match="eos_token_id"):
         Qwen3Config.from_dict(dict(TINY_A, eos_token_id="7"))
+
+
+def test_random_weights_specification(tmp_path):
+    """``--random-weights NAME[:SEED]`` or ``CONFIG.JSON[:SEED]`` stands in for ``--model``."""
+    from ullm_amd.config import parse_random_weights, preset_names
+    assert {"qwen3-0.6b", "qwen3-8b", "qwen3-14b", "qwen3-32b"} <= set(preset_names())
+    cfg, seed = parse_random_weights("qwen3-8b")
+    c = Qwen3Config.from_dict(cfg)
+    assert seed == 0 and (c.hidden_size, c.num_hidden_layers, c.num_attention_heads, c.num_key_value_heads, c.head_dim,
+                          c.intermediate_size, c.vocab_size) == (4096, 36, 32, 8, 128, 12288, 151936)
+    cfg, seed = parse_random_weights("Qwen3-32B:7")
+    c = Qwen3Config.from_dict(cfg)
+    assert seed == 7 and (c.hidden_size, c.num_hidden_layers, c.num_attention_heads, c.intermediate_size) == (5120, 64, 64, 25600)
+    path = tmp_path / "config.json"
+    path.write_text(json.dumps(TINY_B))
+    assert parse_random_weights(f"{path}:3") == (TINY_B, 3) and parse_random_weights(str(path)) == (TINY_B, 0)
+    with pytest.raises(ConfigError, match="neither"):
+        parse_random_weights("qwen3-9000b")
+    ap = argparse.ArgumentParser()
+    EngineConfig.add_cli_args(ap)
+    ec = EngineConfig.from_args(ap.parse_args(["--random-weights", "qwen3-14b:2"]))
+    assert ec.model is None and ec.random_weights == "qwen3-14b:2" and ec.generation_defaults() == {}
+    with pytest.raises(ConfigError, match="either"):
+        EngineConfig.from_args(ap.parse_args([]))
+    with pytest.raises(ConfigError, match="either"):
+        EngineConfig(model="x", random_weights="qwen3-8b")

@@ -453,3 +453,21 @@ def test_command_line(model_dirs, plain_models, capsys):
     lines = [json.loads(x) for x in capsys.readouterr().out.strip().splitlines() if x.startswith("{")]
     assert [x["token_ids"] for x in lines] == [plain.greedy_generate(w, cfg, [5, 17, 3], 4),
                                                plain.greedy_generate(w, cfg, [9, 8], 4)]
+
+
+def test_command_line_with_random_weights(tmp_path, capsys):
+    """``--random-weights CONFIG.JSON:SEED`` draws the weights on the device: the same seed gives the same tokens,
+    another seed other tokens."""
+    from conftest import TINY_B
+    from ullm_amd.cli import main
+    path = tmp_path / "config.json"
+    path.write_text(json.dumps(TINY_B))
+    runs = []
+    for seed in (4, 4, 5):
+        rc = main(["--random-weights", f"{path}:{seed}", "--dtype", "float32", "--prompt-ids", "5,17,3,99,200",
+                   "--temperature", "0", "--max-new-tokens", "6", "--ignore-eos", "--context-len", "64", "--num-pages", "16",
+                   "--max-bs", "4"])
+        assert rc == 0
+        lines = [json.loads(x) for x in capsys.readouterr().out.strip().splitlines() if x.startswith("{")]
+        runs.append(lines[0]["token_ids"])
+    assert len(runs[0]) == 6 and runs[0] == runs[1] and runs[0] != runs[2]

@@ -83,6 +83,29 @@ def test_silu_mul(ops, dtype):
     assert torch.all(ops.silu_mul(gu) == 0)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_add_bias(ops, dtype):
+    """The bias of a library product is added by a kernel of our own, in 32-bit, in place, also into a view."""
+    torch.manual_seed(3)
+    y = (torch.randn(37, 203, device=DEV) * 3).to(dtype)
+    bias = torch.randn(203, device=DEV)
+    want = (y.float() + bias).to(dtype)
+    assert ops.add_bias(y, bias) is y and torch.equal(y, want)
+    wide = (torch.randn(5, 64, device=DEV)).to(dtype)
+    keep = wide.clone()
+    ops.add_bias(wide[:, 8:40], bias[:32].contiguous())
+    assert torch.equal(wide[:, 8:40], (keep[:, 8:40].float() + bias[:32]).to(dtype))
+    assert torch.equal(wide[:, :8], keep[:, :8]) and torch.equal(wide[:, 40:], keep[:, 40:])
+    # through the dispatch: a biased bfloat16 product with more rows than the weight-streaming kernel takes
+    if dtype == torch.bfloat16:
+        a, w = torch.randn(40, 64, device=DEV).to(dtype), torch.randn(96, 64, device=DEV).to(dtype)
+        b = torch.randn(96, device=DEV)
+        for out_dtype in (torch.bfloat16, torch.float32):
+            got = ops.gemm_bf16(a, w, b, out_dtype=out_dtype)
+            ref = a.float() @ w.float().T + b
+            assert got.dtype == out_dtype and (got.float() - ref).abs().max() <= tol(dtype, ref)
+
+
 @pytest.mark.parametrize("shape", [(1, 50, 70), (5, 129, 33), (70, 64, 16), (3, 503, 96)])
 def test_gemm_simple(ops, shape):
     torch.manual_seed(3)

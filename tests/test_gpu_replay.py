@@ -313,6 +313,27 @@ def test_random_configurations(tmp_path, trial, matrix_cores):
         close(np.concatenate(outs), want, dtype)
 
 
+def test_bfloat16_attention_off_the_matrix_cores_is_announced(model_dirs, caplog):
+    """Head sizes and page sizes the matrix-core kernels do not take run on the general kernel: right, but
+    many times slower, so it is said once per shape."""
+    import logging
+    from ullm_amd.kernels import ops
+    from ullm_amd.replay import Replayer
+    ops._warned_general_attention.clear()
+    with caplog.at_level(logging.WARNING, logger="ullm_amd"):
+        rep = Replayer(model_dirs["C"], "bfloat16", 128, 16, DEV)                 # head_dim 48
+        for i in range(3):
+            rep.step({"step": i, "entries": [{"id": "r", "tokens": [1, 2, 3], "want": []}], "end": []})
+        rep = Replayer(model_dirs["D"], "bfloat16", 128, 8, DEV)                  # pages of 8
+        rep.step({"step": 0, "entries": [{"id": "r", "tokens": [1, 2, 3], "want": []}], "end": []})
+        rep = Replayer(model_dirs["D"], "bfloat16", 128, 16, DEV)                 # taken by the matrix cores: silent
+        rep.step({"step": 0, "entries": [{"id": "r", "tokens": [1, 2, 3], "want": []}], "end": []})
+        rep = Replayer(model_dirs["C"], "float32", 128, 16, DEV)                  # 32-bit never goes there: silent
+        rep.step({"step": 0, "entries": [{"id": "r", "tokens": [1, 2, 3], "want": []}], "end": []})
+    said = [r.getMessage() for r in caplog.records if "general kernel" in r.getMessage()]
+    assert len(said) == 2 and "head_dim 48" in said[0] and "page size 8" in said[1]
+
+
 def test_pool_too_small_is_an_error_not_a_wrong_result(replayers):
     rep = replayers("A", "float32", max_tokens=64)
     with pytest.raises(RuntimeError, match="pages"):

@@ -1,4 +1,4 @@
-from .engine_config import EngineConfig, normalize_dtype
+from .engine_config import EngineConfig, normalize_dtype, parse_random_weights, preset_names
 from .model_config import ConfigError, Qwen3Config, read_config_json
 
-__all__ = ["EngineConfig", "normalize_dtype", "ConfigError", "Qwen3Config", "read_config_json"]
+__all__ = ["EngineConfig", "normalize_dtype", "parse_random_weights", "preset_names", "ConfigError", "Qwen3Config", "read_config_json"]

@@ -29,9 +29,33 @@ def normalize_dtype(name: str) -> str:
     return _DTYPES[key]
 
 
+PRESET_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "presets")
+
+
+def preset_names() -> List[str]:
+    """Named sizes ``random_weights`` knows: config.json files that ship with the package."""
+    return sorted(f[:-5] for f in os.listdir(PRESET_DIR) if f.endswith(".json"))
+
+
+def parse_random_weights(spec: str):
+    """(config.json dict, seed) of a ``NAME[:SEED]`` / ``PATH[:SEED]`` specification."""
+    name, seed = spec, 0
+    if ":" in spec and spec.rsplit(":", 1)[1].lstrip("-").isdigit():
+        name, seed = spec.rsplit(":", 1)[0], int(spec.rsplit(":", 1)[1])
+    path = os.path.join(PRESET_DIR, name.lower() + ".json") if name.lower() in preset_names() else name
+    if not os.path.isfile(path):
+        raise ConfigError(f"random weights {spec!r}: {name!r} is neither a config.json nor one of {preset_names()}")
+    with open(path, "r", encoding="utf-8") as f:
+        try:
+            config = json.load(f)
+        except json.JSONDecodeError as e:
+            raise ConfigError(f"{path}: not valid JSON ({e})") from None
+    return config, seed
+
+
 @dataclass
 class EngineConfig:
-    model: str                                  # folder with config.json and *.safetensors
+    model: Optional[str] = None                 # folder with config.json and *.safetensors
     gpu_memory_utilization: float = 0.9         # share of free device memory the cache may take
     max_bs: int = 50                            # most live requests (= request slots)
     tp_size: int = 1
@@ -53,9 +77,14 @@ class EngineConfig:
     enable_prefix_cache: bool = False           # share whole pages of equal prompt prefixes
     seed: int = 0                               # default seed for requests that bring none
     device: str = "cuda:0"
+    # instead of ``model``: NAME[:SEED] or PATH[:SEED], a named size (see ``preset_names``) or a config.json,
+    # whose weights are drawn on the device from the seed (default 0)
+    random_weights: Optional[str] = None
 
     def __post_init__(self):
         self.dtype = normalize_dtype(self.dtype)
+        if (self.model is None) == (self.random_weights is None):
+            raise ConfigError("give either a model folder (model) or a random-weights specification, not both or neither")
         if self.tp_size != 1 or self.pp_size != 1:
             raise ConfigError("this engine runs on one GPU: tp_size and pp_size must be 1")
         if self.device_ids is not None:
@@ -77,7 +106,10 @@ class EngineConfig:
     def add_cli_args(parser: argparse.ArgumentParser) -> None:
         """Options with the reference's names and defaults (ullm/entrypoints/api_server.py:130-183)
         followed by this engine's own."""
-        parser.add_argument("--model", type=str, required=True, help="Model folder")
+        parser.add_argument("--model", type=str, default=None, help="Model folder")
+        parser.add_argument("--random-weights", type=str, default=None, metavar="SPEC",
+                            help="instead of --model: NAME[:SEED] or CONFIG.JSON[:SEED], random weights drawn on the "
+                                 f"device; names: {', '.join(preset_names())}")
         parser.add_argument("--gpu-memory-utilization", type=float, default=0.9,
                             help="GPU memory utilization")
         parser.add_argument("--max-bs", type=int, default=50, help="Maximum batch size")
@@ -127,14 +159,15 @@ class EngineConfig:
             max_prefill_chunk=args.max_prefill_chunk,
             enable_prefix_cache=args.enable_prefix_cache,
             seed=args.seed,
+            random_weights=getattr(args, "random_weights", None),
         )
 
     def generation_defaults(self) -> dict:
         """Sampling defaults from generation_config.json beside the model, for the keys the
         reference copies (ullm/config.py:46-67): temperature, top_k, top_p, min_p."""
-        path = os.path.join(self.model, "generation_config.json")
         out = {}
-        if os.path.isfile(path):
+        path = os.path.join(self.model, "generation_config.json") if self.model else ""
+        if path and os.path.isfile(path):
             with open(path, "r", encoding="utf-8") as f:
                 d = json.load(f)
             for key in ("temperature", "top_k", "top_p", "min_p"):

@@ -209,6 +209,30 @@ extern "C" int ullm_residual_add(const void* branch, float* residual, long long 
   ULLM_LAUNCH_CHECK();
 }
 
+// ------------------------------------------------------------------ y[t, :] += bias (float32 [N]), in place
+template <typename T>
+__global__ void add_bias_kernel(T* __restrict__ y, const float* __restrict__ bias, int N, long long row_stride, size_t total) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const size_t t = idx / N;
+  const int n = (int)(idx - t * N);
+  T* p = y + t * row_stride + n;
+  st_f32(p, ld_f32(p) + bias[n]);
+}
+
+extern "C" int ullm_add_bias(void* y, const float* bias, int T_, int N, long long row_stride, int dtype, hipStream_t stream) {
+  if (T_ <= 0 || N <= 0) return 0;
+  const size_t total = (size_t)T_ * N;
+  dim3 block(256), grid((unsigned)((total + 255) / 256));
+  if (dtype == ULLM_F32)
+    hipLaunchKernelGGL(add_bias_kernel<float>, grid, block, 0, stream, (float*)y, bias, N, row_stride, total);
+  else if (dtype == ULLM_BF16)
+    hipLaunchKernelGGL(add_bias_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)y, bias, N, row_stride, total);
+  else
+    return ULLM_ERR_DTYPE;
+  ULLM_LAUNCH_CHECK();
+}
+
 // ------------------------------------------------------------------ SiLU(gate) * up
 template <typename T>
 __global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int I, size_t total) {

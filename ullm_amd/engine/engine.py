@@ -14,7 +14,7 @@ import torch
 
 from ..config.engine_config import EngineConfig
 from ..sampling import Sampler, SamplingParams
-from .loading import load_model
+from .loading import load_model, random_model
 from .request import EngineStepResult, FinishReason, Request, RequestStatus, Scheduled
 from .runner import UNKNOWN_TOKEN, ModelRunner, PreparedStep, StepEntry
 from .scheduler import Scheduler
@@ -57,7 +57,9 @@ class Engine:
         device, tests); otherwise the folder ``config.model`` is loaded."""
         self.config = config
         logging.basicConfig(level=getattr(logging, config.log_level.upper(), logging.INFO))
-        if model is None:
+        if model is None and config.random_weights is not None:
+            model_config, model, env = random_model(config.random_weights, config.dtype, config.device, config.context_len)
+        elif model is None:
             model_config, model, env = load_model(config.model, config.dtype, config.device, config.context_len)
         self.model_config, self.model, self.env = model_config, model, env
         if config.num_pages is not None:

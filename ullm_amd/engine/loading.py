@@ -33,3 +33,15 @@ def load_model(model_dir: str, dtype: str, device: str, context_len: int):
     env = make_env(dtype, device, context_len)
     load_weights(model, model_dir, env)
     return cfg, model, env
+
+
+def random_model(spec: str, dtype: str, device: str, context_len: int):
+    """(typed config, model with random weights drawn on the device, env) for a specification
+    ``NAME[:SEED]`` / ``CONFIG.JSON[:SEED]`` (see :func:`ullm_amd.config.parse_random_weights`)."""
+    from ..config.engine_config import parse_random_weights
+    from ..weights.random_init import bind_random_weights
+    config_dict, seed = parse_random_weights(spec)
+    cfg, model = build_model(config_dict)
+    env = make_env(dtype, device, context_len)
+    bind_random_weights(model, env, seed)
+    return cfg, model, env

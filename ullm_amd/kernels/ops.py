@@ -5,6 +5,7 @@ A non-zero return of a launcher raises ``KernelError``; nothing falls back to an
 from __future__ import annotations
 
 import ctypes
+import logging
 from typing import Optional
 
 import torch
@@ -12,6 +13,7 @@ import torch
 from . import build
 
 F32, BF16 = 0, 1
+logger = logging.getLogger("ullm_amd")
 
 
 class KernelError(RuntimeError):
@@ -135,6 +137,16 @@ def residual_add(branch: torch.Tensor, residual: torch.Tensor) -> None:
     lib = build.load("elementwise")
     _check(lib.ullm_residual_add(_p(branch), _p(residual), ctypes.c_longlong(residual.numel()), _c_int(_dt(branch)),
                                  _stream()), "residual_add")
+
+
+def add_bias(y: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
+    """y [T, N] += bias (float32 [N]) in place, the sum taken in 32-bit; returns y."""
+    T, N = y.shape
+    _need(y.stride(1) == 1, "y must have unit stride along its rows")
+    _need(bias.dtype == torch.float32 and bias.numel() == N and bias.is_contiguous(), "bias must be float32 [N]")
+    _check(build.load("elementwise").ullm_add_bias(_p(y), _p(bias), _c_int(T), _c_int(N), ctypes.c_longlong(y.stride(0)),
+                                                   _c_int(_dt(y)), _stream()), "add_bias")
+    return y
 
 
 def silu_mul(gate_up: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -380,10 +392,10 @@ def gemm_bf16(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = N
         return gemm_skinny(a, w, bias, out_dtype=out_dtype)
     if library and out_dtype == torch.float32 and a.is_contiguous() and w.is_contiguous() and _MM_TAKES_OUT_DTYPE:
         y = torch.mm(a, w.t(), out_dtype=torch.float32)
-        return y if bias is None else y + bias
+        return y if bias is None else add_bias(y, bias)
     if library and out_dtype == torch.bfloat16:
         y = torch.nn.functional.linear(a, w)
-        return y if bias is None else (y.float() + bias).to(torch.bfloat16)
+        return y if bias is None else add_bias(y, bias)
     if out_dtype == torch.float32 and M <= 64 and gemm_skinny_supports(a, w):
         return gemm_skinny(a, w, bias, out_dtype=out_dtype)
     return gemm_simple(a, w, bias, out_dtype=out_dtype)
@@ -478,6 +490,24 @@ def attention_prefill_mfma(q, out, k_pool, v_pool, tiles: torch.Tensor, n_tiles:
         "attention_prefill")
 
 
+_warned_general_attention = set()
+
+
+def _warn_general_attention(hd: int, page_size: int) -> None:
+    """Said once per shape: bfloat16 attention that the matrix-core kernels do not take runs on the general
+    kernel (one block per token and head), which is right but many times slower."""
+    if (hd, page_size) in _warned_general_attention:
+        return
+    _warned_general_attention.add((hd, page_size))
+    why = []
+    if hd not in (32, 64, 96, 128, 256):
+        why.append(f"head_dim {hd} is not one of 32, 64, 96, 128, 256")
+    if page_size % 16:
+        why.append(f"page size {page_size} is not a multiple of 16")
+    logger.warning("bfloat16 attention runs on the general kernel, not on the matrix cores (%s): expect it to be "
+                   "many times slower", "; ".join(why) or "shape not supported")
+
+
 def paged_attention(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, ctx, group, nq: int,
                     nkv: int, hd: int, scale: float, window: int) -> torch.Tensor:
     """Attention of the batch's queries over their requests' cached keys and values (the new
@@ -485,6 +515,8 @@ def paged_attention(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
     the one-token entries, one for the tiles of longer entries); everything else, and float32
     always, takes the general kernel.  Every choice computes the same function."""
     if not attention_mfma_supports(q.dtype, hd, group.page_size, nq, nkv):
+        if q.dtype == torch.bfloat16:
+            _warn_general_attention(hd, group.page_size)
         return paged_attention_generic(q, k_pool, v_pool, ctx.positions, ctx.token_entry, group.block_table,
                                        group.page_size, nq, nkv, hd, scale, window)
     out = torch.empty((q.shape[0], nq * hd), dtype=q.dtype, device=q.device)
