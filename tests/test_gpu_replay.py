@@ -171,6 +171,31 @@ def test_portions_whose_projections_come_as_stacks_of_partial_sums(model_dirs, p
     close(np.concatenate(got), want, "bfloat16")
 
 
+def test_portions_of_17_to_64_tokens_through_the_kernel_for_those_row_counts(model_dirs, plain_models, monkeypatch):
+    """Steps of 17 to 64 tokens take the q|k|v and gate|up projections through the kernel for those row counts where
+    the matrices are large; here the size limit is lifted so that a tiny model (A: width 64, a whole stage of K)
+    takes that way too, beside steps that do not."""
+    from ullm_amd.kernels import ops
+    from ullm_amd.replay import Replayer
+    monkeypatch.setattr(ops, "ROWS_MIN_COLUMNS", 0)
+    calls, inner = [], ops.gemm_rows
+    monkeypatch.setattr(ops, "gemm_rows", lambda a, w, bias=None, silu=False: calls.append((a.shape[0], silu)) or inner(a, w, bias, silu))
+    rep = Replayer(model_dirs["A"], "bfloat16", 512, 16, DEV)
+    vocab = plain_models["A"][0]["vocab_size"]
+    toks = make_tokens(vocab, 250, 32)
+    want = oracle(plain_models, "A", toks)
+    sizes = [17, 3, 64, 40, 1, 60, 16, 25, 24]
+    assert sum(sizes) == 250
+    got, i = [], 0
+    for s, n in enumerate(sizes):
+        got.append(rep.step({"step": s, "entries": [{"id": "r", "tokens": toks[i:i + n], "want": list(range(n))}],
+                             "end": ["r"] if i + n == 250 else []}))
+        i += n
+    assert {n for n, _ in calls} == {n for n in sizes if 17 <= n <= 64}
+    assert {silu for _, silu in calls} == {False, True}               # q|k|v and gate|up
+    close(np.concatenate(got), want, "bfloat16")
+
+
 @pytest.mark.parametrize("name,dtype", [("B", "float32"), ("C", "bfloat16"), ("C", "float32"), ("D", "bfloat16"),
                                         ("E", "bfloat16")])
 def test_long_decoding(replayers, plain_models, name, dtype):

@@ -48,6 +48,19 @@ __device__ __forceinline__ uint4 ld_stream16(const void* p) {
   return make_uint4(v.x, v.y, v.z, v.w);
 }
 
+// 16 bytes as one vector load / store.  (Copying a uint4 through a cast pointer is a memcpy to the compiler,
+// which can keep registers that hold loads in flight in scratch memory; a native vector type is a plain load.)
+__device__ __forceinline__ uint4 ld16(const void* p) {
+  typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
+  const u32x4 v = *reinterpret_cast<const u32x4*>(p);
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ void st16(void* p, const uint4& v) {
+  typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
+  const u32x4 t = {v.x, v.y, v.z, v.w};
+  *reinterpret_cast<u32x4*>(p) = t;
+}
+
 __device__ __forceinline__ uint2 ld_stream8(const void* p) {
   typedef __attribute__((ext_vector_type(2))) unsigned int u32x2;
   const u32x2 v = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(p));

@@ -1,0 +1,257 @@
+// C[M, N] = X[M, K] * W[N, K]^T for 17 to 64 rows, bfloat16 in and out, 32-bit accumulation, with what
+// follows the product folded in:
+//   STORE : C = result (+ bias)
+//   SILU  : W is the stacked gate|up matrix [2 N, K]; C[M, N] = silu(gate) * up on the 32-bit sums
+//           (ullm/layers/activation.py:16-18 after gate_up_proj, ullm/models/qwen3.py:43-45)
+//
+// At these row counts the product is still a read of W from HBM, once, and its time is set by how many
+// bytes of W the chip keeps on their way.  So the matrix is cut into as many blocks as there are compute
+// units (a block's columns need not be a multiple of 16: the last tile of a wave is used in part), and a
+// wave keeps four to six stages of 64 values of K of its tiles of W in flight in registers.  The rows of X
+// are shared: a stage of X goes through shared memory once per block and every wave reads its operand
+// from there.  A result column is summed by one wave in the order of K, so it does not depend on timing
+// or on the batch.
+//
+// A operand of v_mfma_f32_16x16x32_bf16 = a W tile (lane (r, g) holds W[n0 + r][k + 8g .. +8]), B
+// operand = 16 rows of X; W tiles reach that layout through the wave's own part of shared memory (a
+// wave fetches whole 128-byte lines, 8 rows per instruction).  Shared-memory rows are 128 bytes; piece
+// c of row r lies at piece c ^ ((r >> 1) & 7), which keeps the 16-byte writes and reads of the
+// hardware's lane groups on different banks.  Weights are [out, in] (ullm/layers/linear.py:165).
+#include "common.h"
+#include <type_traits>
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+
+union Pack8 {
+  bf16x8_t v;
+  uint4 u4;
+};
+
+enum { ROWS_STORE = 0, ROWS_SILU = 1 };
+
+// f(0), f(1), .. f(N - 1) with the index a constant of the language, not of the optimiser: registers that
+// hold stages in flight are then never indexed by a variable, and so never end up in scratch memory
+template <int I, int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    static_for<I + 1, N>(f);
+  }
+}
+
+#define ROWS_MAX_WAVES 8   // waves of a block (512 threads: two waves a SIMD, 256 registers each)
+
+// Stages of W and of X a wave has in flight (of X as many as of W: loads complete in order, so waiting for a stage
+// of X waits for every load issued before it, and a stage of X fetched later than a stage of W would cut short
+// what W has in flight).  As many as about 150 registers hold: ntw tiles of W (two 16-byte pieces each) and xq
+// pieces of X per stage.
+__host__ __device__ constexpr int rows_depth(int ntw, int xq) {
+  const int d = 150 / ((2 * ntw + xq) * 4);
+  return d < 3 ? 3 : (d > 8 ? 8 : d);
+}
+
+// MT = 16-row tiles of X (M <= 16 MT); XQ = 16-byte pieces of a stage of X per thread (MT * 128 pieces over the
+// block's threads).  Wave wn of a block's WN owns columns n0 .. n0 + cols_per_wave of the block's cols_per_block.
+template <int MT, int XQ, int EPI>
+__global__ void __launch_bounds__(64 * ROWS_MAX_WAVES)
+gemm_rows_kernel(const bf16_t* __restrict__ X, int ldx, const bf16_t* __restrict__ W, int ldw,
+                 const float* __restrict__ bias, bf16_t* __restrict__ C, int ldc, int M, int N, int K,
+                 int WN, int cols_per_wave, int cols_per_block) {
+  constexpr int NTW = EPI == ROWS_SILU ? 2 : 1;         // tiles of W per wave: gate and up rows of the same columns
+  constexpr int D = rows_depth(NTW, XQ);
+  constexpr int TILE = 16 * 128;                        // 16 rows x 64 values
+  constexpr int XB = MT * TILE;                         // a stage of X
+  __shared__ __attribute__((aligned(16))) unsigned char xs[2 * XB + 64 * 16];   // two stages, then a spare place per lane
+  __shared__ __attribute__((aligned(16))) unsigned char ws[ROWS_MAX_WAVES * NTW * TILE];
+  const int tid = threadIdx.x, lane = tid & 63, wn = tid >> 6;
+  const int g = lane >> 4, r = lane & 15, lrow = lane >> 3, lcol = lane & 7;
+  const int block_n0 = blockIdx.x * cols_per_block;
+  const int block_end = block_n0 + cols_per_block < N ? block_n0 + cols_per_block : N;
+  const int n0 = block_n0 + wn * cols_per_wave;
+  const int n_end = n0 + cols_per_wave < block_end ? n0 + cols_per_wave : block_end;   // may lie below n0: a wave without columns
+  // W: a lane fetches rows lrow and 8 + lrow of each of the wave's tiles, piece lcol.  No load stands
+  // under a condition and no loaded value under a select (either makes the compiler wait for every load
+  // in flight at the next use, which would undo the stages in flight).  Nothing needs one: a row of W
+  // past the wave's columns reads the wave's last row again (a line the same instruction fetches anyway)
+  // and only feeds result columns that are never stored; a row of X past M reads row 0 and only feeds
+  // result rows that are never stored; K is a whole number of stages, so no stage has a tail; and the
+  // stages fetched past the end of the loop read the matrix's last stage again and are not used.
+  const bf16_t* wsrc[NTW][2];
+  int put[2], get[2];
+  const int last_col = n_end > n0 ? n_end - 1 : 0;
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int row = 8 * h + lrow, col = n0 + row;
+    put[h] = row * 128 + ((lcol ^ ((row >> 1) & 7)) << 4);
+    get[h] = r * 128 + (((4 * h + g) ^ ((r >> 1) & 7)) << 4);       // h here: the step of 32 inside the stage
+#pragma unroll
+    for (int i = 0; i < NTW; ++i)
+      wsrc[i][h] = W + ((size_t)(col < n_end ? col : last_col) + (size_t)i * N) * ldw + 8 * lcol;
+  }
+  // X: piece p = tid + 64 WN q of the stage is row p / 8, piece p % 8.  Where the piece goes in shared
+  // memory: xput + (stage & 1) * xstep.  A thread whose piece lies past the stage reads piece 0 and stores
+  // to a spare place instead of skipping either (a store of a loaded value under a condition would again
+  // wait for every load in flight).
+  const bf16_t* xsrc[XQ];
+  int xput[XQ], xstep[XQ];
+#pragma unroll
+  for (int q = 0; q < XQ; ++q) {
+    const int p = tid + 64 * WN * q;
+    const bool ok = p < MT * 128;
+    const int row = ok ? p >> 3 : 0, col = ok ? p & 7 : 0;
+    xsrc[q] = X + (size_t)(row < M ? row : 0) * ldx + 8 * col;
+    xput[q] = ok ? (row >> 4) * TILE + (row & 15) * 128 + ((col ^ (((row & 15) >> 1) & 7)) << 4) : 2 * XB + 16 * lane;
+    xstep[q] = ok ? XB : 0;
+  }
+  unsigned char* const mine = ws + wn * NTW * TILE;
+  f32x4_t acc[NTW][MT];
+#pragma unroll
+  for (int i = 0; i < NTW; ++i)
+#pragma unroll
+    for (int t = 0; t < MT; ++t) acc[i][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  struct Stage { uint4 w[NTW][2], x[XQ]; };
+  const int k_last = K - 64;                                        // first value of the matrix's last stage
+  auto fetch = [&](Stage& s, int k0) __attribute__((always_inline)) {
+    const int k = k0 < k_last ? k0 : k_last;
+    static_for<0, NTW>([&](auto i) {
+      static_for<0, 2>([&](auto h) { s.w[i][h] = ld_stream16(wsrc[i][h] + k); });
+    });
+    static_for<0, XQ>([&](auto q) { s.x[q] = ld16(xsrc[q] + k); });
+  };
+  // One stage: the registers that hold stage s go to shared memory and are refilled with the stage that
+  // will need them next; a barrier; the products.  Stage s goes to the X buffer that was last read two
+  // stages ago, before the previous barrier.
+  auto stage = [&](Stage& st, int s) __attribute__((always_inline)) {
+    unsigned char* xb = xs + (s & 1) * XB;
+    static_for<0, XQ>([&](auto q) { st16(xs + xput[q] + (s & 1) * xstep[q], st.x[q]); });
+    static_for<0, NTW>([&](auto i) {
+      static_for<0, 2>([&](auto h) { st16(mine + i * TILE + put[h], st.w[i][h]); });
+    });
+    fetch(st, 64 * (s + D));
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      Pack8 wf[NTW], xf[MT];
+#pragma unroll
+      for (int i = 0; i < NTW; ++i) wf[i].u4 = *reinterpret_cast<const uint4*>(mine + i * TILE + get[j]);
+#pragma unroll
+      for (int t = 0; t < MT; ++t) xf[t].u4 = *reinterpret_cast<const uint4*>(xb + t * TILE + get[j]);
+#pragma unroll
+      for (int i = 0; i < NTW; ++i)
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+          acc[i][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[i].v, xf[t].v, acc[i][t], 0, 0, 0);
+    }
+  };
+  // D stages in flight: registers st[d] hold the stages s = d (mod D)
+  Stage st[D];
+  const int stages = K / 64;
+  static_for<0, D>([&](auto d) { fetch(st[d], 64 * d); });
+  int s = 0;
+  for (; s + D <= stages; s += D) static_for<0, D>([&](auto d) { stage(st[d], s + d); });
+  static_for<0, D - 1>([&](auto d) {
+    if (s + d < stages) stage(st[d], s + d);
+  });
+  // acc[i][t][j] = sum for row m = 16 t + r, column n0 + 4 g + j (of half i of the stacked matrix)
+  const int nn = n0 + 4 * g;
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    const int m = 16 * t + r;
+    if (m >= M || nn >= n_end) continue;
+    float v[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if (EPI == ROWS_SILU) v[j] = fast_silu(acc[0][t][j]) * acc[NTW - 1][t][j];
+      else v[j] = acc[0][t][j] + (bias && nn + j < n_end ? bias[nn + j] : 0.f);
+    }
+    bf16_t* cp = C + (size_t)m * ldc + nn;
+    if (nn + 3 < n_end) {
+      *reinterpret_cast<uint2*>(cp) = make_uint2(pack2_bf16(v[0], v[1]), pack2_bf16(v[2], v[3]));
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (nn + j < n_end) cp[j] = f32_to_bf16_bits(v[j]);
+    }
+  }
+}
+
+static int rows_compute_units() {
+  static int units[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (units[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    units[dev] = n;
+  }
+  return units[dev];
+}
+
+struct RowsShape {
+  int cols_per_block, cols_per_wave, wn, xq, blocks;
+};
+
+// How a matrix of N result columns is cut: a whole number of rounds of one block per compute unit, and
+// the block's columns over its waves in steps of 4 (at most 16 per wave).  A function of the matrix, the
+// epilogue and the number of 16-row tiles of X alone.
+static bool rows_shape(int N, int mt, int units, RowsShape* s) {
+  const int rounds = (N + units * 16 * ROWS_MAX_WAVES - 1) / (units * 16 * ROWS_MAX_WAVES);
+  int cpb = (N + rounds * units - 1) / (rounds * units);
+  cpb = (cpb + 3) / 4 * 4;
+  if (cpb < 8) cpb = 8;
+  int wn = (cpb + 15) / 16;
+  if (wn < 2) wn = 2;                                   // at least two waves: a wave alone hides no latency of the other's products
+  if (wn > ROWS_MAX_WAVES) return false;
+  int cpw = (cpb + wn - 1) / wn;
+  cpw = (cpw + 3) / 4 * 4;
+  s->cols_per_block = cpb;
+  s->cols_per_wave = cpw;
+  s->wn = wn;
+  s->xq = (mt * 128 + 64 * wn - 1) / (64 * wn);
+  s->blocks = (N + cpb - 1) / cpb;
+  return true;
+}
+
+// N: columns of the result (with epi 1 the weights have 2 N rows)
+extern "C" int ullm_gemm_rows_supports(int M, int N, int K, int ldx, int ldw, int ldc, int epi) {
+  RowsShape s;
+  return M >= 1 && M <= 64 && N >= 4 && K >= 64 && K % 64 == 0 && ldx % 8 == 0 && ldw % 8 == 0 && ldc % 4 == 0 &&
+         ldc >= N && (epi == ROWS_STORE || epi == ROWS_SILU) && rows_shape(N, (M + 15) / 16, rows_compute_units(), &s);
+}
+
+// X bfloat16 [M <= 64, K], K a multiple of 64; W bfloat16 [N, K] (epi 1: [2 N, K], gate rows then up rows);
+// C bfloat16 [M, N] with row stride ldc; bias float32 [N] or null (epi 0 only).
+extern "C" int ullm_gemm_rows(const void* X, int ldx, const void* W, int ldw, const float* bias, void* C, int ldc,
+                              int M, int N, int K, int epi, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (!ullm_gemm_rows_supports(M, N, K, ldx, ldw, ldc, epi)) return ULLM_ERR_SHAPE;
+  if (((uintptr_t)X & 15) || ((uintptr_t)W & 15) || ((uintptr_t)C & 7)) return ULLM_ERR_SHAPE;
+  if (epi == ROWS_SILU && bias) return ULLM_ERR_UNSUPPORTED;
+  const int mt = (M + 15) / 16;
+  RowsShape s;
+  rows_shape(N, mt, rows_compute_units(), &s);
+  dim3 grid(s.blocks), block(64 * s.wn);
+#define GO(MT, XQ, EPI) hipLaunchKernelGGL((gemm_rows_kernel<MT, XQ, EPI>), grid, block, 0, stream, (const bf16_t*)X, ldx, \
+    (const bf16_t*)W, ldw, bias, (bf16_t*)C, ldc, M, N, K, s.wn, s.cols_per_wave, s.cols_per_block)
+#define GO_XQ(MT, EPI)                                    \
+  do {                                                    \
+    if (s.xq <= 1) GO(MT, 1, EPI);                        \
+    else if (s.xq == 2) { if constexpr (MT >= 2) GO(MT, 2, EPI); } \
+    else if (s.xq == 3) { if constexpr (MT >= 3) GO(MT, 3, EPI); } \
+    else { if constexpr (MT >= 4) GO(MT, 4, EPI); }       \
+  } while (0)
+#define GO_MT(EPI)                         \
+  do {                                     \
+    if (mt == 1) GO_XQ(1, EPI);            \
+    else if (mt == 2) GO_XQ(2, EPI);       \
+    else if (mt == 3) GO_XQ(3, EPI);       \
+    else GO_XQ(4, EPI);                    \
+  } while (0)
+  if (epi == ROWS_SILU) GO_MT(ROWS_SILU);
+  else GO_MT(ROWS_STORE);
+#undef GO_MT
+#undef GO_XQ
+#undef GO
+  ULLM_LAUNCH_CHECK();
+}

@@ -1,0 +1,175 @@
+"""Times single kernels at given shapes: ``python -m ullm_amd.kernels.microbench <what> [options]``.
+
+Every measurement records its calls as nodes of one HIP graph (so that a call costs what it costs
+inside a decode graph, without the host's launch time) and rotates over several copies of the large
+operands (weights, cache pages), enough of them that no call finds its data in the 256 MB memory-side
+cache: the figures are those of a cold read from HBM, as in a model whose weights exceed that cache.
+
+  decode-attention   one token per request over its cache: every (splits, waves) shape of the launch
+  prefill-attention  prompt tiles of one request
+  projection         a [rows, K] x [N, K]^T product by each kernel that can take it, and the library
+"""
+from __future__ import annotations
+
+import argparse
+from typing import Callable, List
+
+import torch
+
+from . import ops
+
+DEV = "cuda:0"
+
+
+def graph_time(calls: List[Callable[[], None]], replays: int = 5) -> float:
+    """Mean microseconds per call of ``calls`` when they run as one HIP graph."""
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for f in calls:
+            f()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        for f in calls:
+            f()
+    g.replay()
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(replays):
+        g.replay()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / replays / len(calls) * 1e3
+
+
+def copies_for(nbytes: int, at_least: int = 4) -> int:
+    """How many copies of an operand of this size make 1.5 GB, several times the memory-side cache."""
+    return max(at_least, min(64, -(-(3 << 29) // max(1, nbytes))))
+
+
+def decode_attention(args) -> None:
+    nq, nkv, hd, P = args.heads, args.kv_heads, args.head_dim, args.page_size
+    for B in args.batch:
+        for ctx in args.context:
+            pages_per = -(-ctx // P)
+            kv_bytes = B * ctx * nkv * hd * 2 * 2
+            nv = copies_for(kv_bytes, 8)
+            n_pages = nv * B * pages_per
+            k_pool = torch.randn(n_pages, nkv, P, hd, device=DEV).bfloat16()
+            v_pool = torch.randn(n_pages, nkv, hd, P, device=DEV).bfloat16()
+            tables = torch.randperm(n_pages).int().reshape(nv, B, pages_per).to(DEV)
+            q = torch.randn(B, nq * hd, device=DEV).bfloat16()
+            out = torch.empty_like(q)
+            pos = torch.full((B,), ctx - 1, dtype=torch.int32, device=DEV)
+            ent = torch.arange(B, dtype=torch.int32, device=DEV)
+            groups = -(-(nq // nkv) // 16)
+            auto = ops.decode_split(B, nkv, groups, ctx, hd)
+            cells = []
+            for splits, waves in [(0, 0)] + [(s, w) for w in (4, 8, 1) for s in (1, 2, 4, 8, 16, 32)]:
+                if splits * B * nkv * groups > 2048 or (hd == 256 and waves == 8):
+                    continue
+                calls = [(lambda v=v: ops.attention_decode_mfma(q, out, k_pool, v_pool, None, B, pos, ent, tables[v], P, nq,
+                                                                nkv, hd, hd ** -0.5, 0, ctx, splits=splits, waves=waves))
+                         for v in range(nv)]
+                t = graph_time(calls)
+                name = f"chosen {auto[1]}x{auto[0]}" if splits == 0 else f"{splits}x{waves}"
+                cells.append(f"{name}: {t:.1f}")
+            print(f"decode attention, batch {B}, context {ctx}, {nq}/{nkv} heads of {hd} ({kv_bytes / 1e6:.0f} MB of cache); "
+                  f"us by splits x waves: " + "  ".join(cells), flush=True)
+            del k_pool, v_pool
+
+
+def prefill_attention(args) -> None:
+    nq, nkv, hd, P = args.heads, args.kv_heads, args.head_dim, args.page_size
+    for T in args.context:
+        pages_per = -(-T // P)
+        nv = 4
+        n_pages = nv * pages_per
+        k_pool = torch.randn(n_pages, nkv, P, hd, device=DEV).bfloat16()
+        v_pool = torch.randn(n_pages, nkv, hd, P, device=DEV).bfloat16()
+        tables = torch.randperm(n_pages).int().reshape(nv, 1, pages_per).to(DEV)
+        q = torch.randn(T, nq * hd, device=DEV).bfloat16()
+        out = torch.empty_like(q)
+        pos = torch.arange(T, dtype=torch.int32, device=DEV)
+        ent = torch.zeros(T, dtype=torch.int32, device=DEV)
+        tile = ops.PREFILL_TILE
+        tiles = torch.tensor([[i, min(tile, T - i)] for i in range(0, T, tile)], dtype=torch.int32, device=DEV)
+        keys = [min(i + tile, T) for i in range(0, T, tile)]
+        flops = 4 * nq * hd * T * (T + 1) / 2
+        cells = []
+        for halves in (0, 1, 2):
+            calls = [(lambda v=v: ops.attention_prefill_mfma(q, out, k_pool, v_pool, tiles, tiles.shape[0], pos, ent, tables[v],
+                                                             P, nq, nkv, hd, hd ** -0.5, 0, halves=halves,
+                                                             keys_total=sum(keys), keys_max=max(keys)))
+                     for v in range(nv)]
+            t = graph_time(calls)
+            cells.append(f"halves {halves or 'chosen'}: {t:.1f} us = {flops / t / 1e6:.0f} TFLOP/s")
+        print(f"prompt attention, {T} tokens, {nq}/{nkv} heads of {hd}: " + "  ".join(cells), flush=True)
+        del k_pool, v_pool
+
+
+def projection(args) -> None:
+    N, K = args.columns, args.inner
+    w_bytes = N * K * 2
+    nv = copies_for(w_bytes)
+    ws = [torch.randn(N, K, device=DEV).bfloat16() * 0.02 for _ in range(nv)]
+    gain = torch.ones(K, device=DEV)
+    for M in args.rows:
+        x = torch.randn(M, K, device=DEV).bfloat16()
+        stream = torch.randn(M, K, device=DEV)
+        resid = torch.zeros(M, N, device=DEV)
+        cells = []
+
+        def timed(name, make):
+            try:
+                make(0)()
+            except ops.KernelError:
+                return
+            cells.append(f"{name}: {graph_time([make(v) for v in range(nv)]):.1f}")
+        timed("library", lambda v: (lambda: torch.nn.functional.linear(x, ws[v])))
+        if ops.gemm_skinny_supports(x, ws[0]):
+            timed("skinny", lambda v: (lambda: ops.gemm_skinny(x, ws[v])))
+            timed("skinny+add", lambda v: (lambda: ops.gemm_skinny_add(x, ws[v], resid)))
+            if N % 2 == 0:
+                timed("skinny+silu", lambda v: (lambda: ops.gemm_skinny_silu(x, ws[v])))
+        if ops.gemm_skinny_normed_supports(stream, gain, ws[0]):
+            timed("skinny+norm", lambda v: (lambda: ops.gemm_skinny_normed(stream, gain, 1e-6, ws[v])))
+        if ops.gemm_rows_supports(x, ws[0]):
+            timed("rows", lambda v: (lambda: ops.gemm_rows(x, ws[v])))
+        if N % 2 == 0 and ops.gemm_rows_supports(x, ws[0], silu=True):
+            timed("rows+silu", lambda v: (lambda: ops.gemm_rows(x, ws[v], silu=True)))
+        if ops.gemm_partial_sums_supports(x, ws[0]):
+            timed("partial sums", lambda v: (lambda: ops.gemm_partial_sums(x, ws[v])))
+        if N % 2 == 0:
+            timed("library+silu", lambda v: (lambda: ops.silu_mul(torch.nn.functional.linear(x, ws[v]))))
+        floor = w_bytes / 8e12 * 1e6
+        print(f"projection [{M}, {K}] x [{N}, {K}]^T ({w_bytes / 1e6:.0f} MB of weights, {floor:.1f} us at 8 TB/s); us: "
+              + "  ".join(cells), flush=True)
+
+
+def main(argv=None) -> int:
+    ap = argparse.ArgumentParser(prog="ullm_amd.kernels.microbench", description=__doc__.split("\n\n")[0])
+    sub = ap.add_subparsers(dest="what", required=True)
+    ints = lambda s: [int(x) for x in s.split(",")]   # noqa: E731
+    for name in ("decode-attention", "prefill-attention"):
+        p = sub.add_parser(name)
+        p.add_argument("--heads", type=int, default=32)
+        p.add_argument("--kv-heads", type=int, default=8)
+        p.add_argument("--head-dim", type=int, default=128)
+        p.add_argument("--page-size", type=int, default=16)
+        p.add_argument("--batch", type=ints, default=[1, 8, 64], help="comma-separated batch sizes (decode)")
+        p.add_argument("--context", type=ints, default=[1100], help="comma-separated context lengths / prompt lengths")
+    p = sub.add_parser("projection")
+    p.add_argument("--columns", type=int, required=True, help="rows of the weight matrix (columns of the result)")
+    p.add_argument("--inner", type=int, required=True)
+    p.add_argument("--rows", type=ints, default=[1, 8, 16, 32, 64, 128], help="comma-separated numbers of rows of x")
+    args = ap.parse_args(argv)
+    {"decode-attention": decode_attention, "prefill-attention": prefill_attention, "projection": projection}[args.what](args)
+    return 0
+
+
+if __name__ == "__main__":
+    raise SystemExit(main())

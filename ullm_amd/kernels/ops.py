@@ -367,6 +367,41 @@ def gemm_partial_sums(a: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     return out
 
 
+ROWS_MAX_ROWS = 64
+# fewest columns of the result for which the 17-to-64-row kernel is chosen over the library: with fewer, its
+# blocks (one per compute unit, at least 8 columns each) would not fill the chip
+ROWS_MIN_COLUMNS = 2048
+
+
+def gemm_rows_supports(a: torch.Tensor, w: torch.Tensor, silu: bool = False) -> bool:
+    M, K = a.shape
+    n_out = w.shape[0] // 2 if silu else w.shape[0]
+    return (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and a.stride(1) == 1 and w.stride(1) == 1
+            and w.shape[1] == K and (not silu or w.shape[0] % 2 == 0) and a.data_ptr() % 16 == 0
+            and w.data_ptr() % 16 == 0 and n_out % 4 == 0
+            and bool(build.load("gemm_rows").ullm_gemm_rows_supports(
+                _c_int(M), _c_int(n_out), _c_int(K), _c_int(a.stride(0)), _c_int(w.stride(0)), _c_int(n_out),
+                _c_int(1 if silu else 0))))
+
+
+def gemm_rows(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, silu: bool = False) -> torch.Tensor:
+    """a (bfloat16 [M <= 64, K]) times w (bfloat16 [N, K]) transposed (+ bias float32 [N]) as bfloat16 [M, N];
+    with ``silu``, w is gate | up [2 I, K] and the result silu(gate) * up [M, I] on the 32-bit sums.  The
+    matrix is cut into one block per compute unit and every wave keeps several stages of its rows of w in
+    flight: for the row counts between the few-rows kernel and the library."""
+    M, K = a.shape
+    _need(gemm_rows_supports(a, w, silu), "gemm_rows takes bfloat16, M <= 64, K a multiple of 8, N a multiple of 4")
+    n_out = w.shape[0] // 2 if silu else w.shape[0]
+    if bias is not None:
+        _need(not silu and bias.dtype == torch.float32 and bias.numel() == n_out and bias.is_contiguous(),
+              "bias must be float32 [N] (and there is none with silu)")
+    out = torch.empty((M, n_out), dtype=torch.bfloat16, device=a.device)
+    _check(build.load("gemm_rows").ullm_gemm_rows(_p(a), _c_int(a.stride(0)), _p(w), _c_int(w.stride(0)), _p(bias), _p(out),
+                                                  _c_int(n_out), _c_int(M), _c_int(n_out), _c_int(K),
+                                                  _c_int(1 if silu else 0), _stream()), "gemm_rows")
+    return out
+
+
 SKINNY_MAX_ROWS = 16     # up to here the weight-streaming kernel beats the library product
 # torch.mm(..., out_dtype=float32) stores the 32-bit accumulator of a bfloat16 product; older torch lacks it
 _MM_TAKES_OUT_DTYPE = "out_dtype" in (torch.mm.__doc__ or "")
@@ -390,6 +425,8 @@ def gemm_bf16(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = N
     if (out_dtype == torch.float32 and M <= WIDE_HEAD_SKINNY_MAX_ROWS and w.shape[0] >= WIDE_HEAD_MIN_COLUMNS
             and gemm_skinny_supports(a, w)):
         return gemm_skinny(a, w, bias, out_dtype=out_dtype)
+    if (out_dtype == torch.bfloat16 and M <= ROWS_MAX_ROWS and w.shape[0] >= ROWS_MIN_COLUMNS and gemm_rows_supports(a, w)):
+        return gemm_rows(a, w, bias)
     if library and out_dtype == torch.float32 and a.is_contiguous() and w.is_contiguous() and _MM_TAKES_OUT_DTYPE:
         y = torch.mm(a, w.t(), out_dtype=torch.float32)
         return y if bias is None else add_bias(y, bias)
@@ -412,19 +449,22 @@ def attention_mfma_supports(dtype: torch.dtype, hd: int, page_size: int, nq: int
 
 def decode_split(n_items: int, nkv: int, groups: int, max_kv: int, hd: int = 128):
     """(waves, num_splits) of the decode attention launch.  A wave walks its keys one 32-key tile after
-    the other, each a round trip to memory, so few (token, kv head) pairs are cut further: up to one
-    block per compute unit, down to about one tile per wave; a second small kernel adds the blocks'
-    partial results.  From 256 pairs on there are blocks enough and a token's keys stay in one block;
-    from 1024 pairs on a block is a single wave that walks all keys of its pair, so that the waves of
-    a compute unit start and end independently and one's start overlaps the others' streaming."""
+    the other, each a round trip to memory, so few (token, kv head) pairs with many keys are cut over
+    several blocks, up to one block per compute unit (more would run in a second round), and a second
+    small kernel adds the blocks' partial results; that kernel costs about as much as walking eight more
+    tiles, so short contexts are not cut.  From 256 pairs on there are blocks enough and a token's keys
+    stay in one block; from 1024 pairs on a block is a single wave that walks all keys of its pair, so
+    that the waves of a compute unit start and end independently and one's start overlaps the others'
+    streaming.  (Timings behind these choices: profiles/decode_attention_shapes_qwen3_8b.md.)"""
     pairs = max(1, n_items * nkv * groups)
     if pairs >= 1024:
         return 1, 1
-    waves = 8 if (pairs <= 512 and hd != 256) else 4
-    if pairs >= 256:
-        return waves, 1
     tiles = -(-max_kv // 32)
-    return waves, max(1, min(256 // pairs, tiles // waves))
+    splits = 1
+    if pairs < 256 and tiles > 16:
+        splits = max(1, min(256 // pairs, tiles // 3))
+    waves = 8 if (splits == 1 and pairs < 256 and hd != 256) else 4
+    return waves, splits
 
 
 def attention_decode_mfma(q, out, k_pool, v_pool, token_list: Optional[torch.Tensor], n_items: int,

@@ -13,12 +13,12 @@ from .base import FeedForward, PartEnv, StepContext, WeightDecl, register_part
 from .linear import can_fuse, linear, linear_into_stream, linear_of_norm
 
 
-# Rows up to which the weight-streaming kernel with the activation folded in beats the library product plus the
-# activation kernel (in a graph, gate|up of Qwen3-8B / 14B / 32B): at 16 rows 33 / 68 / 95 us against 46 / 87 / 97 us;
-# at 17 to 32 rows 36-40 / 71-83 / 98-115 us against 48-52 / 85-89 / 96-99 us; from 33 rows on the library is ahead
-# everywhere.  So up to 32 rows, but only up to 16 for matrices beyond Qwen3-14B's 178 M elements.
+# gate|up with the activation folded in, by rows of the batch (timings: profiles/projections_by_rows.md):
+# up to 16 rows the few-rows kernel; from 17 to 64 rows the kernel for those row counts, except that up to 32 rows
+# the few-rows kernel is still ahead on matrices up to Qwen3-8B's size; beyond 64 rows the library product and
+# the activation kernel.
 GATE_UP_SKINNY_MAX_ROWS = 32
-GATE_UP_SKINNY_WIDE_MAX_WEIGHT = 200_000_000     # elements of gate|up up to which 17 to 32 rows take that kernel too
+GATE_UP_SKINNY_WIDE_MAX_WEIGHT = 200_000_000     # elements of gate|up up to which 17 to 32 rows take the few-rows kernel
 
 
 @register_part("ffn", "swiglu")
@@ -47,6 +47,9 @@ class SwiGLU(FeedForward):
                 and (rows <= 16 or self.w_gate_up.numel() <= GATE_UP_SKINNY_WIDE_MAX_WEIGHT)
                 and ops.gemm_skinny_supports(x, self.w_gate_up)):
             act = ops.gemm_skinny_silu(x, self.w_gate_up)
+        elif (x.dtype == torch.bfloat16 and 16 < rows <= ops.ROWS_MAX_ROWS and self.intermediate_size >= ops.ROWS_MIN_COLUMNS
+                and ops.gemm_rows_supports(x, self.w_gate_up, silu=True)):
+            act = ops.gemm_rows(x, self.w_gate_up, silu=True)
         else:
             act = ops.silu_mul(linear(x, self.w_gate_up))
         return linear_into_stream(act, self.w_down, ctx)
