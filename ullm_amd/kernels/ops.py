@@ -452,18 +452,24 @@ def decode_split(n_items: int, nkv: int, groups: int, max_kv: int, hd: int = 128
     the other, each a round trip to memory, so few (token, kv head) pairs with many keys are cut over
     several blocks, up to one block per compute unit (more would run in a second round), and a second
     small kernel adds the blocks' partial results; that kernel costs about as much as walking eight more
-    tiles, so short contexts are not cut.  From 256 pairs on there are blocks enough and a token's keys
-    stay in one block; from 1024 pairs on a block is a single wave that walks all keys of its pair, so
-    that the waves of a compute unit start and end independently and one's start overlaps the others'
-    streaming.  (Timings behind these choices: profiles/decode_attention_shapes_qwen3_8b.md.)"""
+    tiles, so short contexts are not cut.  Mostly a block is a single wave (several are resident on a
+    SIMD, they start and end independently and one's start overlaps the others' streaming, and their number
+    need not be a multiple of the compute units); four waves a block where few pairs have very many keys.
+    (Timings behind these choices: profiles/decode_attention_shapes_qwen3_8b.md.)"""
     pairs = max(1, n_items * nkv * groups)
     if pairs >= 1024:
         return 1, 1
     tiles = -(-max_kv // 32)
-    splits = 1
-    if pairs < 256 and tiles > 16:
-        splits = max(1, min(256 // pairs, tiles // 3))
-    waves = 8 if (splits == 1 and pairs < 256 and hd != 256) else 4
+    if pairs > 256:
+        # single waves, two to four to a SIMD, so that the launch has no rounds of whole blocks (four-wave blocks,
+        # one to a compute unit, take 49 us at 264 pairs against 30 us at 256); up to 576 pairs cut in two
+        return 1, (2 if pairs <= 576 and tiles > 16 else 1)
+    if pairs == 256:
+        return (4 if tiles > 16 else 1), 1
+    splits = min(16, max(1, 512 // pairs), tiles)
+    if tiles > 8 * splits:
+        splits = min(16, max(1, 1024 // pairs), tiles)
+    waves = 4 if (tiles > 4 * splits and pairs * splits * 4 <= 1024) else 1
     return waves, splits
 
 
