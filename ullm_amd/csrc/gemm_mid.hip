@@ -127,8 +127,7 @@ gemm_partial_sums_kernel(const bf16_t* __restrict__ X, int ldx, const bf16_t* __
 
 // Slices of K for a matrix [N, K]: as many as give at most one block per compute unit (256 on this
 // part), so that all blocks run side by side: one more slice, and the blocks left over for a second
-// round cost half as much again (down projection of Qwen3-14B at 256 rows: 72 us with 6 slices = 240
-// blocks, 107 us with 7 = 280).  Every slice is a multiple of 64 and at least 256 values long.  A
+// round cost half as much again.  Every slice is a multiple of 64 and at least 256 values long.  A
 // function of the matrix alone, so that the order of the sums does not depend on the batch.
 extern "C" int ullm_gemm_partial_sums_slices(int N, int K) {
   if (N <= 0 || K <= 0) return 0;

@@ -128,8 +128,7 @@ __device__ __forceinline__ void skinny_finish(f32x4_t (&acc)[NT][MT], RedT& red,
 // c ^ ((r >> 1) & 7), which keeps both the 16-byte writes and the 16-byte reads of the hardware's lane
 // groups on different banks.  No barrier in the loop: a wave only reads what it wrote.
 // (Loading the operands straight from memory in the matrix layout, 64 bytes of each of 16 rows per
-// instruction and of X as many rows as the batch has, was slower the more rows X had: 92 against 80 us
-// for the four projections of a Qwen3-8B layer at 8 rows, 105 against 83 us at 16.)
+// instruction and of X as many rows as the batch has, was slower the more rows X had.)
 // NORMX: X is float32 and gain [K] float32, see above; else X is bfloat16.
 // XH: 8-row halves of a tile of X that are fetched: 1 for M <= 8 (then MT = 1), where the other half
 // stays zero in shared memory and costs neither loads nor the registers that hold them in flight
@@ -359,15 +358,13 @@ extern "C" int ullm_gemm_skinny(const void* X, int ldx, const void* W, int ldw, 
   else if (tiles16 >= 4096) nt = mt >= 2 ? 4 : 2;
   else if (tiles16 >= 1024 && mt >= 2) nt = 2;
   // with the norm folded in, a tile of X costs a wave as much as a tile of W: two tiles of W per tile of X
-  // (projection to q|k|v of Qwen3-8B at 8 rows: 15.6 us against 16.5)
   if (gain && force_nt <= 0) nt = 2;
   if (epi == EPI_SILU) nt = (force_nt == 4 || mt >= 4) ? 4 : 2;   // gate and up tiles come in pairs
   if (nt != 1 && nt != 2 && nt != 4) return ULLM_ERR_UNSUPPORTED;
   if (nt == 4 && mt == 1) nt = 2;                       // not instantiated
   // Columns of the result per block.  Up to 16 rows of X, a matrix that fills the chip is spread evenly over
   // the compute units; for store and add that may take two tiles of W a block of which only a part is used
-  // (5120 columns: 256 blocks of 20 instead of 320 of 16; down projection of Qwen3-32B at 8 rows 63.9 -> 50.4 us,
-  // of Qwen3-14B 44.1 -> 34.6 us; q|k|v of Qwen3-8B, 6144 columns in 256 blocks of 24, 14.8 -> 14.0 us).
+  // (5120 columns: 256 blocks of 20 instead of 320 of 16, which would leave most units idle in a second round).
   int rows = 16 * (epi == EPI_SILU ? nt / 2 : nt);
   const int units = skinny_compute_units();
   if (force_rows <= 0 && mt == 1 && N >= 16 * units) {
@@ -385,7 +382,7 @@ extern "C" int ullm_gemm_skinny(const void* X, int ldx, const void* W, int ldw, 
     rows = force_rows;
   }
   const int tiles = (N + rows - 1) / rows;
-  // waves per block: 8 tiles of W in flight per block (measured: 8 waves with one tile each, 4 with two),
+  // waves per block: 8 tiles of W in flight per block (8 waves with one tile each, 4 with two),
   // each wave with at least 128 values of K
   const int max_waves = sk_max_waves(mt, nt);
   int waves = 1;

@@ -408,7 +408,7 @@ _MM_TAKES_OUT_DTYPE = "out_dtype" in (torch.mm.__doc__ or "")
 
 
 # 32-bit results over very many columns (the logits head) up to 32 rows: four tiles of W a block, four waves,
-# 235-256 us against the library's 270-281 us for Qwen3's 151 936 x 4096 head at 17 to 32 rows
+# ahead of the library there
 WIDE_HEAD_SKINNY_MAX_ROWS, WIDE_HEAD_MIN_COLUMNS = 32, 65536
 
 

@@ -20,8 +20,8 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
     return ops.gemm_bf16(x, weight, bias, out_dtype=out_dtype)
 
 
-# Rows up to which folding the norm into the product pays: 37.6 against 39.8 us for gate|up of Qwen3-8B
-# and 15.6 against 16.5 us for q|k|v at 8 rows in a graph; at 16 rows 42.7 against 40.3 and 18.4 against 18.7.
+# Rows up to which folding the norm into the product pays: beyond, the float32 rows of X cost every block more
+# registers and loads than the saved launch is worth.
 NORM_FOLDED_MAX_ROWS = 8
 
 
@@ -55,8 +55,8 @@ def can_fuse(residual: torch.Tensor, dtype: torch.dtype, *weights: torch.Tensor)
 
 
 STACKED_MIN_ROWS, STACKED_MAX_ROWS = 17, 256
-# smallest matrix (elements) that goes this way: below, the stack the norm has to read outweighs the matrix
-# (Qwen3-0.6B's projections, 2-3 M elements: its 256-request workload ran 2% slower with stacks)
+# smallest matrix (elements) that goes this way: below (Qwen3-0.6B's projections, 2-3 M elements), the stack the
+# norm has to read outweighs the matrix
 STACKED_MIN_WEIGHT = 8 << 20
 
 
@@ -64,10 +64,8 @@ def linear_into_stream(x: torch.Tensor, weight: torch.Tensor, ctx) -> torch.Tens
     """The last projection of a mixer or feed-forward, whose result the next norm adds to the residual
     stream.  For 17 to 256 rows in bfloat16, where the model's norms add stacks, it is a stack of
     float32 partial sums over slices of the inner dimension (the slices fill the chip, the norm adds
-    them in order); otherwise the plain product.  Measured against the library product at these
-    shapes: down projection of Qwen3-8B / 14B / 32B at 128 rows 28 / 46 / 68 us against 63 / 147 /
-    180 us, at 256 rows 41 / 72 / 103 us against 51 / 223 / 262 us; output projection at 128 rows
-    14 / 18 / 24 us against 21 / 26 / 37 us, at 256 rows 20 / 27 / 36 us against 20 / 45 / 69 us."""
+    them in order); otherwise the plain product.  For few long rows the library's choice of kernel
+    is two to five times off the memory roofline at these row counts."""
     if (ctx.stacked_branches and x.dtype == torch.bfloat16 and STACKED_MIN_ROWS <= x.shape[0] <= STACKED_MAX_ROWS
             and weight.numel() >= STACKED_MIN_WEIGHT and ops.gemm_partial_sums_supports(x, weight)):
         return ops.gemm_partial_sums(x, weight)
