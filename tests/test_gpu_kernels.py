@@ -454,6 +454,102 @@ def test_attention_on_the_matrix_cores(ops, case):
             break
 
 
+FUSED_CASES = [dict(nq=32, nkv=8, hd=128, P=16, lens=[1153, 31, 32, 33, 1], window=0, norm=True, rope=True),
+               dict(nq=8, nkv=2, hd=64, P=16, lens=[300, 40, 9, 17, 48], window=50, norm=True, rope=True),
+               dict(nq=40, nkv=2, hd=64, P=32, lens=[130, 97], window=0, norm=False, rope=True),      # 20 heads per kv head
+               dict(nq=6, nkv=2, hd=256, P=16, lens=[77, 160], window=0, norm=True, rope=False),
+               dict(nq=4, nkv=1, hd=128, P=48, lens=[1200, 64, 49], window=0, norm=False, rope=False)]
+
+
+@pytest.mark.parametrize("case", FUSED_CASES)
+def test_decode_attention_with_norm_rotation_and_cache_write_folded_in(ops, case):
+    """A step of single new tokens through one kernel: against the plain formulas, and against the two
+    kernels it stands for (the cache it leaves must be the one they leave).  The last entry of the batch is
+    padding as a captured graph has it: position 0, no page; nothing may be written for it."""
+    torch.manual_seed(12)
+    dtype = torch.bfloat16
+    nq, nkv, hd, P, window = (case[k] for k in ("nq", "nkv", "hd", "P", "window"))
+    eps, theta, scale = 1e-5, 5000.0, hd ** -0.5
+    rot, style = (hd, 1) if case["rope"] else (0, 0)
+    assert ops.attention_decode_fused_supports(dtype, hd, P, nq, nkv, rot, style)
+    assert not ops.attention_decode_fused_supports(dtype, hd, P, nq, nkv, hd // 2, 1)      # part of the head rotated
+    assert not ops.attention_decode_fused_supports(dtype, hd, P, nq, nkv, hd, 2)           # adjacent pairs
+    assert not ops.attention_decode_fused_supports(dtype, 96, P, 4, 4, 96, 1)
+    rnd = lambda *s: torch.randn(*s).to(dtype).float()   # noqa: E731
+    lens = case["lens"]
+    B = len(lens) + 1
+    # the cache so far: S - 1 keys per request; the page of the new key exists, its row is unwritten (NaN)
+    ks = [rnd(S, nkv, hd) for S in lens]
+    vs = [rnd(S, nkv, hd) for S in lens]
+    k_pool, v_pool, tables = paged_cache(ks, vs, P, dtype, DEV)
+    for b, S in enumerate(lens):
+        page, row = tables[b][(S - 1) // P], (S - 1) % P
+        k_pool[page, :, row] = float("nan")
+        v_pool[page, :, :, row] = float("nan")
+    positions = torch.tensor([S - 1 for S in lens] + [0], dtype=torch.int32, device=DEV)
+    entry = torch.arange(B, dtype=torch.int32, device=DEV)
+    bt = table_tensor(tables + [[]], DEV)
+    qkv = rnd(B, (nq + 2 * nkv) * hd)
+    qg = (1 + 0.2 * torch.randn(hd)) if case["norm"] else None
+    kg = (1 + 0.2 * torch.randn(hd)) if case["norm"] else None
+    table = None
+    if case["rope"]:
+        inv = 1.0 / (theta ** (torch.arange(0, rot, 2, dtype=torch.float32) / rot))
+        ang = torch.arange(max(lens) + 3, dtype=torch.float32)[:, None] * inv[None]
+        table = torch.cat((ang.cos(), ang.sin()), -1).contiguous().to(DEV)
+    dev = lambda t: None if t is None else t.to(DEV)     # noqa: E731
+    order = sorted(range(B), key=lambda b: -int(positions[b]))      # longest first, as the engine lists them
+    dec = torch.tensor(order, dtype=torch.int32, device=DEV)
+    max_kv = max(lens)
+    # the plain formulas
+    x = qkv[:len(lens)]
+    q = x[:, :nq * hd].view(-1, nq, hd)
+    k = x[:, nq * hd:(nq + nkv) * hd].view(-1, nkv, hd)
+    v = x[:, (nq + nkv) * hd:].view(-1, nkv, hd)
+    if case["norm"]:
+        q, k = plain.rms_norm(q, qg, eps), plain.rms_norm(k, kg, eps)
+    if case["rope"]:
+        cos, sin = plain.rope_cos_sin(positions[:len(lens)].cpu(), rot, theta)
+        q, k = plain.apply_rope_concat_layout(q, cos, sin), plain.apply_rope_concat_layout(k, cos, sin)
+    k, q = k.to(dtype).float(), q.to(dtype).float()
+    full_k = [torch.cat((ks[b][:S - 1], k[b:b + 1])) for b, S in enumerate(lens)]
+    full_v = [torch.cat((vs[b][:S - 1], v[b:b + 1])) for b, S in enumerate(lens)]
+    want = reference_attention([q[b:b + 1] for b in range(len(lens))], full_k, full_v, scale, window).reshape(-1, nq * hd)
+    # the two kernels
+    k_two, v_two = k_pool.clone(), v_pool.clone()
+    q_two = torch.empty(B, nq * hd, dtype=dtype, device=DEV)
+    ops.qk_norm_rope_write(qkv.to(DEV, dtype), q_two, dev(qg), dev(kg), eps, table, rot, style, positions, entry, bt,
+                           k_two, v_two, P, nq, nkv, hd, write_kv=True)
+    out_two = torch.zeros(B, nq * hd, dtype=dtype, device=DEV)
+    ops.attention_decode_mfma(q_two, out_two, k_two, v_two, dec, B, positions, entry, bt, P, nq, nkv, hd, scale, window, max_kv)
+    for splits, waves in ((0, 0), (1, 1), (1, 4), (2, 8), (3, 4), (7, 1), (16, 1)):
+        k_one, v_one = k_pool.clone(), v_pool.clone()
+        out = torch.full((B, nq * hd), float("nan"), dtype=dtype, device=DEV)
+        ops.attention_decode_fused(qkv.to(DEV, dtype), out, dev(qg), dev(kg), eps, table, rot, style, k_one, v_one, dec, B,
+                                   positions, entry, bt, P, nq, nkv, hd, scale, window, max_kv, write_kv=True,
+                                   splits=splits, waves=waves)
+        got = out[:len(lens)].float().cpu()
+        assert not torch.isnan(got).any(), (splits, waves)
+        assert (got - want).abs().max() <= tol(dtype, want), (splits, waves)
+        assert (got - out_two[:len(lens)].float().cpu()).abs().max() <= 0.25 * tol(dtype, want), (splits, waves)
+        # the cache: the same rows written, keys within a rounding of the other kernel's, values bit for bit
+        assert torch.equal(torch.isnan(k_one), torch.isnan(k_two)) and torch.equal(torch.isnan(v_one), torch.isnan(v_two))
+        assert torch.equal(torch.nan_to_num(v_one.float()), torch.nan_to_num(v_two.float()))
+        dk = (torch.nan_to_num(k_one.float()) - torch.nan_to_num(k_two.float())).abs()
+        assert float(dk.max()) <= 2 ** -7 * float(torch.nan_to_num(k_two.float()).abs().max()), (splits, waves)
+        assert float((dk > 0).float().mean()) < 1e-3
+        for b, S in enumerate(lens):
+            page, row = tables[b][(S - 1) // P], (S - 1) % P
+            assert (k_one[page, :, row].float().cpu() - k[b]).abs().max() <= tol(dtype, k)
+    # a layer that reads a cache another layer wrote: nothing is written, the cache's own newest key is used
+    k_read, v_read = k_two.clone(), v_two.clone()
+    out = torch.full((B, nq * hd), float("nan"), dtype=dtype, device=DEV)
+    ops.attention_decode_fused(qkv.to(DEV, dtype), out, dev(qg), dev(kg), eps, table, rot, style, k_read, v_read, dec, B,
+                               positions, entry, bt, P, nq, nkv, hd, scale, window, max_kv, write_kv=False)
+    assert torch.equal(torch.nan_to_num(k_read.float()), torch.nan_to_num(k_two.float()))
+    assert (out[:len(lens)].float().cpu() - want).abs().max() <= tol(dtype, want)
+
+
 def test_matrix_core_attention_finds_one_far_key_at_every_edge(ops):
     torch.manual_seed(9)
     dtype = torch.bfloat16

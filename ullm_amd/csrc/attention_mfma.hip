@@ -97,14 +97,18 @@ __device__ __forceinline__ void load_tile(KVTile<NQK>& t, int key0, const PageWi
 
 // Scores, softmax update and value product for one tile held in registers, for NG groups of 16
 // columns that share the tile (each group has its own queries, limits, maximum, sum and output).
-template <int NQK, int NG>
+// `own` (or null): the key (head_dim values) and value (head_dim values) of the token itself, at
+// position max_hi, in shared memory.  The tile that holds that position takes them from there instead
+// of from the cache, where the same kernel is only just writing them.
+template <int NQK, int NG, bool OWN>
 __device__ __forceinline__ void process_tile(const KVTile<NQK>& cur, int key0, const Pack8 (&qreg)[NG][NQK],
                                              const int (&col_lo)[NG], const int (&col_hi)[NG], int max_hi,
                                              float scale_log2e, f32x4_t (&acc)[NG][2 * NQK], float (&m)[NG],
-                                             float (&l)[NG]) {
+                                             float (&l)[NG], const bf16_t* own) {
+  constexpr int HD = 32 * NQK;
   const int lane = threadIdx.x & 63, g = lane >> 4;
   const bool edge = key0 + 32 > max_hi + 1;     // some keys of the tile hold no written data
-  Pack8 vals[2 * NQK];
+  Pack8 vals[2 * NQK], keys[2][NQK];
 #pragma unroll
   for (int n = 0; n < 2 * NQK; ++n) {
     vals[n].u2[0] = cur.v[n][0];
@@ -115,6 +119,35 @@ __device__ __forceinline__ void process_tile(const KVTile<NQK>& cur, int key0, c
         if (key0 + 16 * (j >> 2) + 4 * g + (j & 3) > max_hi) vals[n].h[j] = 0;
     }
   }
+  const Pack8 (*kp)[NQK] = cur.k;
+  if constexpr (OWN) {
+#pragma unroll
+    for (int sb = 0; sb < 2; ++sb)
+#pragma unroll
+      for (int ch = 0; ch < NQK; ++ch) keys[sb][ch] = cur.k[sb][ch];
+    kp = keys;
+  }
+  if (OWN && own && key0 + 32 > max_hi) {
+    const int c = lane & 15;
+    const int at = max_hi - key0;               // 0 .. 31: sub-block at >> 4, row at & 15, which lane group at >> 2 & 3 holds
+    if (c == (at & 15)) {
+#pragma unroll
+      for (int ch = 0; ch < NQK; ++ch) {
+        const uint4 k = ld16(own + 32 * ch + 8 * g);
+        if (at < 16) keys[0][ch].u4 = k;
+        else keys[1][ch].u4 = k;
+      }
+    }
+    if (g == ((at >> 2) & 3)) {
+#pragma unroll
+      for (int n = 0; n < 2 * NQK; ++n) {
+        const bf16_t v = own[HD + 16 * n + c];
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          if (j == 4 * (at >> 4) + (at & 3)) vals[n].h[j] = v;
+      }
+    }
+  }
 #pragma unroll
   for (int q = 0; q < NG; ++q) {
     f32x4_t s[2];
@@ -123,7 +156,7 @@ __device__ __forceinline__ void process_tile(const KVTile<NQK>& cur, int key0, c
       s[sb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int ch = 0; ch < NQK; ++ch)
-        s[sb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.k[sb][ch].v, qreg[q][ch].v, s[sb], 0, 0, 0);
+        s[sb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kp[sb][ch].v, qreg[q][ch].v, s[sb], 0, 0, 0);
     }
     // scores of keys key0 + 16 sb + 4 g + r for this lane's column; mask, running maximum
     float tile_max = NEG_BIG;
@@ -167,7 +200,10 @@ __device__ __forceinline__ void process_tile(const KVTile<NQK>& cur, int key0, c
 }
 
 // The work of one wave.  NQK = head_dim / 32; NG groups of 16 columns share every tile.
-//   col_q[q]      : pointer to this lane's column's query row in group q (null if padding)
+//   queries       : fetch() queues the loads of what the queries are made from, before the loads of the
+//                   first tiles; finish(qreg), behind them, fills qreg[q][ch] = this lane's column's
+//                   query in group q, dims 32 ch + 8 g .. +8 (zeros if padding), while the tiles are on
+//                   their way, and returns where the token's own key and value lie (or null)
 //   col_lo/hi[q]  : first and last key the column may see (hi < lo for padding)
 //   key_begin/key_end : the wave's key range [begin, end), begin a multiple of 32
 //   max_hi     : largest key position that holds written data for this request
@@ -175,12 +211,11 @@ __device__ __forceinline__ void process_tile(const KVTile<NQK>& cur, int key0, c
 // lane's share of the sum; the four lanes of a column add up to the column's sum).
 // Page ids are fetched 1024 keys at a time; the loads of the next DEPTH (1 or 2) tiles are in flight
 // while the current one is worked on.
-template <int NQK, int NG, int DEPTH>
+template <int NQK, int NG, int DEPTH, bool OWN, class Queries>
 __device__ __forceinline__ void attend_range(
-    const bf16_t* const (&col_q)[NG], const int (&col_lo)[NG], const int (&col_hi)[NG], int key_begin, int key_end,
+    Queries& queries, const int (&col_lo)[NG], const int (&col_hi)[NG], int key_begin, int key_end,
     int max_hi, const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool, const int* __restrict__ bt,
     int page_size, int nkv, int kvh, float scale_log2e, f32x4_t (&acc)[NG][2 * NQK], float (&m)[NG], float (&l)[NG]) {
-  const int lane = threadIdx.x & 63, g = lane >> 4;
 #pragma unroll
   for (int q = 0; q < NG; ++q) {
 #pragma unroll
@@ -189,46 +224,45 @@ __device__ __forceinline__ void attend_range(
     l[q] = 0.f;
   }
   if (key_begin >= key_end) return;
+  queries.fetch();
   PageWindow pw = load_pages(key_begin, key_end, bt, page_size);
   Pack8 qreg[NG][NQK];
-#pragma unroll
-  for (int q = 0; q < NG; ++q)
-#pragma unroll
-    for (int ch = 0; ch < NQK; ++ch) {
-      if (col_q[q]) qreg[q][ch].u4 = *reinterpret_cast<const uint4*>(col_q[q] + 32 * ch + 8 * g);
-      else qreg[q][ch].u4 = make_uint4(0, 0, 0, 0);
-    }
+  const bf16_t* own = nullptr;
 #define TILE_LOAD(T, K0) load_tile<NQK>(T, K0, pw, k_pool, v_pool, page_size, nkv, kvh)
-#define TILE_WORK(T, K0) process_tile<NQK, NG>(T, K0, qreg, col_lo, col_hi, max_hi, scale_log2e, acc, m, l)
-  for (int base = key_begin; base < key_end; base += 1024) {
-    if (base != key_begin) pw = load_pages(base, key_end, bt, page_size);
-    const int stop = base + 1024 < key_end ? base + 1024 : key_end;
+#define TILE_WORK(T, K0) process_tile<NQK, NG, OWN>(T, K0, qreg, col_lo, col_hi, max_hi, scale_log2e, acc, m, l, own)
+  KVTile<NQK> t0, t1, t2;                                 // DEPTH 1 takes two of them in turns, DEPTH 2 all three
+  int base = key_begin, stop = base + 1024 < key_end ? base + 1024 : key_end;
+  TILE_LOAD(t0, base);
+  if (DEPTH == 2 && base + 32 < stop) TILE_LOAD(t1, base + 32);
+  own = queries.finish(qreg);
+  for (;;) {
     if (DEPTH == 1) {
-      KVTile<NQK> a, b;
-      TILE_LOAD(a, base);
       for (int key0 = base; key0 < stop; key0 += 64) {
-        if (key0 + 32 < stop) TILE_LOAD(b, key0 + 32);
-        TILE_WORK(a, key0);
+        if (key0 + 32 < stop) TILE_LOAD(t1, key0 + 32);
+        TILE_WORK(t0, key0);
         if (key0 + 32 >= stop) break;
-        if (key0 + 64 < stop) TILE_LOAD(a, key0 + 64);
-        TILE_WORK(b, key0 + 32);
+        if (key0 + 64 < stop) TILE_LOAD(t0, key0 + 64);
+        TILE_WORK(t1, key0 + 32);
       }
-      continue;
+    } else {
+      // three buffers in rotation: while tile i is worked on, tiles i+1 and i+2 are loading
+      for (int key0 = base; key0 < stop; key0 += 96) {
+        if (key0 + 64 < stop) TILE_LOAD(t2, key0 + 64);
+        TILE_WORK(t0, key0);
+        if (key0 + 32 >= stop) break;
+        if (key0 + 96 < stop) TILE_LOAD(t0, key0 + 96);
+        TILE_WORK(t1, key0 + 32);
+        if (key0 + 64 >= stop) break;
+        if (key0 + 128 < stop) TILE_LOAD(t1, key0 + 128);
+        TILE_WORK(t2, key0 + 64);
+      }
     }
-    KVTile<NQK> t0, t1, t2;
+    base += 1024;
+    if (base >= key_end) break;
+    pw = load_pages(base, key_end, bt, page_size);        // the next 1024 keys' page ids
+    stop = base + 1024 < key_end ? base + 1024 : key_end;
     TILE_LOAD(t0, base);
-    if (base + 32 < stop) TILE_LOAD(t1, base + 32);
-    // three buffers in rotation: while tile i is worked on, tiles i+1 and i+2 are loading
-    for (int key0 = base; key0 < stop; key0 += 96) {
-      if (key0 + 64 < stop) TILE_LOAD(t2, key0 + 64);
-      TILE_WORK(t0, key0);
-      if (key0 + 32 >= stop) break;
-      if (key0 + 96 < stop) TILE_LOAD(t0, key0 + 96);
-      TILE_WORK(t1, key0 + 32);
-      if (key0 + 64 >= stop) break;
-      if (key0 + 128 < stop) TILE_LOAD(t1, key0 + 128);
-      TILE_WORK(t2, key0 + 64);
-    }
+    if (DEPTH == 2 && base + 32 < stop) TILE_LOAD(t1, base + 32);
   }
 #undef TILE_LOAD
 #undef TILE_WORK
@@ -286,17 +320,172 @@ __device__ __forceinline__ void merge_waves(f32x4_t (&acc)[NG][2 * NQK], float (
 // a second, small kernel adds the splits in split order.  (A single kernel in which the last block to
 // finish does that sum needs a device-wide memory fence per block, which on a part with one L2 per
 // XCD costs far more than the second launch.)
-template <int NQK, int WAVES>
+//
+// FUSE: `q` is the row of the fused projection q | k | v, not yet normed or rotated.  Every wave norms
+// and rotates its queries itself (a few hundred operations on values it loads anyway), and the one wave
+// whose keys end at the token's own position does the same for the token's key, writes key and value
+// to the cache for the steps to come, and hands them to its last tile through shared memory: a decode
+// step then needs no kernel of its own for norm, rotation and cache write.
+struct DecodeFuse {
+  const float* q_gain;    // per-head norm gains [head_dim], or null: no norm
+  const float* k_gain;
+  float eps;
+  const float* cos_sin;   // [table_rows, head_dim]: cos of the head_dim / 2 angles, then sin; or null: no rotation
+  int table_rows;
+  bf16_t* k_pool;         // the pools again, writable; null: this layer reads a cache that another layer writes
+  bf16_t* v_pool;
+};
+
+// Queries as the projection left them (bfloat16, normed and rotated by an earlier kernel).
+template <int NQK>
+struct ReadyQueries {
+  const bf16_t* row;                    // the column's head, or null for a padding column
+  int g;
+  Pack8 raw[NQK];
+  __device__ __forceinline__ void fetch() {
+#pragma unroll
+    for (int ch = 0; ch < NQK; ++ch) {
+      if (row) raw[ch].u4 = *reinterpret_cast<const uint4*>(row + 32 * ch + 8 * g);
+      else raw[ch].u4 = make_uint4(0, 0, 0, 0);
+    }
+  }
+  __device__ __forceinline__ const bf16_t* finish(Pack8 (&qreg)[1][NQK]) {
+#pragma unroll
+    for (int ch = 0; ch < NQK; ++ch) qreg[0][ch] = raw[ch];
+    return nullptr;
+  }
+};
+
+// Queries, and for one wave the token's own key and value, from the raw projection row.
+template <int NQK>
+struct RawQueries {
+  static constexpr int HD = 32 * NQK;
+  const DecodeFuse& fuse;
+  const bf16_t* q_head;                 // the column's query head in the projection row
+  const bf16_t* k_head;                 // the token's key and value heads there, if this wave's keys end with the
+  const bf16_t* v_head;                 //   token itself and the layer writes its cache; else null
+  const float* cs;                      // the position's row of the table, or null
+  bf16_t* k_dst;                        // where key and value go in the cache (null: nowhere)
+  bf16_t* v_dst;
+  int page_size, g, c;
+  bf16_t* own_kv;                       // shared memory: head_dim values of the key, then of the value
+  Pack8 q_raw[NQK], k_raw[NQK];
+  bf16_t v_raw[2 * NQK];
+  float q_gain[NQK][8], k_gain[NQK][8], cos_[NQK / 2][8], sin_[NQK / 2][8];
+
+  __device__ __forceinline__ static void load8(float (&to)[8], const float* from) {
+    const float4 a = *reinterpret_cast<const float4*>(from), b = *reinterpret_cast<const float4*>(from + 4);
+    to[0] = a.x; to[1] = a.y; to[2] = a.z; to[3] = a.w; to[4] = b.x; to[5] = b.y; to[6] = b.z; to[7] = b.w;
+  }
+  __device__ __forceinline__ void fetch() {
+#pragma unroll
+    for (int ch = 0; ch < NQK; ++ch) q_raw[ch].u4 = ld16(q_head + 32 * ch + 8 * g);
+    if (k_head) {
+#pragma unroll
+      for (int ch = 0; ch < NQK; ++ch) k_raw[ch].u4 = ld16(k_head + 32 * ch + 8 * g);
+#pragma unroll
+      for (int n = 0; n < 2 * NQK; ++n) v_raw[n] = v_head[16 * n + c];
+    }
+    if (cs) {
+#pragma unroll
+      for (int ch = 0; ch < NQK / 2; ++ch) {
+        load8(cos_[ch], cs + 32 * ch + 8 * g);
+        load8(sin_[ch], cs + HD / 2 + 32 * ch + 8 * g);
+      }
+    }
+    if (fuse.q_gain) {
+#pragma unroll
+      for (int ch = 0; ch < NQK; ++ch) load8(q_gain[ch], fuse.q_gain + 32 * ch + 8 * g);
+    }
+    if (fuse.k_gain && k_head) {
+#pragma unroll
+      for (int ch = 0; ch < NQK; ++ch) load8(k_gain[ch], fuse.k_gain + 32 * ch + 8 * g);
+    }
+  }
+  // Per-head norm and half-split rotation of a head held by the four lanes of a column: chunk ch,
+  // element j = dim 32 ch + 8 g + j.  The same formulas as ullm_qk_norm_rope_write (which serves prompt
+  // portions), so that a key is the same whichever of the two wrote it; the partner of a dim in the
+  // first half is the dim head_dim / 2 further on, which for head sizes of 64, 128 and 256 lies in the
+  // same lane.
+  __device__ __forceinline__ void norm_rotate(const Pack8 (&raw)[NQK], const float (*gain)[8], Pack8 (&to)[NQK]) const {
+    static_assert(NQK % 2 == 0, "the partner dim must lie in the same lane");
+    float x[NQK][8];
+#pragma unroll
+    for (int ch = 0; ch < NQK; ++ch)
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        x[ch][2 * w] = __uint_as_float(raw[ch].w[w] << 16);
+        x[ch][2 * w + 1] = __uint_as_float(raw[ch].w[w] & 0xffff0000u);
+      }
+    if (gain) {
+      float ss = 0.f;
+#pragma unroll
+      for (int ch = 0; ch < NQK; ++ch)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) ss += x[ch][j] * x[ch][j];
+      ss += __shfl_xor(ss, 16, 64);
+      ss += __shfl_xor(ss, 32, 64);
+      const float rs = rsqrtf(ss / (float)HD + fuse.eps);
+#pragma unroll
+      for (int ch = 0; ch < NQK; ++ch)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) x[ch][j] = (x[ch][j] * rs) * gain[ch][j];
+    }
+    if (cs) {
+#pragma unroll
+      for (int ch = 0; ch < NQK / 2; ++ch)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const float a = x[ch][j], b = x[ch + NQK / 2][j];
+          x[ch][j] = a * cos_[ch][j] - b * sin_[ch][j];
+          x[ch + NQK / 2][j] = b * cos_[ch][j] + a * sin_[ch][j];
+        }
+    }
+#pragma unroll
+    for (int ch = 0; ch < NQK; ++ch)
+#pragma unroll
+      for (int w = 0; w < 4; ++w) to[ch].w[w] = pack2_bf16(x[ch][2 * w], x[ch][2 * w + 1]);
+  }
+  __device__ __forceinline__ const bf16_t* finish(Pack8 (&qreg)[1][NQK]) {
+    norm_rotate(q_raw, fuse.q_gain ? q_gain : nullptr, qreg[0]);
+    if (!k_head) return nullptr;
+    // only one wave of the block gets here, so the one place in shared memory is its own
+    Pack8 key[NQK];
+    norm_rotate(k_raw, fuse.k_gain ? k_gain : nullptr, key);
+    if (c == 0) {
+#pragma unroll
+      for (int ch = 0; ch < NQK; ++ch) {
+        st16(own_kv + 32 * ch + 8 * g, key[ch].u4);
+        if (k_dst) st16(k_dst + 32 * ch + 8 * g, key[ch].u4);
+      }
+    }
+    if (g == 0) {
+#pragma unroll
+      for (int n = 0; n < 2 * NQK; ++n) {
+        own_kv[HD + 16 * n + c] = v_raw[n];
+        if (v_dst) v_dst[(size_t)(16 * n + c) * page_size] = v_raw[n];
+      }
+    }
+    // the lanes of this wave read each other's values from there at the last tile
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    return own_kv;
+  }
+};
+
+template <int NQK, int WAVES, bool FUSE>
 __global__ void __launch_bounds__(64 * WAVES)
 attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
                         const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
                         const int* __restrict__ token_list, const int* __restrict__ positions,
                         const int* __restrict__ token_entry, const int* __restrict__ block_table,
                         int bt_stride, int page_size, int nq, int nkv, float scale_log2e, int window,
-                        int num_splits, float* __restrict__ part) {
+                        int num_splits, float* __restrict__ part, DecodeFuse fuse) {
   constexpr int HD = 32 * NQK;
   constexpr int ROW = HD + 4;                       // output dims, then maximum and sum (rows stay 16-byte aligned)
   __shared__ float merge[(WAVES > 1 ? WAVES / 2 : 1) * (WAVES > 1 ? (8 * NQK + 2) * 64 : 1)];   // [writer][value][lane]: conflict-free
+  __shared__ __attribute__((aligned(16))) bf16_t own_kv[FUSE ? 2 * HD : 8];   // the token's own key, then its value
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g = lane >> 4, c = lane & 15;
   const int split = blockIdx.x;
   const int G = nq / nkv;
@@ -317,11 +506,31 @@ attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __re
   f32x4_t accs[1][2 * NQK];
   float ms[1], ls[1];
   {
-    const bf16_t* const cq[1] = {col_ok ? q + (size_t)t * q_stride + (size_t)head * HD : nullptr};
+    const int* const bt = block_table + (size_t)token_entry[t] * bt_stride;
+    const bf16_t* const row = q + (size_t)t * q_stride;
     const int clo[1] = {lo}, chi[1] = {col_ok ? pos : -1};
-    attend_range<NQK, 1, (WAVES > 4 || NQK >= 8 ? 1 : 2)>(cq, clo, chi, begin, end, pos, k_pool, v_pool,
-                                              block_table + (size_t)token_entry[t] * bt_stride, page_size, nkv, kvh,
-                                              scale_log2e, accs, ms, ls);
+    constexpr int DEPTH = WAVES > 4 || NQK >= 8 ? 1 : 2;
+    if constexpr (FUSE) {
+      const bool has_own = fuse.k_pool && begin < end && end == pos + 1;
+      // no page (a padding entry), no write, as in the kernel for prompt portions; one block per kv head writes
+      const int page = has_own && cg == 0 ? bt[pos / page_size] : -1;
+      const int off = pos % page_size;
+      RawQueries<NQK> queries{
+          fuse,
+          row + (size_t)(col_ok ? head : kvh * G) * HD,      // a padding column takes the group's first head: never stored
+          has_own ? row + (size_t)(nq + kvh) * HD : nullptr,
+          has_own ? row + (size_t)(nq + nkv + kvh) * HD : nullptr,
+          fuse.cos_sin ? fuse.cos_sin + (size_t)(pos < fuse.table_rows ? pos : fuse.table_rows - 1) * HD : nullptr,
+          page >= 0 ? fuse.k_pool + (((size_t)page * nkv + kvh) * page_size + off) * HD : nullptr,
+          page >= 0 ? fuse.v_pool + ((size_t)page * nkv + kvh) * HD * page_size + off : nullptr,
+          page_size, g, c, own_kv};
+      attend_range<NQK, 1, DEPTH, true>(queries, clo, chi, begin, end, pos, k_pool, v_pool, bt, page_size, nkv, kvh,
+                                        scale_log2e, accs, ms, ls);
+    } else {
+      ReadyQueries<NQK> queries{col_ok ? row + (size_t)head * HD : nullptr, g};
+      attend_range<NQK, 1, DEPTH, false>(queries, clo, chi, begin, end, pos, k_pool, v_pool, bt, page_size, nkv, kvh,
+                                         scale_log2e, accs, ms, ls);
+    }
   }
   merge_waves<NQK, 1, WAVES>(accs, ms, ls, merge);
   f32x4_t (&acc)[2 * NQK] = accs[0];
@@ -842,7 +1051,7 @@ static int decode_launch(
     const void* q, int q_stride, void* out, int out_stride, const void* k_pool, const void* v_pool,
     const int* token_list, int n_items, const int* positions, const int* token_entry,
     const int* block_table, int bt_stride, int page_size, int nq, int nkv, int hd, float scale, int window,
-    int num_splits, int waves, float* workspace, hipStream_t stream) {
+    int num_splits, int waves, float* workspace, hipStream_t stream, const DecodeFuse* fuse = nullptr) {
   if (n_items <= 0) return 0;
   if (!ullm_attention_mfma_supports(hd, page_size, nq, nkv)) return ULLM_ERR_UNSUPPORTED;
   if (waves != 1 && waves != 4 && waves != 8) return ULLM_ERR_UNSUPPORTED;
@@ -853,15 +1062,27 @@ static int decode_launch(
   if (n_items > 65535 || nkv * groups > 65535) return ULLM_ERR_SHAPE;
   const float sl = scale * 1.4426950408889634f;
   dim3 grid(num_splits, nkv * groups, n_items), block(64 * waves);
+  const DecodeFuse f = fuse ? *fuse : DecodeFuse{nullptr, nullptr, 0.f, nullptr, 0, nullptr, nullptr};
 #define ARGS (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool, token_list, \
-    positions, token_entry, block_table, bt_stride, page_size, nq, nkv, sl, window, num_splits, workspace
-#define CALL(N) do {                                                                                        \
-    if (waves == 8) hipLaunchKernelGGL((attention_decode_kernel<N, 8>), grid, block, 0, stream, ARGS);      \
-    else if (waves == 4) hipLaunchKernelGGL((attention_decode_kernel<N, 4>), grid, block, 0, stream, ARGS); \
-    else hipLaunchKernelGGL((attention_decode_kernel<N, 1>), grid, block, 0, stream, ARGS);                 \
+    positions, token_entry, block_table, bt_stride, page_size, nq, nkv, sl, window, num_splits, workspace, f
+#define CALL_AS(N, F) do {                                                                                     \
+    if (waves == 8) hipLaunchKernelGGL((attention_decode_kernel<N, 8, F>), grid, block, 0, stream, ARGS);      \
+    else if (waves == 4) hipLaunchKernelGGL((attention_decode_kernel<N, 4, F>), grid, block, 0, stream, ARGS); \
+    else hipLaunchKernelGGL((attention_decode_kernel<N, 1, F>), grid, block, 0, stream, ARGS);                 \
   } while (0)
-  DISPATCH_NQK(hd, CALL)
+  if (fuse) {
+    switch (hd) {
+      case 64: CALL_AS(2, true); break;
+      case 128: CALL_AS(4, true); break;
+      case 256: CALL_AS(8, true); break;
+      default: return ULLM_ERR_UNSUPPORTED;
+    }
+  } else {
+#define CALL(N) CALL_AS(N, false)
+    DISPATCH_NQK(hd, CALL)
 #undef CALL
+  }
+#undef CALL_AS
 #undef ARGS
   int rc = (int)hipGetLastError();
   if (rc != 0 || num_splits == 1) return rc;
@@ -878,6 +1099,40 @@ extern "C" int ullm_attention_decode(
   return decode_launch(q, q_stride, out, out_stride, k_pool, v_pool, token_list, n_items, positions, token_entry,
                        block_table, bt_stride, page_size, nq, nkv, hd, scale, window, num_splits, waves, workspace,
                        stream);
+}
+
+// Head sizes and position encodings the fused decode step takes: rotation of the whole head in
+// half-split pairs (style 1, rot == hd) or none (style 0 or rot 0), head sizes whose halves are whole
+// 32-dim chunks.
+extern "C" int ullm_attention_decode_fused_supports(int hd, int page_size, int nq, int nkv, int rot, int style) {
+  if (!ullm_attention_mfma_supports(hd, page_size, nq, nkv)) return 0;
+  if (hd != 64 && hd != 128 && hd != 256) return 0;
+  const bool rotates = style != 0 && rot > 0;
+  return !rotates || (style == 1 && rot == hd);
+}
+
+// ullm_attention_decode with the per-head norm, the rotation and the cache write of the step folded in:
+// `qkv` [tokens, (nq + 2 nkv) * hd] is the fused projection as it leaves the matrix product.  q_gain /
+// k_gain float32 [hd] or null (no norm); cos_sin float32 [table_rows, rot] or null; write_kv = 0 for a
+// layer that reads a cache another layer writes (then k and v of the projection are not used).
+// Every item must be the last token of its request so far (its position is the newest key).
+extern "C" int ullm_attention_decode_fused(
+    const void* qkv, int qkv_stride, void* out, int out_stride, void* k_pool, void* v_pool,
+    const int* token_list, int n_items, const int* positions, const int* token_entry,
+    const int* block_table, int bt_stride, int page_size, int nq, int nkv, int hd, float scale, int window,
+    int num_splits, int waves, float* workspace, const float* q_gain, const float* k_gain, float eps,
+    const float* cos_sin, int table_rows, int rot, int style, int write_kv, hipStream_t stream) {
+  if (!ullm_attention_decode_fused_supports(hd, page_size, nq, nkv, rot, style)) return ULLM_ERR_UNSUPPORTED;
+  const bool rotates = style != 0 && rot > 0;
+  if (rotates && (!cos_sin || table_rows <= 0)) return ULLM_ERR_SHAPE;
+  if ((qkv_stride & 7) || ((uintptr_t)qkv & 15) || ((uintptr_t)k_pool & 15) || ((uintptr_t)q_gain & 15) ||
+      ((uintptr_t)k_gain & 15) || ((uintptr_t)cos_sin & 15))
+    return ULLM_ERR_SHAPE;
+  const DecodeFuse f = {q_gain, k_gain, eps, rotates ? cos_sin : nullptr, table_rows,
+                        write_kv ? (bf16_t*)k_pool : nullptr, write_kv ? (bf16_t*)v_pool : nullptr};
+  return decode_launch(qkv, qkv_stride, out, out_stride, k_pool, v_pool, token_list, n_items, positions, token_entry,
+                       block_table, bt_stride, page_size, nq, nkv, hd, scale, window, num_splits, waves, workspace,
+                       stream, &f);
 }
 
 // ------------------------------------------------------------------------------- no allocation

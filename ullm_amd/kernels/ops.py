@@ -508,6 +508,65 @@ def attention_decode_mfma(q, out, k_pool, v_pool, token_list: Optional[torch.Ten
         _c_int(splits), _c_int(waves), _p(ws), _stream()), "attention_decode")
 
 
+def attention_decode_fused_supports(dtype: torch.dtype, hd: int, page_size: int, nq: int, nkv: int,
+                                    rotary_dim: int, style: int) -> bool:
+    """Whether the decode kernel can also do the step's per-head norm, rotation and cache write."""
+    if dtype != torch.bfloat16:
+        return False
+    lib = build.load("attention_mfma")
+    return bool(lib.ullm_attention_decode_fused_supports(_c_int(hd), _c_int(page_size), _c_int(nq), _c_int(nkv),
+                                                         _c_int(rotary_dim), _c_int(style)))
+
+
+def attention_decode_fused(qkv, out, q_gain: Optional[torch.Tensor], k_gain: Optional[torch.Tensor], eps: float,
+                           cos_sin: Optional[torch.Tensor], rotary_dim: int, style: int, k_pool, v_pool,
+                           token_list: Optional[torch.Tensor], n_items: int, positions, token_entry, block_table,
+                           page_size: int, nq: int, nkv: int, hd: int, scale: float, window: int, max_kv: int,
+                           write_kv: bool, splits: int = 0, waves: int = 0) -> None:
+    """``attention_decode_mfma`` for a step in which every item is its request's newest token, with what
+    ``qk_norm_rope_write`` does folded in: ``qkv`` [T, (nq + 2 nkv) * hd] is the fused projection as the
+    matrix product left it; the kernel norms and rotates q and k itself and writes k and v to the cache."""
+    _check_pools(k_pool, v_pool, nkv, page_size, hd, torch.bfloat16)
+    _need(qkv.dtype == torch.bfloat16 and qkv.dim() == 2 and qkv.stride(1) == 1 and qkv.shape[1] == (nq + 2 * nkv) * hd,
+          "qkv must be bfloat16 [T, (nq + 2 nkv) * hd]")
+    _need(out.dtype == torch.bfloat16 and out.stride(1) == 1 and out.shape == (qkv.shape[0], nq * hd), "bad attention output")
+    _i32(positions, "positions")
+    _i32(token_entry, "token_entry")
+    if token_list is not None:
+        _i32(token_list, "token_list", n_items)
+    else:
+        _need(n_items <= qkv.shape[0], "more items than tokens")
+    _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.stride(1) == 1,
+          "block_table must be int32 [B, stride]")
+    _need(-(-max_kv // page_size) <= block_table.shape[1], "block table narrower than the longest context")
+    for gn, nm in ((q_gain, "q_gain"), (k_gain, "k_gain")):
+        if gn is not None:
+            _need(gn.dtype == torch.float32 and gn.numel() == hd and gn.is_contiguous(), f"{nm} must be float32 [hd]")
+    table_rows = 0
+    if style != 0 and rotary_dim > 0:
+        _need(cos_sin is not None and cos_sin.dtype == torch.float32 and cos_sin.dim() == 2
+              and cos_sin.shape[1] == rotary_dim and cos_sin.is_contiguous(),
+              "cos_sin must be float32 [positions, rotary_dim]")
+        table_rows = cos_sin.shape[0]
+    groups = -(-(nq // nkv) // 16)
+    auto_waves, auto_splits = decode_split(n_items, nkv, groups, max_kv, hd)
+    waves = waves or auto_waves
+    if hd == 256 and waves == 8:
+        waves = 4
+    splits = splits or auto_splits
+    lib = build.load("attention_mfma")
+    ws = None
+    if splits > 1:
+        ws = torch.empty(n_items * nq * splits * (hd + 4), dtype=torch.float32, device=qkv.device)
+    _check(lib.ullm_attention_decode_fused(
+        _p(qkv), _c_int(qkv.stride(0)), _p(out), _c_int(out.stride(0)), _p(k_pool), _p(v_pool), _p(token_list),
+        _c_int(n_items), _p(positions), _p(token_entry), _p(block_table), _c_int(block_table.stride(0)),
+        _c_int(page_size), _c_int(nq), _c_int(nkv), _c_int(hd), _c_float(scale), _c_int(window),
+        _c_int(splits), _c_int(waves), _p(ws), _p(q_gain), _p(k_gain), _c_float(eps), _p(cos_sin),
+        _c_int(table_rows), _c_int(rotary_dim), _c_int(style), _c_int(1 if write_kv else 0), _stream()),
+        "attention_decode_fused")
+
+
 PREFILL_TILE = 32      # tokens of one request per prompt tile (two groups of 16 columns for every wave of a block)
 
 

@@ -85,10 +85,20 @@ class GQAttention(Mixer):
         T = qkv.shape[0]
         x = qkv
         group = ctx.groups[cache.group]
-        q = torch.empty((T, self.nq * self.hd), dtype=x.dtype, device=x.device)
         table, rot, style = self.position.kernel_args() if self.position is not None else (None, 0, 0)
+        eps = self.qk_norm_eps if self.qk_norm_eps is not None else 0.0
+        if (ctx.num_decode == T and not ctx.num_tiles and ops.attention_decode_fused_supports(
+                x.dtype, self.hd, group.page_size, self.nq, self.nkv, rot, style)):
+            # a step of single new tokens: norm, rotation and cache write happen inside the attention kernel
+            out = torch.empty((T, self.nq * self.hd), dtype=x.dtype, device=x.device)
+            ops.attention_decode_fused(
+                qkv, out, self.q_gain, self.k_gain, eps, table, rot, style, cache.k_pool, cache.v_pool,
+                ctx.decode_tokens, ctx.num_decode, ctx.positions, ctx.token_entry, group.block_table, group.page_size,
+                self.nq, self.nkv, self.hd, self.scale, self.window, ctx.max_decode_kv, write_kv=cache.owner)
+            return out
+        q = torch.empty((T, self.nq * self.hd), dtype=x.dtype, device=x.device)
         ops.qk_norm_rope_write(
-            qkv, q, self.q_gain, self.k_gain, self.qk_norm_eps if self.qk_norm_eps is not None else 0.0,
+            qkv, q, self.q_gain, self.k_gain, eps,
             table, rot, style, ctx.positions, ctx.token_entry, group.block_table,
             cache.k_pool, cache.v_pool, group.page_size, self.nq, self.nkv, self.hd, write_kv=cache.owner)
         return ops.paged_attention(q, cache.k_pool, cache.v_pool, ctx, group, self.nq, self.nkv, self.hd,
