@@ -17,6 +17,12 @@ from .base import KVNeed, LayerCache, Mixer, PartEnv, PositionEncoding, StepCont
 from .linear import can_fuse, linear, linear_into_stream, linear_of_norm
 
 
+# Up to this many single new tokens a step, the attention kernel norms, rotates and writes the new keys itself.
+# With more, its waves fill the chip and the extra work at each wave's start is no longer hidden behind the
+# others' loads: the kernel of its own, which does it for all tokens at once, is then the faster way.
+FUSED_DECODE_MAX_TOKENS = 64
+
+
 @register_part("mixer", "gqa_attention")
 class GQAttention(Mixer):
     folds_norm = True
@@ -87,8 +93,8 @@ class GQAttention(Mixer):
         group = ctx.groups[cache.group]
         table, rot, style = self.position.kernel_args() if self.position is not None else (None, 0, 0)
         eps = self.qk_norm_eps if self.qk_norm_eps is not None else 0.0
-        if (ctx.num_decode == T and not ctx.num_tiles and ops.attention_decode_fused_supports(
-                x.dtype, self.hd, group.page_size, self.nq, self.nkv, rot, style)):
+        if (ctx.num_decode == T and not ctx.num_tiles and T <= FUSED_DECODE_MAX_TOKENS
+                and ops.attention_decode_fused_supports(x.dtype, self.hd, group.page_size, self.nq, self.nkv, rot, style)):
             # a step of single new tokens: norm, rotation and cache write happen inside the attention kernel
             out = torch.empty((T, self.nq * self.hd), dtype=x.dtype, device=x.device)
             ops.attention_decode_fused(
