@@ -636,6 +636,7 @@ struct PrefillStage {                     // one 32-key tile on its way from the
   static constexpr int KROW = 2 * HD + 32, VROW = 64 + 32;     // bytes
   static constexpr int KBYTES = 32 * KROW, VBYTES = HD * VROW;
   uint4 k[PER_THREAD], v[PER_THREAD];
+  int ok;                                 // bit j: piece j comes from a page that exists (the same in the whole wave)
 };
 
 // What a thread's pieces need that does not change from tile to tile: byte offsets in the cache
@@ -667,10 +668,27 @@ __device__ __forceinline__ PrefillLanes<NQK> prefill_lanes(int page_size) {
   return pl;
 }
 
+// Page ids for the prompt kernel's loads: as load_pages, but the table is read by every lane (a lane
+// past the end of the data reads the entry of the last key) and the result is made -1 by arithmetic,
+// so the load stands outside any condition and the compiler can count it among the loads in flight.
+__device__ __forceinline__ PageWindow prefill_pages(int key_from, int key_end, const int* __restrict__ bt, int page_size) {
+  PageWindow w;
+  w.base = key_from >> 4;
+  const int kb = (w.base + (int)(threadIdx.x & 63)) << 4;
+  const int at = kb < key_end ? kb : key_end - 1;
+  w.page = bt[at / page_size] | ((key_end - 1 - kb) >> 31);
+  w.off = kb % page_size;
+  return w;
+}
+
 // Queue the loads of the tile at key0.  A wave's 64 pieces of one round lie in one 16-key sub-block,
 // so its page id is a single lane of the page window and the cache address is a base common to the
 // wave (scalar registers) plus the thread's own 32-bit offset.  `k_head` / `v_head` point at this kv
-// head inside page 0; `page_elems` is the distance between pages.
+// head inside page 0; `page_elems` is the distance between pages.  Every load is issued whatever the
+// page table says, so that the waits in the loop are for the loads of two steps ago and not for all
+// of them: a sub-block without a page (given back behind a window, or past the end of the data) reads
+// page 0 instead.  Its keys are never seen (it lies in a tile with tests, and they fail for such a
+// key), and its values are replaced by zeros on the way to LDS.
 template <int NQK>
 __device__ __forceinline__ void stage_load(PrefillStage<NQK>& st, int key0, const PageWindow& pw,
                                            const PrefillLanes<NQK>& pl, const bf16_t* __restrict__ k_head,
@@ -678,35 +696,22 @@ __device__ __forceinline__ void stage_load(PrefillStage<NQK>& st, int key0, cons
   using S = PrefillStage<NQK>;
   constexpr int HD = S::HD;
   const int tid = threadIdx.x & (S::THREADS - 1);
+  st.ok = 0;
 #pragma unroll
   for (int j = 0; j < S::PER_THREAD; ++j) {
     const int piece = tid + j * S::THREADS;
-    const int sub = __builtin_amdgcn_readfirstlane(piece / (2 * HD)) + (key0 >> 4) - pw.base;
-    const int page = piece < S::CHUNKS ? __builtin_amdgcn_readlane(pw.page, sub & 63) : -1;
-    if (page < 0) {
-      st.k[j] = make_uint4(0, 0, 0, 0);
-      st.v[j] = make_uint4(0, 0, 0, 0);
-      continue;
-    }
+    const int sub = (__builtin_amdgcn_readfirstlane(piece / (2 * HD)) + (key0 >> 4) - pw.base) & 63;
+    const int page = __builtin_amdgcn_readlane(pw.page, sub);
     const unsigned off = (unsigned)__builtin_amdgcn_readlane(pw.off, sub);
-    const size_t base = (size_t)(unsigned)page * page_elems;
-    const char* kp = reinterpret_cast<const char*>(k_head + base + off * HD);
-    const char* vp = reinterpret_cast<const char*>(v_head + base + off);
-    st.k[j] = *reinterpret_cast<const uint4*>(kp + pl.kofs[j]);
-    st.v[j] = *reinterpret_cast<const uint4*>(vp + pl.vofs[j]);
+    const size_t base = (size_t)(unsigned)(page < 0 ? 0 : page) * page_elems;
+    st.ok |= (page < 0 ? 0 : 1) << j;
+    st.k[j] = ld16(reinterpret_cast<const char*>(k_head + base + off * HD) + pl.kofs[j]);
+    st.v[j] = ld16(reinterpret_cast<const char*>(v_head + base + off) + pl.vofs[j]);
   }
 }
 
-template <int NQK>
-__device__ __forceinline__ void stage_zero(PrefillStage<NQK>& st) {
-#pragma unroll
-  for (int j = 0; j < PrefillStage<NQK>::PER_THREAD; ++j) {
-    st.k[j] = make_uint4(0, 0, 0, 0);
-    st.v[j] = make_uint4(0, 0, 0, 0);
-  }
-}
-
-// Write a loaded tile to LDS; values of keys past max_hi (never written, may hold anything) become 0.
+// Write a loaded tile to LDS; values of keys past max_hi (never written, may hold anything) and of
+// sub-blocks without a page become 0.
 template <int NQK>
 __device__ __forceinline__ void stage_store(const PrefillStage<NQK>& st, int key0, int max_hi,
                                             const PrefillLanes<NQK>& pl, unsigned char* __restrict__ kl,
@@ -714,13 +719,13 @@ __device__ __forceinline__ void stage_store(const PrefillStage<NQK>& st, int key
   using S = PrefillStage<NQK>;
   constexpr int HD = S::HD;
   const int tid = threadIdx.x & (S::THREADS - 1);
-  const bool edge = key0 + 32 > max_hi + 1;
+  const bool plain = key0 + 32 <= max_hi + 1 && st.ok == (1 << S::PER_THREAD) - 1;
 #pragma unroll
   for (int j = 0; j < S::PER_THREAD; ++j) {
     const int piece = tid + j * S::THREADS;
     if (piece >= S::CHUNKS) continue;
-    *reinterpret_cast<uint4*>(kl + pl.klds[j]) = st.k[j];
-    if (!edge) {
+    st16(kl + pl.klds[j], st.k[j]);
+    if (plain) {
       *reinterpret_cast<uint2*>(vl + pl.vlds[j]) = make_uint2(st.v[j].x, st.v[j].y);       // keys 8 half .. +4
       *reinterpret_cast<uint2*>(vl + pl.vlds[j] + 16) = make_uint2(st.v[j].z, st.v[j].w);  // keys 8 half + 4 .. +4
       continue;
@@ -728,9 +733,10 @@ __device__ __forceinline__ void stage_store(const PrefillStage<NQK>& st, int key
     Pack8 v;
     v.u4 = st.v[j];
     const int sb = piece / (2 * HD), half = piece % 2;
+    const bool ok = (st.ok >> j) & 1;
 #pragma unroll
     for (int e = 0; e < 8; ++e)
-      if (key0 + 16 * sb + 8 * half + e > max_hi) v.h[e] = 0;
+      if (!ok || key0 + 16 * sb + 8 * half + e > max_hi) v.h[e] = 0;
     *reinterpret_cast<uint2*>(vl + pl.vlds[j]) = v.u2[0];
     *reinterpret_cast<uint2*>(vl + pl.vlds[j] + 16) = v.u2[1];
   }
@@ -848,7 +854,7 @@ __device__ __forceinline__ void process_tile_lds(const unsigned char* __restrict
 // lasts half as long and a compute unit holds one block at a time, so that blocks that finish early
 // (tiles with few keys) make room for the next ones instead of idling beside a long one.
 template <int NQK, int KS>
-__global__ void __launch_bounds__(64 * PREFILL_WAVES * KS)
+__global__ void __launch_bounds__(64 * PREFILL_WAVES * KS, NQK <= 4 ? 2 / KS : 1)
 attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
                          const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
                          const int* __restrict__ tiles, const int* __restrict__ positions,
@@ -926,29 +932,22 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __r
     negm[qg] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     l[qg] = 0.f;
   }
-  // the page window serves the loads, which run ahead of the products
-  PageWindow pw = load_pages(my_begin < key_end ? my_begin : key_begin, key_end, bt, page_size);
+  // The page window serves the loads, which run ahead of the products.  It holds 32 tiles; every 16
+  // steps the next one takes over, fetched 16 steps earlier.
+  PageWindow pw = prefill_pages(my_begin, key_end, bt, page_size);
   PrefillStage<NQK> st0, st1;
   const PrefillLanes<NQK> lanes = prefill_lanes<NQK>(page_size);
   const unsigned page_elems = (unsigned)(nkv * page_size * HD);
   const bf16_t* const k_head = k_pool + (size_t)kvh * page_size * HD;
   const bf16_t* const v_head = v_pool + (size_t)kvh * page_size * HD;
-#define STAGE_LOAD(ST, K0)                                                         \
-  do {                                                                             \
-    if ((K0) < my_end) {                                                           \
-      if ((K0) >= 16 * (pw.base + 64)) pw = load_pages((K0), key_end, bt, page_size); \
-      stage_load<NQK>(ST, (K0), pw, lanes, k_head, v_head, page_elems);           \
-    } else {                                                                       \
-      stage_zero<NQK>(ST);                                                         \
-    }                                                                              \
-  } while (0)
+#define STAGE_LOAD(ST, K0) stage_load<NQK>(ST, (K0), pw, lanes, k_head, v_head, page_elems)
 #define STAGE_STORE(ST, K0, BUF)                                                   \
   stage_store<NQK>(ST, (K0), last_pos, lanes, tile_lds + (BUF) * TILE_BYTES,       \
                    tile_lds + (BUF) * TILE_BYTES + S::KBYTES)
   // The tile at K0 is in LDS tile BUF; NEXT holds the tile after it, which goes to the other LDS tile
   // (last read one step ago, before the barrier) and is then refilled with the tile three further on.
   // Every wave runs every step: a wave without a head has no visible key (its limits are empty), and
-  // a step past the end of this half's keys finds a tile of zeros whose keys no column sees, so
+  // a step past the end of this half's keys finds keys that no column sees and values of zero, so
   // neither changes a sum and the loop needs no test around the products.
 #define STAGE_WORK(K0, BUF, NEXT)                                                  \
   do {                                                                             \
@@ -966,11 +965,32 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __r
   STAGE_STORE(st0, my_begin, 0);
   STAGE_LOAD(st0, my_begin + 64);
   __syncthreads();
-  for (int i = 0; i < steps; i += 2) {                    // the same number of barriers in both halves
-    STAGE_WORK(my_begin + 32 * i, 0, st1);
-    if (i + 1 >= steps) break;
-    STAGE_WORK(my_begin + 32 * i + 32, 1, st0);
+#define STAGE_PRODUCTS(K0, BUF)                                                    \
+  do {                                                                             \
+    const unsigned char* kl = tile_lds + (BUF) * TILE_BYTES;                       \
+    if ((K0) + 31 > first_pos || (K0) < open_lo)                                   \
+      process_tile_lds<NQK, NG, true>(kl, kl + S::KBYTES, (K0), qreg, clo, chi, acc, m, negm, l);  \
+    else                                                                           \
+      process_tile_lds<NQK, NG, false>(kl, kl + S::KBYTES, (K0), qreg, clo, chi, acc, m, negm, l); \
+  } while (0)
+  // Steps go in pairs, so that the two register stages and the two LDS tiles take turns in a way the
+  // compiler can see (it then waits for the loads of two steps ago only); an odd last step follows the
+  // loops and has nothing left to fetch.  Both halves pass the same number of barriers.
+  const int paired = steps & ~1;
+  for (int o = 0; o < paired; o += 16) {
+    const PageWindow pw_next = prefill_pages(my_begin + 32 * (o + 16), key_end, bt, page_size);
+    const int n = paired - o < 16 ? paired - o : 16;
+    for (int j = 0; j < n; j += 2) {
+      STAGE_WORK(my_begin + 32 * (o + j), 0, st1);
+      STAGE_WORK(my_begin + 32 * (o + j) + 32, 1, st0);
+    }
+    pw = pw_next;
   }
+  if (steps & 1) {
+    STAGE_PRODUCTS(my_begin + 32 * paired, 0);
+    if (KS == 2) __syncthreads();                         // the merge below reuses the tiles' memory
+  }
+#undef STAGE_PRODUCTS
 #undef STAGE_STORE
 #undef STAGE_LOAD
 #undef STAGE_WORK
