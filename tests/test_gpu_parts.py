@@ -81,6 +81,47 @@ def test_toy_mixer_with_state_registers_builds_and_steps(tmp_path, dtype, cuts):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_state_mixer_steps_replayed_from_graphs(tmp_path, dtype):
+    """A state mixer that says its single-token step can be captured keeps the model on HIP graphs:
+    three requests (a batch padded to four, the padding entries' state going to the spare row) decode
+    side by side from graphs, a fourth joins and one leaves on the way, and every step equals the plain
+    forward: the state moves on once per step, also in the step that captures a graph."""
+    from ullm_amd.replay import Replayer
+    from ullm_amd.weights.random_init import write_random_model
+    from safetensors.torch import load_file
+    cfg = base_cfg([ATT, TOY, dict(ATT, heads=4, kv_heads=1, head_dim=32), TOY])
+    d = write_random_model(cfg, str(tmp_path / "m"), seed=21)
+    w = load_file(os.path.join(d, "model.safetensors"))
+    rep = Replayer(d, dtype, 512, 8, DEV, use_graphs=True)
+    if not rep.runner.use_graphs:
+        pytest.skip("graphs need the GPU")
+    g = torch.Generator().manual_seed(5)
+    reqs = {r: torch.randint(0, cfg["vocab_size"], (n,), generator=g).tolist() for r, n in (("a", 40), ("b", 33), ("c", 47), ("d", 30))}
+    wants = {r: toy_arch.toy_forward(w, cfg, t).numpy() for r, t in reqs.items()}
+    done = {r: 0 for r in reqs}
+    plan = [[("a", 12), ("b", 9), ("c", 20)]] + [[("a", 1), ("b", 1), ("c", 1)]] * 6 + [[("d", 11)]] + \
+           [[("a", 1), ("b", 1), ("c", 1), ("d", 1)]] * 5 + [[("a", 1), ("c", 1), ("d", 1)]] * 8 + [[("c", 1)]] * 3
+    ended = set()
+    for s, step in enumerate(plan):
+        entries = []
+        for r, n in step:
+            n = min(n, len(reqs[r]) - done[r])
+            if n > 0:
+                entries.append({"id": r, "tokens": reqs[r][done[r]:done[r] + n], "want": list(range(n))})
+        end = ["b"] if s == 13 and "b" not in ended else []
+        ended.update(end)
+        out = rep.step({"step": s, "entries": entries, "end": end})
+        row = 0
+        for e in entries:
+            n = len(e["tokens"])
+            want = wants[e["id"]][done[e["id"]]:done[e["id"]] + n]
+            assert float(np.abs(out[row:row + n] - want).max()) <= REL[dtype] * float(np.abs(want).max()) + 1e-6, (s, e["id"])
+            done[e["id"]] += n
+            row += n
+    assert len(rep.runner._graphs) >= 2          # batches of 4 (3 padded, and 4) and of 1
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_only_state_layers_need_no_pages(tmp_path, dtype):
     cfg = base_cfg([TOY, TOY], tie=True)
     rep, _ = run_and_compare(tmp_path, cfg, dtype, CUTS[2])

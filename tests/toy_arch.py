@@ -26,7 +26,8 @@ class RunningMean(Mixer):
         self.w = None
 
     def cache_need(self):
-        return StateNeed((self.hidden_size + 1,), torch.float32)
+        # a step of single tokens takes the slots from the device (below), so it may be captured
+        return StateNeed((self.hidden_size + 1,), torch.float32, graph_safe=True)
 
     def weights(self):
         return [WeightDecl(f"{self.prefix}.mean_proj.weight", (self.hidden_size, self.hidden_size))]
@@ -36,6 +37,15 @@ class RunningMean(Mixer):
 
     def forward(self, x, ctx, cache):
         H = self.hidden_size
+        if ctx.decode_only:
+            # one token per entry, token i = entry i: gather the entries' rows, move them on, scatter them
+            # back (the padding entries of a captured batch all name the spare row)
+            slots = ctx.entry_slot.long()
+            rows = cache.state[slots]
+            sums, counts = rows[:, :H] + x.float(), rows[:, H] + 1.0
+            if cache.owner:
+                cache.state[slots] = torch.cat((sums, counts[:, None]), dim=1)
+            return linear((sums / counts[:, None]).to(x.dtype), self.w)
         means = torch.empty(x.shape, dtype=torch.float32, device=x.device)
         t = 0
         for n, slot in zip(ctx.host["lens"], ctx.host["slots"]):
@@ -55,6 +65,7 @@ class Top1Experts(FeedForward):
     """Every token goes to the one expert its router scores highest (scores in float32, first index
     on ties); y = softmax(scores)[e] * down_e(relu(up_e x)).  Tokens are gathered per expert, run
     through the framework's linear, and scattered back."""
+    graph_safe = False      # each expert gathers the rows routed to it: sizes that depend on the tokens
 
     def __init__(self, hidden_size: int, expert_size: int, num_experts: int, prefix: str):
         self.hidden_size, self.expert_size, self.num_experts, self.prefix = hidden_size, expert_size, num_experts, prefix

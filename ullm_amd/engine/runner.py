@@ -64,8 +64,9 @@ class ModelRunner:
                     group=g, k_pool=torch.zeros(k_shape, dtype=env.dtype, device=env.device),
                     v_pool=torch.zeros(v_shape, dtype=env.dtype, device=env.device))
         for key, need in states.items():
+            # one row more than requests: the slot of a captured batch's padding entries
             views[key] = LayerCache(
-                state=torch.zeros((max_requests,) + tuple(need.shape), dtype=need.dtype, device=env.device))
+                state=torch.zeros((max_requests + 1,) + tuple(need.shape), dtype=need.dtype, device=env.device))
         self._views = views
         # per cache id what its block sees: the one view, or one view per declared need
         self.caches: Dict[int, LayerCache] = {}
@@ -76,9 +77,13 @@ class ModelRunner:
         self.feed_source: Optional[torch.Tensor] = None
         self.vocab_size = model.plan.vocab_size
         # Steps in which every entry brings one token are replayed from HIP graphs, one graph per
-        # (batch size bucket, context length bucket).  Padding entries would disturb per-request state,
-        # so a model with state mixers always runs eagerly.
-        self.use_graphs = bool(use_graphs) and env.device.type == "cuda" and not states
+        # (batch size bucket, context length bucket), unless a part says that its work cannot be captured
+        # (Part.graph_safe); with state mixers only if each of them says that its single-token step can be
+        # (StateNeed.graph_safe).
+        self.use_graphs = (bool(use_graphs) and env.device.type == "cuda"
+                           and all(need.graph_safe for need in states.values())
+                           and all(part.graph_safe for part in model.parts()))
+        self.padding_slot = max_requests
         self.max_graph_batch = max_graph_batch
         self._graphs: Dict[tuple, "_DecodeGraph"] = {}
         self._graph_pool = None
@@ -189,6 +194,7 @@ class ModelRunner:
             raise StepError(f"request {bad.request_id!r}: token id outside [0, {self.vocab_size})")
         ids[:n_tok] = tok
         slot[:n_real] = slots
+        slot[n_real:] = self.padding_slot
         start[:n_real] = starts
         r = 0
         for b, e in enumerate(entries):
@@ -216,7 +222,7 @@ class ModelRunner:
                      num_tiles=len(tile_list) // 2, tile_keys_total=sum(k for k, _, _ in tile_keys),
                      tile_keys_max=tile_keys[-1][0] if tile_keys else 0, max_q=max(lens), max_kv=max_kv,
                      decode_only=all(n == 1 for n in lens), lens=lens + [1] * n_pad,
-                     starts=starts + [0] * n_pad, slots=slots + [0] * n_pad, unknown=unknown)
+                     starts=starts + [0] * n_pad, slots=slots + [self.padding_slot] * n_pad, unknown=unknown)
         return host, offs, facts
 
     def _context(self, dev: torch.Tensor, offs, facts) -> tuple:
@@ -337,12 +343,17 @@ class ModelRunner:
         self._upload(host, into=static_dev)
         ctx, rows = self._context(static_dev, offs, facts)
         with torch.no_grad():
-            # once eagerly on a side stream: loads the kernels and sizes the library's workspaces
+            # once eagerly on a side stream: loads the kernels and sizes the library's workspaces.  Keys and
+            # values written twice are the same keys and values; state that a step moves on is put back.
+            states = [c.state for c in self._views.values() if c.state is not None]
+            saved = [t.clone() for t in states]
             side = torch.cuda.Stream()
             side.wait_stream(torch.cuda.current_stream())
             with torch.cuda.stream(side):
                 self._feed(static_dev, offs)
                 self.model.forward(ctx, self.caches, rows)
+                for t, was in zip(states, saved):
+                    t.copy_(was)
             torch.cuda.current_stream().wait_stream(side)
             if self._graph_pool is None:
                 self._graph_pool = torch.cuda.graph_pool_handle()

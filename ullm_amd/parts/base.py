@@ -45,9 +45,17 @@ class KVNeed:
 
 @dataclass(frozen=True)
 class StateNeed:
-    """A mixer that keeps state of fixed size per request (zeroed at admission)."""
+    """A mixer that keeps state of fixed size per request (zeroed at admission).
+
+    ``graph_safe``: the mixer's step for single new tokens (``ctx.decode_only``) takes everything from
+    device tensors (``ctx.entry_slot``, not the host lists), so it may be captured into a HIP graph and
+    replayed with other requests in the same places.  The state tensor has one row more than there are
+    requests; the padding entries of a captured batch carry that row's index as their slot, so whatever a
+    step does to their state lands where no request looks.  One mixer that does not say so keeps the
+    whole model on eager steps."""
     shape: Tuple[int, ...]
     dtype: torch.dtype = torch.float32
+    graph_safe: bool = False
 
 
 CacheNeed = Union[KVNeed, StateNeed, None]
@@ -163,8 +171,14 @@ class PartEnv:
 
 
 class Part:
-    """Base of every part.  ``weights()`` declares tensors; ``bind`` receives them."""
+    """Base of every part.  ``weights()`` declares tensors; ``bind`` receives them.
+
+    ``graph_safe``: the part's work in a step of single new tokens can be captured into a HIP graph: it
+    queues the same kernels whatever the tokens are and never waits for the device (no sizes that
+    depend on values, as a routed feed-forward that gathers each expert's rows has).  One part that
+    says no keeps the whole model on eager steps."""
     kind = ""
+    graph_safe = True
 
     def weights(self) -> List[WeightDecl]:
         return []
