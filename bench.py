@@ -184,6 +184,9 @@ class Sized:
         """(tokens/s, ms, fraction of the dtype's matrix peak) of one prompt of n_tokens, best of three."""
         from ullm_amd import SamplingParams
         torch = self.torch
+        if n_tokens >= self.context_len:
+            # the engine would keep the prompt's last context_len tokens and the figures would be of those
+            raise SystemExit(f"a prompt of {n_tokens} tokens needs --context-len above {n_tokens} (it is {self.context_len})")
         eng = self.engine(max_bs=1, num_pages=-(-(n_tokens + 16) // 16), max_num_batched_tokens=n_tokens,
                           max_prefill_chunk=n_tokens)
         best = None

@@ -21,8 +21,11 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
 
 
 # Rows up to which folding the norm into the product pays: beyond, the float32 rows of X cost every block more
-# registers and loads than the saved launch is worth.
+# registers and loads than the saved launch is worth.  A small matrix (q|k|v of the 8B and 14B sizes) has few
+# blocks to pay that price, and the launch of the norm's own kernel weighs more beside its short product: there
+# the norm is folded in for every row count the kernel takes.
 NORM_FOLDED_MAX_ROWS = 8
+NORM_FOLDED_SMALL_WEIGHT = 40 << 20     # elements
 
 
 def linear_of_norm(x, weight: torch.Tensor, bias: Optional[torch.Tensor] = None, silu: bool = False) -> torch.Tensor:
@@ -32,7 +35,8 @@ def linear_of_norm(x, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
     and the result silu(gate) * up."""
     from .base import PendingNorm
     if isinstance(x, PendingNorm):
-        if (x.out_dtype == torch.bfloat16 and x.stream.shape[0] <= NORM_FOLDED_MAX_ROWS
+        if (x.out_dtype == torch.bfloat16
+                and (x.stream.shape[0] <= NORM_FOLDED_MAX_ROWS or weight.numel() <= NORM_FOLDED_SMALL_WEIGHT)
                 and ops.gemm_skinny_normed_supports(x.stream, x.gain, weight)):
             return ops.gemm_skinny_normed(x.stream, x.gain, x.eps, weight, bias, silu=silu)
         x = x.apply()
