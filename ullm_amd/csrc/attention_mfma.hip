@@ -1043,6 +1043,411 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __r
   }
 }
 
+// ------------------------------------------------------------------------------- prompt portions, tiles straight to LDS
+// The same work split as attention_prefill_kernel, for head sizes 64 and 128, with the 32-key tiles of
+// keys and values fetched by loads that write shared memory themselves (global_load_lds_dwordx4: a
+// wave's 64 lanes fill 1024 consecutive bytes, every lane from an address of its own).  No register
+// holds a tile on its way, no instruction copies it, and four tiles of shared memory take turns, so the
+// loads run three tiles ahead of the products.
+//   keys   32 rows of head_dim values, unpadded; the 16-byte piece p of key k lies at piece p ^ f(k),
+//          f such that the 16 keys a product's lanes read together fall into 16 different bank groups
+//   values one row of 32 keys per dim (64 bytes); piece p of dim d lies at piece p ^ (d / 4 % 4)
+// A score product's 16 rows are the keys 8 (r / 4) + 4 sb + r % 4 of the tile (sb = which of the two
+// products), so that in its result a lane group holds eight consecutive keys (4 from each product): the
+// order in which a 16-byte piece of the values holds them, and the value product needs no shuffle.
+// The loads are issued in inline assembly: the compiler, which cannot tell which of such loads a read of
+// shared memory depends on, would otherwise wait for all of them before every read.  The waits for them
+// stand in the code, by count (a wave's loads complete in order), and the loop holds no load of the
+// compiler's own whose wait could be off by the ones it does not see: the page ids lie in shared memory.
+#define DMA_TILES 4                       // tiles of shared memory that take turns
+#define DMA_TABLE_TILES 128               // tiles whose page ids shared memory holds at a time (and 4 more, for the loads ahead)
+
+// 16 bytes per lane from `src` to shared memory at lds_base + 16 * lane (lds_base the same in the whole wave).
+// The instruction takes the place in shared memory from M0, which the compiler keeps for itself and warns
+// about; nothing else in these kernels uses it.
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+__device__ __forceinline__ void load16_to_lds(const void* src, unsigned char* lds_base) {
+#ifdef __HIP_DEVICE_COMPILE__
+  typedef __attribute__((address_space(3))) unsigned char lds_byte_t;
+  const unsigned at = (unsigned)__builtin_amdgcn_readfirstlane((int)(uintptr_t)(lds_byte_t*)lds_base);
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(at) : "memory", "m0");
+#else
+  __builtin_amdgcn_global_load_lds(src, lds_base, 16, 0, 0);
+#endif
+}
+#pragma clang diagnostic pop
+// at most N of this wave's loads are still on their way
+template <int N>
+__device__ __forceinline__ void loads_left() {
+  static_assert(N >= 0 && N < 64, "the counter has six bits");
+#ifdef __HIP_DEVICE_COMPILE__
+  asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
+#endif
+}
+
+template <int NQK>
+struct DmaTile {
+  static constexpr int HD = 32 * NQK;
+  static constexpr int PR = HD / 8;       // 16-byte pieces of a key row
+  static constexpr int ROUNDS = NQK / 2;  // load instructions per wave for a tile's keys, and as many for its values
+  static constexpr int KBYTES = 32 * 2 * HD, VBYTES = HD * 64;
+  static constexpr int BYTES = KBYTES + VBYTES;
+  static_assert(NQK == 2 || NQK == 4, "head sizes 64 and 128");
+  // the row that key k (0 .. 31) has in its score product, and what its pieces' places are xor-ed with
+  __host__ __device__ static constexpr int row_of_key(int k) { return (k & 3) | (((k >> 3) & 3) << 2); }
+  __host__ __device__ static constexpr int key_swizzle(int k) { return PR == 16 ? row_of_key(k) : row_of_key(k) >> 1; }
+};
+
+// What a lane's loads need that does not change from tile to tile.
+template <int NQK>
+struct DmaLanes {
+  unsigned k_off[DmaTile<NQK>::ROUNDS];   // bytes from the first key row of the instruction's 16-key sub-block
+  int k_sub[DmaTile<NQK>::ROUNDS];        // which of the tile's two sub-blocks (the same in the whole wave)
+  unsigned v_off[DmaTile<NQK>::ROUNDS];   // bytes from the sub-block's first key in dim 0
+  int v_sub[DmaTile<NQK>::ROUNDS];        // which sub-block this lane's piece lies in
+  int dest[DmaTile<NQK>::ROUNDS];         // where the instruction's 1024 bytes go inside the tile's keys (and values)
+};
+
+template <int NQK>
+__device__ __forceinline__ DmaLanes<NQK> dma_lanes(int page_size) {
+  using T = DmaTile<NQK>;
+  DmaLanes<NQK> d;
+  const int lane = threadIdx.x & 63, wave = (threadIdx.x >> 6) % PREFILL_WAVES;
+#pragma unroll
+  for (int rd = 0; rd < T::ROUNDS; ++rd) {
+    const int ins = wave + PREFILL_WAVES * rd;
+    const int at = 64 * ins + lane;                       // the lane's place among the tile's pieces, as they lie in LDS
+    const int key = at / T::PR, kpiece = (at % T::PR) ^ T::key_swizzle(key);
+    d.k_sub[rd] = __builtin_amdgcn_readfirstlane(key >> 4);
+    d.k_off[rd] = 2u * (unsigned)((key & 15) * T::HD + 8 * kpiece);
+    const int dim = 16 * ins + (lane >> 2), vpiece = (lane & 3) ^ ((dim >> 2) & 3);
+    d.v_sub[rd] = vpiece >> 1;
+    d.v_off[rd] = 2u * (unsigned)(dim * page_size + 8 * (vpiece & 1));
+    d.dest[rd] = 1024 * ins;
+  }
+  return d;
+}
+
+// Start the loads of the tile at key0 into the tile of shared memory at `tile` (keys, then values); page0 / page1
+// are the page ids of its two 16-key sub-blocks.  A sub-block without a page reads page 0: its keys are
+// never seen, and its values count as zero in the products.
+template <int NQK>
+__device__ __forceinline__ void dma_tile_load(unsigned char* tile, int key0, int page0, int page1, int page_size,
+                                              const DmaLanes<NQK>& dl, const bf16_t* __restrict__ k_head,
+                                              const bf16_t* __restrict__ v_head, unsigned page_elems) {
+  using T = DmaTile<NQK>;
+  const unsigned off0 = (unsigned)(key0 % page_size), off1 = (unsigned)((key0 + 16) % page_size);
+  const size_t base0 = (size_t)(unsigned)(page0 < 0 ? 0 : page0) * page_elems;
+  const size_t base1 = (size_t)(unsigned)(page1 < 0 ? 0 : page1) * page_elems;
+  const char* const k0 = reinterpret_cast<const char*>(k_head + base0 + off0 * T::HD);
+  const char* const k1 = reinterpret_cast<const char*>(k_head + base1 + off1 * T::HD);
+  const char* const v0 = reinterpret_cast<const char*>(v_head + base0 + off0);
+  const char* const v1 = reinterpret_cast<const char*>(v_head + base1 + off1);
+#pragma unroll
+  for (int rd = 0; rd < T::ROUNDS; ++rd) load16_to_lds((dl.k_sub[rd] ? k1 : k0) + dl.k_off[rd], tile + dl.dest[rd]);
+#pragma unroll
+  for (int rd = 0; rd < T::ROUNDS; ++rd)
+    load16_to_lds((dl.v_sub[rd] ? v1 : v0) + dl.v_off[rd], tile + T::KBYTES + dl.dest[rd]);
+}
+
+// Scores, softmax update and value product of one wave for the tile in shared memory; as process_tile_lds,
+// with the keys' order and the tile's layout as described above.
+template <int NQK, int NG, bool masked>
+__device__ __forceinline__ void dma_tile_products(const unsigned char* __restrict__ tile, int key0, const Pack8 (&qreg)[NG][NQK],
+                                                  const int (&col_lo)[NG], const int (&col_hi)[NG],
+                                                  f32x4_t (&acc)[NG][2 * NQK], float (&m)[NG], f32x4_t (&negm)[NG],
+                                                  float (&l)[NG], const int (&k_at)[2][NQK], int v_at, int max_hi,
+                                                  bool ok0, bool ok1) {
+  using T = DmaTile<NQK>;
+  const int lane = threadIdx.x & 63, g = lane >> 4;
+  f32x4_t s[NG][2];
+#pragma unroll
+  for (int sb = 0; sb < 2; ++sb)
+#pragma unroll
+    for (int ch = 0; ch < NQK; ++ch) {
+      Pack8 kf;
+      kf.u4 = ld16(tile + k_at[sb][ch]);
+#pragma unroll
+      for (int q = 0; q < NG; ++q)
+        s[q][sb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qreg[q][ch].v, ch == 0 ? negm[q] : s[q][sb], 0, 0, 0);
+    }
+  // s[q][sb][r] is the exponent of key key0 + 8 g + 4 sb + r for this lane's column
+  float lane_max[NG], alpha[NG];
+  bool exceeds = false;
+#pragma unroll
+  for (int q = 0; q < NG; ++q) {
+    lane_max[q] = NEG_BIG;
+    alpha[q] = 1.f;
+#pragma unroll
+    for (int sb = 0; sb < 2; ++sb)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        if (masked) {
+          const int kk = key0 + 8 * g + 4 * sb + r;
+          if (!(kk >= col_lo[q] && kk <= col_hi[q])) s[q][sb][r] = NEG_BIG;
+        }
+        lane_max[q] = fmaxf(lane_max[q], s[q][sb][r]);
+      }
+    const bool sees = !masked || lane_max[q] > 0.5f * NEG_BIG;
+    exceeds = exceeds || (sees && (lane_max[q] > RESCALE_STEP || m[q] < 0.5f * NEG_BIG));
+  }
+  if (__any(exceeds)) {
+#pragma unroll
+    for (int q = 0; q < NG; ++q) {
+      float col_max = lane_max[q];
+      col_max = fmaxf(col_max, __shfl_xor(col_max, 16, 64));
+      col_max = fmaxf(col_max, __shfl_xor(col_max, 32, 64));
+      const bool had = m[q] > 0.5f * NEG_BIG;
+      const bool moves = col_max > 0.5f * NEG_BIG && (!had || col_max > RESCALE_STEP);
+      if (moves) {
+        m[q] = (had ? m[q] : 0.f) + col_max;
+        negm[q] = f32x4_t{-m[q], -m[q], -m[q], -m[q]};
+        if (had) alpha[q] = fast_exp2(-col_max);
+#pragma unroll
+        for (int sb = 0; sb < 2; ++sb)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) s[q][sb][r] -= col_max;     // a hidden score stays far below
+      }
+#pragma unroll
+      for (int n = 0; n < 2 * NQK; ++n)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          float o = acc[q][n][r] * alpha[q];
+#ifdef __HIP_DEVICE_COMPILE__
+          asm volatile("" : "+v"(o));       // pins the multiply inside the branch: most tiles skip it
+#endif
+          acc[q][n][r] = o;
+        }
+    }
+  }
+  Pack8 p[NG];
+#pragma unroll
+  for (int q = 0; q < NG; ++q) {
+    float psum = l[q] * alpha[q];
+#pragma unroll
+    for (int sb = 0; sb < 2; ++sb) {
+      float e[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        e[r] = (!masked || s[q][sb][r] > 0.5f * NEG_BIG) ? fast_exp2(s[q][sb][r]) : 0.f;
+      p[q].w[2 * sb] = pack2_bf16(e[0], e[1]);
+      p[q].w[2 * sb + 1] = pack2_bf16(e[2], e[3]);
+      psum = add_pair_bf16(p[q].w[2 * sb], psum);
+      psum = add_pair_bf16(p[q].w[2 * sb + 1], psum);
+    }
+    l[q] = psum;
+  }
+  // masked tiles only: which of this lane's eight keys (8 g ..) hold written values.  The others (past the end
+  // of the data, or in a sub-block without a page, which reads page 0) may hold anything and must count as 0.
+  uint32_t live[4] = {0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu};
+  if (masked) {
+    const bool ok = g >> 1 ? ok1 : ok0;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const int kk = key0 + 8 * g + 2 * w;
+      live[w] = (ok && kk <= max_hi ? 0x0000ffffu : 0u) | (ok && kk + 1 <= max_hi ? 0xffff0000u : 0u);
+    }
+  }
+#pragma unroll
+  for (int n = 0; n < 2 * NQK; ++n) {
+    Pack8 vf;
+    vf.u4 = ld16(tile + T::KBYTES + v_at + 1024 * n);
+    if (masked) {
+#pragma unroll
+      for (int w = 0; w < 4; ++w) vf.w[w] &= live[w];
+    }
+#pragma unroll
+    for (int q = 0; q < NG; ++q) acc[q][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, p[q].v, acc[q][n], 0, 0, 0);
+  }
+}
+
+template <int NQK, int KS>
+__global__ void __launch_bounds__(64 * PREFILL_WAVES * KS, 2 / KS)
+attention_prefill_dma_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
+                             const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
+                             const int* __restrict__ tiles, const int* __restrict__ positions,
+                             const int* __restrict__ token_entry, const int* __restrict__ block_table,
+                             int bt_stride, int page_size, int nq, int nkv, float scale_log2e, int window,
+                             int n_tiles) {
+  using T = DmaTile<NQK>;
+  constexpr int HD = 32 * NQK;
+  constexpr int NG = PREFILL_GROUPS;
+  constexpr int PER_LANE = NG * (8 * NQK + 2);            // floats a lane hands over in the merge
+  constexpr int PER = 2 * T::ROUNDS;                      // load instructions of a wave per tile
+  constexpr int TABLE = 2 * (DMA_TABLE_TILES + 4);        // page ids in shared memory, one per 16-key sub-block
+  static_assert(KS == 1 || PREFILL_WAVES * PER_LANE * 64 * 4 <= KS * DMA_TILES * T::BYTES, "the merge reuses the tiles' memory");
+  __shared__ __attribute__((aligned(1024))) unsigned char lds[KS * DMA_TILES * T::BYTES];   // [half][tile][keys | values]
+  __shared__ int page_ids[KS][TABLE];
+  const int wave_id = (int)(threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63, wave = wave_id % PREFILL_WAVES, half = wave_id / PREFILL_WAVES;
+  const int g = lane >> 4, c = lane & 15;
+  unsigned char* const tile_lds = lds + half * DMA_TILES * T::BYTES;
+  int* const pages = page_ids[half];
+  const int G = nq / nkv, chunks = (G + PREFILL_WAVES - 1) / PREFILL_WAVES, per_kv = n_tiles * chunks;
+  int kvh, rest;
+  if (nkv % 8 == 0) {
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    kvh = (slot / per_kv) * 8 + xcd;
+    rest = slot % per_kv;
+  } else {
+    kvh = blockIdx.x / per_kv;
+    rest = blockIdx.x % per_kv;
+  }
+  const int tile_idx = n_tiles - 1 - rest / chunks;
+  const int head_in_group = (rest % chunks) * PREFILL_WAVES + wave;
+  const bool head_ok = head_in_group < G;                 // a wave without a head still helps to load
+  const int head = kvh * G + (head_ok ? head_in_group : G - 1);
+  const int first = tiles[2 * tile_idx], count = tiles[2 * tile_idx + 1];
+  int clo[NG], chi[NG], tok[NG];
+  Pack8 qreg[NG][NQK];
+#pragma unroll
+  for (int qg = 0; qg < NG; ++qg) {
+    const bool ok = head_ok && 16 * qg + c < count;
+    tok[qg] = first + (16 * qg + c < count ? 16 * qg + c : 0);
+    const int pos = positions[tok[qg]];
+    clo[qg] = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+    chi[qg] = ok ? pos : -1;
+    const bf16_t* qp = q + (size_t)tok[qg] * q_stride + (size_t)head * HD + 8 * g;
+#pragma unroll
+    for (int ch = 0; ch < NQK; ++ch) {
+      if (ok) qreg[qg][ch].u4 = *reinterpret_cast<const uint4*>(qp + 32 * ch);
+      else qreg[qg][ch].u4 = make_uint4(0, 0, 0, 0);
+      // scale * log2(e) goes into the queries once, so that a score is its weight's exponent
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        const uint32_t two = qreg[qg][ch].w[w];
+        qreg[qg][ch].w[w] = pack2_bf16(__uint_as_float(two << 16) * scale_log2e,
+                                       __uint_as_float(two & 0xffff0000u) * scale_log2e);
+      }
+    }
+  }
+  const int last_pos = positions[first + count - 1];
+  const int first_pos = positions[first];
+  const int open_lo = (window > 0 && last_pos - window + 1 > 0) ? last_pos - window + 1 : 0;
+  const int key_begin = ((window > 0 && first_pos - window + 1 > 0) ? first_pos - window + 1 : 0) & ~31;
+  const int key_end = last_pos + 1;
+  const int steps = ((key_end - key_begin + 31) / 32 + KS - 1) / KS;    // this half's share of the 32-key tiles
+  const int my_begin = key_begin + half * steps * 32;
+  const int* bt = block_table + (size_t)token_entry[first] * bt_stride;
+  f32x4_t acc[NG][2 * NQK];
+  float m[NG], l[NG];
+  f32x4_t negm[NG];
+#pragma unroll
+  for (int qg = 0; qg < NG; ++qg) {
+#pragma unroll
+    for (int n = 0; n < 2 * NQK; ++n) acc[qg][n] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    m[qg] = NEG_BIG;
+    negm[qg] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    l[qg] = 0.f;
+  }
+  // where this lane reads its operands inside a tile: key row 8 (c / 4) + 4 sb + c % 4, piece 4 ch + g; dim 16 n + c, piece g
+  int k_at[2][NQK];
+#pragma unroll
+  for (int sb = 0; sb < 2; ++sb)
+#pragma unroll
+    for (int ch = 0; ch < NQK; ++ch) {
+      const int key = 8 * (c >> 2) + 4 * sb + (c & 3);
+      k_at[sb][ch] = key * 2 * HD + 16 * ((4 * ch + g) ^ T::key_swizzle(key));
+    }
+  const int v_at = c * 64 + 16 * (g ^ (c >> 2));
+  const DmaLanes<NQK> dl = dma_lanes<NQK>(page_size);
+  const unsigned page_elems = (unsigned)(nkv * page_size * HD);
+  const bf16_t* const k_head = k_pool + (size_t)kvh * page_size * HD;
+  const bf16_t* const v_head = v_pool + (size_t)kvh * page_size * HD;
+  // Tile i of this half is loaded with the page ids pages[2 (i - t0)], pages[2 (i - t0) + 1].
+#define TILE_LOAD(I, T0) dma_tile_load<NQK>(tile_lds + ((I) % DMA_TILES) * T::BYTES, my_begin + 32 * (I), pages[2 * ((I) - (T0))], \
+                                            pages[2 * ((I) - (T0)) + 1], page_size, dl, k_head, v_head, page_elems)
+  // Tiles 0, 1 and 2 go on their way; in step i tile i + 3 follows, into the place of tile i - 1, which every wave
+  // has left behind when it passes the step's barrier.  Loads are started for the tiles of this half's steps only,
+  // so the last steps wait for fewer loads to be left.
+  for (int t0 = 0; t0 < steps; t0 += DMA_TABLE_TILES) {
+    // page ids of the tiles t0 .. t0 + DMA_TABLE_TILES + 3 (the loads run up to three tiles ahead of the steps)
+    __syncthreads();
+    for (int e = threadIdx.x & (64 * PREFILL_WAVES - 1); e < TABLE; e += 64 * PREFILL_WAVES) {
+      const int kb = my_begin + 32 * t0 + 16 * e;
+      pages[e] = kb < key_end ? bt[kb / page_size] : -1;
+    }
+    __syncthreads();
+    if (t0 == 0) {
+      if (steps > 0) TILE_LOAD(0, 0);
+      if (steps > 1) TILE_LOAD(1, 0);
+      if (steps > 2) TILE_LOAD(2, 0);
+    }
+    const int t1 = t0 + DMA_TABLE_TILES < steps ? t0 + DMA_TABLE_TILES : steps;
+    for (int i = t0; i < t1; ++i) {
+      const int K0 = my_begin + 32 * i;
+      unsigned char* const tile = tile_lds + (i % DMA_TILES) * T::BYTES;
+      // this wave's part of tile i has landed once only the loads of the tiles after it are left
+      if (i + 2 < steps) loads_left<2 * PER>();
+      else if (i + 1 < steps) loads_left<PER>();
+      else loads_left<0>();
+      // The bare barrier: with the fence of __syncthreads the compiler would wait here for every load it
+      // knows of.  No access to memory may move across it: the next loads overwrite what other waves read
+      // until here.
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+      if (i + 3 < steps) TILE_LOAD(i + 3, t0);
+      if (K0 + 31 > first_pos || K0 < open_lo) {
+        const bool ok0 = pages[2 * (i - t0)] >= 0, ok1 = pages[2 * (i - t0) + 1] >= 0;
+        dma_tile_products<NQK, NG, true>(tile, K0, qreg, clo, chi, acc, m, negm, l, k_at, v_at, last_pos, ok0, ok1);
+      } else {
+        dma_tile_products<NQK, NG, false>(tile, K0, qreg, clo, chi, acc, m, negm, l, k_at, v_at, last_pos, true, true);
+      }
+    }
+  }
+#undef TILE_LOAD
+  // nothing is on its way any more, and every wave is done with the tiles: their memory serves the merge
+  loads_left<0>();
+  __syncthreads();
+  if (KS == 2) {
+    float* w = reinterpret_cast<float*>(lds) + (size_t)wave * PER_LANE * 64 + lane;
+    if (half == 1) {
+#pragma unroll
+      for (int qg = 0; qg < NG; ++qg) {
+#pragma unroll
+        for (int n = 0; n < 2 * NQK; ++n)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) w[(qg * (8 * NQK + 2) + 4 * n + e) * 64] = acc[qg][n][e];
+        w[(qg * (8 * NQK + 2) + 8 * NQK) * 64] = m[qg];
+        w[(qg * (8 * NQK + 2) + 8 * NQK + 1) * 64] = l[qg];
+      }
+    }
+    __syncthreads();
+    if (half == 0) {
+#pragma unroll
+      for (int qg = 0; qg < NG; ++qg) {
+        const float m_b = w[(qg * (8 * NQK + 2) + 8 * NQK) * 64], l_b = w[(qg * (8 * NQK + 2) + 8 * NQK + 1) * 64];
+        const float M = fmaxf(m[qg], m_b);
+        const float fa = fast_exp2(m[qg] - M), fb = fast_exp2(m_b - M);
+#pragma unroll
+        for (int n = 0; n < 2 * NQK; ++n)
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            acc[qg][n][e] = acc[qg][n][e] * fa + w[(qg * (8 * NQK + 2) + 4 * n + e) * 64] * fb;
+        l[qg] = l[qg] * fa + l_b * fb;
+        m[qg] = M;
+      }
+    }
+    if (half == 1) return;
+  }
+#pragma unroll
+  for (int qg = 0; qg < NG; ++qg) {
+    float lt = l[qg];
+    lt += __shfl_xor(lt, 16, 64);
+    lt += __shfl_xor(lt, 32, 64);
+    if (chi[qg] < 0) continue;
+    const float inv = lt > 0.f ? 1.f / lt : 0.f;
+    bf16_t* op = out + (size_t)tok[qg] * out_stride + (size_t)head * HD;
+#pragma unroll
+    for (int n = 0; n < 2 * NQK; ++n)
+      *reinterpret_cast<uint2*>(op + 16 * n + 4 * g) =
+          make_uint2(pack2_bf16(acc[qg][n][0] * inv, acc[qg][n][1] * inv),
+                     pack2_bf16(acc[qg][n][2] * inv, acc[qg][n][3] * inv));
+  }
+}
+
 // tokens of one request a prompt tile may hold
 extern "C" int ullm_attention_prefill_tile(void) { return 16 * PREFILL_GROUPS; }
 
@@ -1192,7 +1597,16 @@ extern "C" int ullm_attention_decode_static(
 }
 
 template <int N, typename... Args>
-static void prefill_launch(int halves, unsigned blocks, hipStream_t stream, Args... args) {
+static void prefill_launch(int halves, bool staged, unsigned blocks, hipStream_t stream, Args... args) {
+  if constexpr (N == 2 || N == 4) {
+    if (!staged) {                                        // tiles straight to shared memory
+      if (halves == 2)
+        hipLaunchKernelGGL((attention_prefill_dma_kernel<N, 2>), dim3(blocks), dim3(64 * PREFILL_WAVES * 2), 0, stream, args...);
+      else
+        hipLaunchKernelGGL((attention_prefill_dma_kernel<N, 1>), dim3(blocks), dim3(64 * PREFILL_WAVES), 0, stream, args...);
+      return;
+    }
+  }
   if constexpr (N <= 4) {
     if (halves == 2) {
       hipLaunchKernelGGL((attention_prefill_kernel<N, 2>), dim3(blocks), dim3(64 * PREFILL_WAVES * 2), 0, stream, args...);
@@ -1229,6 +1643,8 @@ extern "C" int ullm_attention_prefill(
     long long keys_total, int keys_max, hipStream_t stream) {
   if (n_tiles <= 0) return 0;
   if (!ullm_attention_mfma_supports(hd, page_size, nq, nkv)) return ULLM_ERR_UNSUPPORTED;
+  const bool staged = halves >= 10;                       // 10, 11, 12: as 0, 1, 2 with the kernel that stages tiles in registers
+  if (staged) halves -= 10;
   if (window < 0 || halves < 0 || halves > 2) return ULLM_ERR_SHAPE;
   const int chunks = (nq / nkv + PREFILL_WAVES - 1) / PREFILL_WAVES;
   const long long blocks = (long long)n_tiles * nkv * chunks;
@@ -1250,7 +1666,7 @@ extern "C" int ullm_attention_prefill(
     halves = (enough && blocks >= 2 * units) ? 1 : 2;
   }
   const float sl = scale * 1.4426950408889634f;
-#define CALL(N) prefill_launch<N>(halves, (unsigned)blocks, stream, (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, \
+#define CALL(N) prefill_launch<N>(halves, staged, (unsigned)blocks, stream, (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, \
     (const bf16_t*)k_pool, (const bf16_t*)v_pool, tiles, positions, token_entry, block_table, bt_stride, page_size,    \
     nq, nkv, sl, window, n_tiles)
   DISPATCH_NQK(hd, CALL)

@@ -100,13 +100,15 @@ def prefill_attention(args) -> None:
         keys = [min(i + tile, T) for i in range(0, T, tile)]
         flops = 4 * nq * hd * T * (T + 1) / 2
         cells = []
-        for halves in (0, 1, 2):
+        # 11, 12: the kernel that stages tiles in registers, where the one that loads them straight to LDS would run
+        for halves in (0, 1, 2, 11, 12):
             calls = [(lambda v=v: ops.attention_prefill_mfma(q, out, k_pool, v_pool, tiles, tiles.shape[0], pos, ent, tables[v],
                                                              P, nq, nkv, hd, hd ** -0.5, 0, halves=halves,
                                                              keys_total=sum(keys), keys_max=max(keys)))
                      for v in range(nv)]
             t = graph_time(calls)
-            cells.append(f"halves {halves or 'chosen'}: {t:.1f} us = {flops / t / 1e6:.0f} TFLOP/s")
+            name = {0: "chosen", 11: "staged, halves 1", 12: "staged, halves 2"}.get(halves, f"halves {halves}")
+            cells.append(f"{name}: {t:.1f} us = {flops / t / 1e6:.0f} TFLOP/s")
         print(f"prompt attention, {T} tokens, {nq}/{nkv} heads of {hd}: " + "  ".join(cells), flush=True)
         del k_pool, v_pool
 
