@@ -437,7 +437,10 @@ def test_attention_on_the_matrix_cores(ops, case):
         t0 += n
     # prompt tiles: two halves of a block sharing the keys, one block taking all, and the chooser with
     # figures that send it either way
-    halves = ((0, {}), (1, {}), (2, {}), (0, dict(keys_total=10 ** 9, keys_max=1)), (0, dict(keys_total=1, keys_max=10 ** 6)))
+    # (11, 12: the kernel that stages tiles in registers, also where head size 128 has the one that loads them
+    # straight to shared memory)
+    halves = ((0, {}), (1, {}), (2, {}), (0, dict(keys_total=10 ** 9, keys_max=1)), (0, dict(keys_total=1, keys_max=10 ** 6)),
+              (11, {}), (12, {}))
     for i, (splits, waves) in enumerate(((0, 0), (1, 4), (1, 8), (2, 8), (3, 4), (7, 8), (1, 1), (2, 1))):
         out = torch.full((q.shape[0], nq * hd), float("nan"), dtype=dtype, device=DEV)
         if dec:
@@ -626,7 +629,7 @@ def test_matrix_core_attention_finds_one_far_key_beyond_a_thousand_keys(ops, hd)
             for n in (5, 40):                     # one tile, and two tiles (the last query in the second)
                 qd, k_pool, v_pool, positions, entry, bt, v = _dominant_key_problem(hd, S, n, target, nq, nkv, P, seed=1)
                 tiles = [x for f in range(0, n, ops.PREFILL_TILE) for x in (f, min(ops.PREFILL_TILE, n - f))]
-                for halves in (1, 2):
+                for halves in (1, 2, 11, 12):
                     out = torch.zeros(n, nq * hd, dtype=torch.bfloat16, device=DEV)
                     ops.attention_prefill_mfma(qd, out, k_pool, v_pool, torch.tensor(tiles, dtype=torch.int32, device=DEV),
                                                len(tiles) // 2, positions, entry, bt, P, nq, nkv, hd, 1.0, window,
@@ -645,12 +648,57 @@ def test_matrix_core_attention_finds_one_far_key_beyond_a_thousand_keys(ops, hd)
                 got = out.float().cpu().view(nq, hd)
                 assert (got[0] - v[target, 0]).abs().max() > 0.1, ("decode sees past its window", window, splits, waves)
             qd, k_pool, v_pool, positions, entry, bt, v = _dominant_key_problem(hd, S, 5, target, nq, nkv, P, seed=3)
-            for halves in (1, 2):
+            for halves in (1, 2, 11, 12):
                 out = torch.zeros(5, nq * hd, dtype=torch.bfloat16, device=DEV)
                 ops.attention_prefill_mfma(qd, out, k_pool, v_pool, torch.tensor([0, 5], dtype=torch.int32, device=DEV), 1,
                                            positions, entry, bt, P, nq, nkv, hd, 1.0, window, halves=halves)
                 got = out.float().cpu().view(5, nq, hd)[-1]
                 assert (got[0] - v[target, 0]).abs().max() > 0.1, ("a prompt tile sees past its window", window, halves)
+
+
+def test_prompt_attention_over_more_keys_than_its_page_table_holds(ops):
+    """The prompt kernel for head size 128 keeps the page ids of 128 tiles (4096 keys) in shared memory and
+    refills them on the way: a dominant key on either side of every refill (one block taking all keys: 4096,
+    8192; two halves of a block: each half's own 4096th key) must be found, with and without a window, and all
+    query rows must agree with a plain softmax over the keys."""
+    hd, nq, nkv, P, S, n = 128, 4, 1, 16, 9001, 37
+    for window in (0, 6000):
+        lo = 0 if window == 0 else S - window
+        half = lo // 32 * 32 + ((S - lo // 32 * 32 + 31) // 32 + 1) // 2 * 32       # first key of the second half
+        seams = {lo, 4095, 4096, 4097, 8191, 8192, 8193, half - 1, half, half + 4095, half + 4096, S - 40, S - 1}
+        for target in sorted(t for t in seams if lo <= t < S):
+            qd, k_pool, v_pool, positions, entry, bt, v = _dominant_key_problem(hd, S, n, target, nq, nkv, P, seed=4)
+            tiles = [x for f in range(0, n, ops.PREFILL_TILE) for x in (f, min(ops.PREFILL_TILE, n - f))]
+            for halves in (1, 2, 12):
+                out = torch.zeros(n, nq * hd, dtype=torch.bfloat16, device=DEV)
+                ops.attention_prefill_mfma(qd, out, k_pool, v_pool, torch.tensor(tiles, dtype=torch.int32, device=DEV),
+                                           len(tiles) // 2, positions, entry, bt, P, nq, nkv, hd, 1.0, window, halves=halves)
+                got = out.float().cpu().view(n, nq, hd)
+                if target <= S - n:            # visible to every query of the portion; the last query looks straight at it
+                    for h in range(nq):
+                        assert (got[-1, h] - v[target, 0]).abs().max() < 3e-2, (window, target, halves, h)
+    # random data, every query row against a plain softmax
+    torch.manual_seed(6)
+    k = torch.randn(S, nkv, hd).bfloat16().float()
+    vv = torch.randn(S, nkv, hd).bfloat16().float()
+    q = torch.randn(n, nq, hd).bfloat16().float()
+    k_pool, v_pool, tables = paged_cache([k], [vv], P, torch.bfloat16, DEV, seed=3)
+    positions = torch.arange(S - n, S).int().to(DEV)
+    entry = torch.zeros(n, dtype=torch.int32, device=DEV)
+    bt = table_tensor(tables, DEV)
+    tiles = torch.tensor([x for f in range(0, n, ops.PREFILL_TILE) for x in (f, min(ops.PREFILL_TILE, n - f))], dtype=torch.int32, device=DEV)
+    scale = hd ** -0.5
+    for window in (0, 6000):
+        scores = torch.einsum("qhd,kd->qhk", q, k[:, 0]) * scale
+        pos = torch.arange(S - n, S)[:, None, None]
+        keys = torch.arange(S)[None, None, :]
+        hidden = (keys > pos) | ((keys <= pos - window) if window else torch.zeros_like(keys > pos))
+        want = torch.einsum("qhk,kd->qhd", torch.softmax(scores.masked_fill(hidden, float("-inf")), -1), vv[:, 0]).reshape(n, -1)
+        for halves in (0, 1, 2):
+            out = torch.zeros(n, nq * hd, dtype=torch.bfloat16, device=DEV)
+            ops.attention_prefill_mfma(q.reshape(n, -1).to(DEV, torch.bfloat16), out, k_pool, v_pool, tiles, tiles.numel() // 2,
+                                       positions, entry, bt, P, nq, nkv, hd, scale, window, halves=halves)
+            assert (out.float().cpu() - want).abs().max() <= tol(torch.bfloat16, want), (window, halves)
 
 
 def test_matrix_core_attention_with_scores_that_climb(ops):

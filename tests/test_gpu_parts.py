@@ -270,7 +270,12 @@ def test_norm_left_to_the_feed_forwards_first_projection(monkeypatch):
     from ullm_amd.kernels import ops
     seen, inner = [], ops.gemm_skinny_normed
     monkeypatch.setattr(ops, "gemm_skinny_normed", lambda *a, **k: seen.append(1) or inner(*a, **k))
-    for T, folded in ((1, True), (7, True), (8, True), (9, False), (16, False)):
+    # a small matrix keeps the norm inside for every row count the kernel takes, a large one up to 8 rows
+    from ullm_amd.parts import linear as linear_rules
+    cases = [(T, True, None) for T in (1, 7, 8, 9, 16)] + [(T, T <= 8, 0) for T in (8, 9, 16)]
+    for T, folded, small in cases:
+        if small is not None:
+            monkeypatch.setattr(linear_rules, "NORM_FOLDED_SMALL_WEIGHT", small)
         stream = torch.randn(T, H) * torch.logspace(-2, 2, T)[:, None]
         want = stream + plain.qwen3_mlp(plain.rms_norm(stream, gain, eps), {k: v.float() for k, v in w.items()}, "f")
         got = stream.clone().to(DEV)

@@ -1044,7 +1044,7 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __r
 }
 
 // ------------------------------------------------------------------------------- prompt portions, tiles straight to LDS
-// The same work split as attention_prefill_kernel, for head sizes 64 and 128, with the 32-key tiles of
+// The same work split as attention_prefill_kernel, for head size 128, with the 32-key tiles of
 // keys and values fetched by loads that write shared memory themselves (global_load_lds_dwordx4: a
 // wave's 64 lanes fill 1024 consecutive bytes, every lane from an address of its own).  No register
 // holds a tile on its way, no instruction copies it, and four tiles of shared memory take turns, so the
@@ -1093,7 +1093,7 @@ struct DmaTile {
   static constexpr int ROUNDS = NQK / 2;  // load instructions per wave for a tile's keys, and as many for its values
   static constexpr int KBYTES = 32 * 2 * HD, VBYTES = HD * 64;
   static constexpr int BYTES = KBYTES + VBYTES;
-  static_assert(NQK == 2 || NQK == 4, "head sizes 64 and 128");
+  static_assert(NQK == 4, "head size 128 (with 64 the staged kernel is the faster one)");
   // the row that key k (0 .. 31) has in its score product, and what its pieces' places are xor-ed with
   __host__ __device__ static constexpr int row_of_key(int k) { return (k & 3) | (((k >> 3) & 3) << 2); }
   __host__ __device__ static constexpr int key_swizzle(int k) { return PR == 16 ? row_of_key(k) : row_of_key(k) >> 1; }
@@ -1598,7 +1598,7 @@ extern "C" int ullm_attention_decode_static(
 
 template <int N, typename... Args>
 static void prefill_launch(int halves, bool staged, unsigned blocks, hipStream_t stream, Args... args) {
-  if constexpr (N == 2 || N == 4) {
+  if constexpr (N == 4) {
     if (!staged) {                                        // tiles straight to shared memory
       if (halves == 2)
         hipLaunchKernelGGL((attention_prefill_dma_kernel<N, 2>), dim3(blocks), dim3(64 * PREFILL_WAVES * 2), 0, stream, args...);
