@@ -122,6 +122,17 @@ def test_state_mixer_steps_replayed_from_graphs(tmp_path, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_scaled_embedding_head_bias_and_capped_logits(tmp_path, dtype):
+    """What a plan may say about the two ends of the model: the token rows scaled on their way into the
+    stream, a bias on the logits, and a soft cap on them (tight enough here to bend the largest logits)."""
+    cfg = base_cfg([ATT, dict(ATT, heads=4, kv_heads=2, head_dim=32)], embed_scale=72 ** 0.5, head_bias=True, logit_cap=3.0)
+    rep, w = run_and_compare(tmp_path, cfg, dtype, CUTS[2], seed=13)
+    assert "head.bias" in w and float(w["head.bias"].abs().max()) > 0
+    cfg = base_cfg([ATT], tie=True, embed_scale=0.5, logit_cap=50.0)
+    run_and_compare(tmp_path, cfg, dtype, CUTS[1], seed=14)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_only_state_layers_need_no_pages(tmp_path, dtype):
     cfg = base_cfg([TOY, TOY], tie=True)
     rep, _ = run_and_compare(tmp_path, cfg, dtype, CUTS[2])

@@ -182,7 +182,8 @@ def toy_plan(cfg: dict) -> ModelPlan:
     return ModelPlan(vocab_size=cfg["vocab_size"], hidden_size=H, embedding_weight="tok.weight", layers=layers,
                      final_norm=Choice("norm", "rmsnorm", dict(size=H, eps=eps, weight_name="out_norm.weight")),
                      head_weight="head.weight", tie_head_to_embedding=cfg.get("tie", False), run_order=order,
-                     init_std=cfg.get("init_std", 0.05))
+                     init_std=cfg.get("init_std", 0.05), embedding_scale=cfg.get("embed_scale", 1.0),
+                     head_bias="head.bias" if cfg.get("head_bias") else None, logit_softcap=cfg.get("logit_cap", 0.0))
 
 
 register_architecture("ToyStackForCausalLM", toy_config_from_dict, toy_plan)
@@ -214,7 +215,7 @@ def toy_forward(w: Dict[str, torch.Tensor], cfg: dict, token_ids: List[int]) -> 
     w = {k: v.float() for k, v in w.items()}
     T, eps = len(token_ids), cfg["eps"]
     positions = torch.arange(T)
-    h = w["tok.weight"][torch.tensor(token_ids)]
+    h = w["tok.weight"][torch.tensor(token_ids)] * cfg.get("embed_scale", 1.0)
     order = cfg.get("run_order") or [[i, i] for i in range(len(cfg["layers"]))]
     kv_of: Dict[int, tuple] = {}
     for layer, cache_id in order:
@@ -257,4 +258,6 @@ def toy_forward(w: Dict[str, torch.Tensor], cfg: dict, token_ids: List[int]) -> 
                             plain.linear(x, w[f"{p}.ffn.up_proj.weight"])), -1)
             h = h + plain.linear(plain.silu_and_mul(gu), w[f"{p}.ffn.down_proj.weight"])
     x = plain.rms_norm(h, w["out_norm.weight"], eps)
-    return plain.linear(x, w["head.weight"] if "head.weight" in w else w["tok.weight"])
+    logits = plain.linear(x, w["head.weight"] if "head.weight" in w else w["tok.weight"], w.get("head.bias"))
+    cap = cfg.get("logit_cap", 0.0)
+    return cap * torch.tanh(logits / cap) if cap else logits

@@ -31,10 +31,10 @@ __device__ __forceinline__ void st4_f32(bf16_t* p, float4 v) {
 
 
 // ------------------------------------------------------------------ embedding
-// residual[t, :] = float(table[ids[t], :]); ids outside [0, V) give a zero row.
+// residual[t, :] = scale * float(table[ids[t], :]); ids outside [0, V) give a zero row.
 template <typename T>
 __global__ void embedding_kernel(const int* __restrict__ ids, const T* __restrict__ table,
-                                 float* __restrict__ residual, int H, int V) {
+                                 float* __restrict__ residual, int H, int V, float scale) {
   const int t = blockIdx.x;
   const int id = ids[t];
   float* out = residual + (size_t)t * H;
@@ -44,24 +44,43 @@ __global__ void embedding_kernel(const int* __restrict__ ids, const T* __restric
   }
   const T* row = table + (size_t)id * H;
   if (H % 4 == 0 && !(((uintptr_t)table | (uintptr_t)residual) & 15)) {
-    for (int i = 4 * threadIdx.x; i < H; i += 4 * blockDim.x)
-      *reinterpret_cast<float4*>(out + i) = ld4_f32(row + i);
+    for (int i = 4 * threadIdx.x; i < H; i += 4 * blockDim.x) {
+      const float4 v = ld4_f32(row + i);
+      *reinterpret_cast<float4*>(out + i) = make_float4(v.x * scale, v.y * scale, v.z * scale, v.w * scale);
+    }
     return;
   }
-  for (int i = threadIdx.x; i < H; i += blockDim.x) out[i] = ld_f32(row + i);
+  for (int i = threadIdx.x; i < H; i += blockDim.x) out[i] = ld_f32(row + i) * scale;
 }
 
 extern "C" int ullm_embedding(const int* ids, const void* table, float* residual, int T_, int H,
-                              int V, int dtype, hipStream_t stream) {
+                              int V, int dtype, float scale, hipStream_t stream) {
   if (T_ <= 0) return 0;
   if (H <= 0 || V <= 0) return ULLM_ERR_SHAPE;
   dim3 grid(T_), block(256);
   if (dtype == ULLM_F32)
-    hipLaunchKernelGGL(embedding_kernel<float>, grid, block, 0, stream, ids, (const float*)table, residual, H, V);
+    hipLaunchKernelGGL(embedding_kernel<float>, grid, block, 0, stream, ids, (const float*)table, residual, H, V, scale);
   else if (dtype == ULLM_BF16)
-    hipLaunchKernelGGL(embedding_kernel<bf16_t>, grid, block, 0, stream, ids, (const bf16_t*)table, residual, H, V);
+    hipLaunchKernelGGL(embedding_kernel<bf16_t>, grid, block, 0, stream, ids, (const bf16_t*)table, residual, H, V, scale);
   else
     return ULLM_ERR_DTYPE;
+  ULLM_LAUNCH_CHECK();
+}
+
+// ------------------------------------------------------------------ a soft cap on the logits
+// x = cap * tanh(x / cap), in place, float32 [rows, cols] with row stride ld
+__global__ void softcap_kernel(float* __restrict__ x, int cols, int ld, float cap) {
+  float* row = x + (size_t)blockIdx.y * ld;
+  const float inv = 1.f / cap;
+  for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < cols; i += gridDim.x * blockDim.x) row[i] = cap * tanhf(row[i] * inv);
+}
+
+extern "C" int ullm_softcap(float* x, int rows, int cols, int ld, float cap, hipStream_t stream) {
+  if (rows <= 0 || cols <= 0) return 0;
+  if (!(cap > 0.f) || ld < cols || rows > 65535) return ULLM_ERR_SHAPE;
+  int bx = (cols + 1023) / 1024;
+  if (bx > 256) bx = 256;
+  hipLaunchKernelGGL(softcap_kernel, dim3(bx, rows), dim3(256), 0, stream, x, cols, ld, cap);
   ULLM_LAUNCH_CHECK();
 }
 

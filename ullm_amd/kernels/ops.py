@@ -72,8 +72,8 @@ def _check_pools(k_pool, v_pool, nkv: int, page_size: int, hd: int, dtype) -> No
 
 # ---------------------------------------------------------------------------------- elementwise
 
-def embedding(ids: torch.Tensor, table: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """float32 [T, H] rows of ``table`` [V, H] at ``ids`` [T] (int32)."""
+def embedding(ids: torch.Tensor, table: torch.Tensor, out: Optional[torch.Tensor] = None, scale: float = 1.0) -> torch.Tensor:
+    """float32 [T, H] rows of ``table`` [V, H] at ``ids`` [T] (int32), times ``scale``."""
     T = ids.numel()
     V, H = table.shape
     _i32(ids, "ids")
@@ -83,8 +83,16 @@ def embedding(ids: torch.Tensor, table: torch.Tensor, out: Optional[torch.Tensor
     _need(out.dtype == torch.float32 and out.is_contiguous() and out.shape == (T, H), "bad embedding output")
     lib = build.load("elementwise")
     _check(lib.ullm_embedding(_p(ids), _p(table), _p(out), _c_int(T), _c_int(H), _c_int(V),
-                              _c_int(_dt(table)), _stream()), "embedding")
+                              _c_int(_dt(table)), _c_float(scale), _stream()), "embedding")
     return out
+
+
+def softcap_(x: torch.Tensor, cap: float) -> torch.Tensor:
+    """x = cap * tanh(x / cap) in place, float32 [rows, cols]."""
+    _need(x.dtype == torch.float32 and x.dim() == 2 and x.stride(1) == 1 and cap > 0, "softcap takes float32 [rows, cols] and a cap > 0")
+    _check(build.load("elementwise").ullm_softcap(_p(x), _c_int(x.shape[0]), _c_int(x.shape[1]), _c_int(x.stride(0)),
+                                                  _c_float(cap), _stream()), "softcap")
+    return x
 
 
 def feed_tokens(ids: torch.Tensor, feed: torch.Tensor, source: torch.Tensor) -> None:

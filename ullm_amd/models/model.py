@@ -40,6 +40,9 @@ class ModelPlan:
     final_norm: Choice
     head_weight: str                         # tensor name of the output matrix [vocab, hidden]
     tie_head_to_embedding: bool = False      # bind the token table where the head tensor is absent
+    embedding_scale: float = 1.0             # the token rows are multiplied by this on their way into the stream
+    head_bias: Optional[str] = None          # tensor name of a bias [vocab] on the logits, float32
+    logit_softcap: float = 0.0               # > 0: logits = cap * tanh(logits / cap)
     # The order layers run in: (layer, cache id).  A layer may appear more than once (with a cache id
     # of its own each time, or the same one).  The first entry that names a cache id owns that cache
     # and writes it; later entries with the same id only read it, so a layer can read the cache
@@ -64,6 +67,7 @@ class Model:
             self.cache_owner.setdefault(cache_id, idx)
         self.embedding: Optional[torch.Tensor] = None
         self.head: Optional[torch.Tensor] = None
+        self.head_bias: Optional[torch.Tensor] = None
         self.env: Optional[PartEnv] = None
 
     # ------------------------------------------------------------------ weights
@@ -79,12 +83,15 @@ class Model:
             decls.extend(part.weights())
         decls.append(WeightDecl(p.head_weight, (p.vocab_size, p.hidden_size),
                                 alias_of=p.embedding_weight if p.tie_head_to_embedding else None))
+        if p.head_bias:
+            decls.append(WeightDecl(p.head_bias, (p.vocab_size,), keep_fp32=True))
         return decls
 
     def bind(self, tensors: Dict[str, torch.Tensor], env: PartEnv) -> None:
         self.env = env
         self.embedding = tensors[self.plan.embedding_weight].contiguous()
         self.head = tensors[self.plan.head_weight].contiguous()
+        self.head_bias = tensors[self.plan.head_bias].contiguous() if self.plan.head_bias else None
         for part in self.parts():
             part.bind(tensors, env)
 
@@ -122,7 +129,7 @@ class Model:
     def forward(self, ctx: StepContext, caches: Dict[int, LayerCache], logit_rows: Optional[torch.Tensor]):
         """Runs the batch through every layer of the run order and returns float32 logits
         [len(logit_rows), vocab] (None if no row is wanted)."""
-        residual = ops.embedding(ctx.token_ids, self.embedding)
+        residual = ops.embedding(ctx.token_ids, self.embedding, scale=self.plan.embedding_scale)
         pending = None
         for idx, (layer, cache_id) in enumerate(self.run_order):
             cache = caches.get(cache_id)
@@ -134,4 +141,7 @@ class Model:
         if logit_rows is None or logit_rows.numel() == 0:
             return None
         x = self.final_norm.add_norm(pending, residual, rows=logit_rows, out_dtype=ctx.dtype)
-        return linear(x, self.head, out_dtype=torch.float32)
+        logits = linear(x, self.head, self.head_bias, out_dtype=torch.float32)
+        if self.plan.logit_softcap > 0:
+            ops.softcap_(logits, self.plan.logit_softcap)
+        return logits
