@@ -470,8 +470,9 @@ def decode_split(n_items: int, nkv: int, groups: int, max_kv: int, hd: int = 128
     tiles = -(-max_kv // 32)
     if pairs > 256:
         # single waves, two to four to a SIMD, so that the launch has no rounds of whole blocks (four-wave blocks,
-        # one to a compute unit, take 49 us at 264 pairs against 30 us at 256); up to 576 pairs cut in two
-        return 1, (2 if pairs <= 576 and tiles > 16 else 1)
+        # one to a compute unit, take 49 us at 264 pairs against 30 us at 256); up to 576 pairs cut in three where
+        # that still gives at most one wave per SIMD and compute unit, else in two
+        return 1, (max(2, min(3, 1024 // pairs)) if pairs <= 576 and tiles > 16 else 1)
     if pairs == 256:
         return (4 if tiles > 16 else 1), 1
     splits = min(16, max(1, 512 // pairs), tiles)
