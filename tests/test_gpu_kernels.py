@@ -677,6 +677,16 @@ def test_prompt_attention_over_more_keys_than_its_page_table_holds(ops):
                 if target <= S - n:            # visible to every query of the portion; the last query looks straight at it
                     for h in range(nq):
                         assert (got[-1, h] - v[target, 0]).abs().max() < 3e-2, (window, target, halves, h)
+    # the same seams for a single decoded token, whose kernel fetches page ids 1024 keys at a time
+    for target in (1023, 1024, 4095, 4096, 8191, 8192, S - 1):
+        qd, k_pool, v_pool, positions, entry, bt, v = _dominant_key_problem(hd, S, 1, target, nq, nkv, P, seed=5)
+        for splits, waves in ((1, 1), (1, 8), (2, 8), (16, 1), (5, 4)):
+            out = torch.zeros(1, nq * hd, dtype=torch.bfloat16, device=DEV)
+            ops.attention_decode_mfma(qd, out, k_pool, v_pool, None, 1, positions, entry, bt, P, nq, nkv, hd, 1.0, 0, S,
+                                      splits=splits, waves=waves)
+            got = out.float().cpu().view(nq, hd)
+            for h in range(nq):
+                assert (got[h] - v[target, 0]).abs().max() < 3e-2, ("decode", target, splits, waves, h)
     # random data, every query row against a plain softmax
     torch.manual_seed(6)
     k = torch.randn(S, nkv, hd).bfloat16().float()
