@@ -164,3 +164,15 @@ def test_prefix_sharing_skips_cached_pages_at_admission():
     sched.add(req(1, 10))                                  # the same tokens
     out = run_step(sched, cache)
     assert [(s.start, s.num_tokens) for s in out] == [(8, 2)]
+
+
+def test_batch_buckets_of_the_captured_decode_graphs():
+    """A decode step replays the graph of the next bucket: never smaller than the batch, less than half as large again
+    from 33 requests on, and the same bucket for every batch up to it."""
+    from ullm_amd.engine.runner import batch_bucket
+    assert [batch_bucket(n) for n in (1, 2, 3, 8, 9, 16, 17, 32)] == [1, 2, 4, 8, 16, 16, 32, 32]
+    assert [batch_bucket(n) for n in (33, 48, 49, 64, 65, 96, 97, 128, 129, 192, 193, 256)] == \
+        [48, 48, 64, 64, 96, 96, 128, 128, 192, 192, 256, 256]
+    for n in range(1, 600):
+        b = batch_bucket(n)
+        assert b >= n and batch_bucket(b) == b and (n <= 32 or 2 * b < 3 * n)

@@ -38,6 +38,16 @@ class StepError(RuntimeError):
 UNKNOWN_TOKEN = -2         # stands for a token that is still being sampled when the step is prepared
 
 
+def batch_bucket(n: int) -> int:
+    """The batch size of the captured graph that a decode step of ``n`` requests replays: the next power of
+    two, or three quarters of it from 48 on (48, 96, 192: whole 16-row tiles, and the projections' cost
+    follows the number of such tiles from there on; below, the kernels take 16 or 32 rows at one cost)."""
+    b = 1
+    while b < n:
+        b *= 2
+    return b * 3 // 4 if b >= 64 and n <= b * 3 // 4 else b
+
+
 class ModelRunner:
     def __init__(self, model: Model, env: PartEnv, page_size: int, num_pages, max_requests: int,
                  enable_prefix_cache: bool = False, use_graphs: bool = True, max_graph_batch: int = 256):
@@ -259,10 +269,7 @@ class ModelRunner:
         must already be in the state in which the step will find them."""
         entries = list(entries)
         if (self.use_graphs and len(entries) <= self.max_graph_batch and all(len(e.tokens) == 1 for e in entries)):
-            B = len(entries)
-            b_pad = 1
-            while b_pad < B:
-                b_pad *= 2
+            b_pad = batch_bucket(len(entries))
             longest = max(e.cache.num_computed + 1 for e in entries)
             kv_bucket = 256
             while kv_bucket < longest:
