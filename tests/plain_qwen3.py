@@ -127,10 +127,12 @@ def qwen3_mlp(x, w: Dict[str, torch.Tensor], prefix: str):
 def window_of_layer(cfg: dict, layer: int) -> int:
     """The reference reads none of the sliding-window keys (0 everywhere).  When a config switches
     ``use_sliding_window`` on, layers from ``max_window_layers`` on look back ``sliding_window``
-    keys, the current one included."""
-    if cfg.get("use_sliding_window", False) and layer >= cfg.get("max_window_layers", cfg["num_hidden_layers"]):
-        return int(cfg["sliding_window"])
-    return 0
+    keys, the current one included; a list ``layer_types`` names the layers that do instead."""
+    if not cfg.get("use_sliding_window", False):
+        return 0
+    if cfg.get("layer_types"):
+        return int(cfg["sliding_window"]) if cfg["layer_types"][layer] == "sliding_attention" else 0
+    return int(cfg["sliding_window"]) if layer >= cfg.get("max_window_layers", cfg["num_hidden_layers"]) else 0
 
 
 def qwen3_forward(w: Dict[str, torch.Tensor], cfg: dict, token_ids: List[int]) -> torch.Tensor:

@@ -51,6 +51,18 @@ def test_bad_values_are_refused():
 def test_window_is_chosen_layer_by_layer():
     c = Qwen3Config.from_dict(TINY_C)
     assert [c.window_of_layer(i) for i in range(3)] == [0, 24, 24]
+    # a list of the layers' kinds wins over max_window_layers; without use_sliding_window it may name no window
+    kinds = ["sliding_attention", "full_attention", "sliding_attention"]
+    listed = Qwen3Config.from_dict(dict(TINY_C, layer_types=kinds))
+    assert [listed.window_of_layer(i) for i in range(3)] == [24, 0, 24] and listed.to_dict()["layer_types"] == kinds
+    plain = Qwen3Config.from_dict(dict(TINY_A, layer_types=["full_attention"] * TINY_A["num_hidden_layers"]))
+    assert all(plain.window_of_layer(i) == 0 for i in range(plain.num_hidden_layers))
+    with pytest.raises(ConfigError, match="layer_types"):
+        Qwen3Config.from_dict(dict(TINY_C, layer_types=kinds[:2]))
+    with pytest.raises(ConfigError, match="layer_types"):
+        Qwen3Config.from_dict(dict(TINY_C, layer_types=["full_attention", "chunked", "full_attention"]))
+    with pytest.raises(ConfigError, match="use_sliding_window"):
+        Qwen3Config.from_dict(dict(TINY_C, use_sliding_window=False, layer_types=kinds))
     _, model = build_model(TINY_C)
     groups, cache_group, states = model.cache_layout()
     assert len(groups) == 2 and not states

@@ -317,6 +317,8 @@ def test_random_configurations(tmp_path, trial, matrix_cores):
         cfg["head_dim"] = rng.choice([32, 64, 96, 128, 256])
         cfg["use_sliding_window"] = trial % 2 == 0
         page_size, n = rng.choice([16, 32, 64]), rng.choice([97, 150, 230])
+    if cfg["use_sliding_window"] and trial % 3 == 0:          # the windowed layers named one by one
+        cfg["layer_types"] = [rng.choice(["full_attention", "sliding_attention"]) for _ in range(cfg["num_hidden_layers"])]
     assert ops.attention_mfma_supports(torch.bfloat16, cfg["head_dim"], page_size, cfg["num_attention_heads"], nkv) == matrix_cores \
         or not matrix_cores
     d = write_random_model(cfg, str(tmp_path / "m"), seed=trial)

@@ -76,6 +76,7 @@ class Qwen3Config:
     use_sliding_window: bool
     sliding_window: int
     max_window_layers: int
+    layer_types: tuple            # per layer "full_attention" / "sliding_attention", or () where config.json has no list
     torch_dtype: str
     eos_token_id: int             # the first stop id config.json names (-1: none)
     eos_token_ids: tuple          # all of them: config.json may hold a list
@@ -107,6 +108,16 @@ class Qwen3Config:
         if use_window and window <= 0:
             raise ConfigError("config.json: use_sliding_window is true but 'sliding_window' "
                               "is missing or not positive")
+        kinds = d.get("layer_types")
+        if kinds is None:
+            kinds = ()
+        elif (not isinstance(kinds, (list, tuple)) or len(kinds) != layers
+              or any(k not in ("full_attention", "sliding_attention") for k in kinds)):
+            raise ConfigError(f"config.json: layer_types={kinds!r} must name 'full_attention' or 'sliding_attention' "
+                              f"for each of the {layers} layers")
+        elif "sliding_attention" in kinds and not use_window:
+            raise ConfigError("config.json: layer_types names sliding_attention layers but use_sliding_window is "
+                              "not true: which keys such a layer sees is not defined")
         act = _take(d, "hidden_act", str, "silu")
         if act != "silu":
             raise ConfigError(f"config.json: hidden_act={act!r}; this architecture's "
@@ -146,6 +157,7 @@ class Qwen3Config:
             use_sliding_window=use_window,
             sliding_window=window,
             max_window_layers=max_window_layers,
+            layer_types=tuple(kinds),
             torch_dtype=dtype,
             eos_token_id=int(eos_ids[0]) if eos_ids else -1,
             eos_token_ids=tuple(int(e) for e in eos_ids),
@@ -164,13 +176,21 @@ class Qwen3Config:
     def to_dict(self) -> dict:
         d = asdict(self)
         d["architectures"] = list(self.architectures)
+        d["eos_token_ids"] = list(self.eos_token_ids)
+        if self.layer_types:
+            d["layer_types"] = list(self.layer_types)
+        else:
+            del d["layer_types"]
         return d
 
     def window_of_layer(self, layer: int) -> int:
-        """Keys a query of this layer may look back over, itself included; 0 = all."""
-        if self.use_sliding_window and layer >= self.max_window_layers:
-            return self.sliding_window
-        return 0
+        """Keys a query of this layer may look back over, itself included; 0 = all.  A per-layer list in
+        config.json decides where there is one, else the layers from ``max_window_layers`` on have the window."""
+        if not self.use_sliding_window:
+            return 0
+        if self.layer_types:
+            return self.sliding_window if self.layer_types[layer] == "sliding_attention" else 0
+        return self.sliding_window if layer >= self.max_window_layers else 0
 
 
 def read_config_json(model_dir: str) -> dict:
