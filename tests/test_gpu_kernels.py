@@ -534,7 +534,9 @@ def test_decode_attention_with_norm_rotation_and_cache_write_folded_in(ops, case
         got = out[:len(lens)].float().cpu()
         assert not torch.isnan(got).any(), (splits, waves)
         assert (got - want).abs().max() <= tol(dtype, want), (splits, waves)
-        assert (got - out_two[:len(lens)].float().cpu()).abs().max() <= 0.25 * tol(dtype, want), (splits, waves)
+        # against the two kernels: a quarter of the tolerance, or one bfloat16 step of the largest output
+        near = max(0.25 * tol(dtype, want), 2.0 ** -7 * float(want.abs().max()))
+        assert (got - out_two[:len(lens)].float().cpu()).abs().max() <= near, (splits, waves)
         # the cache: the same rows written, keys within a rounding of the other kernel's, values bit for bit
         assert torch.equal(torch.isnan(k_one), torch.isnan(k_two)) and torch.equal(torch.isnan(v_one), torch.isnan(v_two))
         assert torch.equal(torch.nan_to_num(v_one.float()), torch.nan_to_num(v_two.float()))
