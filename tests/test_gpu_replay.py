@@ -340,6 +340,69 @@ def test_random_configurations(tmp_path, trial, matrix_cores):
         close(np.concatenate(outs), want, dtype)
 
 
+@pytest.mark.parametrize("trial", range(16))
+def test_random_mixed_traces(tmp_path, trial):
+    """Random configurations under random traces: up to four live requests in a pool that holds just them,
+    each cut in its own manner (portions of changing size, most of it at once and then single tokens, single
+    tokens from its middle on), some left out of a step; a request is admitted as soon as the pool has room,
+    on pages that others gave back.  Every position's logits equal the plain model's, in both dtypes."""
+    import random
+    from ullm_amd.replay import Replayer
+    from ullm_amd.weights.random_init import write_random_model
+    rng = random.Random(5000 + trial)
+    nkv = rng.choice([1, 2, 3, 4, 8])
+    cfg = dict(architectures=["Qwen3ForCausalLM"], hidden_size=rng.choice([40, 72, 96, 136, 200, 264]),
+               num_hidden_layers=rng.choice([1, 2, 3]), num_attention_heads=nkv * rng.choice([1, 2, 3, 4, 5, 7, 8]),
+               num_key_value_heads=nkv, head_dim=rng.choice([16, 32, 48, 64, 80, 96, 112, 128, 256]),
+               intermediate_size=rng.choice([56, 104, 200, 328]), vocab_size=rng.choice([101, 257, 503, 1000]),
+               rope_theta=rng.choice([1e4, 1e6]), rms_norm_eps=rng.choice([1e-5, 1e-6]), max_position_embeddings=1024,
+               tie_word_embeddings=rng.random() < 0.5, attention_bias=rng.random() < 0.3, initializer_range=0.05,
+               use_sliding_window=rng.random() < 0.4, sliding_window=rng.choice([7, 33, 100, 150]),
+               max_window_layers=rng.choice([0, 1]))
+    page_size = rng.choice([4, 8, 16, 32])
+    if trial % 2:                                             # shapes the matrix-core attention takes
+        cfg["head_dim"], page_size = rng.choice([32, 64, 96, 128, 256]), rng.choice([16, 32, 64])
+    d = write_random_model(cfg, str(tmp_path / "m"), seed=trial)
+    pc, w = plain.load_model_folder(d)
+    lens = [rng.choice([3, 20, 64, 65, 130, 257, 400]) for _ in range(rng.choice([2, 3, 4, 5, 6]))]
+    toks = {f"r{i}": [rng.randrange(cfg["vocab_size"]) for _ in range(n)] for i, n in enumerate(lens)}
+    want = {r: plain.qwen3_forward(w, pc, t).numpy() for r, t in toks.items()}
+    held = lambda r: -(-len(toks[r]) // 64) * 64             # noqa: E731
+    pool = max(sum(sorted((held(r) for r in toks), reverse=True)[:4]), 128)
+    manner = {r: rng.choice(["portions", "most, then single", "single from the middle"]) for r in toks}
+    steps, done, live, queue = [], {r: 0 for r in toks}, [], list(toks)
+    while queue or live:
+        while queue and len(live) < 4 and sum(held(x) for x in live) + held(queue[0]) <= pool:
+            live.append(queue.pop(0))
+        entries, end = [], []
+        for r in [r for r in live if rng.random() < 0.8] or [live[0]]:
+            left = len(toks[r]) - done[r]
+            if manner[r] == "portions":
+                n = min(left, rng.choice([1, 2, 3, 5, 17, 31, 32, 33, 64, 100]))
+            elif manner[r] == "most, then single":
+                n = left - 12 if left > 12 else 1
+            else:
+                n = min(left, rng.choice([2, 40])) if done[r] < len(toks[r]) // 2 else 1
+            entries.append((r, done[r], n))
+            done[r] += n
+            if done[r] == len(toks[r]):
+                end.append(r)
+        steps.append((entries, end))
+        live = [r for r in live if r not in end]
+    for dtype in ("float32", "bfloat16"):
+        rep = Replayer(d, dtype, pool, page_size, DEV)
+        for s, (entries, end) in enumerate(steps):
+            got = rep.step({"step": s, "end": end, "entries": [
+                {"id": r, "tokens": toks[r][at:at + n], "want": list(range(n))} for r, at, n in entries]})
+            row = 0
+            for r, at, n in entries:
+                bound = REL[dtype] * float(np.abs(want[r]).max()) + 1e-6
+                err = float(np.abs(got[row:row + n] - want[r][at:at + n]).max())
+                assert err <= bound, f"{dtype} step {s} request {r} tokens {at}..{at + n - 1}: {err:.3e} > {bound:.3e}"
+                row += n
+        assert not rep.live and rep.runner.cache.num_free_pages() == rep.max_tokens // page_size
+
+
 def test_bfloat16_attention_off_the_matrix_cores_is_announced(model_dirs, caplog):
     """Head sizes and page sizes the matrix-core kernels do not take run on the general kernel: right, but
     many times slower, so it is said once per shape."""
