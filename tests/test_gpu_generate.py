@@ -471,3 +471,78 @@ def test_command_line_with_random_weights(tmp_path, capsys):
         lines = [json.loads(x) for x in capsys.readouterr().out.strip().splitlines() if x.startswith("{")]
         runs.append(lines[0]["token_ids"])
     assert len(runs[0]) == 6 and runs[0] == runs[1] and runs[0] != runs[2]
+
+
+@pytest.mark.parametrize("trial", range(10))
+def test_random_engine_settings_change_no_token(tmp_path, trial):
+    """The same requests (seeded sampling, stop ids, every kind of length limit) through a roomy engine that runs
+    eagerly and waits for every step, and through one with settings drawn at random (pages for little more than
+    one request, small budgets and portions, prefix sharing, graphs, steps queued ahead); requests join while
+    others run and one may be aborted.  In 32-bit: the same tokens and the same reasons to stop."""
+    import random
+    from ullm_amd import LLM, EngineConfig, SamplingParams
+    from ullm_amd.weights.random_init import write_random_model
+    rng = random.Random(77000 + trial)
+    nkv = rng.choice([1, 2, 4])
+    cfg = dict(architectures=["Qwen3ForCausalLM"], hidden_size=rng.choice([40, 72, 96]), num_hidden_layers=rng.choice([1, 2]),
+               num_attention_heads=nkv * rng.choice([1, 2, 4]), num_key_value_heads=nkv, head_dim=rng.choice([16, 32, 64, 128]),
+               intermediate_size=rng.choice([56, 104]), vocab_size=rng.choice([31, 101, 257]), rope_theta=1e4,
+               rms_norm_eps=1e-6, max_position_embeddings=512, tie_word_embeddings=rng.random() < 0.5,
+               initializer_range=0.08, use_sliding_window=rng.random() < 0.3, sliding_window=rng.choice([7, 33]),
+               max_window_layers=rng.choice([0, 1]))
+    stop_ids = rng.choice([None, 3, [3, 5, 9]])
+    if stop_ids is not None:
+        cfg["eos_token_id"] = stop_ids
+    d = write_random_model(cfg, str(tmp_path / "m"), seed=trial)
+    V, page_size, n_req = cfg["vocab_size"], rng.choice([4, 8, 16]), rng.choice([2, 5, 9, 14])
+    shared = [rng.randrange(V) for _ in range(rng.choice([0, 0, 9, 40]))]
+    prompts = [shared + [rng.randrange(V) for _ in range(rng.choice([1, 2, 5, 17, 40, 70]))] for _ in range(n_req)]
+    params = []
+    for p in prompts:
+        kw = dict(temperature=rng.choice([0.0, 0.7, 1.0, 1.5]), top_k=rng.choice([-1, 5, 20]), top_p=rng.choice([1.0, 0.9]),
+                  min_p=rng.choice([0.0, 0.05]), seed=rng.randrange(1 << 20), ignore_eos=rng.random() < 0.3,
+                  stop_token_ids=rng.choice([[], [], [1, 2], [rng.randrange(V)]]))
+        limit = rng.choice(["new", "total", "both", "context"])
+        if limit in ("new", "both"):
+            kw["max_new_tokens"] = rng.choice([1, 2, 8, 30, 60])
+        if limit in ("total", "both"):
+            kw["max_tokens"] = len(p) + rng.choice([1, 3, 25])
+        if rng.random() < 0.3:
+            kw["eos_token_id"] = rng.randrange(V)
+        params.append(SamplingParams(**kw))
+    context_len = 160
+    one_request = -(-context_len // page_size) + 1
+    pages = rng.choice([one_request, one_request + 3, 2 * one_request, 8 * one_request])
+    base = dict(model=d, dtype="float32", context_len=context_len, page_size=page_size, device=DEV)
+    ids = [f"q{i}" for i in range(n_req)]
+    roomy = LLM(EngineConfig(**base, max_bs=16, num_pages=16 * one_request, enforce_eager=True, disable_async_scheduling=True))
+    want = roomy.generate(prompts, params, ids)
+    eng = LLM(EngineConfig(**base, max_bs=rng.choice([2, 4, 8, 16]), num_pages=pages,
+                           max_num_batched_tokens=rng.choice([8, 16, 33, 256]), max_prefill_chunk=rng.choice([3, 7, 16, 256]),
+                           enable_prefix_cache=rng.random() < 0.5, enforce_eager=rng.random() < 0.4,
+                           disable_async_scheduling=rng.random() < 0.3)).engine
+    abort = rng.randrange(n_req) if rng.random() < 0.3 and n_req > 2 else None
+    got, pending, steps = {}, list(range(n_req)), 0
+    while pending or eng.has_unfinished_requests():
+        for _ in range(rng.choice([0, 1, 1, 3])):
+            if pending:
+                i = pending.pop(0)
+                eng.add_request(ids[i], prompts[i], params[i])
+        if not eng.has_unfinished_requests():
+            continue
+        for out in eng.step():
+            got.setdefault(out.seq_id, []).append(out)
+        steps += 1
+        assert steps < 5000
+        if abort is not None and steps == 3:
+            if ids[abort] in eng.scheduler.requests:
+                eng.abort_request(ids[abort])
+            else:
+                abort = None
+    for i in range(n_req):
+        if i == abort:
+            continue
+        assert [o.new_token_id for o in got[ids[i]]] == want[i].token_ids
+        assert got[ids[i]][-1].finish_reason == want[i].finish_reason
+    eng.runner.cache.check()
+    assert eng.config.enable_prefix_cache or eng.runner.cache.num_free_pages() == pages
