@@ -713,6 +713,65 @@ def test_prompt_attention_over_more_keys_than_its_page_table_holds(ops):
             assert (out.float().cpu() - want).abs().max() <= tol(torch.bfloat16, want), (window, halves)
 
 
+@pytest.mark.parametrize("dtype,hd,nq", [(torch.bfloat16, 128, 8), (torch.float32, 64, 4)])
+def test_cache_pools_beyond_four_gibi_elements(ops, dtype, hd, nq):
+    """A cache sized for this GPU's memory: pools of five gibi-elements each (10 and 20 GiB) with the live pages
+    at their far end, where 32-bit element and byte offsets have wrapped.  Every kernel that touches the cache
+    (rotary + write, decode and prompt attention on the matrix cores, the fused decode step, the general
+    attention) must give, bit for bit, what it gives on a small pool, and write nowhere else."""
+    free, _ = torch.cuda.mem_get_info()
+    if free < (48 << 30):
+        pytest.skip("needs 48 GiB of free device memory")
+    torch.manual_seed(3)
+    nkv, P, lens = 2, 16, [(1, 300), (1, 37), (40, 200), (70, 70)]
+    rnd = lambda *s: torch.randn(*s).to(dtype).float()   # noqa: E731
+    ks, vs = [rnd(S, nkv, hd) for _, S in lens], [rnd(S, nkv, hd) for _, S in lens]
+    k_small, v_small, tables = paged_cache(ks, vs, P, dtype, DEV, fill=0.0)
+    n_small, big_pages = k_small.shape[0], (5 << 30) // (nkv * P * hd)
+    shift = big_pages - n_small
+    k_big = torch.zeros((big_pages, nkv, P, hd), dtype=dtype, device=DEV)
+    v_big = torch.zeros((big_pages, nkv, hd, P), dtype=dtype, device=DEV)
+    k_big[shift:], v_big[shift:] = k_small, v_small
+    positions = torch.cat([torch.arange(S - n, S) for n, S in lens]).int().to(DEV)
+    entry = torch.cat([torch.full((n,), b) for b, (n, _) in enumerate(lens)]).int().to(DEV)
+    T = positions.numel()
+    qkv = rnd(T, (nq + 2 * nkv) * hd).to(DEV, dtype)
+    gain = (1 + 0.1 * torch.randn(hd)).to(DEV)
+    inv = 1.0 / (10000.0 ** (torch.arange(0, hd, 2, dtype=torch.float32) / hd))
+    ang = torch.arange(302, dtype=torch.float32)[:, None] * inv[None]
+    table = torch.cat((ang.cos(), ang.sin()), -1).contiguous().to(DEV)
+    dec = torch.tensor([0, 1], dtype=torch.int32, device=DEV)
+    tiles = torch.tensor([x for t0, n in ((2, 40), (42, 70)) for f in range(0, n, ops.PREFILL_TILE)
+                          for x in (t0 + f, min(ops.PREFILL_TILE, n - f))], dtype=torch.int32, device=DEV)
+    scale, results = hd ** -0.5, []
+    for kp, vp, tb in ((k_small.clone(), v_small.clone(), tables), (k_big, v_big, [[p + shift for p in t] for t in tables])):
+        bt, res = table_tensor(tb, DEV), {}
+        q = torch.empty(T, nq * hd, dtype=dtype, device=DEV)
+        ops.qk_norm_rope_write(qkv, q, gain, gain, 1e-6, table, hd, 1, positions, entry, bt, kp, vp, P, nq, nkv, hd, write_kv=True)
+        res["q"] = q
+        new = lambda: torch.zeros(T, nq * hd, dtype=dtype, device=DEV)   # noqa: E731
+        if dtype == torch.bfloat16:
+            for splits, waves in ((0, 0), (1, 4), (3, 1)):
+                res[f"decode {splits}x{waves}"] = out = new()
+                ops.attention_decode_mfma(q, out, kp, vp, dec, 2, positions, entry, bt, P, nq, nkv, hd, scale, 0, 300,
+                                          splits=splits, waves=waves)
+            for halves in (1, 2, 11, 12):
+                res[f"prompt {halves}"] = out = new()
+                ops.attention_prefill_mfma(q, out, kp, vp, tiles, tiles.numel() // 2, positions, entry, bt, P, nq, nkv, hd,
+                                           scale, 0, halves=halves)
+            res["fused"] = out = new()
+            ops.attention_decode_fused(qkv, out, gain, gain, 1e-6, table, hd, 1, kp, vp, dec, 2, positions, entry, bt, P, nq,
+                                       nkv, hd, scale, 0, 300, write_kv=True)
+        res["general"] = ops.paged_attention_generic(q, kp, vp, positions, entry, bt, P, nq, nkv, hd, scale, 0, out=new())
+        res["keys"], res["values"] = kp[-n_small:].clone(), vp[-n_small:].clone()
+        results.append(res)
+    for name, small in results[0].items():
+        assert float(small.float().abs().max()) > 0 and torch.equal(small, results[1][name]), name
+    assert float(k_big[:shift].abs().max()) == 0 and float(v_big[:shift].abs().max()) == 0
+    del k_big, v_big, kp, vp, results
+    torch.cuda.empty_cache()           # the pools go back to the device, not to torch's cache
+
+
 def test_matrix_core_attention_with_scores_that_climb(ops):
     """The reference value of the exponentials follows the running maximum only in steps: scores that
     rise a little with every tile (so it lags, then jumps) and scores that fall must both come out right."""
