@@ -742,34 +742,20 @@ __device__ __forceinline__ void stage_store(const PrefillStage<NQK>& st, int key
   }
 }
 
-// Scores, softmax update and value product of one wave for the tile in LDS.  `masked` = some key of
-// the tile is hidden from some column (diagonal, window or end of data); otherwise no per-score test.
-// The queries come multiplied by scale * log2(e), and the first product of a score starts from minus
-// the column's reference value (`negm`, the same in all four elements) instead of zero, so the
-// products deliver the exponent itself: exp2 of it is the weight.  A column without a reference
-// value yet (m == NEG_BIG) counts from zero, and the first tile that shows it a key gives it one.
-template <int NQK, int NG, bool masked>
-__device__ __forceinline__ void process_tile_lds(const unsigned char* __restrict__ kl, const unsigned char* __restrict__ vl,
-                                                 int key0, const Pack8 (&qreg)[NG][NQK],
-                                                 const int (&col_lo)[NG], const int (&col_hi)[NG],
-                                                 f32x4_t (&acc)[NG][2 * NQK], float (&m)[NG], f32x4_t (&negm)[NG],
-                                                 float (&l)[NG]) {
-  using S = PrefillStage<NQK>;
-  const int lane = threadIdx.x & 63, g = lane >> 4, c = lane & 15;
-  f32x4_t s[NG][2];
-#pragma unroll
-  for (int sb = 0; sb < 2; ++sb)
-#pragma unroll
-    for (int ch = 0; ch < NQK; ++ch) {
-      Pack8 kf;
-      kf.u4 = *reinterpret_cast<const uint4*>(kl + (16 * sb + c) * S::KROW + 64 * ch + 16 * g);
-#pragma unroll
-      for (int q = 0; q < NG; ++q)
-        s[q][sb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qreg[q][ch].v, ch == 0 ? negm[q] : s[q][sb], 0, 0, 0);
-    }
-  // Does any exponent exceed RESCALE_STEP, or does a column meet its first key?  Each lane looks at
-  // its own scores only and the wave votes.  Most tiles pass, and then no value crosses lanes and
-  // nothing is rescaled.
+// The softmax step both prompt kernels share, between the score products and the value products of a tile.
+// `s[q][sb][r]` holds the exponents of this lane's eight keys for column q (the products started from minus
+// the column's reference value); `key_of(sb, r)` is the key's offset in the tile.  Does any exponent exceed
+// RESCALE_STEP, or does a column meet its first key?  Each lane looks at its own scores only and the wave votes;
+// most tiles pass, and then no value crosses lanes and nothing is rescaled.  Otherwise the columns' maxima are
+// formed (a column's keys lie in four lanes); where one is more than RESCALE_STEP above the reference value, or
+// there was none (m == NEG_BIG counts from zero), it becomes the new one, and the exponents and the output so
+// far are brought to it.  Leaves the weights in `p`, rounded to bfloat16 as they multiply the values, and adds
+// those rounded weights to the sums `l`, two per instruction.
+template <int NQK, int NG, bool masked, typename KeyOf>
+__device__ __forceinline__ void prompt_tile_softmax(f32x4_t (&s)[NG][2], int key0, KeyOf key_of,
+                                                    const int (&col_lo)[NG], const int (&col_hi)[NG],
+                                                    f32x4_t (&acc)[NG][2 * NQK], float (&m)[NG], f32x4_t (&negm)[NG],
+                                                    float (&l)[NG], Pack8 (&p)[NG]) {
   float lane_max[NG], alpha[NG];
   bool exceeds = false;
 #pragma unroll
@@ -781,7 +767,7 @@ __device__ __forceinline__ void process_tile_lds(const unsigned char* __restrict
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         if (masked) {
-          const int kk = key0 + 16 * sb + 4 * g + r;
+          const int kk = key0 + key_of(sb, r);
           if (!(kk >= col_lo[q] && kk <= col_hi[q])) s[q][sb][r] = NEG_BIG;
         }
         lane_max[q] = fmaxf(lane_max[q], s[q][sb][r]);
@@ -790,9 +776,6 @@ __device__ __forceinline__ void process_tile_lds(const unsigned char* __restrict
     exceeds = exceeds || (sees && (lane_max[q] > RESCALE_STEP || m[q] < 0.5f * NEG_BIG));
   }
   if (__any(exceeds)) {
-    // the columns' maxima (a column's keys lie in four lanes); where one is more than RESCALE_STEP
-    // above the reference value, or there was none, it becomes the new one: the exponents and the
-    // output so far are brought to it
 #pragma unroll
     for (int q = 0; q < NG; ++q) {
       float col_max = lane_max[q];
@@ -821,7 +804,6 @@ __device__ __forceinline__ void process_tile_lds(const unsigned char* __restrict
         }
     }
   }
-  Pack8 p[NG];
 #pragma unroll
   for (int q = 0; q < NG; ++q) {
     float psum = l[q] * alpha[q];
@@ -833,12 +815,41 @@ __device__ __forceinline__ void process_tile_lds(const unsigned char* __restrict
         e[r] = (!masked || s[q][sb][r] > 0.5f * NEG_BIG) ? fast_exp2(s[q][sb][r]) : 0.f;
       p[q].w[2 * sb] = pack2_bf16(e[0], e[1]);
       p[q].w[2 * sb + 1] = pack2_bf16(e[2], e[3]);
-      // the sum takes the rounded weights, the ones that multiply the values, two per instruction
       psum = add_pair_bf16(p[q].w[2 * sb], psum);
       psum = add_pair_bf16(p[q].w[2 * sb + 1], psum);
     }
     l[q] = psum;
   }
+}
+
+// Scores, softmax update and value product of one wave for the tile in LDS.  `masked` = some key of
+// the tile is hidden from some column (diagonal, window or end of data); otherwise no per-score test.
+// The queries come multiplied by scale * log2(e), and the first product of a score starts from minus
+// the column's reference value (`negm`, the same in all four elements) instead of zero, so the
+// products deliver the exponent itself: exp2 of it is the weight.  A column without a reference
+// value yet (m == NEG_BIG) counts from zero, and the first tile that shows it a key gives it one.
+template <int NQK, int NG, bool masked>
+__device__ __forceinline__ void process_tile_lds(const unsigned char* __restrict__ kl, const unsigned char* __restrict__ vl,
+                                                 int key0, const Pack8 (&qreg)[NG][NQK],
+                                                 const int (&col_lo)[NG], const int (&col_hi)[NG],
+                                                 f32x4_t (&acc)[NG][2 * NQK], float (&m)[NG], f32x4_t (&negm)[NG],
+                                                 float (&l)[NG]) {
+  using S = PrefillStage<NQK>;
+  const int lane = threadIdx.x & 63, g = lane >> 4, c = lane & 15;
+  f32x4_t s[NG][2];
+#pragma unroll
+  for (int sb = 0; sb < 2; ++sb)
+#pragma unroll
+    for (int ch = 0; ch < NQK; ++ch) {
+      Pack8 kf;
+      kf.u4 = *reinterpret_cast<const uint4*>(kl + (16 * sb + c) * S::KROW + 64 * ch + 16 * g);
+#pragma unroll
+      for (int q = 0; q < NG; ++q)
+        s[q][sb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qreg[q][ch].v, ch == 0 ? negm[q] : s[q][sb], 0, 0, 0);
+    }
+  Pack8 p[NG];
+  prompt_tile_softmax<NQK, NG, masked>(s, key0, [g](int sb, int r) { return 16 * sb + 4 * g + r; }, col_lo, col_hi,
+                                       acc, m, negm, l, p);
 #pragma unroll
   for (int n = 0; n < 2 * NQK; ++n) {
     Pack8 vf;
@@ -1173,71 +1184,9 @@ __device__ __forceinline__ void dma_tile_products(const unsigned char* __restric
         s[q][sb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qreg[q][ch].v, ch == 0 ? negm[q] : s[q][sb], 0, 0, 0);
     }
   // s[q][sb][r] is the exponent of key key0 + 8 g + 4 sb + r for this lane's column
-  float lane_max[NG], alpha[NG];
-  bool exceeds = false;
-#pragma unroll
-  for (int q = 0; q < NG; ++q) {
-    lane_max[q] = NEG_BIG;
-    alpha[q] = 1.f;
-#pragma unroll
-    for (int sb = 0; sb < 2; ++sb)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        if (masked) {
-          const int kk = key0 + 8 * g + 4 * sb + r;
-          if (!(kk >= col_lo[q] && kk <= col_hi[q])) s[q][sb][r] = NEG_BIG;
-        }
-        lane_max[q] = fmaxf(lane_max[q], s[q][sb][r]);
-      }
-    const bool sees = !masked || lane_max[q] > 0.5f * NEG_BIG;
-    exceeds = exceeds || (sees && (lane_max[q] > RESCALE_STEP || m[q] < 0.5f * NEG_BIG));
-  }
-  if (__any(exceeds)) {
-#pragma unroll
-    for (int q = 0; q < NG; ++q) {
-      float col_max = lane_max[q];
-      col_max = fmaxf(col_max, __shfl_xor(col_max, 16, 64));
-      col_max = fmaxf(col_max, __shfl_xor(col_max, 32, 64));
-      const bool had = m[q] > 0.5f * NEG_BIG;
-      const bool moves = col_max > 0.5f * NEG_BIG && (!had || col_max > RESCALE_STEP);
-      if (moves) {
-        m[q] = (had ? m[q] : 0.f) + col_max;
-        negm[q] = f32x4_t{-m[q], -m[q], -m[q], -m[q]};
-        if (had) alpha[q] = fast_exp2(-col_max);
-#pragma unroll
-        for (int sb = 0; sb < 2; ++sb)
-#pragma unroll
-          for (int r = 0; r < 4; ++r) s[q][sb][r] -= col_max;     // a hidden score stays far below
-      }
-#pragma unroll
-      for (int n = 0; n < 2 * NQK; ++n)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          float o = acc[q][n][r] * alpha[q];
-#ifdef __HIP_DEVICE_COMPILE__
-          asm volatile("" : "+v"(o));       // pins the multiply inside the branch: most tiles skip it
-#endif
-          acc[q][n][r] = o;
-        }
-    }
-  }
   Pack8 p[NG];
-#pragma unroll
-  for (int q = 0; q < NG; ++q) {
-    float psum = l[q] * alpha[q];
-#pragma unroll
-    for (int sb = 0; sb < 2; ++sb) {
-      float e[4];
-#pragma unroll
-      for (int r = 0; r < 4; ++r)
-        e[r] = (!masked || s[q][sb][r] > 0.5f * NEG_BIG) ? fast_exp2(s[q][sb][r]) : 0.f;
-      p[q].w[2 * sb] = pack2_bf16(e[0], e[1]);
-      p[q].w[2 * sb + 1] = pack2_bf16(e[2], e[3]);
-      psum = add_pair_bf16(p[q].w[2 * sb], psum);
-      psum = add_pair_bf16(p[q].w[2 * sb + 1], psum);
-    }
-    l[q] = psum;
-  }
+  prompt_tile_softmax<NQK, NG, masked>(s, key0, [g](int sb, int r) { return 8 * g + 4 * sb + r; }, col_lo, col_hi,
+                                       acc, m, negm, l, p);
   // masked tiles only: which of this lane's eight keys (8 g ..) hold written values.  The others (past the end
   // of the data, or in a sub-block without a page, which reads page 0) may hold anything and must count as 0.
   uint32_t live[4] = {0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu};
