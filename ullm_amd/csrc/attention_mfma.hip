@@ -403,10 +403,10 @@ struct RawQueries {
     }
   }
   // Per-head norm and half-split rotation of a head held by the four lanes of a column: chunk ch,
-  // element j = dim 32 ch + 8 g + j.  The same formulas as ullm_qk_norm_rope_write (which serves prompt
-  // portions), so that a key is the same whichever of the two wrote it; the partner of a dim in the
-  // first half is the dim head_dim / 2 further on, which for head sizes of 64, 128 and 256 lies in the
-  // same lane.
+  // element j = dim 32 ch + 8 g + j.  The same operations in the same order as ullm_qk_norm_rope_write's
+  // kernel for these head sizes (which serves prompt portions), multiply-adds spelled out in both, so
+  // that a key has the same bits whichever of the two wrote it; the partner of a dim in the first half
+  // is the dim head_dim / 2 further on, which for head sizes of 64, 128 and 256 lies in the same lane.
   __device__ __forceinline__ void norm_rotate(const Pack8 (&raw)[NQK], const float (*gain)[8], Pack8 (&to)[NQK]) const {
     static_assert(NQK % 2 == 0, "the partner dim must lie in the same lane");
     float x[NQK][8];
@@ -418,13 +418,24 @@ struct RawQueries {
         x[ch][2 * w + 1] = __uint_as_float(raw[ch].w[w] & 0xffff0000u);
       }
     if (gain) {
-      float ss = 0.f;
+      // the sum of squares in the order of ullm_qk_norm_rope_write's kernel for these head sizes: runs of
+      // 8 consecutive dims summed in turn, then the runs pairwise, the most distant pairs first (run p of
+      // the head is chunk p / 4 of lane group p % 4 here)
+      float part[NQK];
 #pragma unroll
-      for (int ch = 0; ch < NQK; ++ch)
+      for (int ch = 0; ch < NQK; ++ch) {
+        float a = 0.f;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) ss += x[ch][j] * x[ch][j];
-      ss += __shfl_xor(ss, 16, 64);
+        for (int j = 0; j < 8; ++j) a = fmaf(x[ch][j], x[ch][j], a);
+        part[ch] = a;
+      }
+#pragma unroll
+      for (int m = NQK / 2; m >= 1; m >>= 1)
+#pragma unroll
+        for (int ch = 0; ch < m; ++ch) part[ch] += part[ch + m];
+      float ss = part[0];
       ss += __shfl_xor(ss, 32, 64);
+      ss += __shfl_xor(ss, 16, 64);
       const float rs = rsqrtf(ss / (float)HD + fuse.eps);
 #pragma unroll
       for (int ch = 0; ch < NQK; ++ch)
@@ -437,8 +448,8 @@ struct RawQueries {
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
           const float a = x[ch][j], b = x[ch + NQK / 2][j];
-          x[ch][j] = a * cos_[ch][j] - b * sin_[ch][j];
-          x[ch + NQK / 2][j] = b * cos_[ch][j] + a * sin_[ch][j];
+          x[ch][j] = fmaf(a, cos_[ch][j], -(b * sin_[ch][j]));
+          x[ch + NQK / 2][j] = fmaf(b, cos_[ch][j], a * sin_[ch][j]);
         }
     }
 #pragma unroll

@@ -492,7 +492,9 @@ qk_norm_rope_write_vec_kernel(
   if (gain) {
     float ss = 0.f;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) ss += x[j] * x[j];
+    for (int j = 0; j < 8; ++j) ss = fmaf(x[j], x[j], ss);
+    // pairwise, the most distant lanes of a head first: the decode attention kernel, which does this
+    // norm itself for single new tokens, adds in the same order (multiply-adds spelled out in both)
     for (int m = lph >> 1; m > 0; m >>= 1) ss += __shfl_xor(ss, m, WAVE);
     const float rs = rsqrtf(ss / (float)hd + eps);
     if (arith) {
@@ -519,7 +521,7 @@ qk_norm_rope_write_vec_kernel(
         const float c[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
         const float sn[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
 #pragma unroll
-        for (int j = 0; j < 8; ++j) x[j] = first ? x[j] * c[j] - y[j] * sn[j] : x[j] * c[j] + y[j] * sn[j];
+        for (int j = 0; j < 8; ++j) x[j] = first ? fmaf(x[j], c[j], -(y[j] * sn[j])) : fmaf(x[j], c[j], y[j] * sn[j]);
       }
     } else if (arith) {
 #pragma unroll
