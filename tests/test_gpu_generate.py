@@ -443,6 +443,55 @@ def test_prefix_cache_gives_the_same_tokens(model_dirs, plain_models):
     llm.engine.runner.cache.check()
 
 
+def test_bfloat16_prefix_cache_along_each_requests_own_path(tmp_path):
+    """Prefix sharing on the bfloat16 path (config D, head size 64, pages of 16): a first portion that starts
+    behind shared pages goes through the matrix-core prompt kernel with keys it did not write itself.  Requests
+    share 40, 40 and 33 tokens of a prompt (two whole pages), one shares nothing; each is checked along its own
+    path against the plain implementation, and the shared pages must have been found, not recomputed."""
+    from ullm_amd import SamplingParams
+    d, (cfg, w) = untied(tmp_path, "D", 23)
+    shared = prompts_of(cfg["vocab_size"], (40,), 10)[0]
+    other = prompts_of(cfg["vocab_size"], (21,), 11)[0]
+    llm = make_llm(d, dtype="bfloat16", page_size=16, num_pages=32, enable_prefix_cache=True, max_prefill_chunk=24)
+    sp = SamplingParams(temperature=0.0, max_new_tokens=6, ignore_eos=True)
+    _, checked = run_and_check_own_path(llm, cfg, w, [shared + [1, 2, 3]], [sp])
+    tree = llm.engine.runner.cache.prefix_tree
+    assert tree.num_nodes >= 2
+    eng = llm.engine
+    computed = []
+    launch = eng.runner.launch
+
+    def counting(prepared):
+        computed.append(sum(len(e.tokens) for e in prepared.entries))
+        return launch(prepared)
+    eng.runner.launch = counting
+    prompts = [shared + [9], shared[:33] + [7, 7], other, shared + [1, 2, 3, 4]]
+    for i, p in enumerate(prompts):                      # under fresh ids: the checker names requests r0, r1, ...
+        eng.add_request(f"r{i}", p, sp)
+    got = {}
+    seen = {}
+    eng.on_logits = lambda sampling, logits: [seen.setdefault(s_.request.request_id, []).append((s_.request.num_tokens, row))
+                                              for s_, row in zip(sampling, logits.float().cpu())]
+    while eng.has_unfinished_requests():
+        for r in eng.step():
+            if r.new_token_id >= 0:
+                got.setdefault(r.seq_id, []).append(r.new_token_id)
+    for i, p in enumerate(prompts):
+        seq = p + got[f"r{i}"]
+        full = plain.qwen3_forward(w, cfg, seq)
+        bound = 3e-2 * float(full.abs().max()) + 1e-6
+        for pos, row in seen[f"r{i}"]:
+            if pos >= len(seq):
+                continue
+            assert float((row - full[pos - 1]).abs().max()) <= bound, (i, pos)
+            assert seq[pos] == int(row.argmax()), (i, pos)
+            checked += 1
+    assert checked >= 30
+    # 41 + 35 + 21 + 44 prompt tokens and 4 x 5 decoded ones; two pages of 16 were found for three of the requests
+    assert sum(computed) == 41 + 35 + 21 + 44 + 4 * 5 - 3 * 32, computed
+    eng.runner.cache.check()
+
+
 def test_command_line(model_dirs, plain_models, capsys):
     from ullm_amd.cli import main
     cfg, w = plain_models["A"]
