@@ -171,3 +171,32 @@ def test_random_weights_specification(tmp_path):
         EngineConfig.from_args(ap.parse_args([]))
     with pytest.raises(ConfigError, match="either"):
         EngineConfig(model="x", random_weights="qwen3-8b")
+
+
+def test_a_windowed_configuration_is_announced_as_this_engines_own_reading(caplog):
+    """The reference reads none of the sliding-window keys (ullm/models/qwen3.py builds every layer with full
+    attention), so a config that switches windows on gets logits no reference run pins: said once per model."""
+    import logging
+    with caplog.at_level(logging.WARNING, logger="ullm_amd"):
+        build_model(TINY_A)
+    assert not [r for r in caplog.records if "sliding-window" in r.getMessage()]
+    with caplog.at_level(logging.WARNING, logger="ullm_amd"):
+        build_model(TINY_C)
+    said = [r.getMessage() for r in caplog.records if "sliding-window" in r.getMessage()]
+    assert len(said) == 1 and "2 of 3 layers look back 24 keys" in said[0] and "the reference applies no window" in said[0]
+
+
+def test_a_context_past_the_models_positions_is_refused(caplog):
+    """The reference's rotary table has max_position_embeddings rows (ullm/models/qwen3.py:142,
+    ullm/layers/rotary_embedding.py:69); an engine with a longer context is refused when it is built.  Trace
+    replay, whose number is a pool's size and whose traces are given, says so once and goes on."""
+    import logging
+    from ullm_amd.engine.loading import context_within_model
+    cfg, _ = build_model(TINY_A)                       # max_position_embeddings = 128
+    assert context_within_model(cfg, 128) == 128 and context_within_model(cfg, 64) == 64
+    with pytest.raises(ConfigError, match="max_position_embeddings=128"):
+        context_within_model(cfg, 129)
+    with caplog.at_level(logging.WARNING, logger="ullm_amd"):
+        assert context_within_model(cfg, 512, strict=False) == 512
+    assert any("max_position_embeddings=128" in r.getMessage() for r in caplog.records)
+    assert context_within_model({"no": "such key"}, 10 ** 6) == 10 ** 6     # a configuration without the key has no limit

@@ -457,6 +457,38 @@ def test_attention_on_the_matrix_cores(ops, case):
             break
 
 
+@pytest.mark.parametrize("row", [(5,), (7, 3), (64,), (1,), (4, 1000)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.uint8])
+def test_state_rows_of_requests_that_start_afresh_are_zeroed(ops, row, dtype):
+    """Rows of any size and type (16-, 4- and 1-byte words): only the slots of entries that start at 0 are
+    zeroed, slots outside the tensor are ignored, nothing else is touched."""
+    torch.manual_seed(1)
+    slots = 9
+    state = (torch.rand((slots,) + row, device=DEV) * 200 + 1).to(dtype)
+    before = state.clone()
+    entry_slot = torch.tensor([3, 0, 8, 5, 11, 2], dtype=torch.int32, device=DEV)
+    entry_start = torch.tensor([0, 7, 0, 1, 0, 0], dtype=torch.int32, device=DEV)
+    ops.zero_fresh_rows(state, entry_slot, entry_start, 5)                  # the sixth entry is not part of the batch
+    for s_ in range(slots):
+        want = torch.zeros_like(before[s_]) if s_ in (3, 8) else before[s_]
+        assert torch.equal(state[s_], want), s_
+    # an odd base address: a view that starts one row further on
+    if dtype == torch.uint8 and row == (5,):
+        view = state[1:]
+        ops.zero_fresh_rows(view, torch.tensor([0], dtype=torch.int32, device=DEV), torch.tensor([0], dtype=torch.int32, device=DEV), 1)
+        assert int(state[1].sum()) == 0 and torch.equal(state[2], before[2])
+
+
+@pytest.mark.parametrize("cols", [503, 1024, 151936])
+def test_rows_gathered_by_an_index_on_the_device(ops, cols):
+    torch.manual_seed(2)
+    src = torch.randn(7, cols + 8, device=DEV)[:, :cols]                    # rows with a stride of their own
+    index = torch.tensor([6, 0, 3, 3, 9, -1], dtype=torch.int32, device=DEV)
+    got = ops.gather_rows(src, index)
+    assert got.shape == (6, cols)
+    assert torch.equal(got[:4], src[[6, 0, 3, 3]]) and float(got[4:].abs().max()) == 0.0
+
+
 FUSED_CASES = [dict(nq=32, nkv=8, hd=128, P=16, lens=[1153, 31, 32, 33, 1], window=0, norm=True, rope=True),
                dict(nq=8, nkv=2, hd=64, P=16, lens=[300, 40, 9, 17, 48], window=50, norm=True, rope=True),
                dict(nq=40, nkv=2, hd=64, P=32, lens=[130, 97], window=0, norm=False, rope=True),      # 20 heads per kv head

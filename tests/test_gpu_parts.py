@@ -80,6 +80,33 @@ def test_toy_mixer_with_state_registers_builds_and_steps(tmp_path, dtype, cuts):
     assert float(np.abs(out - want.numpy()).max()) <= REL[dtype] * float(want.abs().max()) + 1e-6
 
 
+KEYS = dict(mixer="keys_only", dim=24, ffn_size=60)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("cuts", CUTS)
+def test_toy_mixer_that_keeps_one_row_per_token_and_plans_its_own_work(tmp_path, dtype, cuts):
+    """A mixer defined in the tests that keeps keys only (one float32 row per token, no values) and takes its
+    work list from a planner of its own: the step function allocates the one pool it declares, runs its planner
+    beside the attention kernels' and hands it the result, with no change to the framework's files.  Layer 3
+    reads the cache layer 1 wrote."""
+    cfg = base_cfg([ATT, KEYS, dict(KEYS, dim=40), KEYS], run_order=[[0, 0], [1, 1], [2, 2], [3, 1]])
+    rep, _ = run_and_compare(tmp_path, cfg, dtype, cuts, seed=19)
+    runner = rep.runner
+    assert sorted(runner._planners) == ["attention", "toy_spans"]
+    assert [(g.head_dim, g.rows) for g in runner.cache.groups] == [(16, None), (24, ((1, 24, 4),)), (40, ((1, 40, 4),))]
+    for cache_id, dim in ((1, 24), (2, 40)):
+        view = runner.caches[cache_id]
+        assert sorted(view.pools) == ["latent"] and view.k_pool is None and view.v_pool is None
+        assert view.pools["latent"].dtype == torch.float32 and view.pools["latent"].shape[1:] == (1, 8, dim)
+    attention = runner.caches[0]
+    assert sorted(attention.pools) == ["k", "v"] and attention.k_pool is attention.pools["k"]
+    pages = runner.cache.allocators[0].num_pages
+    item = 4 if dtype == "float32" else 2
+    assert runner.cache_bytes() == pages * 8 * (2 * 3 * 16 * item + 24 * 4 + 40 * 4)
+    assert runner.cache.groups[1].bytes_per_token(item) == 24 * 4
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_state_mixer_steps_replayed_from_graphs(tmp_path, dtype):
     """A state mixer that says its single-token step can be captured keeps the model on HIP graphs:
@@ -203,6 +230,7 @@ def test_a_block_that_keeps_keys_and_values_and_state(tmp_path, dtype):
 def test_parts_are_found_by_name_and_unknown_names_fail():
     from ullm_amd.parts import build_part, registered_parts
     assert "toy_running_mean" in registered_parts("mixer") and "gqa_attention" in registered_parts("mixer")
+    assert "toy_keys_only" in registered_parts("mixer")
     assert "swiglu" in registered_parts("ffn") and registered_parts("block") == ["prenorm", "toy_two_mixers"]
     with pytest.raises(KeyError, match="no mixer part named"):
         build_part("mixer", "does_not_exist")

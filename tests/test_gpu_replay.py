@@ -470,7 +470,11 @@ def test_graph_replays_equal_eager_steps(model_dirs, plain_models, name, dtype):
         for r, n in step:
             n = min(n, len(reqs[r]) - done[r])
             if n > 0:
-                entries.append({"id": r, "tokens": reqs[r][done[r]:done[r] + n], "want": list(range(n))})
+                # in some steps of single tokens one entry wants nothing: its row is then left out of the
+                # replayed graph's logits on the device
+                skip = s % 4 == 3 and r == "b" and all(m == 1 for _, m in step) and len(step) > 1
+                entries.append({"id": r, "tokens": reqs[r][done[r]:done[r] + n], "want": [] if skip else list(range(n)),
+                                "at": done[r]})
                 done[r] += n
         if not entries:
             continue
@@ -479,8 +483,15 @@ def test_graph_replays_equal_eager_steps(model_dirs, plain_models, name, dtype):
         close(a, b, dtype)
         row = 0
         for e in entries:
-            got[e["id"]].append(a[row:row + len(e["tokens"])])
-            row += len(e["tokens"])
+            n = len(e["want"])
+            got[e["id"]].append((e["at"], a[row:row + n]))
+            row += n
+        assert row == len(a)
     assert len(graphs.runner._graphs) >= 2 and not eager.runner._graphs
+    skipped = 0
     for r in reqs:
-        close(np.concatenate(got[r]), wants[r][:done[r]], dtype)
+        for at, rows in got[r]:
+            if len(rows):
+                close(rows, wants[r][at:at + len(rows)], dtype)
+            skipped += len(rows) == 0
+    assert skipped >= 3

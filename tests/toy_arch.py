@@ -1,18 +1,21 @@
 """A test-only architecture, registered from outside the framework: a stack whose layers are chosen
-one by one in the config (attention with any position encoding, window, norm and bias option, or a
-toy mixer with per-request state of fixed size; a dense feed-forward or a toy one that routes every
+one by one in the config (attention with any position encoding, window, norm and bias option, a
+toy mixer with per-request state of fixed size, or a toy mixer that keeps one row per token in pages and
+plans its own work lists; a dense feed-forward or a toy one that routes every
 token to one of several experts; a toy position encoding with angles of its own), with an optional
 run order that names a layer twice or lets a layer read another layer's cache.  Beside it, its plain whole-sequence forward.
 Nothing here is a model of anyone's; it exists to show that the framework's parts, cache manager and
 step function take new parts without a change to the framework's files."""
 from typing import Dict, List
 
+import numpy as np
 import torch
 
 import plain_qwen3 as plain
 from ullm_amd.models import Choice, ModelPlan, register_architecture
 from ullm_amd.kernels import ops
-from ullm_amd.parts import Block, FeedForward, Mixer, PositionEncoding, StateNeed, WeightDecl, register_part
+from ullm_amd.parts import (Block, CacheRows, FeedForward, KVNeed, Mixer, PositionEncoding, StateNeed, StepPlan, StepShape,
+                            WeightDecl, register_part)
 from ullm_amd.parts.linear import linear
 
 
@@ -58,6 +61,61 @@ class RunningMean(Mixer):
                 state[H] = counts[-1]
             t += n
         return linear(means.to(x.dtype), self.w)
+
+
+def plan_spans(shape: StepShape) -> StepPlan:
+    """The work list of the keys-only mixer below, made by the step function through the planner hook: one
+    (first token, tokens, keys before them) triple per entry, in batch order."""
+    spans, t0 = [], 0
+    for n, start in zip(shape.lens, shape.starts):
+        spans += [t0, n, start]
+        t0 += n
+    return StepPlan(arrays={"spans": np.asarray(spans, dtype=np.int32)}, facts={"count": len(shape.lens)})
+
+
+@register_part("mixer", "toy_keys_only")
+class KeysOnly(Mixer):
+    """One head whose keys are also its values: y_t = Wo * sum_j softmax_j(q_t . k_j / sqrt(d)) k_j over j <= t.
+    It keeps a single row of ``dim`` values per token, in float32 whatever the compute dtype, and says so in
+    its need: the step function then allocates that one pool and no value pool.  Its work list comes from a
+    planner of its own, named in ``step_planners``."""
+    graph_safe = False          # it reads its work list on the host
+    step_planners = {"toy_spans": plan_spans}
+
+    def __init__(self, hidden_size: int, dim: int, prefix: str):
+        self.hidden_size, self.dim, self.prefix = hidden_size, dim, prefix
+
+    def cache_need(self):
+        return KVNeed(1, self.dim, rows=(CacheRows("latent", 1, self.dim, dtype=torch.float32),))
+
+    def weights(self):
+        p, H, d = self.prefix, self.hidden_size, self.dim
+        return [WeightDecl(f"{p}.q.weight", (d, H)), WeightDecl(f"{p}.k.weight", (d, H)), WeightDecl(f"{p}.o.weight", (H, d))]
+
+    def bind(self, tensors, env):
+        p = self.prefix
+        self.wq, self.wk, self.wo = (tensors[f"{p}.{n}.weight"].contiguous() for n in ("q", "k", "o"))
+
+    def forward(self, x, ctx, cache):
+        d = self.dim
+        group = ctx.groups[cache.group]
+        pool, P = cache.pools["latent"], group.page_size            # [pages, 1, page_size, dim] float32
+        q, k = linear(x, self.wq).float(), linear(x, self.wk).float()
+        if cache.owner:
+            page = group.block_table[ctx.token_entry.long(), (ctx.positions // P).long()].long()
+            pool[page, 0, (ctx.positions % P).long()] = k
+        plan = ctx.plans["toy_spans"]
+        spans = plan.arrays["spans"].view(-1, 3).tolist()
+        assert len(spans) == plan.facts["count"] == ctx.num_entries
+        out = torch.empty_like(q)
+        for b, (first, n, start) in enumerate(spans):
+            total = start + n
+            pages = group.block_table[b, :-(-total // P)].long()
+            keys = pool[pages, 0].reshape(-1, d)[:total]
+            scores = (q[first:first + n] @ keys.T) * d ** -0.5
+            seen = torch.arange(total, device=x.device)[None, :] <= (start + torch.arange(n, device=x.device))[:, None]
+            out[first:first + n] = torch.softmax(scores.masked_fill(~seen, float("-inf")), dim=-1) @ keys
+        return linear(out.to(x.dtype), self.wo)
 
 
 @register_part("ffn", "toy_top1_experts")
@@ -163,6 +221,8 @@ def toy_plan(cfg: dict) -> ModelPlan:
                 hidden_size=H, num_heads=L["heads"], num_kv_heads=L["kv_heads"], head_dim=L["head_dim"],
                 prefix=f"{p}.attn", position=position, qk_norm_eps=eps if L.get("qk_norm", True) else None,
                 bias=L.get("bias", False), window=L.get("window", 0), scale=L.get("scale")))
+        elif L["mixer"] == "keys_only":
+            mixer = Choice("mixer", "toy_keys_only", dict(hidden_size=H, dim=L["dim"], prefix=f"{p}.lat"))
         else:
             mixer = Choice("mixer", "toy_running_mean", dict(hidden_size=H, prefix=f"{p}.mix"))
         norm = lambda n: Choice("norm", "rmsnorm", dict(size=H, eps=eps, weight_name=f"{p}.{n}.weight"))  # noqa: E731
@@ -239,7 +299,15 @@ def toy_forward(w: Dict[str, torch.Tensor], cfg: dict, token_ids: List[int]) -> 
             scale = L.get("scale") or d ** -0.5
             o = plain.causal_gqa_attention(q, k, v, scale, L.get("window", 0))
             a = plain.linear(o.reshape(T, nq * d), w[f"{p}.attn.o_proj.weight"])
-        if L["mixer"] != "attention":
+        if L["mixer"] == "keys_only":
+            d = L["dim"]
+            q, k = plain.linear(x, w[f"{p}.lat.q.weight"]), plain.linear(x, w[f"{p}.lat.k.weight"])
+            if cache_id not in kv_of:
+                kv_of[cache_id] = (k, k)
+            k = kv_of[cache_id][0]
+            o = plain.causal_gqa_attention(q.view(T, 1, d), k.view(T, 1, d), k.view(T, 1, d), d ** -0.5)
+            a = plain.linear(o.reshape(T, d), w[f"{p}.lat.o.weight"])
+        elif L["mixer"] != "attention":
             means = torch.cumsum(x, 0) / torch.arange(1, T + 1, dtype=torch.float32)[:, None]
             a = a + plain.linear(means, w[f"{p}.mix.mean_proj.weight"])
         h = h + a

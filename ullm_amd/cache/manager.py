@@ -10,8 +10,8 @@ from a pool of ``max_bs``.  Here
   * a group with a window gives pages back as soon as the window has passed them;
   * pages are handed out per portion (``reserve``) and a request's progress is recorded after the
     step (``commit``); ``release`` gives everything back;
-  * a request *slot* (0 .. max_requests-1) stands for the request's rows of fixed-size state;
-    freshly admitted slots are reported so that their state can be zeroed before the first step.
+  * a request *slot* (0 .. max_requests-1) stands for the request's rows of fixed-size state (the step
+    function zeroes the rows of every request that steps from its first token).
 """
 from __future__ import annotations
 
@@ -31,9 +31,13 @@ class CacheGroupSpec:
     head_dim: int
     window: int                   # 0 = every earlier key
     layers: tuple                 # the caches of this group, one set of pools each (any hashable names)
+    # what a token keeps in each layer's pools: (heads, dim, bytes per value or None = the compute dtype's)
+    # per pool; None = one key row and one value row per kv head
+    rows: Optional[tuple] = None
 
     def bytes_per_token(self, itemsize: int) -> int:
-        return 2 * self.num_kv_heads * self.head_dim * itemsize * len(self.layers)
+        rows = self.rows if self.rows is not None else ((self.num_kv_heads, self.head_dim, None),) * 2
+        return sum(heads * dim * (size or itemsize) for heads, dim, size in rows) * len(self.layers)
 
 
 class CacheFull(RuntimeError):
@@ -65,7 +69,6 @@ class CacheManager:
         self.max_requests = max_requests
         self.allocators = [PageAllocator(n) for n in num_pages]
         self._free_slots: List[int] = list(range(max_requests - 1, -1, -1))
-        self._fresh_slots: List[int] = []
         # the block tables once more as one int32 matrix per group, row = slot, -1 where a table holds
         # no page: a step gathers its rows from here instead of converting Python lists
         self._rows = [np.full((max_requests, 16), -1, dtype=np.int32) for _ in groups]
@@ -98,7 +101,6 @@ class CacheManager:
                 self._put_row(g, slot, 0, rc.tables[g])
             rc.num_computed = len(matched) * self.page_size
         self.requests[request_id] = rc
-        self._fresh_slots.append(slot)
         return rc
 
     def _put_row(self, g: int, slot: int, start: int, pages: Sequence[int]) -> None:
@@ -118,11 +120,6 @@ class CacheManager:
             return rows[slots, :width]
         out = np.full((len(slots), width), -1, dtype=np.int32)
         out[:, :rows.shape[1]] = rows[slots]
-        return out
-
-    def take_fresh_slots(self) -> List[int]:
-        """Slots admitted since the last call: their state rows must be zeroed before they step."""
-        out, self._fresh_slots = self._fresh_slots, []
         return out
 
     # ------------------------------------------------------------------ pages
@@ -196,8 +193,6 @@ class CacheManager:
             self._rows[g][rc.slot] = -1
         rc.released = True
         self._free_slots.append(rc.slot)
-        if rc.slot in self._fresh_slots:
-            self._fresh_slots.remove(rc.slot)
         del self.requests[rc.request_id]
 
     def rewind(self, rc: RequestCache) -> None:
@@ -210,8 +205,6 @@ class CacheManager:
             self._rows[g][rc.slot] = -1
             rc.first_live[g] = 0
         rc.num_computed = 0
-        if rc.slot not in self._fresh_slots:
-            self._fresh_slots.append(rc.slot)
 
     # ------------------------------------------------------------------ figures and checks
     def num_free_pages(self, group: int = 0) -> int:

@@ -104,6 +104,71 @@ extern "C" int ullm_feed_tokens(int* ids, const int* feed, const int* source, in
   ULLM_LAUNCH_CHECK();
 }
 
+// ------------------------------------------------------------------ rows of per-request state, rows of results
+// The state rows (row_bytes bytes each) of the requests that step from their first token are zeroed:
+// entry b's row is slot[b], and it starts afresh if start[b] == 0.  grid (entries, pieces of a row).
+// The words of a row are 16, 4 or 1 bytes wide, whichever the row size and the base address allow.
+template <typename W>
+__global__ void zero_fresh_rows_kernel(unsigned char* __restrict__ state, long long row_bytes, int n_rows,
+                                       const int* __restrict__ slot, const int* __restrict__ start) {
+  const int b = blockIdx.x;
+  if (start[b] != 0) return;
+  const int row = slot[b];
+  if (row < 0 || row >= n_rows) return;
+  W* words = reinterpret_cast<W*>(state + (size_t)row * row_bytes);
+  const long long n = row_bytes / (long long)sizeof(W);
+  W zero;
+  memset(&zero, 0, sizeof(W));
+  for (long long i = (long long)blockIdx.y * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.y * blockDim.x)
+    words[i] = zero;
+}
+
+extern "C" int ullm_zero_fresh_rows(void* state, long long row_bytes, int n_rows, const int* slot, const int* start,
+                                    int n_entries, hipStream_t stream) {
+  if (n_entries <= 0 || row_bytes <= 0) return 0;
+  if (n_rows <= 0) return ULLM_ERR_SHAPE;
+  const int width = (row_bytes % 16 == 0 && ((uintptr_t)state & 15) == 0) ? 16
+                    : (row_bytes % 4 == 0 && ((uintptr_t)state & 3) == 0) ? 4 : 1;
+  long long pieces = (row_bytes / width + 255) / 256;
+  if (pieces > 64) pieces = 64;
+  dim3 grid(n_entries, (unsigned)pieces), block(256);
+  if (width == 16)
+    hipLaunchKernelGGL(zero_fresh_rows_kernel<uint4>, grid, block, 0, stream, (unsigned char*)state, row_bytes, n_rows, slot, start);
+  else if (width == 4)
+    hipLaunchKernelGGL(zero_fresh_rows_kernel<uint32_t>, grid, block, 0, stream, (unsigned char*)state, row_bytes, n_rows, slot, start);
+  else
+    hipLaunchKernelGGL(zero_fresh_rows_kernel<unsigned char>, grid, block, 0, stream, (unsigned char*)state, row_bytes, n_rows, slot, start);
+  ULLM_LAUNCH_CHECK();
+}
+
+// out[i, :] = src[index[i], :] for float32 rows (an index outside [0, n_src) gives a row of zeros).
+// grid (rows, pieces of a row).
+__global__ void gather_rows_kernel(const float* __restrict__ src, long long src_stride, int n_src,
+                                   const int* __restrict__ index, float* __restrict__ out, int cols, int vec) {
+  const int i = blockIdx.x;
+  const int from = index[i];
+  const bool ok = from >= 0 && from < n_src;
+  const float* row = src + (size_t)(ok ? from : 0) * src_stride;
+  float* dst = out + (size_t)i * cols;
+  if (vec) {
+    for (int c = 4 * (blockIdx.y * blockDim.x + threadIdx.x); c < cols; c += 4 * gridDim.y * blockDim.x)
+      *reinterpret_cast<float4*>(dst + c) = ok ? ld4_f32_stream(row + c) : make_float4(0.f, 0.f, 0.f, 0.f);
+    return;
+  }
+  for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < cols; c += gridDim.y * blockDim.x) dst[c] = ok ? row[c] : 0.f;
+}
+
+extern "C" int ullm_gather_rows(const float* src, long long src_stride, int n_src, const int* index, float* out,
+                                int n, int cols, hipStream_t stream) {
+  if (n <= 0 || cols <= 0) return 0;
+  if (n_src <= 0 || src_stride < cols) return ULLM_ERR_SHAPE;
+  const int vec = cols % 4 == 0 && src_stride % 4 == 0 && !(((uintptr_t)src | (uintptr_t)out) & 15);
+  int pieces = (cols / (vec ? 4 : 1) + 255) / 256;
+  if (pieces > 256) pieces = 256;
+  hipLaunchKernelGGL(gather_rows_kernel, dim3(n, pieces), dim3(256), 0, stream, src, src_stride, n_src, index, out, cols, vec);
+  ULLM_LAUNCH_CHECK();
+}
+
 // ------------------------------------------------------------------ add + RMS norm
 // For output row r (input row i = rows ? rows[r] : r):
 //   s = residual[i] + float(branch[i])      (branch may be null: s = residual[i]; it may also be a stack

@@ -16,9 +16,8 @@ import torch
 
 from ..cache.manager import CacheManager, RequestCache
 from ..kernels import ops
-from ..kernels.ops import PREFILL_TILE as Q_TILE   # tokens of one request per prompt-portion attention tile
 from ..models.model import Model
-from ..parts import GroupView, LayerCache, PartEnv, StepContext
+from ..parts import GroupView, LayerCache, PartEnv, StepContext, StepPlan, StepShape
 from ..staging import StagedUpload
 
 
@@ -65,19 +64,27 @@ class ModelRunner:
                                   enable_prefix_cache=enable_prefix_cache and not states)
         self.max_table = -(-env.context_len // page_size)
         views: Dict[tuple, LayerCache] = {}      # (cache id, index of the need in its block) -> view
-        for g, spec in enumerate(groups):
-            k_shape = (num_pages[g], spec.num_kv_heads, page_size, spec.head_dim)
-            v_shape = (num_pages[g], spec.num_kv_heads, spec.head_dim, page_size)   # transposed inside a page
+        for g, (spec, need) in enumerate(zip(groups, model.group_needs())):
             for key in spec.layers:
-                # zeroed once so that no row ever holds a non-finite bit pattern before it is written
-                views[key] = LayerCache(
-                    group=g, k_pool=torch.zeros(k_shape, dtype=env.dtype, device=env.device),
-                    v_pool=torch.zeros(v_shape, dtype=env.dtype, device=env.device))
+                pools = {}
+                for rows in need.pools():
+                    shape = ((num_pages[g], rows.heads, rows.dim, page_size) if rows.transposed
+                             else (num_pages[g], rows.heads, page_size, rows.dim))
+                    # zeroed once so that no row ever holds a non-finite bit pattern before it is written
+                    pools[rows.name] = torch.zeros(shape, dtype=rows.dtype or env.dtype, device=env.device)
+                views[key] = LayerCache.of_pools(g, pools)
         for key, need in states.items():
             # one row more than requests: the slot of a captured batch's padding entries
             views[key] = LayerCache(
                 state=torch.zeros((max_requests + 1,) + tuple(need.shape), dtype=need.dtype, device=env.device))
         self._views = views
+        self._states = [c.state.view(c.state.shape[0], -1) for c in views.values() if c.state is not None]
+        # what the parts' kernels want to know about a step beside the flat batch (Part.step_planners)
+        self._planners: Dict[str, object] = {}
+        for part in model.parts():
+            for name, planner in part.step_planners.items():
+                if self._planners.setdefault(name, planner) is not planner:
+                    raise StepError(f"two parts name different step planners {name!r}")
         # per cache id what its block sees: the one view, or one view per declared need
         self.caches: Dict[int, LayerCache] = {}
         for cache_id in sorted({c for c, _ in views}):
@@ -102,16 +109,18 @@ class ModelRunner:
     def cache_bytes(self) -> int:
         total = 0
         for c in self._views.values():
-            for t in (c.k_pool, c.v_pool, c.state):
+            for t in list(c.pools.values()) + [c.state]:
                 if t is not None:
                     total += t.numel() * t.element_size()
         return total
 
     def _pack(self, entries: Sequence[StepEntry], pad_entries: int = 0, table_stride: Optional[int] = None,
-              allow_unknown: bool = False):
-        """Flatten the entries into one int32 host array.  Returns (host array, offsets, facts).
+              allow_unknown: bool = False, kv_bucket: Optional[int] = None):
+        """Flatten the entries into one int32 host array.  Returns (host array, layout, facts); the layout
+        maps a field's name to its (first, end) in the array.
         ``pad_entries`` > len(entries) appends one-token entries that hold no pages (their cache
-        writes are skipped and their outputs ignored), so that a batch fits a captured graph.
+        writes are skipped and their outputs ignored), so that a batch fits a captured graph; every entry's
+        only token is then a wanted row and ``picked`` lists the entries that asked for it.
         With ``allow_unknown`` a token may be UNKNOWN_TOKEN (its id is filled in before the launch);
         ``facts["unknown"]`` lists such tokens as (index into the array, entry, index in the entry)."""
         P = self.page_size
@@ -120,6 +129,7 @@ class ModelRunner:
         if n_real == 0 or sum(lens) == 0:
             raise StepError("a step needs at least one token")
         n_pad = max(0, pad_entries - n_real)
+        for_graph = pad_entries > 0
         B = n_real + n_pad
         T = sum(lens) + n_pad
         groups = self.cache.groups
@@ -131,31 +141,6 @@ class ModelRunner:
                     raise StepError("a block table is wider than the captured graph's")
                 widest = table_stride
             strides.append(widest)
-        n_want = sum(len(e.want) for e in entries) + n_pad
-        # attention work lists: tokens of one-token entries; tiles of <= Q_TILE tokens of longer entries
-        dec_keys, tile_keys, max_dec_kv, t0 = [], [], 0, 0
-        for e, n in zip(entries, lens):
-            if n == 1:
-                dec_keys.append((-e.cache.num_computed, t0))
-                max_dec_kv = max(max_dec_kv, e.cache.num_computed + 1)
-            else:
-                for first in range(0, n, Q_TILE):
-                    count = min(Q_TILE, n - first)
-                    tile_keys.append((e.cache.num_computed + first + count, t0 + first, count))
-            t0 += n
-        tile_keys.sort()                                  # the attention kernel wants rising numbers of keys
-        dec_keys.sort()                                   # longest contexts first: the short ones fill the tail
-        dec_list = [t for _, t in dec_keys]
-        tile_list = [x for _, first, count in tile_keys for x in (first, count)]
-        dec_list.extend(range(t0, t0 + n_pad))
-        ng = len(groups)
-        sizes = [T, T, T, B + 1, B, B, n_want] + [B * s for s in strides] + [len(dec_list), len(tile_list), T]
-        offs = np.concatenate(([0], np.cumsum(sizes)))
-        host = np.zeros(int(offs[-1]), dtype=np.int32)
-        ids, pos, ent = host[offs[0]:offs[1]], host[offs[1]:offs[2]], host[offs[2]:offs[3]]
-        q_start, slot, start = host[offs[3]:offs[4]], host[offs[4]:offs[5]], host[offs[5]:offs[6]]
-        rows = host[offs[6]:offs[7]]
-        host[offs[9 + ng]:offs[10 + ng]] = -1             # per token: where the device takes its id from (-1: from ids)
         caches = [e.cache for e in entries]
         starts = [rc.num_computed for rc in caches]
         slots = [rc.slot for rc in caches]
@@ -175,6 +160,28 @@ class ModelRunner:
                 if rc.slot in seen:
                     raise StepError(f"request {rc.request_id!r} appears twice in one step")
                 seen.add(rc.slot)
+        picked = [b for b, e in enumerate(entries) if len(e.want)] if for_graph else []
+        n_want = B if for_graph else sum(len(e.want) for e in entries)
+        shape = StepShape(tuple(lens), tuple(starts), n_pad, kv_bucket)
+        plans = {name: planner(shape) for name, planner in self._planners.items()}
+        fields = [("ids", T), ("positions", T), ("token_entry", T), ("q_start", B + 1), ("slot", B), ("start", B),
+                  ("rows", n_want), ("picked", B if for_graph else 0)]
+        fields += [(f"table{g}", B * stride) for g, stride in enumerate(strides)]
+        for name, plan in plans.items():
+            for key, arr in plan.arrays.items():
+                arr = np.asarray(arr)
+                if arr.dtype != np.int32 or arr.ndim != 1:
+                    raise StepError(f"step planner {name!r}: array {key!r} must be a flat int32 array")
+                fields.append((f"plan.{name}.{key}", arr.size))
+        fields.append(("feed", T))
+        layout, at = {}, 0
+        for name, size in fields:
+            layout[name] = (at, at + size)
+            at += size
+        host = np.zeros(at, dtype=np.int32)
+        part = lambda name: host[layout[name][0]:layout[name][1]]   # noqa: E731
+        ids, pos, ent, q_start, rows = part("ids"), part("positions"), part("token_entry"), part("q_start"), part("rows")
+        part("feed")[:] = -1                             # per token: where the device takes its id from (-1: from ids)
         n_tok = T - n_pad
         tok = np.empty(n_tok, dtype=np.int64)
         if n_tok == n_real:                              # one token each: no per-entry array work
@@ -197,23 +204,22 @@ class ModelRunner:
             first_of = q_start[:n_real]
             for t in np.nonzero(tok == UNKNOWN_TOKEN)[0].tolist():
                 b = int(ent[t])
-                unknown.append((t, b, t - int(first_of[b])))
+                unknown.append((layout["ids"][0] + t, layout["feed"][0] + t, b, t - int(first_of[b])))
             tok[tok == UNKNOWN_TOKEN] = 0
         if int(tok.min()) < 0 or int(tok.max()) >= self.vocab_size:
             bad = next(rc for rc, e in zip(caches, entries) if min(e.tokens) < 0 or max(e.tokens) >= self.vocab_size)
             raise StepError(f"request {bad.request_id!r}: token id outside [0, {self.vocab_size})")
         ids[:n_tok] = tok
-        slot[:n_real] = slots
-        slot[n_real:] = self.padding_slot
-        start[:n_real] = starts
+        part("slot")[:n_real] = slots
+        part("slot")[n_real:] = self.padding_slot
+        part("start")[:n_real] = starts
         r = 0
         for b, e in enumerate(entries):
-            for w in e.want:
+            for w in ([0] if for_graph else e.want):
                 if not (0 <= w < lens[b]):
                     raise StepError(f"request {caches[b].request_id!r}: wanted place {w} outside its {lens[b]} tokens")
                 rows[r] = q_start[b] + w
                 r += 1
-        max_kv = max(s0 + n for s0, n in zip(starts, lens))
         t = n_tok
         for b in range(n_real, B):                       # padding entries: token 0 at position 0, no pages
             ent[t] = b
@@ -222,38 +228,48 @@ class ModelRunner:
             t += 1
             r += 1
         q_start[B] = T
-        for g, s in enumerate(strides):
-            bt = host[offs[7 + g]:offs[8 + g]].reshape(B, s)
-            bt[:n_real] = self.cache.table_rows(g, slots, s)
+        part("picked")[:len(picked)] = picked
+        for g, stride in enumerate(strides):
+            bt = part(f"table{g}").reshape(B, stride)
+            bt[:n_real] = self.cache.table_rows(g, slots, stride)
             bt[n_real:] = -1
-        host[offs[7 + ng]:offs[8 + ng]] = dec_list
-        host[offs[8 + ng]:offs[9 + ng]] = tile_list
-        facts = dict(T=T, B=B, strides=strides, n_want=n_want, num_decode=len(dec_list), max_dec_kv=max_dec_kv,
-                     num_tiles=len(tile_list) // 2, tile_keys_total=sum(k for k, _, _ in tile_keys),
-                     tile_keys_max=tile_keys[-1][0] if tile_keys else 0, max_q=max(lens), max_kv=max_kv,
+        for name, plan in plans.items():
+            for key, arr in plan.arrays.items():
+                part(f"plan.{name}.{key}")[:] = arr
+        facts = dict(T=T, B=B, strides=strides, n_want=n_want, picked=picked, max_q=max(lens),
+                     max_kv=kv_bucket or max(s0 + n for s0, n in zip(starts, lens)),
                      decode_only=all(n == 1 for n in lens), lens=lens + [1] * n_pad,
-                     starts=starts + [0] * n_pad, slots=slots + [self.padding_slot] * n_pad, unknown=unknown)
-        return host, offs, facts
+                     starts=starts + [0] * n_pad, slots=slots + [self.padding_slot] * n_pad, unknown=unknown,
+                     plans={name: plan.facts for name, plan in plans.items()},
+                     plan_arrays={name: list(plan.arrays) for name, plan in plans.items()})
+        return host, layout, facts
 
-    def _context(self, dev: torch.Tensor, offs, facts) -> tuple:
+    def _context(self, dev: torch.Tensor, layout, facts) -> tuple:
         """Views into the uploaded buffer as a StepContext, and the wanted rows."""
         groups = self.cache.groups
-        ng = len(groups)
         B, T = facts["B"], facts["T"]
-        view = lambda i: dev[int(offs[i]):int(offs[i + 1])]  # noqa: E731
-        gviews = [GroupView(view(7 + g).view(B, facts["strides"][g]), facts["strides"][g], self.page_size,
-                            groups[g].window) for g in range(ng)]
+        view = lambda name: dev[layout[name][0]:layout[name][1]]  # noqa: E731
+        gviews = [GroupView(view(f"table{g}").view(B, facts["strides"][g]), facts["strides"][g], self.page_size,
+                            groups[g].window) for g in range(len(groups))]
+        plans = {name: StepPlan({key: view(f"plan.{name}.{key}") for key in facts["plan_arrays"][name]}, dict(numbers))
+                 for name, numbers in facts["plans"].items()}
         ctx = StepContext(
-            num_tokens=T, num_entries=B, token_ids=view(0), positions=view(1), token_entry=view(2),
-            q_start=view(3), entry_slot=view(4), entry_start=view(5), groups=gviews,
-            max_q_len=facts["max_q"], max_kv_len=facts["max_kv"], decode_only=facts["decode_only"],
-            dtype=self.env.dtype,
-            decode_tokens=view(7 + ng) if facts["num_decode"] else None, num_decode=facts["num_decode"],
-            max_decode_kv=facts["max_dec_kv"], tiles=view(8 + ng).view(-1, 2) if facts["num_tiles"] else None,
-            num_tiles=facts["num_tiles"], tile_keys_total=facts["tile_keys_total"],
-            tile_keys_max=facts["tile_keys_max"], stacked_branches=self._stacked_branches,
-            host={"lens": facts["lens"], "starts": facts["starts"], "slots": facts["slots"]})
-        return ctx, (view(6) if facts["n_want"] else None)
+            num_tokens=T, num_entries=B, token_ids=view("ids"), positions=view("positions"),
+            token_entry=view("token_entry"), q_start=view("q_start"), entry_slot=view("slot"),
+            entry_start=view("start"), groups=gviews, max_q_len=facts["max_q"], max_kv_len=facts["max_kv"],
+            decode_only=facts["decode_only"], dtype=self.env.dtype, stacked_branches=self._stacked_branches,
+            host={"lens": facts["lens"], "starts": facts["starts"], "slots": facts["slots"]}, plans=plans)
+        return ctx, (view("rows") if facts["n_want"] else None)
+
+    def _forward(self, dev: torch.Tensor, layout, ctx: StepContext, rows) -> Optional[torch.Tensor]:
+        """The device work of a step, the same whether it runs now or is captured: late token ids, the state
+        rows of requests that start at their first token zeroed, the model."""
+        if self.feed_source is not None:
+            ops.feed_tokens(dev[layout["ids"][0]:layout["ids"][1]], dev[layout["feed"][0]:layout["feed"][1]],
+                            self.feed_source)
+        for state in self._states:
+            ops.zero_fresh_rows(state, ctx.entry_slot, ctx.entry_start, ctx.num_entries)
+        return self.model.forward(ctx, self.caches, rows)
 
     # ------------------------------------------------------------------ the step
     def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
@@ -275,12 +291,11 @@ class ModelRunner:
             while kv_bucket < longest:
                 kv_bucket *= 2
             kv_bucket = min(kv_bucket, self.max_table * self.page_size)
-            packed = [StepEntry(e.cache, e.tokens, [0]) for e in entries]
-            host, offs, facts = self._pack(packed, pad_entries=b_pad, table_stride=self.max_table,
-                                           allow_unknown=allow_unknown)
-            return PreparedStep(entries, host, offs, facts, (b_pad, kv_bucket))
-        host, offs, facts = self._pack(entries, allow_unknown=allow_unknown)
-        return PreparedStep(entries, host, offs, facts, None)
+            host, layout, facts = self._pack(entries, pad_entries=b_pad, table_stride=self.max_table,
+                                             allow_unknown=allow_unknown, kv_bucket=kv_bucket)
+            return PreparedStep(entries, host, layout, facts, (b_pad, kv_bucket))
+        host, layout, facts = self._pack(entries, allow_unknown=allow_unknown)
+        return PreparedStep(entries, host, layout, facts, None)
 
     def stage(self, prepared: "PreparedStep") -> None:
         """Copy a prepared step's description into pinned memory ahead of its launch (optional: the
@@ -297,34 +312,21 @@ class ModelRunner:
         if prepared.facts["unknown"]:
             raise StepError("a prepared step still holds tokens without an id")
         entries = prepared.entries
-        fresh = self.cache.take_fresh_slots()
-        if fresh:
-            for c in self._views.values():
-                if c.state is not None:
-                    c.state[torch.tensor(fresh, device=c.state.device)] = 0
         if prepared.graph_key is not None:
             logits = self._launch_graph(prepared)
         else:
             dev = self._send(prepared)
-            self._feed(dev, prepared.offs)
-            ctx, rows = self._context(dev, prepared.offs, prepared.facts)
+            ctx, rows = self._context(dev, prepared.layout, prepared.facts)
             with torch.no_grad():
-                logits = self.model.forward(ctx, self.caches, rows)
+                logits = self._forward(dev, prepared.layout, ctx, rows)
         for e in entries:
             self.cache.commit(e.cache, len(e.tokens))
         return logits
 
-    def _feed(self, dev: torch.Tensor, offs) -> None:
-        """Token ids that the step before has sampled and the host has not seen (see
-        :meth:`PreparedStep.feed_token`) are taken from ``feed_source`` on the device."""
-        if self.feed_source is not None:
-            last = len(offs) - 1
-            ops.feed_tokens(dev[int(offs[0]):int(offs[1])], dev[int(offs[last - 1]):int(offs[last])], self.feed_source)
-
     def build_context(self, entries: Sequence[StepEntry]):
         """Flatten the entries into device tensors (one host-to-device copy)."""
-        host, offs, facts = self._pack(entries)
-        return self._context(self._upload(host), offs, facts)
+        host, layout, facts = self._pack(entries)
+        return self._context(self._upload(host), layout, facts)
 
     # ------------------------------------------------------------------ HIP graphs for decode steps
     def _launch_graph(self, prepared: "PreparedStep") -> Optional[torch.Tensor]:
@@ -332,23 +334,26 @@ class ModelRunner:
         B = len(entries)
         graph = self._graphs.get(prepared.graph_key)
         if graph is None:
-            graph = self._capture(prepared.graph_key, prepared.host, prepared.offs, prepared.facts)
+            graph = self._capture(prepared.graph_key, prepared.host, prepared.layout, prepared.facts)
         else:
+            if prepared.layout != graph.layout or prepared.facts["plans"] != graph.plan_facts:
+                raise StepError("a step planner gave a decode step of the same batch and context bucket another "
+                                "layout or other numbers than the captured graph has")
             self._send(prepared, into=graph.static_dev)
         graph.graph.replay()
-        wanted = [b for b, e in enumerate(entries) if len(e.want)]
-        if not wanted:
+        picked = prepared.facts["picked"]
+        if not picked:
             return None
-        if len(wanted) == B:
+        if len(picked) == B:
             return graph.logits[:B]
-        return graph.logits[torch.tensor(wanted, device=graph.logits.device)]
+        # some entries want nothing: their rows are left out by a gather fed from the packed buffer
+        first = prepared.layout["picked"][0]
+        return ops.gather_rows(graph.logits, graph.static_dev[first:first + len(picked)])
 
-    def _capture(self, key, host: np.ndarray, offs, facts) -> "_DecodeGraph":
-        b_pad, kv_bucket = key
-        facts = dict(facts, max_dec_kv=kv_bucket, max_kv=kv_bucket)    # the kernels' split of the keys is fixed
+    def _capture(self, key, host: np.ndarray, layout, facts) -> "_DecodeGraph":
         static_dev = torch.empty(host.size, dtype=torch.int32, device=self.env.device)
         self._upload(host, into=static_dev)
-        ctx, rows = self._context(static_dev, offs, facts)
+        ctx, rows = self._context(static_dev, layout, facts)
         with torch.no_grad():
             # once eagerly on a side stream: loads the kernels and sizes the library's workspaces.  Keys and
             # values written twice are the same keys and values; state that a step moves on is put back.
@@ -357,8 +362,7 @@ class ModelRunner:
             side = torch.cuda.Stream()
             side.wait_stream(torch.cuda.current_stream())
             with torch.cuda.stream(side):
-                self._feed(static_dev, offs)
-                self.model.forward(ctx, self.caches, rows)
+                self._forward(static_dev, layout, ctx, rows)
                 for t, was in zip(states, saved):
                     t.copy_(was)
             torch.cuda.current_stream().wait_stream(side)
@@ -366,9 +370,8 @@ class ModelRunner:
                 self._graph_pool = torch.cuda.graph_pool_handle()
             g = torch.cuda.CUDAGraph()
             with torch.cuda.graph(g, pool=self._graph_pool):
-                self._feed(static_dev, offs)
-                logits = self.model.forward(ctx, self.caches, rows)
-        graph = _DecodeGraph(g, static_dev, logits)
+                logits = self._forward(static_dev, layout, ctx, rows)
+        graph = _DecodeGraph(g, static_dev, logits, dict(layout), dict(facts["plans"]))
         self._graphs[key] = graph
         return graph
 
@@ -378,26 +381,25 @@ class PreparedStep:
     """A step whose host work is done (see :meth:`ModelRunner.prepare`)."""
     entries: List[StepEntry]
     host: np.ndarray                  # the packed batch description
-    offs: np.ndarray
+    layout: dict                      # field name -> (first, end) in it
     facts: dict
     graph_key: Optional[tuple]        # (batch bucket, context bucket) if the step replays a graph
     staged: Optional[torch.Tensor] = None   # the description already in pinned memory (see ModelRunner.stage)
 
     def unknown_tokens(self) -> List[tuple]:
         """(entry, index among the entry's tokens) of every token that still needs an id."""
-        return [(b, j) for _, b, j in self.facts["unknown"]]
+        return [(b, j) for _, _, b, j in self.facts["unknown"]]
 
     def fill_token(self, k: int, token: int) -> None:
         """Give the k-th unknown token its id."""
-        at = int(self.offs[0]) + self.facts["unknown"][k][0]
+        at = self.facts["unknown"][k][0]
         self.host[at] = token
         if self.staged is not None:
             self.staged[at] = token
 
     def feed_token(self, k: int, index: int) -> None:
         """The k-th unknown token is entry ``index`` of the runner's ``feed_source`` when the step runs."""
-        t = self.facts["unknown"][k][0]
-        at = int(self.offs[len(self.offs) - 2]) + t
+        at = self.facts["unknown"][k][1]
         self.host[at] = index
         if self.staged is not None:
             self.staged[at] = index
@@ -411,3 +413,5 @@ class _DecodeGraph:
     graph: "torch.cuda.CUDAGraph"
     static_dev: torch.Tensor          # the packed batch description the captured kernels read
     logits: torch.Tensor              # float32 [batch bucket, vocab], rewritten by every replay
+    layout: dict                      # where the captured kernels read each field
+    plan_facts: dict                  # the planners' numbers the kernels were launched with

@@ -106,6 +106,32 @@ def feed_tokens(ids: torch.Tensor, feed: torch.Tensor, source: torch.Tensor) -> 
                                                       _c_int(source.numel()), _stream()), "feed_tokens")
 
 
+def zero_fresh_rows(state: torch.Tensor, entry_slot: torch.Tensor, entry_start: torch.Tensor, n_entries: int) -> None:
+    """state[entry_slot[b]] = 0 for every entry b < n_entries with entry_start[b] == 0: the per-request state
+    rows (``state`` contiguous [slots, anything]) of requests that step from their first token.  Takes
+    everything from device tensors, so it can be part of a captured step."""
+    _need(state.is_contiguous() and state.dim() >= 1, "state must be contiguous [slots, ...]")
+    _i32(entry_slot, "entry_slot", n_entries)
+    _i32(entry_start, "entry_start", n_entries)
+    rows = state.shape[0]
+    row_bytes = (state.numel() // max(1, rows)) * state.element_size()
+    _check(build.load("elementwise").ullm_zero_fresh_rows(_p(state), ctypes.c_longlong(row_bytes), _c_int(rows),
+                                                         _p(entry_slot), _p(entry_start), _c_int(n_entries), _stream()),
+           "zero_fresh_rows")
+
+
+def gather_rows(src: torch.Tensor, index: torch.Tensor) -> torch.Tensor:
+    """src[index] for float32 ``src`` [n, cols] and int32 ``index`` on the device: no index travels from the
+    host and nothing waits for the device."""
+    _need(src.dtype == torch.float32 and src.dim() == 2 and src.stride(1) == 1, "gather_rows takes float32 [n, cols]")
+    _i32(index, "index")
+    n, cols = index.numel(), src.shape[1]
+    out = torch.empty((n, cols), dtype=torch.float32, device=src.device)
+    _check(build.load("elementwise").ullm_gather_rows(_p(src), ctypes.c_longlong(src.stride(0)), _c_int(src.shape[0]),
+                                                     _p(index), _p(out), _c_int(n), _c_int(cols), _stream()), "gather_rows")
+    return out
+
+
 def add_rmsnorm(branch: Optional[torch.Tensor], residual: torch.Tensor, gain: torch.Tensor, eps: float,
                 out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None,
                 out: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -455,7 +481,19 @@ def attention_mfma_supports(dtype: torch.dtype, hd: int, page_size: int, nq: int
         _c_int(hd), _c_int(page_size), _c_int(nq), _c_int(nkv)))
 
 
-def decode_split(n_items: int, nkv: int, groups: int, max_kv: int, hd: int = 128):
+_units_of_device = {}
+
+
+def compute_units(device=None) -> int:
+    """Compute units of the device the kernels run on (256 on an MI355X)."""
+    index = torch.cuda.current_device() if device is None else torch.device(device).index or 0
+    n = _units_of_device.get(index)
+    if n is None:
+        n = _units_of_device[index] = int(torch.cuda.get_device_properties(index).multi_processor_count)
+    return n
+
+
+def decode_split(n_items: int, nkv: int, groups: int, max_kv: int, hd: int = 128, window: int = 0, units: int = 256):
     """(waves, num_splits) of the decode attention launch.  A wave walks its keys one 32-key tile after
     the other, each a round trip to memory, so few (token, kv head) pairs with many keys are cut over
     several blocks, up to one block per compute unit (more would run in a second round), and a second
@@ -463,22 +501,26 @@ def decode_split(n_items: int, nkv: int, groups: int, max_kv: int, hd: int = 128
     tiles, so short contexts are not cut.  Mostly a block is a single wave (several are resident on a
     SIMD, they start and end independently and one's start overlaps the others' streaming, and their number
     need not be a multiple of the compute units); four waves a block where few pairs have very many keys.
-    (Timings behind these choices: profiles/decode_attention_shapes_qwen3_8b.md.)"""
+    With a window a token reads at most the window's keys (and up to 31 before them, to the tile's edge),
+    however long its context is.  ``units``: the device's compute units, four SIMDs each."""
     pairs = max(1, n_items * nkv * groups)
-    if pairs >= 1024:
+    simds = 4 * units
+    if pairs >= simds:
         return 1, 1
+    if window > 0:
+        max_kv = min(max_kv, window + 31)
     tiles = -(-max_kv // 32)
-    if pairs > 256:
+    if pairs > units:
         # single waves, two to four to a SIMD, so that the launch has no rounds of whole blocks (four-wave blocks,
-        # one to a compute unit, take 49 us at 264 pairs against 30 us at 256); up to 576 pairs cut in three where
-        # that still gives at most one wave per SIMD and compute unit, else in two
-        return 1, (max(2, min(3, 1024 // pairs)) if pairs <= 576 and tiles > 16 else 1)
-    if pairs == 256:
+        # one to a compute unit, take 49 us at 264 pairs against 30 us at 256); up to 2.25 pairs a unit cut in three
+        # where that still gives at most one wave per SIMD and compute unit, else in two
+        return 1, (max(2, min(3, simds // pairs)) if pairs <= units * 9 // 4 and tiles > 16 else 1)
+    if pairs == units:
         return (4 if tiles > 16 else 1), 1
-    splits = min(16, max(1, 512 // pairs), tiles)
+    splits = min(16, max(1, 2 * units // pairs), tiles)
     if tiles > 8 * splits:
-        splits = min(16, max(1, 1024 // pairs), tiles)
-    waves = 4 if (tiles > 4 * splits and pairs * splits * 4 <= 1024) else 1
+        splits = min(16, max(1, simds // pairs), tiles)
+    waves = 4 if (tiles > 4 * splits and pairs * splits * 4 <= simds) else 1
     return waves, splits
 
 
@@ -501,7 +543,7 @@ def attention_decode_mfma(q, out, k_pool, v_pool, token_list: Optional[torch.Ten
           "block_table must be int32 [B, stride]")
     _need(-(-max_kv // page_size) <= block_table.shape[1], "block table narrower than the longest context")
     groups = -(-(nq // nkv) // 16)
-    auto_waves, auto_splits = decode_split(n_items, nkv, groups, max_kv, hd)
+    auto_waves, auto_splits = decode_split(n_items, nkv, groups, max_kv, hd, window, compute_units(q.device))
     waves = waves or auto_waves
     if hd == 256 and waves == 8:
         waves = 4
@@ -558,7 +600,7 @@ def attention_decode_fused(qkv, out, q_gain: Optional[torch.Tensor], k_gain: Opt
               "cos_sin must be float32 [positions, rotary_dim]")
         table_rows = cos_sin.shape[0]
     groups = -(-(nq // nkv) // 16)
-    auto_waves, auto_splits = decode_split(n_items, nkv, groups, max_kv, hd)
+    auto_waves, auto_splits = decode_split(n_items, nkv, groups, max_kv, hd, window, compute_units(qkv.device))
     waves = waves or auto_waves
     if hd == 256 and waves == 8:
         waves = 4
@@ -623,25 +665,29 @@ def _warn_general_attention(hd: int, page_size: int) -> None:
 
 
 def paged_attention(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, ctx, group, nq: int,
-                    nkv: int, hd: int, scale: float, window: int) -> torch.Tensor:
+                    nkv: int, hd: int, scale: float, window: int, plan=None) -> torch.Tensor:
     """Attention of the batch's queries over their requests' cached keys and values (the new
     tokens' rows included).  bfloat16 shapes the matrix-core kernels take go there (one launch for
-    the one-token entries, one for the tiles of longer entries); everything else, and float32
-    always, takes the general kernel.  Every choice computes the same function."""
+    the one-token entries, one for the tiles of longer entries, both listed in ``plan``: arrays
+    ``decode_tokens`` and ``tiles``, numbers ``num_decode``, ``max_decode_kv``, ``num_tiles``,
+    ``tile_keys_total``, ``tile_keys_max``); everything else, and float32 always, takes the general
+    kernel.  Every choice computes the same function."""
     if not attention_mfma_supports(q.dtype, hd, group.page_size, nq, nkv):
         if q.dtype == torch.bfloat16:
             _warn_general_attention(hd, group.page_size)
         return paged_attention_generic(q, k_pool, v_pool, ctx.positions, ctx.token_entry, group.block_table,
                                        group.page_size, nq, nkv, hd, scale, window)
+    _need(plan is not None, "the matrix-core attention kernels need the step's work lists (a step plan)")
     out = torch.empty((q.shape[0], nq * hd), dtype=q.dtype, device=q.device)
-    if ctx.num_decode:
-        attention_decode_mfma(q, out, k_pool, v_pool, ctx.decode_tokens, ctx.num_decode, ctx.positions,
+    n = plan.facts
+    if n["num_decode"]:
+        attention_decode_mfma(q, out, k_pool, v_pool, plan.arrays["decode_tokens"], n["num_decode"], ctx.positions,
                               ctx.token_entry, group.block_table, group.page_size, nq, nkv, hd, scale, window,
-                              ctx.max_decode_kv)
-    if ctx.num_tiles:
-        attention_prefill_mfma(q, out, k_pool, v_pool, ctx.tiles, ctx.num_tiles, ctx.positions, ctx.token_entry,
-                               group.block_table, group.page_size, nq, nkv, hd, scale, window,
-                               keys_total=ctx.tile_keys_total, keys_max=ctx.tile_keys_max)
+                              n["max_decode_kv"])
+    if n["num_tiles"]:
+        attention_prefill_mfma(q, out, k_pool, v_pool, plan.arrays["tiles"], n["num_tiles"], ctx.positions,
+                               ctx.token_entry, group.block_table, group.page_size, nq, nkv, hd, scale, window,
+                               keys_total=n["tile_keys_total"], keys_max=n["tile_keys_max"])
     return out
 
 

@@ -100,19 +100,22 @@ class Model:
         """Groups of caches with equal needs, and the per-request state needs.  A cache is named by
         (cache id, index of the need among those its block declares).
         Returns (groups, {(cache id, need index): group index}, {(cache id, need index): StateNeed})."""
-        keyed: Dict[Tuple[int, int, int], List[Tuple[int, int]]] = {}
+        keyed: Dict[KVNeed, List[Tuple[int, int]]] = {}
         states: Dict[Tuple[int, int], StateNeed] = {}
         for cache_id, idx in self.cache_owner.items():
             for i, need in enumerate(cache_needs_of(self.blocks[self.run_order[idx][0]])):
                 if isinstance(need, KVNeed):
-                    keyed.setdefault((need.num_kv_heads, need.head_dim, need.window), []).append((cache_id, i))
+                    keyed.setdefault(need, []).append((cache_id, i))
                 else:
                     states[(cache_id, i)] = need
         groups, cache_group = [], {}
-        for (nkv, hd, window), keys in keyed.items():
+        for need, keys in keyed.items():
             for c in keys:
                 cache_group[c] = len(groups)
-            groups.append(CacheGroupSpec(nkv, hd, window, tuple(keys)))
+            rows = tuple((r.heads, r.dim, None if r.dtype is None else torch.empty((), dtype=r.dtype).element_size())
+                         for r in need.rows) if need.rows else None
+            groups.append(CacheGroupSpec(need.num_kv_heads, need.head_dim, need.window, tuple(keys), rows))
+        self._group_needs = list(keyed)
         for idx, (layer, cache_id) in enumerate(self.run_order):
             owner_layer = self.run_order[self.cache_owner[cache_id]][0]
             a, b = cache_needs_of(self.blocks[layer]), cache_needs_of(self.blocks[owner_layer])
@@ -120,6 +123,11 @@ class Model:
                 raise ValueError(f"layer {layer} reads cache {cache_id} written by layer {owner_layer} "
                                  f"but their needs differ: {a} vs {b}")
         return groups, cache_group, states
+
+    def group_needs(self) -> List[KVNeed]:
+        """The paged need of every cache group, in the order of :meth:`cache_layout`'s groups."""
+        self.cache_layout()
+        return self._group_needs
 
     def num_needs(self, cache_id: int) -> int:
         """How many needs the block that owns this cache declares."""

@@ -6,13 +6,25 @@ bound in :300-336.
 """
 from __future__ import annotations
 
+import logging
+
 from ..config.model_config import Qwen3Config
 from .model import Choice, ModelPlan
 from .registry import register_architecture
 
+logger = logging.getLogger("ullm_amd")
+
 
 def qwen3_plan(cfg: Qwen3Config) -> ModelPlan:
     layers = []
+    windowed = [i for i in range(cfg.num_hidden_layers) if cfg.window_of_layer(i) > 0]
+    if windowed:
+        # the reference reads none of the sliding-window keys (ullm/models/qwen3.py:48-112 builds every layer
+        # with full attention): which layers look back how far is decided here alone
+        logger.warning("config.json switches sliding-window attention on (%d of %d layers look back %d keys): the "
+                       "reference applies no window, so which layers are windowed and which keys they see is this "
+                       "engine's own reading of use_sliding_window / sliding_window / max_window_layers / layer_types",
+                       len(windowed), cfg.num_hidden_layers, cfg.sliding_window)
     for i in range(cfg.num_hidden_layers):
         p = f"model.layers.{i}"
         position = Choice("position", "rotary", dict(

@@ -10,10 +10,12 @@ from __future__ import annotations
 
 from typing import Dict, List, Optional
 
+import numpy as np
 import torch
 
 from ..kernels import ops
-from .base import KVNeed, LayerCache, Mixer, PartEnv, PositionEncoding, StepContext, WeightDecl, register_part
+from .base import (KVNeed, LayerCache, Mixer, PartEnv, PositionEncoding, StepContext, StepPlan, StepShape, WeightDecl,
+                   register_part)
 from .linear import can_fuse, linear, linear_into_stream, linear_of_norm
 
 
@@ -23,9 +25,37 @@ from .linear import can_fuse, linear, linear_into_stream, linear_of_norm
 FUSED_DECODE_MAX_TOKENS = 64
 
 
+def plan_attention_step(shape: StepShape) -> StepPlan:
+    """How the attention kernels split a batch: the tokens of one-token entries (``decode_tokens``, longest
+    context first: the short ones fill the tail of the launch), and tiles of up to ``ops.PREFILL_TILE``
+    consecutive tokens (first token, count) of the longer entries by rising number of keys (``tiles``), with
+    the numbers the launches are shaped by.  Padding entries of a captured batch are one-token entries."""
+    dec, tiles, max_decode_kv, t0 = [], [], 0, 0
+    for n, start in zip(shape.lens, shape.starts):
+        if n == 1:
+            dec.append((-start, t0))
+            max_decode_kv = max(max_decode_kv, start + 1)
+        else:
+            for first in range(0, n, ops.PREFILL_TILE):
+                count = min(ops.PREFILL_TILE, n - first)
+                tiles.append((start + first + count, t0 + first, count))
+        t0 += n
+    tiles.sort()
+    dec.sort()
+    decode_tokens = [t for _, t in dec] + list(range(t0, t0 + shape.pad_entries))
+    if shape.kv_bucket is not None:
+        max_decode_kv = shape.kv_bucket                   # a captured launch: the split of the keys is fixed
+    return StepPlan(
+        arrays={"decode_tokens": np.asarray(decode_tokens, dtype=np.int32),
+                "tiles": np.asarray([x for _, first, count in tiles for x in (first, count)], dtype=np.int32)},
+        facts={"num_decode": len(decode_tokens), "max_decode_kv": max_decode_kv, "num_tiles": len(tiles),
+               "tile_keys_total": sum(k for k, _, _ in tiles), "tile_keys_max": tiles[-1][0] if tiles else 0})
+
+
 @register_part("mixer", "gqa_attention")
 class GQAttention(Mixer):
     folds_norm = True
+    step_planners = {"attention": plan_attention_step}
 
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, prefix: str,
                  position: Optional[PositionEncoding] = None, qk_norm_eps: Optional[float] = None,
@@ -93,14 +123,17 @@ class GQAttention(Mixer):
         group = ctx.groups[cache.group]
         table, rot, style = self.position.kernel_args() if self.position is not None else (None, 0, 0)
         eps = self.qk_norm_eps if self.qk_norm_eps is not None else 0.0
-        if (ctx.num_decode == T and not ctx.num_tiles and T <= FUSED_DECODE_MAX_TOKENS
+        plan = ctx.plans["attention"]
+        work = plan.facts
+        if (work["num_decode"] == T and not work["num_tiles"] and T <= FUSED_DECODE_MAX_TOKENS
                 and ops.attention_decode_fused_supports(x.dtype, self.hd, group.page_size, self.nq, self.nkv, rot, style)):
             # a step of single new tokens: norm, rotation and cache write happen inside the attention kernel
             out = torch.empty((T, self.nq * self.hd), dtype=x.dtype, device=x.device)
             ops.attention_decode_fused(
                 qkv, out, self.q_gain, self.k_gain, eps, table, rot, style, cache.k_pool, cache.v_pool,
-                ctx.decode_tokens, ctx.num_decode, ctx.positions, ctx.token_entry, group.block_table, group.page_size,
-                self.nq, self.nkv, self.hd, self.scale, self.window, ctx.max_decode_kv, write_kv=cache.owner)
+                plan.arrays["decode_tokens"], work["num_decode"], ctx.positions, ctx.token_entry, group.block_table,
+                group.page_size, self.nq, self.nkv, self.hd, self.scale, self.window, work["max_decode_kv"],
+                write_kv=cache.owner)
             return out
         q = torch.empty((T, self.nq * self.hd), dtype=x.dtype, device=x.device)
         ops.qk_norm_rope_write(
@@ -108,4 +141,4 @@ class GQAttention(Mixer):
             table, rot, style, ctx.positions, ctx.token_entry, group.block_table,
             cache.k_pool, cache.v_pool, group.page_size, self.nq, self.nkv, self.hd, write_kv=cache.owner)
         return ops.paged_attention(q, cache.k_pool, cache.v_pool, ctx, group, self.nq, self.nkv, self.hd,
-                                   self.scale, self.window)
+                                   self.scale, self.window, plan)

@@ -36,11 +36,34 @@ class WeightDecl:
 # --------------------------------------------------------------------------- cache needs
 
 @dataclass(frozen=True)
+class CacheRows:
+    """One pool of a paged cache: per token and head a row of ``dim`` values.  The pool is
+    [pages, heads, page_size, dim], or with ``transposed`` [pages, heads, dim, page_size] (a page's tokens
+    side by side for every dim)."""
+    name: str
+    heads: int
+    dim: int
+    transposed: bool = False
+    dtype: Optional[torch.dtype] = None      # None: the compute dtype
+
+
+@dataclass(frozen=True)
 class KVNeed:
-    """A mixer that keeps one key row and one value row per token and kv head."""
+    """A mixer that keeps rows per token in pages.  By default one key row and one value row per token
+    and kv head (pools "k" [pages, kv_heads, page_size, head_dim] and "v", transposed inside the page,
+    [pages, kv_heads, head_dim, page_size]: the layout the attention kernels read).  A mixer that keeps
+    something else per token (one latent row, keys only, rows in another dtype) names its pools in
+    ``rows``; it then gets exactly those, as ``cache.pools[name]``, and nothing else."""
     num_kv_heads: int
     head_dim: int
     window: int = 0               # keys a query looks back over, itself included; 0 = all
+    rows: Tuple[CacheRows, ...] = ()
+
+    def pools(self) -> Tuple[CacheRows, ...]:
+        if self.rows:
+            return self.rows
+        return (CacheRows("k", self.num_kv_heads, self.head_dim),
+                CacheRows("v", self.num_kv_heads, self.head_dim, transposed=True))
 
 
 @dataclass(frozen=True)
@@ -96,26 +119,55 @@ class LayerCache:
     and hands each of its mixers the one that is its own (``cache.parts[i]``); the outer view's own
     fields then show the first need of each kind, so a block with one need never looks at ``parts``."""
     group: int = -1                        # index into StepContext.groups for KV mixers
-    k_pool: Optional[torch.Tensor] = None  # [num_pages, kv_heads, page_size, head_dim]
-    v_pool: Optional[torch.Tensor] = None  # [num_pages, kv_heads, head_dim, page_size]
+    k_pool: Optional[torch.Tensor] = None  # pools["k"]: [num_pages, kv_heads, page_size, head_dim]
+    v_pool: Optional[torch.Tensor] = None  # pools["v"]: [num_pages, kv_heads, head_dim, page_size]
     state: Optional[torch.Tensor] = None   # [num_slots, *StateNeed.shape]
     owner: bool = True                     # False: reads another layer's cache, writes nothing
     parts: List["LayerCache"] = field(default_factory=list)
+    pools: Dict[str, torch.Tensor] = field(default_factory=dict)   # every pool the need declared, by name
+
+    @staticmethod
+    def of_pools(group: int, pools: Dict[str, torch.Tensor]) -> "LayerCache":
+        return LayerCache(group=group, k_pool=pools.get("k"), v_pool=pools.get("v"), pools=dict(pools))
 
     @staticmethod
     def of_parts(parts: List["LayerCache"]) -> "LayerCache":
         """The view of a block from the views of its needs."""
         if len(parts) == 1:
             return parts[0]
-        kv = next((p for p in parts if p.k_pool is not None), None)
+        kv = next((p for p in parts if p.pools), None)
         st = next((p for p in parts if p.state is not None), None)
         return LayerCache(group=kv.group if kv else -1, k_pool=kv.k_pool if kv else None,
-                          v_pool=kv.v_pool if kv else None, state=st.state if st else None, parts=list(parts))
+                          v_pool=kv.v_pool if kv else None, state=st.state if st else None, parts=list(parts),
+                          pools=dict(kv.pools) if kv else {})
 
     def reader(self) -> "LayerCache":
         """The same cache for a layer that only reads it."""
         return LayerCache(self.group, self.k_pool, self.v_pool, self.state, owner=False,
-                          parts=[p.reader() for p in self.parts])
+                          parts=[p.reader() for p in self.parts], pools=self.pools)
+
+
+@dataclass(frozen=True)
+class StepShape:
+    """What a step planner is told about a batch (host numbers only)."""
+    lens: Tuple[int, ...]         # new tokens of each entry, in batch order
+    starts: Tuple[int, ...]       # tokens each entry's request holds in the cache before the step
+    pad_entries: int = 0          # one-token entries appended behind them for a captured graph: position 0, no pages
+    kv_bucket: Optional[int] = None   # the step replays a captured graph: launch shapes must be those of this context length
+
+
+@dataclass
+class StepPlan:
+    """A kernel family's own view of a step: work lists (int32 arrays; they travel to the device inside
+    the step's one packed buffer and come back as tensors) and host numbers (grid sizes, counts).
+
+    A part names the planners its kernels need in ``Part.step_planners`` ({name: function of a
+    :class:`StepShape`}); the step function runs each once per step and the part finds the result as
+    ``ctx.plans[name]``.  For a step that replays a captured graph (``shape.kv_bucket`` is set) the arrays'
+    sizes may depend only on the number of entries including padding, and the numbers only on that and
+    the bucket: the captured kernels read the arrays at fixed places and were launched with those numbers."""
+    arrays: Dict[str, object] = field(default_factory=dict)   # host: numpy int32 arrays; in a StepContext: device tensors
+    facts: Dict[str, int] = field(default_factory=dict)
 
 
 @dataclass
@@ -135,15 +187,8 @@ class StepContext:
     decode_only: bool             # every entry brings exactly one token
     dtype: torch.dtype = torch.bfloat16          # compute dtype of activations
     host: dict = field(default_factory=dict)   # host-side copies for parts that want them
-    # how attention kernels split the batch: tokens of one-token entries, and tiles of up to 32
-    # consecutive tokens (first token, count) of the longer entries
-    decode_tokens: Optional[torch.Tensor] = None   # int32 [n_decode]: the one-token entries, longest context first
-    num_decode: int = 0
-    max_decode_kv: int = 0
-    tiles: Optional[torch.Tensor] = None           # int32 [n_tiles, 2]
-    num_tiles: int = 0
-    tile_keys_total: int = 0      # sum over the tiles of the keys each tile's last token sees
-    tile_keys_max: int = 0        # the most keys any tile sees (both: how the tiles' work is spread)
+    # what the planners named by the model's parts made of this step (Part.step_planners), by name
+    plans: Dict[str, StepPlan] = field(default_factory=dict)
     # every norm of the model takes a stack [S, T, hidden] of float32 partial sums as its branch and
     # adds them up (Norm.adds_stacks): a mixer or feed-forward may then return such a stack
     stacked_branches: bool = False
@@ -179,6 +224,8 @@ class Part:
     says no keeps the whole model on eager steps."""
     kind = ""
     graph_safe = True
+    # {name: function(StepShape) -> StepPlan}: per-step work lists this part's kernels want (see StepPlan)
+    step_planners: Dict[str, Callable] = {}
 
     def weights(self) -> List[WeightDecl]:
         return []

@@ -45,7 +45,10 @@ class Replayer:
         if max_tokens < 1:
             raise ValueError("max_tokens must be positive")
         self.max_tokens = -(-max_tokens // 64) * 64
-        self.cfg, self.model, self.env = load_model(model_dir, dtype, device, context_len=self.max_tokens)
+        # max_tokens sizes the pool and bounds a request; a trace is replayed as given, also past the positions
+        # the model's configuration names (that is said once, not refused)
+        self.cfg, self.model, self.env = load_model(model_dir, dtype, device, context_len=self.max_tokens,
+                                                    strict_context=False)
         self.runner = ModelRunner(self.model, self.env, page_size=page_size,
                                   num_pages=self.max_tokens // page_size, max_requests=max_requests,
                                   use_graphs=use_graphs)
