@@ -6,12 +6,13 @@
 One JSON line.  ``value`` = decoded tokens per second at batch 8 of Qwen3-8B sizes (every request with a
 1024-token prompt), timed over exactly K engine steps (schedule + model step + sampling) after W untimed
 ones.  ``prefill`` = one 2048-token prompt.  ``roofline`` = bytes a decode step has to read (every weight
-once + the live requests' cache) over its time, against 8 TB/s (``frac``) and against what a plain device
-copy reaches on this GPU (``frac_of_measured``).  ``points`` = tokens per second of the other workloads
-(decode at batch 1 and 64, Qwen3-32B sizes at batch 64 with 4096-token contexts and its 2048-token prefill,
-the 256-request mixed workloads at Qwen3-14B and Qwen3-0.6B sizes); ``points_detail`` says at which context
-each ran and how far from its roofline.  ``measured_peaks`` = the copy and a large bfloat16 product on this
-GPU.  The reference publishes no number for this configuration, so ``vs_baseline`` is null.
+once + the live requests' cache) over its time, against 8 TB/s (``frac``) and against what a kernel that
+only reads reaches on this GPU (``frac_of_measured``).  ``points`` = tokens per second of the other workloads
+(decode at batch 1 and 64; batch 8 at 16K-token, batch 64 at 8K-token and batch 1 at 32K-token contexts; a
+16,384-token prompt; Qwen3-14B and Qwen3-32B sizes at batch 8, Qwen3-32B at batch 64 with 4096-token contexts
+and its 2048-token prefill; the 256-request mixed workloads at Qwen3-14B and Qwen3-0.6B sizes);
+``points_detail`` says at which context each ran and how far from its roofline.  ``measured_peaks`` = a
+streaming read, a device copy and a large bfloat16 product on this GPU.  The reference publishes no number for this configuration, so ``vs_baseline`` is null.
 """
 import argparse
 import json
@@ -28,6 +29,7 @@ PEAK_FLOPS = {"bfloat16": 2.5e15, "float32": 157.3e12}
 # generation lengths uniform in 100..1024, temperature 0.6, no end-of-sequence; 9032.37 tokens/s on an A100 40GB
 REFERENCE_MIXED_TOK_S = 9032.37
 SIZES = ("0.6b", "8b", "14b", "32b")
+LONGEST_CONTEXT = 32768 + 64       # the longest context any point of the default run reaches
 
 
 def parse_args():
@@ -77,10 +79,20 @@ def step_flops(cfg, n_tokens, kv_lens_sum_causal, n_logit_rows):
 
 
 def measured_peaks():
-    """What this GPU reaches on a plain device-to-device copy (bytes read + written per second) and on a large
-    square bfloat16 product of the library: the practical ceilings beside the datasheet's."""
+    """What this GPU reaches with a kernel that only reads (4 GiB, non-temporal 16-byte loads: what a decode
+    step's weight streaming could reach at best), on a plain device-to-device copy (bytes read + written per
+    second) and on a large square bfloat16 product of the library: the practical ceilings beside the datasheet's."""
     import torch
+    from ullm_amd.kernels import ops
     src = torch.empty(1 << 30, dtype=torch.float32, device="cuda:0").normal_()
+    for _ in range(2):
+        ops.stream_read(src)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(5):
+        ops.stream_read(src)
+    torch.cuda.synchronize()
+    read_gbs = 5 * src.numel() * 4 / (time.perf_counter() - t0) / 1e9
     dst = torch.empty_like(src)
     for _ in range(2):
         dst.copy_(src)
@@ -104,13 +116,13 @@ def measured_peaks():
     gemm_tflops = 10 * 2 * n ** 3 / (time.perf_counter() - t0) / 1e12
     del a, b
     torch.cuda.empty_cache()
-    return {"copy_GBs": round(copy_gbs, 1), "gemm_bf16_8192_TFLOPs": round(gemm_tflops, 1)}
+    return {"read_GBs": round(read_gbs, 1), "copy_GBs": round(copy_gbs, 1), "gemm_bf16_8192_TFLOPs": round(gemm_tflops, 1)}
 
 
 class Sized:
     """A model of one named size with random weights on the device, and the runs it is timed on."""
 
-    def __init__(self, size, dtype, context_len, layers=None, eager=False):
+    def __init__(self, size, dtype, context_len, layers=None, eager=False, longest_context=None):
         import torch
         from ullm_amd.config import parse_random_weights
         from ullm_amd.engine.loading import make_env
@@ -122,19 +134,23 @@ class Sized:
         if layers is not None:
             config["num_hidden_layers"] = layers
         self.cfg, self.model = build_model(config)
-        self.env = make_env(dtype, "cuda:0", context_len)
+        # the model (its position table) is built once for the longest context any point runs at; every engine
+        # gets an environment with its own context length (block tables as wide as that context needs)
+        self.env = make_env(dtype, "cuda:0", max(context_len, longest_context or 0))
         bind_random_weights(self.model, self.env, seed=0)
         self.itemsize = 2 if dtype == "bfloat16" else 4
         self.wbytes = weight_bytes(self.model, self.itemsize)
         self.kv_per_token = sum(g.bytes_per_token(self.itemsize) for g in self.model.cache_layout()[0])
         self.gen = torch.Generator().manual_seed(0)
 
-    def engine(self, **kw):
+    def engine(self, context_len=None, **kw):
+        import dataclasses
         from ullm_amd import EngineConfig
         from ullm_amd.engine.engine import Engine
-        ec = EngineConfig(model="(random weights)", dtype=self.dtype, context_len=self.context_len, page_size=16,
+        context_len = context_len or self.context_len
+        ec = EngineConfig(model="(random weights)", dtype=self.dtype, context_len=context_len, page_size=16,
                           enforce_eager=self.eager, **kw)
-        return Engine(ec, model=self.model, env=self.env, model_config=self.cfg)
+        return Engine(ec, model=self.model, env=dataclasses.replace(self.env, context_len=context_len), model_config=self.cfg)
 
     def _check_finite_once(self, eng):
         """The next step's logits must be finite (checked outside the timed steps)."""
@@ -146,14 +162,14 @@ class Sized:
                 raise RuntimeError(f"Qwen3-{self.size}: a step returned logits that are not finite")
         eng.on_logits = check
 
-    def decode(self, batch, steps, warmup, prompt_len, top_k=-1, top_p=1.0):
+    def decode(self, batch, steps, warmup, prompt_len, top_k=-1, top_p=1.0, context_len=None):
         """(tokens/s, ms per step, bytes read per step, mean context) over exactly ``steps`` engine steps."""
         from ullm_amd import SamplingParams
         torch = self.torch
         budget = max(8192, batch)
         # requests that finish their prompt early decode while the others are still in theirs
         new_tokens = warmup + steps + 4 + -(-batch * prompt_len // budget)
-        eng = self.engine(max_bs=batch, num_pages=batch * (-(-(prompt_len + new_tokens + 16) // 16)),
+        eng = self.engine(context_len=context_len, max_bs=batch, num_pages=batch * (-(-(prompt_len + new_tokens + 16) // 16)),
                           max_num_batched_tokens=budget, max_prefill_chunk=2048)
         for i in range(batch):
             prompt = torch.randint(0, self.cfg.vocab_size, (prompt_len,), generator=self.gen).tolist()
@@ -184,11 +200,12 @@ class Sized:
         """(tokens/s, ms, fraction of the dtype's matrix peak) of one prompt of n_tokens, best of three."""
         from ullm_amd import SamplingParams
         torch = self.torch
-        if n_tokens >= self.context_len:
+        context_len = max(self.context_len, n_tokens + 16)
+        if context_len > self.env.context_len:
             # the engine would keep the prompt's last context_len tokens and the figures would be of those
             raise SystemExit(f"a prompt of {n_tokens} tokens needs --context-len above {n_tokens} (it is {self.context_len})")
-        eng = self.engine(max_bs=1, num_pages=-(-(n_tokens + 16) // 16), max_num_batched_tokens=n_tokens,
-                          max_prefill_chunk=n_tokens)
+        eng = self.engine(context_len=context_len, max_bs=1, num_pages=-(-(n_tokens + 16) // 16),
+                          max_num_batched_tokens=n_tokens, max_prefill_chunk=n_tokens)
         best = None
         for rep in range(4):
             prompt = torch.randint(0, self.cfg.vocab_size, (n_tokens,), generator=self.gen).tolist()
@@ -244,11 +261,11 @@ class Sized:
         self.torch.cuda.empty_cache()
 
 
-def decode_detail(tok_s, ms, bytes_step, ctx, copy_gbs):
+def decode_detail(tok_s, ms, bytes_step, ctx, read_gbs):
     achieved = bytes_step / (ms * 1e-3) / 1e9
     return {"tok_s": round(tok_s, 2), "ms_per_step": round(ms, 4), "context": round(ctx, 1),
             "GBs": round(achieved, 1), "frac": round(achieved / HBM_PEAK_GBS, 4),
-            "frac_of_measured": round(achieved / copy_gbs, 4) if copy_gbs else None}
+            "frac_of_measured": round(achieved / read_gbs, 4) if read_gbs else None}
 
 
 def main():
@@ -267,7 +284,9 @@ def main():
                           "baseline": "9032.37 tokens/s, the reference with Qwen3-0.6B on an A100 40GB"}))
         return 0
     args.size = args.size or "8b"
-    m = Sized(args.size, args.dtype, args.context_len, args.layers, args.eager)
+    long_points = not args.no_points and not args.prefill_only
+    m = Sized(args.size, args.dtype, args.context_len, args.layers, args.eager,
+              longest_context=LONGEST_CONTEXT if long_points else args.prefill_only + 16)
     cfg = m.cfg
     if args.prefill_only:
         p_tok_s, p_ms, p_frac = m.prefill(args.prefill_only)
@@ -275,7 +294,7 @@ def main():
                                       "frac": round(p_frac, 4)}}))
         return 0
     peaks = measured_peaks() if not args.no_points else {}
-    copy_gbs = peaks.get("copy_GBs")
+    copy_gbs = peaks.get("read_GBs")        # the denominator of frac_of_measured: a kernel that only reads
     tok_s, ms, bytes_step, ctx = m.decode(args.batch, args.steps, args.warmup, args.prompt_len, args.top_k, args.top_p)
     head = decode_detail(tok_s, ms, bytes_step, ctx, copy_gbs)
     line = {
@@ -309,6 +328,15 @@ def main():
         detail["decode_b64"] = decode_detail(*b64, copy_gbs)
         points = {"decode_b1": round(b1[0], 2), "decode_b64": round(b64[0], 2),
                   f"decode_b{args.batch}_top_k20_top_p95": round(b8f[0], 2)}
+        if args.size == "8b" and args.dtype == "bfloat16":
+            # further contexts: where the cache outweighs the weights
+            for name, batch, ctx in (("decode_b8_ctx16k", 8, 16384), ("decode_b64_ctx8k", 64, 8192), ("decode_b1_ctx32k", 1, 32768)):
+                d = m.decode(batch, 16, 2, ctx - 128, context_len=ctx + 64)
+                detail[name] = decode_detail(*d, copy_gbs)
+                points[name] = round(d[0], 2)
+            p16 = m.prefill(16384)
+            points["prefill_16384"] = round(p16[0], 1)
+            detail["prefill_16384"] = {"tok_s": round(p16[0], 1), "ms": round(p16[1], 3), "frac": round(p16[2], 4)}
         m.close()
         if args.size == "8b" and args.layers is None and args.dtype == "bfloat16":
             # Qwen3-32B sizes: batch 64 with 4096-token contexts (about 69 GB of cache) and a 2048-token prompt
@@ -316,12 +344,18 @@ def main():
             d32 = big.decode(64, 16, 2, 4096 - 32)
             detail["decode_32b_b64_ctx4096"] = decode_detail(*d32, copy_gbs)
             points["decode_32b_b64_ctx4096"] = round(d32[0], 2)
+            d32 = big.decode(8, 16, 2, 1024)
+            detail["decode_32b_b8"] = decode_detail(*d32, copy_gbs)
+            points["decode_32b_b8"] = round(d32[0], 2)
             p32 = big.prefill(2048)
             points["prefill_32b_2048"] = round(p32[0], 1)
             detail["prefill_32b_2048"] = {"tok_s": round(p32[0], 1), "ms": round(p32[1], 3), "frac": round(p32[2], 4)}
             big.close()
             # the 256-request workload at Qwen3-14B sizes, and the reference's own at Qwen3-0.6B sizes
             mid = Sized("14b", args.dtype, 4096, eager=args.eager)
+            d14 = mid.decode(8, 16, 2, 1024)
+            detail["decode_14b_b8"] = decode_detail(*d14, copy_gbs)
+            points["decode_14b_b8"] = round(d14[0], 2)
             m14 = mid.mixed()
             points["mixed_qwen3_14b"] = round(m14[0], 1)
             detail["mixed_qwen3_14b"] = {"output_tok_s": round(m14[0], 1), "output_tokens": m14[1],

@@ -169,6 +169,45 @@ extern "C" int ullm_gather_rows(const float* src, long long src_stride, int n_sr
   ULLM_LAUNCH_CHECK();
 }
 
+// ------------------------------------------------------------------ a plain streaming read, for measurement
+// Every block reads its share of `bytes` once with non-temporal 16-byte loads, eight in flight per thread,
+// and stores one word per block (the xor of what it read, so that no load can be dropped).  What this
+// reaches is the practical ceiling of a kernel that only reads, as a decode step's weight streaming does.
+__global__ void __launch_bounds__(256)
+stream_read_kernel(const uint4* __restrict__ src, long long n16, unsigned* __restrict__ sink) {
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  unsigned acc = 0;
+  for (; i + 7 * stride < n16; i += 8 * stride) {
+    uint4 v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = ld_stream16(src + i + u * stride);
+#pragma unroll
+    for (int u = 0; u < 8; ++u) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+  }
+  for (; i < n16; i += stride) {
+    const uint4 v = ld_stream16(src + i);
+    acc ^= v.x ^ v.y ^ v.z ^ v.w;
+  }
+  for (int m = WAVE / 2; m > 0; m >>= 1) acc ^= __shfl_xor(acc, m, WAVE);
+  if ((threadIdx.x & (WAVE - 1)) == 0) sink[blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE] = acc;
+}
+
+// sink: at least blocks * 4 words.  blocks <= 0: eight per compute unit.
+extern "C" int ullm_stream_read(const void* src, long long bytes, unsigned* sink, int blocks, hipStream_t stream) {
+  if (bytes <= 0) return 0;
+  if (((uintptr_t)src & 15) || bytes % 16) return ULLM_ERR_SHAPE;
+  if (blocks <= 0) {
+    int dev = 0, units = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || units <= 0)
+      units = 256;
+    blocks = 8 * units;
+  }
+  hipLaunchKernelGGL(stream_read_kernel, dim3(blocks), dim3(256), 0, stream, (const uint4*)src, bytes / 16, sink);
+  ULLM_LAUNCH_CHECK();
+}
+
 // ------------------------------------------------------------------ add + RMS norm
 // For output row r (input row i = rows ? rows[r] : r):
 //   s = residual[i] + float(branch[i])      (branch may be null: s = residual[i]; it may also be a stack

@@ -132,6 +132,18 @@ def gather_rows(src: torch.Tensor, index: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def stream_read(src: torch.Tensor, blocks: int = 0) -> torch.Tensor:
+    """Read ``src`` (contiguous, a multiple of 16 bytes) once with a kernel that does nothing else; returns the
+    words the blocks stored (their xor of what they read).  For measuring what a read-only kernel reaches."""
+    nbytes = src.numel() * src.element_size()
+    _need(src.is_contiguous() and nbytes % 16 == 0 and src.data_ptr() % 16 == 0, "stream_read takes contiguous, 16-byte aligned memory")
+    n_blocks = blocks if blocks > 0 else 8 * compute_units(src.device)
+    sink = torch.empty(n_blocks * 4, dtype=torch.int32, device=src.device)
+    _check(build.load("elementwise").ullm_stream_read(_p(src), ctypes.c_longlong(nbytes), _p(sink), _c_int(n_blocks), _stream()),
+           "stream_read")
+    return sink
+
+
 def add_rmsnorm(branch: Optional[torch.Tensor], residual: torch.Tensor, gain: torch.Tensor, eps: float,
                 out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None,
                 out: Optional[torch.Tensor] = None) -> torch.Tensor:

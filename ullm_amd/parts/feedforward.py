@@ -13,7 +13,7 @@ from .base import FeedForward, PartEnv, StepContext, WeightDecl, register_part
 from .linear import can_fuse, linear, linear_into_stream, linear_of_norm
 
 
-# gate|up with the activation folded in, by rows of the batch (timings: profiles/projections_by_rows.md):
+# gate|up with the activation folded in, by rows of the batch (chosen from timings of each kernel at every row count):
 # up to 16 rows the few-rows kernel; from 17 to 64 rows the kernel for those row counts, except that up to 32 rows
 # the few-rows kernel is still ahead on matrices up to Qwen3-8B's size; beyond 64 rows the library product and
 # the activation kernel.
