@@ -602,6 +602,54 @@ def test_decode_attention_with_norm_rotation_and_cache_write_folded_in(ops, case
     assert (out[:len(lens)].float().cpu() - want).abs().max() <= tol(dtype, want)
 
 
+@pytest.mark.parametrize("hd", [64, 128])
+def test_two_large_scores_half_a_unit_apart_weigh_the_same_in_prompt_and_decode_steps(ops, hd):
+    """Two keys whose scores are near 50 in the units of the exponent and half a unit apart, with opposite
+    values: the output is (2^0.5 - 1) / (2^0.5 + 1) of the values' size if the exponents are right to a few
+    thousandths.  A scale that is rounded into the bfloat16 queries moves an exponent of 50 by up to 0.1 and the
+    output by a fifth; scores scaled in 32-bit (as both kinds of kernel do) leave only the weights' own rounding
+    to bfloat16.  Prompt tiles (every shape of launch) and the decode kernel must agree with the 64-bit result."""
+    torch.manual_seed(4)
+    dtype = torch.bfloat16
+    nq, nkv, P, S, n = 2, 1, 16, 200, 40
+    scale = hd ** -0.5
+    unit = scale * 1.4426950408889634                     # an exponent's unit in terms of q . k
+    u = torch.randn(hd)
+    u /= u.norm()
+    k = (torch.randn(S, nkv, hd) * 0.05)
+    q = (torch.randn(n, nq, hd) * 0.05)
+    size = (50.0 / unit) ** 0.5
+    a_at, b_at = 37, 150
+    k[a_at, 0] = size * u
+    k[b_at, 0] = size * u * (49.5 / 50.0)
+    q[-1, :] = size * u
+    k, q = k.to(dtype).double(), q.to(dtype).double()
+    v = torch.zeros(S, nkv, hd)
+    v[a_at], v[b_at] = 1.0, -1.0
+    scores = (k[:, 0] @ q[-1, 0]) * scale
+    want = (torch.softmax(scores, 0)[:, None] * v[:, 0].double()).sum(0)
+    assert 0.1 < float(want[0]) < 0.25 and 45 < float(scores.max()) * 1.4427 < 55      # the case is the one described
+    k_pool, v_pool, tables = paged_cache([k.float()], [v], P, dtype, DEV)
+    bt = table_tensor(tables, DEV)
+    positions = torch.arange(S - n, S, dtype=torch.int32, device=DEV)
+    entry = torch.zeros(n, dtype=torch.int32, device=DEV)
+    qd = q.float().reshape(n, nq * hd).to(DEV, dtype)
+    tiles = torch.tensor([x for f in range(0, n, ops.PREFILL_TILE) for x in (f, min(ops.PREFILL_TILE, n - f))],
+                         dtype=torch.int32, device=DEV)
+    for halves in ((1, 2, 11, 12) if hd == 128 else (1, 2)):
+        out = torch.zeros(n, nq * hd, dtype=dtype, device=DEV)
+        ops.attention_prefill_mfma(qd, out, k_pool, v_pool, tiles, tiles.numel() // 2, positions, entry, bt, P, nq, nkv, hd,
+                                   scale, 0, halves=halves)
+        err = float((out[-1, :hd].double().cpu() - want).abs().max())
+        assert err <= 6e-3, f"prompt tiles, halves {halves}: {err:.4f} from {float(want[0]):.4f}"
+    for splits, waves in ((1, 1), (2, 4), (3, 1)):
+        out = torch.zeros(1, nq * hd, dtype=dtype, device=DEV)
+        ops.attention_decode_mfma(qd[-1:].contiguous(), out, k_pool, v_pool, None, 1, positions[-1:].contiguous(),
+                                  entry[:1], bt, P, nq, nkv, hd, scale, 0, S, splits=splits, waves=waves)
+        err = float((out[0, :hd].double().cpu() - want).abs().max())
+        assert err <= 6e-3, f"decode, {splits} x {waves}: {err:.4f} from {float(want[0]):.4f}"
+
+
 def test_matrix_core_attention_finds_one_far_key_at_every_edge(ops):
     torch.manual_seed(9)
     dtype = torch.bfloat16

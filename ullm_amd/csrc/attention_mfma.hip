@@ -753,6 +753,22 @@ __device__ __forceinline__ void stage_store(const PrefillStage<NQK>& st, int key
   }
 }
 
+// scale * log2(e) = pow2 * frac with pow2 a power of two and 1 <= frac < 2.  The prompt kernels multiply the
+// bfloat16 queries by pow2 (exact) and the 32-bit scores by frac, so a score is the exponent of its weight with
+// no rounding but that of the 32-bit product, as in the decode kernel, which scales the 32-bit score whole.
+struct ScoreScale {
+  float pow2, frac, inv_frac;
+};
+__device__ __forceinline__ ScoreScale split_scale(float scale_log2e) {
+  int e;
+  const float f = frexpf(scale_log2e, &e);              // scale_log2e = f * 2^e, 0.5 <= f < 1
+  ScoreScale sc;
+  sc.frac = 2.f * f;
+  sc.pow2 = ldexpf(1.f, e - 1);
+  sc.inv_frac = 1.f / sc.frac;
+  return sc;
+}
+
 // The softmax step both prompt kernels share, between the score products and the value products of a tile.
 // `s[q][sb][r]` holds the exponents of this lane's eight keys for column q (the products started from minus
 // the column's reference value); `key_of(sb, r)` is the key's offset in the tile.  Does any exponent exceed
@@ -766,7 +782,7 @@ template <int NQK, int NG, bool masked, typename KeyOf>
 __device__ __forceinline__ void prompt_tile_softmax(f32x4_t (&s)[NG][2], int key0, KeyOf key_of,
                                                     const int (&col_lo)[NG], const int (&col_hi)[NG],
                                                     f32x4_t (&acc)[NG][2 * NQK], float (&m)[NG], f32x4_t (&negm)[NG],
-                                                    float (&l)[NG], Pack8 (&p)[NG]) {
+                                                    float (&l)[NG], Pack8 (&p)[NG], const ScoreScale& scale) {
   float lane_max[NG], alpha[NG];
   bool exceeds = false;
 #pragma unroll
@@ -777,6 +793,7 @@ __device__ __forceinline__ void prompt_tile_softmax(f32x4_t (&s)[NG][2], int key
     for (int sb = 0; sb < 2; ++sb)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
+        s[q][sb][r] *= scale.frac;                      // the part of scale * log2(e) that is no power of two, in 32-bit
         if (masked) {
           const int kk = key0 + key_of(sb, r);
           if (!(kk >= col_lo[q] && kk <= col_hi[q])) s[q][sb][r] = NEG_BIG;
@@ -796,7 +813,8 @@ __device__ __forceinline__ void prompt_tile_softmax(f32x4_t (&s)[NG][2], int key
       const bool moves = col_max > 0.5f * NEG_BIG && (!had || col_max > RESCALE_STEP);
       if (moves) {
         m[q] = (had ? m[q] : 0.f) + col_max;
-        negm[q] = f32x4_t{-m[q], -m[q], -m[q], -m[q]};
+        const float start = -m[q] * scale.inv_frac;     // the products start from here and are multiplied by frac
+        negm[q] = f32x4_t{start, start, start, start};
         if (had) alpha[q] = fast_exp2(-col_max);
 #pragma unroll
         for (int sb = 0; sb < 2; ++sb)
@@ -835,16 +853,16 @@ __device__ __forceinline__ void prompt_tile_softmax(f32x4_t (&s)[NG][2], int key
 
 // Scores, softmax update and value product of one wave for the tile in LDS.  `masked` = some key of
 // the tile is hidden from some column (diagonal, window or end of data); otherwise no per-score test.
-// The queries come multiplied by scale * log2(e), and the first product of a score starts from minus
-// the column's reference value (`negm`, the same in all four elements) instead of zero, so the
-// products deliver the exponent itself: exp2 of it is the weight.  A column without a reference
+// The queries come multiplied by the power of two in scale * log2(e), and the first product of a score
+// starts from minus the column's reference value over the remaining factor (`negm`, the same in all four
+// elements) instead of zero, so the products times that factor are the exponent itself: exp2 of it is the weight.  A column without a reference
 // value yet (m == NEG_BIG) counts from zero, and the first tile that shows it a key gives it one.
 template <int NQK, int NG, bool masked>
 __device__ __forceinline__ void process_tile_lds(const unsigned char* __restrict__ kl, const unsigned char* __restrict__ vl,
                                                  int key0, const Pack8 (&qreg)[NG][NQK],
                                                  const int (&col_lo)[NG], const int (&col_hi)[NG],
                                                  f32x4_t (&acc)[NG][2 * NQK], float (&m)[NG], f32x4_t (&negm)[NG],
-                                                 float (&l)[NG]) {
+                                                 float (&l)[NG], const ScoreScale& scale) {
   using S = PrefillStage<NQK>;
   const int lane = threadIdx.x & 63, g = lane >> 4, c = lane & 15;
   f32x4_t s[NG][2];
@@ -860,7 +878,7 @@ __device__ __forceinline__ void process_tile_lds(const unsigned char* __restrict
     }
   Pack8 p[NG];
   prompt_tile_softmax<NQK, NG, masked>(s, key0, [g](int sb, int r) { return 16 * sb + 4 * g + r; }, col_lo, col_hi,
-                                       acc, m, negm, l, p);
+                                       acc, m, negm, l, p, scale);
 #pragma unroll
   for (int n = 0; n < 2 * NQK; ++n) {
     Pack8 vf;
@@ -911,6 +929,7 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __r
   const int first = tiles[2 * tile_idx], count = tiles[2 * tile_idx + 1];
   int clo[NG], chi[NG], tok[NG];
   Pack8 qreg[NG][NQK];
+  const ScoreScale score_scale = split_scale(scale_log2e);
 #pragma unroll
   for (int qg = 0; qg < NG; ++qg) {
     const bool ok = head_ok && 16 * qg + c < count;
@@ -923,12 +942,12 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __r
     for (int ch = 0; ch < NQK; ++ch) {
       if (ok) qreg[qg][ch].u4 = *reinterpret_cast<const uint4*>(qp + 32 * ch);
       else qreg[qg][ch].u4 = make_uint4(0, 0, 0, 0);
-      // scale * log2(e) goes into the queries once, so that a score is its weight's exponent
+      // the power of two in scale * log2(e) goes into the queries once (exact); the scores take the rest
 #pragma unroll
       for (int w = 0; w < 4; ++w) {
         const uint32_t two = qreg[qg][ch].w[w];
-        qreg[qg][ch].w[w] = pack2_bf16(__uint_as_float(two << 16) * scale_log2e,
-                                       __uint_as_float(two & 0xffff0000u) * scale_log2e);
+        qreg[qg][ch].w[w] = pack2_bf16(__uint_as_float(two << 16) * score_scale.pow2,
+                                       __uint_as_float(two & 0xffff0000u) * score_scale.pow2);
       }
     }
   }
@@ -975,9 +994,9 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __r
   do {                                                                             \
     const unsigned char* kl = tile_lds + (BUF) * TILE_BYTES;                       \
     if ((K0) + 31 > first_pos || (K0) < open_lo)                                   \
-      process_tile_lds<NQK, NG, true>(kl, kl + S::KBYTES, (K0), qreg, clo, chi, acc, m, negm, l);  \
+      process_tile_lds<NQK, NG, true>(kl, kl + S::KBYTES, (K0), qreg, clo, chi, acc, m, negm, l, score_scale);  \
     else                                                                           \
-      process_tile_lds<NQK, NG, false>(kl, kl + S::KBYTES, (K0), qreg, clo, chi, acc, m, negm, l); \
+      process_tile_lds<NQK, NG, false>(kl, kl + S::KBYTES, (K0), qreg, clo, chi, acc, m, negm, l, score_scale); \
     STAGE_STORE(NEXT, (K0) + 32, 1 - (BUF));                                       \
     STAGE_LOAD(NEXT, (K0) + 96);                                                   \
     __syncthreads();                                                               \
@@ -991,9 +1010,9 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __r
   do {                                                                             \
     const unsigned char* kl = tile_lds + (BUF) * TILE_BYTES;                       \
     if ((K0) + 31 > first_pos || (K0) < open_lo)                                   \
-      process_tile_lds<NQK, NG, true>(kl, kl + S::KBYTES, (K0), qreg, clo, chi, acc, m, negm, l);  \
+      process_tile_lds<NQK, NG, true>(kl, kl + S::KBYTES, (K0), qreg, clo, chi, acc, m, negm, l, score_scale);  \
     else                                                                           \
-      process_tile_lds<NQK, NG, false>(kl, kl + S::KBYTES, (K0), qreg, clo, chi, acc, m, negm, l); \
+      process_tile_lds<NQK, NG, false>(kl, kl + S::KBYTES, (K0), qreg, clo, chi, acc, m, negm, l, score_scale); \
   } while (0)
   // Steps go in pairs, so that the two register stages and the two LDS tiles take turns in a way the
   // compiler can see (it then waits for the loads of two steps ago only); an odd last step follows the
@@ -1180,7 +1199,7 @@ __device__ __forceinline__ void dma_tile_products(const unsigned char* __restric
                                                   const int (&col_lo)[NG], const int (&col_hi)[NG],
                                                   f32x4_t (&acc)[NG][2 * NQK], float (&m)[NG], f32x4_t (&negm)[NG],
                                                   float (&l)[NG], const int (&k_at)[2][NQK], int v_at, int max_hi,
-                                                  bool ok0, bool ok1) {
+                                                  bool ok0, bool ok1, const ScoreScale& scale) {
   using T = DmaTile<NQK>;
   const int lane = threadIdx.x & 63, g = lane >> 4;
   f32x4_t s[NG][2];
@@ -1197,7 +1216,7 @@ __device__ __forceinline__ void dma_tile_products(const unsigned char* __restric
   // s[q][sb][r] is the exponent of key key0 + 8 g + 4 sb + r for this lane's column
   Pack8 p[NG];
   prompt_tile_softmax<NQK, NG, masked>(s, key0, [g](int sb, int r) { return 8 * g + 4 * sb + r; }, col_lo, col_hi,
-                                       acc, m, negm, l, p);
+                                       acc, m, negm, l, p, scale);
   // masked tiles only: which of this lane's eight keys (8 g ..) hold written values.  The others (past the end
   // of the data, or in a sub-block without a page, which reads page 0) may hold anything and must count as 0.
   uint32_t live[4] = {0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu};
@@ -1261,6 +1280,7 @@ attention_prefill_dma_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t*
   const int first = tiles[2 * tile_idx], count = tiles[2 * tile_idx + 1];
   int clo[NG], chi[NG], tok[NG];
   Pack8 qreg[NG][NQK];
+  const ScoreScale score_scale = split_scale(scale_log2e);
 #pragma unroll
   for (int qg = 0; qg < NG; ++qg) {
     const bool ok = head_ok && 16 * qg + c < count;
@@ -1273,12 +1293,12 @@ attention_prefill_dma_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t*
     for (int ch = 0; ch < NQK; ++ch) {
       if (ok) qreg[qg][ch].u4 = *reinterpret_cast<const uint4*>(qp + 32 * ch);
       else qreg[qg][ch].u4 = make_uint4(0, 0, 0, 0);
-      // scale * log2(e) goes into the queries once, so that a score is its weight's exponent
+      // the power of two in scale * log2(e) goes into the queries once (exact); the scores take the rest
 #pragma unroll
       for (int w = 0; w < 4; ++w) {
         const uint32_t two = qreg[qg][ch].w[w];
-        qreg[qg][ch].w[w] = pack2_bf16(__uint_as_float(two << 16) * scale_log2e,
-                                       __uint_as_float(two & 0xffff0000u) * scale_log2e);
+        qreg[qg][ch].w[w] = pack2_bf16(__uint_as_float(two << 16) * score_scale.pow2,
+                                       __uint_as_float(two & 0xffff0000u) * score_scale.pow2);
       }
     }
   }
@@ -1351,9 +1371,9 @@ attention_prefill_dma_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t*
       if (i + 3 < steps) TILE_LOAD(i + 3, t0);
       if (K0 + 31 > first_pos || K0 < open_lo) {
         const bool ok0 = pages[2 * (i - t0)] >= 0, ok1 = pages[2 * (i - t0) + 1] >= 0;
-        dma_tile_products<NQK, NG, true>(tile, K0, qreg, clo, chi, acc, m, negm, l, k_at, v_at, last_pos, ok0, ok1);
+        dma_tile_products<NQK, NG, true>(tile, K0, qreg, clo, chi, acc, m, negm, l, k_at, v_at, last_pos, ok0, ok1, score_scale);
       } else {
-        dma_tile_products<NQK, NG, false>(tile, K0, qreg, clo, chi, acc, m, negm, l, k_at, v_at, last_pos, true, true);
+        dma_tile_products<NQK, NG, false>(tile, K0, qreg, clo, chi, acc, m, negm, l, k_at, v_at, last_pos, true, true, score_scale);
       }
     }
   }

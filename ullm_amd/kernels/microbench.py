@@ -68,7 +68,7 @@ def decode_attention(args) -> None:
             groups = -(-(nq // nkv) // 16)
             auto = ops.decode_split(B, nkv, groups, ctx, hd)
             cells = []
-            for splits, waves in [(0, 0)] + [(s, w) for w in (4, 8, 1) for s in (1, 2, 4, 8, 16, 32)]:
+            for splits, waves in [(0, 0)] + [(s, w) for w in (4, 8, 1) for s in (1, 2, 4, 8, 16, 32, 64)]:
                 if splits * B * nkv * groups > 2048 or (hd == 256 and waves == 8):
                     continue
                 calls = [(lambda v=v: ops.attention_decode_mfma(q, out, k_pool, v_pool, None, B, pos, ent, tables[v], P, nq,

@@ -529,9 +529,12 @@ def decode_split(n_items: int, nkv: int, groups: int, max_kv: int, hd: int = 128
         return 1, (max(2, min(3, simds // pairs)) if pairs <= units * 9 // 4 and tiles > 16 else 1)
     if pairs == units:
         return (4 if tiles > 16 else 1), 1
-    splits = min(16, max(1, 2 * units // pairs), tiles)
+    # up to 16 blocks a pair; up to 32 where very few pairs have very many keys (one request at 4 096 keys and
+    # more: 134 MB of cache at 32 768 keys in 34 us against 49 us with 16)
+    most = 32 if (pairs * 128 <= simds and tiles >= 128) else 16
+    splits = min(most, max(1, 2 * units // pairs), tiles)
     if tiles > 8 * splits:
-        splits = min(16, max(1, simds // pairs), tiles)
+        splits = min(most, max(1, simds // pairs), tiles)
     waves = 4 if (tiles > 4 * splits and pairs * splits * 4 <= simds) else 1
     return waves, splits
 
