@@ -70,3 +70,42 @@ def test_decode_attention_without_allocation_equals_the_workspace_entry_point():
     rc, out = _call(lib, True, *args, P, nq, nkv, hd, splits, 4)
     assert rc == -4
     assert torch.isnan(out).all()
+
+
+def test_decode_attention_without_allocation_under_graph_capture():
+    """After one call outside capture (the capacity query looks the array up), the entry point is captured
+    into a HIP graph and replayed with other inputs in the same tensors, eager work between the replays; every
+    replay equals the workspace entry point run eagerly, and the call allocates no device memory."""
+    from ullm_amd.kernels import build
+    lib = build.load("attention_mfma")
+    lib.ullm_attention_decode_static_capacity.restype = ctypes.c_longlong
+    assert lib.ullm_attention_decode_static_capacity() > 0          # warm-up on this device, outside capture
+    nq, nkv, hd, P, splits, waves = 32, 8, 128, 16, 5, 4
+    lens = [300, 47, 1025]
+    q, k_pool, v_pool, positions, entry, bt = _problem(7, nq, nkv, hd, P, lens)
+    out = torch.full_like(q, float("nan"))
+
+    def launch(stream):
+        return lib.ullm_attention_decode_static(
+            _ptr(q), ctypes.c_int(q.stride(0)), _ptr(out), ctypes.c_int(out.stride(0)), _ptr(k_pool), _ptr(v_pool),
+            _ptr(None), ctypes.c_int(len(lens)), _ptr(positions), _ptr(entry), _ptr(bt), ctypes.c_int(bt.stride(0)),
+            ctypes.c_int(P), ctypes.c_int(nq), ctypes.c_int(nkv), ctypes.c_int(hd), ctypes.c_float(hd ** -0.5),
+            ctypes.c_int(0), ctypes.c_int(splits), ctypes.c_int(waves), ctypes.c_void_p(stream.cuda_stream))
+    torch.cuda.synchronize()
+    before = torch.cuda.memory_allocated()
+    assert launch(torch.cuda.current_stream()) == 0
+    torch.cuda.synchronize()
+    assert torch.cuda.memory_allocated() == before                  # torch's allocator was not asked for anything
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        assert launch(torch.cuda.current_stream()) == 0
+    for seed in (8, 9, 10):
+        # other numbers in the same tensors (rows of the pools that no request holds stay as they are)
+        q.copy_(torch.randn(q.shape, generator=torch.Generator().manual_seed(seed)).to(q.dtype))
+        k_pool.neg_()
+        v_pool.mul_(0.5)
+        out.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        rc, want = _call(lib, False, q, k_pool, v_pool, positions, entry, bt, P, nq, nkv, hd, splits, waves)
+        assert rc == 0 and torch.equal(out, want), seed

@@ -1548,7 +1548,30 @@ static __device__ __align__(256) float scratch[ULLM_DECODE_SCRATCH_FLOATS];
 #define ULLM_MAX_DEVICES 64
 static float* scratch_ptr[ULLM_MAX_DEVICES];      // per device: that GPU's copy of the array
 
-extern "C" long long ullm_attention_decode_static_capacity(void) { return ULLM_DECODE_SCRATCH_FLOATS; }
+// The current device's copy of the array: looked up at the first call on the device (which is current),
+// kept per device.  0 and *err set if the lookup fails.
+static float* scratch_of_current_device(int* err) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) { *err = (int)e; return nullptr; }
+  if (dev < 0 || dev >= ULLM_MAX_DEVICES) { *err = ULLM_ERR_UNSUPPORTED; return nullptr; }
+  float* ws = __atomic_load_n(&scratch_ptr[dev], __ATOMIC_ACQUIRE);
+  if (!ws) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) { *err = (int)e; return nullptr; }
+    if (!p) { *err = (int)hipErrorInvalidSymbol; return nullptr; }
+    ws = static_cast<float*>(p);
+    __atomic_store_n(&scratch_ptr[dev], ws, __ATOMIC_RELEASE);   // two first callers store the same address
+  }
+  return ws;
+}
+
+extern "C" long long ullm_attention_decode_static_capacity(void) {
+  int err = 0;
+  scratch_of_current_device(&err);                // also the warm-up: the lookup is not stream-ordered
+  return ULLM_DECODE_SCRATCH_FLOATS;
+}
 
 extern "C" int ullm_attention_decode_static(
     const void* q, int q_stride, void* out, int out_stride, const void* k_pool, const void* v_pool,
@@ -1559,19 +1582,9 @@ extern "C" int ullm_attention_decode_static(
   if (num_splits < 1 || nq < 1 || hd < 1) return ULLM_ERR_SHAPE;
   if (ullm_attention_decode_workspace(n_items, nq, hd, num_splits) > (long long)ULLM_DECODE_SCRATCH_FLOATS)
     return ULLM_ERR_SCRATCH;
-  int dev = -1;
-  hipError_t e = hipGetDevice(&dev);
-  if (e != hipSuccess) return (int)e;
-  if (dev < 0 || dev >= ULLM_MAX_DEVICES) return ULLM_ERR_UNSUPPORTED;
-  float* ws = __atomic_load_n(&scratch_ptr[dev], __ATOMIC_ACQUIRE);
-  if (!ws) {                                      // first call on this device, which is current
-    void* p = nullptr;
-    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
-    if (e != hipSuccess) return (int)e;
-    if (!p) return (int)hipErrorInvalidSymbol;
-    ws = static_cast<float*>(p);
-    __atomic_store_n(&scratch_ptr[dev], ws, __ATOMIC_RELEASE);   // two first callers store the same address
-  }
+  int err = 0;
+  float* ws = scratch_of_current_device(&err);
+  if (!ws) return err;
   return decode_launch(q, q_stride, out, out_stride, k_pool, v_pool, token_list, n_items, positions, token_entry,
                        block_table, bt_stride, page_size, nq, nkv, hd, scale, window, num_splits, waves, ws, stream);
 }

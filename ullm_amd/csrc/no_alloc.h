@@ -15,7 +15,10 @@
 // * A call whose partial results need more than ULLM_DECODE_SCRATCH_FLOATS floats
 //   (n_items * nq * num_splits * (hd + 4)) is refused with ULLM_ERR_SCRATCH; nothing is launched.
 // * The array's device address is looked up once per device, with that device current, at the first
-//   call on it (hipGetSymbolAddress); a failure of that lookup is returned as its hipError_t.
+//   call on it (hipGetSymbolAddress); a failure of that lookup is returned as its hipError_t.  The lookup
+//   is not stream-ordered and may load the code object: it must not happen while a stream is capturing.
+//   A caller that captures calls ullm_attention_decode_static_capacity() (or the entry point itself) once
+//   on the device beforehand; every later call only launches kernels on the given stream.
 // * All calls on one GPU share that GPU's array.  Every float a call reads it has written itself in
 //   the same call (the reduce kernel reads exactly the rows the split kernel stored), so nothing
 //   needs clearing between calls; but two calls that overlap in time on one GPU (different streams,
@@ -30,7 +33,8 @@
 extern "C" {
 #endif
 
-// Floats of scratch the static entry point holds per GPU.
+// Floats of scratch the static entry point holds per GPU.  Also looks up the current device's copy of the
+// array, so that a later call under stream capture has nothing left to do but launch.
 long long ullm_attention_decode_static_capacity(void);
 
 // Same arguments and result as ullm_attention_decode, without the workspace.
