@@ -200,3 +200,44 @@ def test_a_context_past_the_models_positions_is_refused(caplog):
         assert context_within_model(cfg, 512, strict=False) == 512
     assert any("max_position_embeddings=128" in r.getMessage() for r in caplog.records)
     assert context_within_model({"no": "such key"}, 10 ** 6) == 10 ** 6     # a configuration without the key has no limit
+
+
+def test_projection_limits_come_from_the_table_or_from_the_size_rules(tmp_path, monkeypatch):
+    """A matrix the table of measurements holds takes its limits from there (missing fields from the rules);
+    any other matrix takes the rules, which speak of the matrix's size only."""
+    import json
+    from ullm_amd.kernels import dispatch
+    small, large = dispatch.default_limits(1024, 1024), dispatch.default_limits(24576, 4096)
+    assert (small.rows, small.fold_norm, small.stacked_from, small.f32_skinny) == (0, 16, 0, 16)
+    assert (large.rows, large.fold_norm, large.silu_skinny, large.stacked_to) == (64, 8, 32, 256)
+    assert dispatch.default_limits(151936, 4096).f32_skinny == 32 and dispatch.default_limits(51200, 5120).silu_skinny == 16
+    table = tmp_path / "table.json"
+    table.write_text(json.dumps({"matrices": {"777x64": {"skinny": 5, "rows": 9, "not a field": 1}}}))
+    monkeypatch.setattr(dispatch, "TABLE_PATH", str(table))
+    monkeypatch.setattr(dispatch, "_table", None)
+    got = dispatch.limits(777, 64)
+    assert (got.skinny, got.rows) == (5, 9) and got.fold_norm == dispatch.default_limits(777, 64).fold_norm
+    assert dispatch.is_tuned(777, 64) and not dispatch.is_tuned(778, 64)
+    assert dispatch.limits(778, 64) == dispatch.default_limits(778, 64)
+    dispatch.write_entry(778, 64, {"skinny": 3})
+    assert dispatch.limits(778, 64).skinny == 3 and dispatch.limits(777, 64).skinny == 5
+    assert dispatch.limits(778, 64).rows == dispatch.default_limits(778, 64).rows
+    with pytest.raises(KeyError):
+        dispatch.write_entry(778, 64, {"no such limit": 3})
+    monkeypatch.setattr(dispatch, "_table", None)             # the real table again for whoever comes next
+
+
+def test_limits_are_derived_from_times_by_the_time_saved_in_total():
+    """One measurement that is off by its noise does not end a kernel's range; a kernel that is never ahead gets
+    none; the norm stays folded only while that beats the norm's own kernel plus the best unfolded product."""
+    from ullm_amd.kernels.microbench import derive_limits
+    rows = [1, 8, 16, 17, 32, 64, 128, 256]
+    stream = {"library>norm": dict(zip(rows, [19, 19, 19, 17, 17, 19, 29, 27])),
+              "partial sums>norm": dict(zip(rows, [13, 14, 14, 15, 17.2, 18, 22, 29]))}
+    assert derive_limits(stream, {"stream"}, 0, 0) == {"stacked_from": 17, "stacked_to": 128}
+    never = {"library>norm": {17: 5.0, 64: 5.0}, "partial sums>norm": {17: 6.0, 64: 9.0}}
+    assert derive_limits(never, {"stream"}, 0, 0) == {"stacked_from": 0, "stacked_to": 0}
+    store = {"norm": {1: 2.5, 8: 2.5, 16: 2.5, 32: 2.5}, "library": {1: 14, 8: 14, 16: 14, 32: 15},
+             "skinny": {1: 10, 8: 10.5, 16: 13, 32: 19}, "rows": {1: 10.5, 8: 10.6, 16: 10.7, 32: 12},
+             "skinny+norm": {1: 11.5, 8: 12.5, 16: 16}}
+    assert derive_limits(store, {"store"}, 0, 0) == {"skinny": 8, "rows": 32, "fold_norm": 8}

@@ -261,9 +261,12 @@ def test_feed_forward_hands_the_norm_a_stack_of_partial_sums(monkeypatch):
     """For 17 to 256 rows in bfloat16 (its down projection has few long rows) the last projection of a feed-forward comes as a stack of float32
     partial sums if every norm of the model adds stacks; the norm's sum is the plain result."""
     from types import SimpleNamespace
-    from ullm_amd.parts import PartEnv, build_part, linear
+    import dataclasses
+    from ullm_amd.kernels import dispatch
+    from ullm_amd.parts import PartEnv, build_part
     from ullm_amd.weights.loader import bind_tensors
-    monkeypatch.setattr(linear, "STACKED_MIN_WEIGHT", 0)      # the test's matrices are small
+    rules = dispatch.default_limits                           # the test's matrices are small: as if they were large
+    monkeypatch.setattr(dispatch, "default_limits", lambda c, k: dataclasses.replace(rules(c, k), stacked_from=17, stacked_to=256))
     torch.manual_seed(5)
     H, I = 96, 224
     env = PartEnv(torch.device(DEV), torch.bfloat16, 16)
@@ -310,11 +313,13 @@ def test_norm_left_to_the_feed_forwards_first_projection(monkeypatch):
     seen, inner = [], ops.gemm_skinny_normed
     monkeypatch.setattr(ops, "gemm_skinny_normed", lambda *a, **k: seen.append(1) or inner(*a, **k))
     # a small matrix keeps the norm inside for every row count the kernel takes, a large one up to 8 rows
-    from ullm_amd.parts import linear as linear_rules
+    import dataclasses
+    from ullm_amd.kernels import dispatch
+    rules = dispatch.default_limits
     cases = [(T, True, None) for T in (1, 7, 8, 9, 16)] + [(T, T <= 8, 0) for T in (8, 9, 16)]
     for T, folded, small in cases:
         if small is not None:
-            monkeypatch.setattr(linear_rules, "NORM_FOLDED_SMALL_WEIGHT", small)
+            monkeypatch.setattr(dispatch, "default_limits", lambda c, k: dataclasses.replace(rules(c, k), fold_norm=8))
         stream = torch.randn(T, H) * torch.logspace(-2, 2, T)[:, None]
         want = stream + plain.qwen3_mlp(plain.rms_norm(stream, gain, eps), {k: v.float() for k, v in w.items()}, "f")
         got = stream.clone().to(DEV)

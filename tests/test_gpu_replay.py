@@ -151,9 +151,12 @@ def test_portions_whose_projections_come_as_stacks_of_partial_sums(model_dirs, p
     """Steps of 17 to 256 tokens hand the output and down projections to the next norm as stacks of
     partial sums where the matrices are large; here the size limit is lifted so that the tiny model
     takes that way too, beside steps that do not."""
+    import dataclasses
+    from ullm_amd.kernels import dispatch
     from ullm_amd.parts import linear
     from ullm_amd.replay import Replayer
-    monkeypatch.setattr(linear, "STACKED_MIN_WEIGHT", 0)
+    rules = dispatch.default_limits
+    monkeypatch.setattr(dispatch, "default_limits", lambda c, k: dataclasses.replace(rules(c, k), stacked_from=17, stacked_to=256))
     calls, inner = [], linear.ops.gemm_partial_sums
     monkeypatch.setattr(linear.ops, "gemm_partial_sums", lambda x, w: calls.append(x.shape[0]) or inner(x, w))
     rep = Replayer(model_dirs[name], "bfloat16", 512, 16, DEV)
@@ -175,9 +178,12 @@ def test_portions_of_17_to_64_tokens_through_the_kernel_for_those_row_counts(mod
     """Steps of 17 to 64 tokens take the q|k|v and gate|up projections through the kernel for those row counts where
     the matrices are large; here the size limit is lifted so that a tiny model (A: width 64, a whole stage of K)
     takes that way too, beside steps that do not."""
-    from ullm_amd.kernels import ops
+    import dataclasses
+    from ullm_amd.kernels import dispatch, ops
     from ullm_amd.replay import Replayer
-    monkeypatch.setattr(ops, "ROWS_MIN_COLUMNS", 0)
+    rules = dispatch.default_limits
+    monkeypatch.setattr(dispatch, "default_limits",
+                        lambda c, k: dataclasses.replace(rules(c, k), rows=64, silu_skinny=16, silu_rows=64))
     calls, inner = [], ops.gemm_rows
     monkeypatch.setattr(ops, "gemm_rows", lambda a, w, bias=None, silu=False: calls.append((a.shape[0], silu)) or inner(a, w, bias, silu))
     rep = Replayer(model_dirs["A"], "bfloat16", 512, 16, DEV)

@@ -8,6 +8,8 @@ cache: the figures are those of a cold read from HBM, as in a model whose weight
   decode-attention   one token per request over its cache: every (splits, waves) shape of the launch
   prefill-attention  prompt tiles of one request
   projection         a [rows, K] x [N, K]^T product by each kernel that can take it, and the library
+  tune               the same for one matrix in the roles it has in a model; writes the row limits up to which
+                     each kernel is ahead into the table that ullm_amd.kernels.dispatch reads
 """
 from __future__ import annotations
 
@@ -16,7 +18,7 @@ from typing import Callable, List
 
 import torch
 
-from . import ops
+from . import dispatch, ops
 
 DEV = "cuda:0"
 
@@ -152,6 +154,124 @@ def projection(args) -> None:
               + "  ".join(cells), flush=True)
 
 
+TUNE_ROWS = [1, 4, 8, 9, 12, 16, 17, 24, 32, 33, 48, 64, 65, 96, 128, 192, 256]
+
+
+def _ahead_up_to(rows, mine, others, start=0):
+    """The row count r > ``start`` up to which taking ``mine`` instead of the best of ``others`` saves the most
+    time in total over the measured row counts in (start, r] (``start`` if it never saves any).  A sum rather
+    than "faster at every row count": one measurement that is off by its noise does not end a range."""
+    best, best_gain, gain = start, 0.0, 0.0
+    for r in rows:
+        if r <= start:
+            continue
+        t = mine.get(r)
+        rest = [o[r] for o in others if r in o]
+        if t is None:
+            break
+        if not rest:
+            continue
+        gain += min(rest) - t
+        if gain > best_gain + 1e-9:
+            best, best_gain = r, gain
+    return best
+
+
+def derive_limits(times: dict, roles, columns: int, inner: int) -> dict:
+    """The fields of :class:`dispatch.Limits` that the measured times of one matrix decide.  ``times`` is
+    {kernel name: {rows: microseconds}} with rows as ints (see :func:`tune` for the names)."""
+    rows = sorted({r for t in times.values() for r in t})
+    get = lambda name: times.get(name, {})   # noqa: E731
+    changes = {}
+    if "store" in roles:
+        changes["skinny"] = _ahead_up_to(rows, get("skinny"), [get("rows"), get("library")])
+        changes["rows"] = _ahead_up_to(rows, get("rows"), [get("library")], start=changes["skinny"])
+        if changes["rows"] == changes["skinny"]:
+            changes["rows"] = 0
+        best = {r: min(t[r] for t in (get("skinny"), get("rows"), get("library")) if r in t) for r in rows}
+        unfolded = {r: best[r] + get("norm")[r] for r in rows if r in get("norm")}
+        changes["fold_norm"] = _ahead_up_to(rows, get("skinny+norm"), [unfolded])
+    if "silu" in roles:
+        changes["silu_skinny"] = _ahead_up_to(rows, get("skinny+silu"), [get("rows+silu"), get("library+silu")])
+        changes["silu_rows"] = _ahead_up_to(rows, get("rows+silu"), [get("library+silu")], start=changes["silu_skinny"])
+        if changes["silu_rows"] == changes["silu_skinny"]:
+            changes["silu_rows"] = 0
+        best = {r: min(t[r] for t in (get("skinny+silu"), get("rows+silu"), get("library+silu")) if r in t) for r in rows}
+        unfolded = {r: best[r] + get("norm")[r] for r in rows if r in get("norm")}
+        changes["fold_norm"] = _ahead_up_to(rows, get("skinny+norm+silu"), [unfolded])
+    if "stream" in roles:
+        # up to 16 rows the few-rows kernel adds into the stream itself; the stacks serve the rows after that
+        upto = _ahead_up_to(rows, get("partial sums>norm"), [get("library>norm")], start=16)
+        changes["stacked_from"], changes["stacked_to"] = (17, upto) if upto > 16 else (0, 0)
+    if "logits" in roles:
+        changes["f32_skinny"] = _ahead_up_to(rows, get("skinny f32"), [get("library f32")])
+    return changes
+
+
+def tune(args) -> None:
+    """Measure one matrix in its roles and write its limits.  Roles: ``store`` (a first projection, bfloat16
+    out, with the norm before it), ``silu`` (gate|up: columns = 2 x intermediate), ``stream`` (a last
+    projection, whose result goes into the residual stream), ``logits`` (32-bit out)."""
+    N, K = args.columns, args.inner
+    roles = set(args.roles)
+    w_bytes = N * K * 2
+    nv = copies_for(w_bytes)
+    ws = [torch.randn(N, K, device=DEV).bfloat16() * 0.02 for _ in range(nv)]
+    gain = torch.ones(K, device=DEV)
+    times = {}
+
+    def timed(name, rows, make):
+        try:
+            make(0)()
+        except (ops.KernelError, RuntimeError):
+            return
+        times.setdefault(name, {})[rows] = round(graph_time([make(v) for v in range(nv)]), 2)
+    for M in TUNE_ROWS:
+        x = torch.randn(M, K, device=DEV).bfloat16()
+        stream = torch.randn(M, K, device=DEV)
+        skinny_ok = ops.gemm_skinny_supports(x, ws[0])
+        if roles & {"store", "silu"}:
+            # the norm kernel that a folded norm saves: the stream [M, K] to bfloat16 rows
+            timed("norm", M, lambda v: (lambda: ops.add_rmsnorm(None, stream, gain, 1e-6, torch.bfloat16)))
+        if "store" in roles:
+            timed("library", M, lambda v: (lambda: torch.nn.functional.linear(x, ws[v])))
+            if skinny_ok:
+                timed("skinny", M, lambda v: (lambda: ops.gemm_skinny(x, ws[v])))
+            if ops.gemm_skinny_normed_supports(stream, gain, ws[0]):
+                timed("skinny+norm", M, lambda v: (lambda: ops.gemm_skinny_normed(stream, gain, 1e-6, ws[v])))
+            if M <= ops.ROWS_MAX_ROWS and ops.gemm_rows_supports(x, ws[0]):
+                timed("rows", M, lambda v: (lambda: ops.gemm_rows(x, ws[v])))
+        if "silu" in roles:
+            timed("library+silu", M, lambda v: (lambda: ops.silu_mul(torch.nn.functional.linear(x, ws[v]))))
+            if skinny_ok:
+                timed("skinny+silu", M, lambda v: (lambda: ops.gemm_skinny_silu(x, ws[v])))
+            if ops.gemm_skinny_normed_supports(stream, gain, ws[0]):
+                timed("skinny+norm+silu", M, lambda v: (lambda: ops.gemm_skinny_normed(stream, gain, 1e-6, ws[v], silu=True)))
+            if M <= ops.ROWS_MAX_ROWS and ops.gemm_rows_supports(x, ws[0], silu=True):
+                timed("rows+silu", M, lambda v: (lambda: ops.gemm_rows(x, ws[v], silu=True)))
+        if "stream" in roles:
+            resid = torch.zeros(M, N, device=DEV)
+            gain_n = torch.ones(N, device=DEV)
+            # the library's product, and the norm that adds it; against the stack and the norm that adds the stack
+            timed("library>norm", M, lambda v: (lambda: ops.add_rmsnorm(torch.nn.functional.linear(x, ws[v]), resid, gain_n, 1e-6,
+                                                                       torch.bfloat16)))
+            if ops.gemm_partial_sums_supports(x, ws[0]):
+                timed("partial sums>norm", M, lambda v: (lambda: ops.add_rmsnorm(ops.gemm_partial_sums(x, ws[v]), resid, gain_n, 1e-6,
+                                                                                 torch.bfloat16)))
+        if "logits" in roles:
+            timed("library f32", M, lambda v: (lambda: torch.mm(x, ws[v].t(), out_dtype=torch.float32)))
+            if skinny_ok and M <= 64:
+                timed("skinny f32", M, lambda v: (lambda: ops.gemm_skinny(x, ws[v], out_dtype=torch.float32)))
+        print(f"rows {M}: " + "  ".join(f"{k}: {v[M]}" for k, v in times.items() if M in v), flush=True)
+    found = dispatch.default_limits(N, K)
+    changes = derive_limits(times, roles, N, K)
+    print(f"limits of {N}x{K}: {changes} (the size rules alone: "
+          f"{ {k: getattr(found, k) for k in changes} })", flush=True)
+    if not args.dry_run:
+        dispatch.write_entry(N, K, changes)
+        print(f"written to {dispatch.TABLE_PATH}", flush=True)
+
+
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(prog="ullm_amd.kernels.microbench", description=__doc__.split("\n\n")[0])
     sub = ap.add_subparsers(dest="what", required=True)
@@ -168,8 +288,15 @@ def main(argv=None) -> int:
     p.add_argument("--columns", type=int, required=True, help="rows of the weight matrix (columns of the result)")
     p.add_argument("--inner", type=int, required=True)
     p.add_argument("--rows", type=ints, default=[1, 8, 16, 32, 64, 128], help="comma-separated numbers of rows of x")
+    p = sub.add_parser("tune")
+    p.add_argument("--columns", type=int, required=True, help="rows of the weight matrix (columns of the result)")
+    p.add_argument("--inner", type=int, required=True)
+    p.add_argument("--roles", type=lambda s: s.split(","), required=True,
+                   help="comma-separated roles of the matrix: store, silu, stream, logits")
+    p.add_argument("--dry-run", action="store_true", help="measure and print, leave the table as it is")
     args = ap.parse_args(argv)
-    {"decode-attention": decode_attention, "prefill-attention": prefill_attention, "projection": projection}[args.what](args)
+    {"decode-attention": decode_attention, "prefill-attention": prefill_attention, "projection": projection,
+     "tune": tune}[args.what](args)
     return 0
 
 

@@ -10,7 +10,7 @@ from typing import Optional
 
 import torch
 
-from . import build
+from . import build, dispatch
 
 F32, BF16 = 0, 1
 logger = logging.getLogger("ullm_amd")
@@ -413,10 +413,7 @@ def gemm_partial_sums(a: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     return out
 
 
-ROWS_MAX_ROWS = 64
-# fewest columns of the result for which the 17-to-64-row kernel is chosen over the library: with fewer, its
-# blocks (one per compute unit, at least 8 columns each) would not fill the chip
-ROWS_MIN_COLUMNS = 2048
+ROWS_MAX_ROWS = 64        # most rows the kernel takes (which matrices it is chosen for: dispatch.limits)
 
 
 def gemm_rows_supports(a: torch.Tensor, w: torch.Tensor, silu: bool = False) -> bool:
@@ -448,30 +445,23 @@ def gemm_rows(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = N
     return out
 
 
-SKINNY_MAX_ROWS = 16     # up to here the weight-streaming kernel beats the library product
 # torch.mm(..., out_dtype=float32) stores the 32-bit accumulator of a bfloat16 product; older torch lacks it
 _MM_TAKES_OUT_DTYPE = "out_dtype" in (torch.mm.__doc__ or "")
 
 
-# 32-bit results over very many columns (the logits head) up to 32 rows: four tiles of W a block, four waves,
-# ahead of the library there
-WIDE_HEAD_SKINNY_MAX_ROWS, WIDE_HEAD_MIN_COLUMNS = 32, 65536
-
-
 def gemm_bf16(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
               out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
-    """bfloat16 operands, 32-bit accumulation.  Few rows go to the weight-streaming kernel; many
-    rows go through the library product (as the reference's linears do, ullm/layers/linear.py:165),
-    which for 32-bit output (logits) stores the accumulator unrounded."""
+    """bfloat16 operands, 32-bit accumulation.  Few rows go to the weight-streaming kernels (up to how many
+    for this matrix: :func:`dispatch.limits`); many rows go through the library product (as the reference's
+    linears do, ullm/layers/linear.py:165), which for 32-bit output (logits) stores the accumulator unrounded."""
     out_dtype = out_dtype or a.dtype
     M = a.shape[0]
     library = a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and a.is_cuda
-    if M <= SKINNY_MAX_ROWS and gemm_skinny_supports(a, w):
+    lim = dispatch.limits(w.shape[0], w.shape[1])
+    few = lim.f32_skinny if out_dtype == torch.float32 else lim.skinny
+    if M <= few and gemm_skinny_supports(a, w):
         return gemm_skinny(a, w, bias, out_dtype=out_dtype)
-    if (out_dtype == torch.float32 and M <= WIDE_HEAD_SKINNY_MAX_ROWS and w.shape[0] >= WIDE_HEAD_MIN_COLUMNS
-            and gemm_skinny_supports(a, w)):
-        return gemm_skinny(a, w, bias, out_dtype=out_dtype)
-    if (out_dtype == torch.bfloat16 and M <= ROWS_MAX_ROWS and w.shape[0] >= ROWS_MIN_COLUMNS and gemm_rows_supports(a, w)):
+    if out_dtype == torch.bfloat16 and M <= min(lim.rows, ROWS_MAX_ROWS) and gemm_rows_supports(a, w):
         return gemm_rows(a, w, bias)
     if library and out_dtype == torch.float32 and a.is_contiguous() and w.is_contiguous() and _MM_TAKES_OUT_DTYPE:
         y = torch.mm(a, w.t(), out_dtype=torch.float32)

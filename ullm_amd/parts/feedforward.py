@@ -10,15 +10,7 @@ import torch
 
 from ..kernels import ops
 from .base import FeedForward, PartEnv, StepContext, WeightDecl, register_part
-from .linear import can_fuse, linear, linear_into_stream, linear_of_norm
-
-
-# gate|up with the activation folded in, by rows of the batch (chosen from timings of each kernel at every row count):
-# up to 16 rows the few-rows kernel; from 17 to 64 rows the kernel for those row counts, except that up to 32 rows
-# the few-rows kernel is still ahead on matrices up to Qwen3-8B's size; beyond 64 rows the library product and
-# the activation kernel.
-GATE_UP_SKINNY_MAX_ROWS = 32
-GATE_UP_SKINNY_WIDE_MAX_WEIGHT = 200_000_000     # elements of gate|up up to which 17 to 32 rows take the few-rows kernel
+from .linear import can_fuse, gate_up, linear_into_stream, linear_of_norm
 
 
 @register_part("ffn", "swiglu")
@@ -42,16 +34,7 @@ class SwiGLU(FeedForward):
         self.w_down = tensors[f"{p}.down_proj.weight"].contiguous()
 
     def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
-        rows = x.shape[0]
-        if (x.dtype == torch.bfloat16 and rows <= GATE_UP_SKINNY_MAX_ROWS
-                and (rows <= 16 or self.w_gate_up.numel() <= GATE_UP_SKINNY_WIDE_MAX_WEIGHT)
-                and ops.gemm_skinny_supports(x, self.w_gate_up)):
-            act = ops.gemm_skinny_silu(x, self.w_gate_up)
-        elif (x.dtype == torch.bfloat16 and 16 < rows <= ops.ROWS_MAX_ROWS and self.intermediate_size >= ops.ROWS_MIN_COLUMNS
-                and ops.gemm_rows_supports(x, self.w_gate_up, silu=True)):
-            act = ops.gemm_rows(x, self.w_gate_up, silu=True)
-        else:
-            act = ops.silu_mul(linear(x, self.w_gate_up))
+        act = gate_up(x, self.w_gate_up)
         return linear_into_stream(act, self.w_down, ctx)
 
     def fusable(self, residual, ctx: StepContext) -> bool:

@@ -9,7 +9,7 @@ from typing import Optional
 
 import torch
 
-from ..kernels import ops
+from ..kernels import dispatch, ops
 
 
 def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
@@ -20,14 +20,6 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
     return ops.gemm_bf16(x, weight, bias, out_dtype=out_dtype)
 
 
-# Rows up to which folding the norm into the product pays: beyond, the float32 rows of X cost every block more
-# registers and loads than the saved launch is worth.  A small matrix (q|k|v of the 8B and 14B sizes) has few
-# blocks to pay that price, and the launch of the norm's own kernel weighs more beside its short product: there
-# the norm is folded in for every row count the kernel takes.
-NORM_FOLDED_MAX_ROWS = 8
-NORM_FOLDED_SMALL_WEIGHT = 40 << 20     # elements
-
-
 def linear_of_norm(x, weight: torch.Tensor, bias: Optional[torch.Tensor] = None, silu: bool = False) -> torch.Tensor:
     """The first projection of a part whose input may be a norm not yet computed
     (:class:`~ullm_amd.parts.base.PendingNorm`): then the norm is folded into the product where the
@@ -35,17 +27,33 @@ def linear_of_norm(x, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
     and the result silu(gate) * up."""
     from .base import PendingNorm
     if isinstance(x, PendingNorm):
+        # folding the norm into the product pays up to a row count that depends on the matrix: beyond, the 32-bit
+        # rows of X cost every block more registers and loads than the saved launch is worth
         if (x.out_dtype == torch.bfloat16
-                and (x.stream.shape[0] <= NORM_FOLDED_MAX_ROWS or weight.numel() <= NORM_FOLDED_SMALL_WEIGHT)
+                and x.stream.shape[0] <= dispatch.limits(weight.shape[0], weight.shape[1]).fold_norm
                 and ops.gemm_skinny_normed_supports(x.stream, x.gain, weight)):
             return ops.gemm_skinny_normed(x.stream, x.gain, x.eps, weight, bias, silu=silu)
         x = x.apply()
     if silu:
-        return ops.gemm_skinny_silu(x, weight)
+        return gate_up(x, weight)
     return linear(x, weight, bias)
 
 
-FUSED_MAX_ROWS = 16      # batches up to this many tokens take the projections with the folded add / activation
+def gate_up(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    """silu(x g^T) * (x u^T) for the stacked weights g | u [2 I, K]: by the few-rows kernel or the kernel for up
+    to 64 rows with the activation on store, up to the row counts the matrix's limits name; else by the
+    library product and the activation kernel (float32 always: the 32-bit product, then the kernel)."""
+    rows = x.shape[0]
+    if x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16:
+        lim = dispatch.limits(weight.shape[0], weight.shape[1])
+        if rows <= lim.silu_skinny and ops.gemm_skinny_supports(x, weight):
+            return ops.gemm_skinny_silu(x, weight)
+        if rows <= min(lim.silu_rows, ops.ROWS_MAX_ROWS) and ops.gemm_rows_supports(x, weight, silu=True):
+            return ops.gemm_rows(x, weight, silu=True)
+    return ops.silu_mul(linear(x, weight))
+
+
+FUSED_MAX_ROWS = 16      # the few-rows kernel adds into the stream itself for up to this many rows (one tile of X)
 
 
 def can_fuse(residual: torch.Tensor, dtype: torch.dtype, *weights: torch.Tensor) -> bool:
@@ -58,19 +66,15 @@ def can_fuse(residual: torch.Tensor, dtype: torch.dtype, *weights: torch.Tensor)
                for w in weights)
 
 
-STACKED_MIN_ROWS, STACKED_MAX_ROWS = 17, 256
-# smallest matrix (elements) that goes this way: below (Qwen3-0.6B's projections, 2-3 M elements), the stack the
-# norm has to read outweighs the matrix
-STACKED_MIN_WEIGHT = 8 << 20
-
-
 def linear_into_stream(x: torch.Tensor, weight: torch.Tensor, ctx) -> torch.Tensor:
     """The last projection of a mixer or feed-forward, whose result the next norm adds to the residual
-    stream.  For 17 to 256 rows in bfloat16, where the model's norms add stacks, it is a stack of
-    float32 partial sums over slices of the inner dimension (the slices fill the chip, the norm adds
-    them in order); otherwise the plain product.  For few long rows the library's choice of kernel
-    is two to five times off the memory roofline at these row counts."""
-    if (ctx.stacked_branches and x.dtype == torch.bfloat16 and STACKED_MIN_ROWS <= x.shape[0] <= STACKED_MAX_ROWS
-            and weight.numel() >= STACKED_MIN_WEIGHT and ops.gemm_partial_sums_supports(x, weight)):
+    stream.  For a range of row counts that depends on the matrix (17 to 256 for all but small ones), in
+    bfloat16 and where the model's norms add stacks, it is a stack of float32 partial sums over slices of
+    the inner dimension (the slices fill the chip, the norm adds them in order); otherwise the plain
+    product.  For few long rows the library's choice of kernel is two to five times off the memory
+    roofline at these row counts."""
+    lim = dispatch.limits(weight.shape[0], weight.shape[1])
+    if (ctx.stacked_branches and x.dtype == torch.bfloat16 and lim.stacked_from > 0
+            and lim.stacked_from <= x.shape[0] <= lim.stacked_to and ops.gemm_partial_sums_supports(x, weight)):
         return ops.gemm_partial_sums(x, weight)
     return linear(x, weight)
