@@ -24,7 +24,9 @@ DEV = "cuda:0"
 
 
 def graph_time(calls: List[Callable[[], None]], replays: int = 5) -> float:
-    """Mean microseconds per call of ``calls`` when they run as one HIP graph."""
+    """Mean microseconds per call of ``calls`` when they run as one HIP graph.  A short list is repeated until
+    the graph holds at least 24 calls, so that the launch of the graph itself is a small share of every call."""
+    calls = list(calls) * max(1, -(-24 // max(1, len(calls))))
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
