@@ -59,10 +59,10 @@ def default_limits(columns: int, inner: int) -> Limits:
         f32_skinny=32 if columns >= 65536 else 16)
 
 
-_table: Optional[Dict[str, Limits]] = None
+_table: Optional[dict] = None
 
 
-def _load() -> Dict[str, Limits]:
+def _load() -> dict:
     global _table
     if _table is None:
         table: Dict[str, Limits] = {}
@@ -85,8 +85,14 @@ def _load() -> Dict[str, Limits]:
 def limits(columns: int, inner: int) -> Limits:
     """The row limits of a weight matrix [columns, inner]: measured ones where the table has the matrix,
     the size rules otherwise."""
-    found = _load().get(f"{columns}x{inner}")
-    return found if found is not None else default_limits(columns, inner)
+    table = _load()
+    found = table.get((columns, inner))                    # by a tuple: this is asked for every projection of every step
+    if found is None:
+        found = table.get(f"{columns}x{inner}")
+        if found is None:
+            return default_limits(columns, inner)
+        table[(columns, inner)] = found
+    return found
 
 
 def is_tuned(columns: int, inner: int) -> bool:
