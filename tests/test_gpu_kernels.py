@@ -1008,6 +1008,73 @@ def test_gemm_skinny_with_the_norm_folded_in(ops, shape):
         assert (got.float().cpu() - want).abs().max() <= 1e-2 * float(want.abs().max())
 
 
+@pytest.mark.parametrize("shape", [(1, 64, 128, 96), (8, 4096, 1024, 6144), (5, 1032, 264, 100), (16, 328, 72, 520),
+                                   (3, 5120, 200, 70000), (13, 24, 512, 36), (9, 8200, 64, 256)])
+def test_a_norm_handed_from_one_product_to_the_next(ops, shape):
+    """A product that adds into the 32-bit stream also leaves, for the norm that comes next, the stream times that
+    norm's gain in bfloat16 and every block's share of the rows' sums of squares; the next product multiplies the
+    former and scales its rows by the latter.  Against the plain add, norm and product, with rows whose scales
+    differ by orders of magnitude (a sum that leaks into another row, or a share of the squares that is lost or
+    counted twice, shows), widths (M, hidden, inner of the first, outputs of the second) that are no multiples of
+    a block's columns, and more blocks than the lanes of the second product fetch at once."""
+    torch.manual_seed(15)
+    M, H, K, N = shape
+    a = torch.randn(M, K, device=DEV).bfloat16()
+    w1 = (torch.randn(H, K, device=DEV) * 0.1).bfloat16()
+    stream0 = torch.randn(M, H, device=DEV) * torch.logspace(-2, 2, M, device=DEV)[:, None]
+    gain = 1.0 + 0.5 * torch.randn(H, device=DEV)
+    w2 = (torch.randn(N, H, device=DEV) * 0.3).bfloat16()
+    b = torch.randn(N, device=DEV)
+    eps = 1e-3
+    for kw in (dict(nt=1, waves=1), dict(nt=2, waves=4), dict(nt=1, rows=12), dict(nt=2, rows=20), {}):
+        plain_stream, stream = stream0.clone(), stream0.clone()
+        ops.gemm_skinny_add(a, w1, plain_stream, **kw)
+        scaled, squares = ops.gemm_skinny_add(a, w1, stream, next_gain=gain, **kw)
+        assert torch.equal(stream, plain_stream), kw                       # the add itself is untouched
+        assert scaled.dtype == torch.bfloat16 and torch.equal(scaled, (stream * gain).bfloat16()), kw
+        assert squares.shape[0] == M and squares.shape[1] % 4 == 0
+        want_sq = stream.double().pow(2).sum(-1)
+        assert ((squares.double().sum(-1) - want_sq).abs() <= 1e-6 * want_sq).all(), kw
+    normed = plain.rms_norm(stream.cpu(), gain.cpu(), eps)
+    want = normed @ w2.float().cpu().T + b.cpu()
+    bound = 1e-2 * float(want.abs().max())
+    results = {"few rows": ops.gemm_skinny(scaled, w2, b, out_dtype=torch.float32, squares=squares, eps=eps),
+               "few rows, one wave": ops.gemm_skinny(scaled, w2, b, out_dtype=torch.float32, squares=squares, eps=eps,
+                                                     nt=1, waves=1),
+               "few rows, two tiles": ops.gemm_skinny(scaled, w2, b, out_dtype=torch.float32, squares=squares, eps=eps,
+                                                      nt=2, waves=2)}
+    if ops.gemm_rows_supports(scaled, w2):
+        results["rows"] = ops.gemm_rows(scaled, w2, b, squares=squares, eps=eps)
+    for name, got in results.items():
+        assert (got.float().cpu() - want).abs().max() <= bound, name
+    # the same arithmetic as the norm folded into the product (x * gain rounded, the product, the scale): the same bits
+    if ops.gemm_skinny_normed_supports(stream, gain, w2):
+        folded = ops.gemm_skinny_normed(stream, gain, eps, w2, b, out_dtype=torch.float32)
+        assert (results["few rows"] - folded).abs().max() <= 2e-6 * float(want.abs().max())
+    # fewer rows of the same stream: every row as before, bit for bit (up to 8 rows and beyond them the lanes share
+    # out the sums of squares differently: across that line the scale may differ in its last bit)
+    for m in {M // 2, M - 1} - {0}:
+        fewer = ops.gemm_skinny(scaled[:m], w2, b, out_dtype=torch.float32, squares=squares[:m].contiguous(), eps=eps)
+        if (m <= 8) == (M <= 8):
+            assert torch.equal(fewer, results["few rows"][:m]), m
+        assert (fewer - results["few rows"][:m]).abs().max() <= 1e-6 * float(want.abs().max())
+    inter = N // 2
+    if inter:
+        wgu = torch.cat([w2[:inter], w2[N - inter:]]).contiguous()
+        want = plain.silu_and_mul(normed @ wgu.float().cpu().T)
+        outs = {"few rows": ops.gemm_skinny_silu(scaled, wgu, squares=squares, eps=eps)}
+        if ops.gemm_rows_supports(scaled, wgu, silu=True):
+            outs["rows"] = ops.gemm_rows(scaled, wgu, silu=True, squares=squares, eps=eps)
+        for name, got in outs.items():
+            assert got.shape == (M, inter) and got.dtype == torch.bfloat16
+            assert (got.float().cpu() - want).abs().max() <= 1e-2 * float(want.abs().max()), name
+    # what the kernels refuse: more than one tile of rows, squares of another batch
+    with pytest.raises(Exception):
+        ops.gemm_skinny(scaled, w2, squares=squares[:, :2].contiguous(), eps=eps)
+    with pytest.raises(Exception):
+        ops.gemm_skinny(torch.cat([scaled] * 3)[:17].contiguous(), w2, squares=torch.ones(17, 4, device=DEV), eps=eps)
+
+
 @pytest.mark.parametrize("shape", [(2, 2, 1536), (1, 4, 1000), (3, 2, 24), (7, 6, 72), (16, 4, 200), (5, 2, 520)])
 def test_folded_norm_on_few_outputs_errs_by_the_rounding_of_its_inputs(ops, shape):
     """silu(gate) * up of rmsnorm(stream) for two to six outputs a row, inner sizes that are no multiple of a

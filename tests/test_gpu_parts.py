@@ -335,6 +335,60 @@ def test_norm_left_to_the_feed_forwards_first_projection(monkeypatch):
     assert isinstance(x, torch.Tensor)
 
 
+def test_a_feed_forward_prepares_the_norm_that_follows_it(monkeypatch):
+    """Told which norm comes next, the feed-forward's last kernel leaves that norm half done (the stream times the
+    gain, the rows' sums of squares) and returns its record; a second feed-forward behind that norm takes the
+    record, and no norm kernel runs in between.  Two feed-forwards in a row against the plain functions, with
+    rows whose sizes differ by orders of magnitude; and the record is only taken for the norm it was made for."""
+    from types import SimpleNamespace
+    from ullm_amd.kernels import ops
+    from ullm_amd.parts import PartEnv, PendingNorm, build_part
+    from ullm_amd.parts.block import PreNormBlock
+    from ullm_amd.weights.loader import bind_tensors
+    torch.manual_seed(8)
+    H, I, eps = 104, 232, 1e-3
+    env = PartEnv(torch.device(DEV), torch.bfloat16, 16)
+    ffns, ws, norms, gains = [], [], [], []
+    for i in range(2):
+        ffn = build_part("ffn", "swiglu", hidden_size=H, intermediate_size=I, prefix=f"f{i}")
+        w = {f"f{i}.{n}.weight": (torch.randn(*shape) * 0.1).bfloat16() for n, shape in
+             (("gate_proj", (I, H)), ("up_proj", (I, H)), ("down_proj", (H, I)))}
+        bind_tensors(ffn, w, env)
+        gain = 1 + 0.3 * torch.randn(H)
+        norm = build_part("norm", "rmsnorm", size=H, eps=eps, weight_name="g")
+        norm.bind({"g": gain.to(DEV)}, env)
+        ffns.append(ffn), ws.append(w), norms.append(norm), gains.append(gain)
+    ctx = SimpleNamespace(stacked_branches=False, dtype=torch.bfloat16)
+    assert ffns[0].hands_norm_ahead
+    norm_kernels, inner = [], ops.add_rmsnorm
+    monkeypatch.setattr(ops, "add_rmsnorm", lambda *a, **k: norm_kernels.append(1) or inner(*a, **k))
+    for T in (1, 5, 8, 9, 16):
+        stream = torch.randn(T, H) * torch.logspace(-2, 2, T)[:, None]
+        mid = stream + plain.qwen3_mlp(plain.rms_norm(stream, gains[0], eps), {k: v.float() for k, v in ws[0].items()}, "f0")
+        want = mid + plain.qwen3_mlp(plain.rms_norm(mid, gains[1], eps), {k: v.float() for k, v in ws[1].items()}, "f1")
+        got = stream.clone().to(DEV)
+        x = PreNormBlock._normed(norms[0], ffns[0], None, got, ctx)
+        record = ffns[0].forward_fused(x, got, ctx, then=norms[1])
+        assert isinstance(record, PendingNorm) and record.norm is norms[1] and record.scaled is not None
+        assert (got.cpu() - mid).abs().max() <= 2e-2 * (mid - stream).abs().max()
+        norm_kernels.clear()
+        x = PreNormBlock._normed(norms[1], ffns[1], record, got, ctx)
+        assert x is record
+        assert ffns[1].forward_fused(x, got, ctx) is None                 # told of no norm: nothing prepared
+        assert not norm_kernels
+        assert (got.cpu() - want).abs().max() <= 2e-2 * (want - stream).abs().max()
+        # a record made for another norm is not taken: the block's own norm runs on the finished stream
+        x = PreNormBlock._normed(norms[0], ffns[1], record, got, ctx)
+        assert x is not record and isinstance(x, PendingNorm) and x.norm is norms[0] and x.scaled is None
+        # a part that wants its input computed gets the normed stream
+        x = PreNormBlock._normed(norms[1], None, record, got, ctx)
+        assert isinstance(x, torch.Tensor) and norm_kernels
+        assert (x.float().cpu() - plain.rms_norm(got.cpu(), gains[1], eps)).abs().max() <= 1e-2 * x.float().abs().max()
+    # beyond the rows the kernels take, nothing is prepared
+    big = torch.randn(40, H, device=DEV)
+    assert not ffns[0].fusable(big, ctx)
+
+
 def test_rotary_part_table_matches_the_plain_angles():
     from ullm_amd.parts import PartEnv, build_part
     rot = build_part("position", "rotary", head_dim=24, theta=777.0, rotary_dim=12, pairing="half")

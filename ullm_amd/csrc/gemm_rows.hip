@@ -12,6 +12,11 @@
 // from there.  A result column is summed by one wave in the order of K, so it does not depend on timing
 // or on the batch.
 //
+// A norm handed ahead by the product before (RowSquares): X is then the stream times the norm's gain in
+// bfloat16, and the 32-bit results of row m are scaled by rsqrt(sum of the parts' squares of row m / K + eps)
+// before the epilogue (ullm/layers/layernorm.py:28-33 with the scale taken out of the product).  The parts are
+// added in a fixed order: a lane's parts in turn, the four lanes of a row, the waves.
+//
 // A operand of v_mfma_f32_16x16x32_bf16 = a W tile (lane (r, g) holds W[n0 + r][k + 8g .. +8]), B
 // operand = 16 rows of X; W tiles reach that layout through the wave's own part of shared memory (a
 // wave fetches whole 128-byte lines, 8 rows per instruction).  Shared-memory rows are 128 bytes; piece
@@ -29,6 +34,16 @@ union Pack8 {
 };
 
 enum { ROWS_STORE = 0, ROWS_SILU = 1 };
+
+// Sums of squares left by the product before (sq == nullptr: none): sq[m][0 .. 4 quads), row stride 4 quads,
+// 16-byte aligned
+struct RowSquares {
+  const float* sq;
+  int quads;
+  float eps;
+};
+
+#define ROWS_SQ_HELD 8   // groups of four partial sums of squares a lane fetches before the product starts
 
 // f(0), f(1), .. f(N - 1) with the index a constant of the language, not of the optimiser: registers that
 // hold stages in flight are then never indexed by a variable, and so never end up in scratch memory
@@ -57,15 +72,31 @@ template <int MT, int XQ, int EPI>
 __global__ void __launch_bounds__(64 * ROWS_MAX_WAVES)
 gemm_rows_kernel(const bf16_t* __restrict__ X, int ldx, const bf16_t* __restrict__ W, int ldw,
                  const float* __restrict__ bias, bf16_t* __restrict__ C, int ldc, int M, int N, int K,
-                 int WN, int cols_per_wave, int cols_per_block) {
+                 int WN, int cols_per_wave, int cols_per_block, RowSquares before) {
   constexpr int NTW = EPI == ROWS_SILU ? 2 : 1;         // tiles of W per wave: gate and up rows of the same columns
   constexpr int D = rows_depth(NTW, XQ);
   constexpr int TILE = 16 * 128;                        // 16 rows x 64 values
   constexpr int XB = MT * TILE;                         // a stage of X
   __shared__ __attribute__((aligned(16))) unsigned char xs[2 * XB + 64 * 16];   // two stages, then a spare place per lane
   __shared__ __attribute__((aligned(16))) unsigned char ws[ROWS_MAX_WAVES * NTW * TILE];
+  __shared__ float sqs[ROWS_MAX_WAVES][16];
   const int tid = threadIdx.x, lane = tid & 63, wn = tid >> 6;
   const int g = lane >> 4, r = lane & 15, lrow = lane >> 3, lcol = lane & 7;
+  // The sums of squares the product before left (one tile of rows): lane (r, g) of wave wn adds groups 4 wn + g,
+  // + 4 WN, ... of row r, the four lanes of a row add theirs, the waves' sums meet in `sqs`.  The loads go out
+  // before the first stages' (unconditional, with the index held in range) and are added while those are on
+  // their way, so nothing waits for them.
+  const bool scaled = MT == 1 && before.sq != nullptr;
+  const int sq_step = 4 * WN, sq_first = 4 * wn + g;
+  float4 held[ROWS_SQ_HELD];
+  const float* const sq_row = before.sq + (size_t)(r < M ? r : M - 1) * 4 * before.quads;
+  if (scaled) {
+#pragma unroll
+    for (int i = 0; i < ROWS_SQ_HELD; ++i) {
+      const int j = sq_first + i * sq_step;
+      held[i] = *reinterpret_cast<const float4*>(sq_row + 4 * (j < before.quads ? j : before.quads - 1));
+    }
+  }
   const int block_n0 = blockIdx.x * cols_per_block;
   const int block_end = block_n0 + cols_per_block < N ? block_n0 + cols_per_block : N;
   const int n0 = block_n0 + wn * cols_per_wave;
@@ -148,11 +179,35 @@ gemm_rows_kernel(const bf16_t* __restrict__ X, int ldx, const bf16_t* __restrict
   Stage st[D];
   const int stages = K / 64;
   static_for<0, D>([&](auto d) { fetch(st[d], 64 * d); });
+  if (scaled) {
+    float q = 0.f;
+#pragma unroll
+    for (int i = 0; i < ROWS_SQ_HELD; ++i) {
+      const float4 v = held[i];
+      q += sq_first + i * sq_step < before.quads ? (v.x + v.y) + (v.z + v.w) : 0.f;
+    }
+    for (int j = sq_first + ROWS_SQ_HELD * sq_step; j < before.quads; j += sq_step) {
+      const float4 v = *reinterpret_cast<const float4*>(sq_row + 4 * j);
+      q += (v.x + v.y) + (v.z + v.w);
+    }
+    q += __shfl_xor(q, 16);
+    q += __shfl_xor(q, 32);
+    if (g == 0) sqs[wn][r] = q;             // read after the barriers of the stages
+  }
   int s = 0;
   for (; s + D <= stages; s += D) static_for<0, D>([&](auto d) { stage(st[d], s + d); });
   static_for<0, D - 1>([&](auto d) {
     if (s + d < stages) stage(st[d], s + d);
   });
+  if (scaled) {
+    float total = 0.f;
+    for (int w = 0; w < WN; ++w) total += sqs[w][r];
+    const float rs = rsqrtf(total / (float)K + before.eps);
+#pragma unroll
+    for (int i = 0; i < NTW; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[i][0][j] *= rs;
+  }
   // acc[i][t][j] = sum for row m = 16 t + r, column n0 + 4 g + j (of half i of the stacked matrix)
   const int nn = n0 + 4 * g;
 #pragma unroll
@@ -222,18 +277,23 @@ extern "C" int ullm_gemm_rows_supports(int M, int N, int K, int ldx, int ldw, in
 
 // X bfloat16 [M <= 64, K], K a multiple of 64; W bfloat16 [N, K] (epi 1: [2 N, K], gate rows then up rows);
 // C bfloat16 [M, N] with row stride ldc; bias float32 [N] or null (epi 0 only).
+// With row_sq (float32 [M <= 16, sq_parts], sq_parts a multiple of 4): the results of row m are scaled by
+// rsqrt(sum of row_sq[m][.] / K + eps) before the epilogue.
 extern "C" int ullm_gemm_rows(const void* X, int ldx, const void* W, int ldw, const float* bias, void* C, int ldc,
-                              int M, int N, int K, int epi, hipStream_t stream) {
+                              int M, int N, int K, int epi, const float* row_sq, int sq_parts, float eps,
+                              hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (!ullm_gemm_rows_supports(M, N, K, ldx, ldw, ldc, epi)) return ULLM_ERR_SHAPE;
   if (((uintptr_t)X & 15) || ((uintptr_t)W & 15) || ((uintptr_t)C & 7)) return ULLM_ERR_SHAPE;
   if (epi == ROWS_SILU && bias) return ULLM_ERR_UNSUPPORTED;
+  if (row_sq && (M > 16 || sq_parts < 4 || sq_parts % 4 || ((uintptr_t)row_sq & 15))) return ULLM_ERR_UNSUPPORTED;
+  const RowSquares before{row_sq, sq_parts / 4, eps};
   const int mt = (M + 15) / 16;
   RowsShape s;
   rows_shape(N, mt, rows_compute_units(), &s);
   dim3 grid(s.blocks), block(64 * s.wn);
 #define GO(MT, XQ, EPI) hipLaunchKernelGGL((gemm_rows_kernel<MT, XQ, EPI>), grid, block, 0, stream, (const bf16_t*)X, ldx, \
-    (const bf16_t*)W, ldw, bias, (bf16_t*)C, ldc, M, N, K, s.wn, s.cols_per_wave, s.cols_per_block)
+    (const bf16_t*)W, ldw, bias, (bf16_t*)C, ldc, M, N, K, s.wn, s.cols_per_wave, s.cols_per_block, before)
 #define GO_XQ(MT, EPI)                                    \
   do {                                                    \
     if (s.xq <= 1) GO(MT, 1, EPI);                        \

@@ -25,6 +25,14 @@
 //     gain and rounds to bfloat16 on the way into shared memory, adds up the squares beside that, and
 //     multiplies the finished sums by rsqrt(mean of squares + eps): y = rs * ((x * gain) W^T).  Against
 //     a norm kernel of its own this saves a launch and a pass, which at these sizes is all latency.
+//
+//   a norm handed from one product to the next (NormAhead, RowSquares)
+//     A product that ends in the stream (RESADD) owns the final values of its columns.  Given the gain of
+//     the norm that comes next it also stores x * gain rounded to bfloat16 and, per block, the sum of the
+//     squares of its columns of every row.  The next product then takes those bfloat16 rows as its X, adds
+//     up the blocks' sums and scales its 32-bit results by rsqrt(mean of squares + eps): the same
+//     arithmetic as NORMX, without a norm kernel between the two and without 32-bit rows of X in the
+//     second.  The sums are added in a fixed order (a lane's blocks in turn, lanes, waves).
 #include "common.h"
 #include <type_traits>
 
@@ -40,6 +48,24 @@ union Pack8 {
 
 enum { EPI_STORE = 0, EPI_RESADD = 1, EPI_SILU = 2 };
 
+// What a RESADD product leaves for the norm that follows it (gain == nullptr: nothing): x[m][n] = stream * gain
+// in bfloat16 (row stride ldx), sq[m][block] = the block's sum of squares of row m of the stream (row stride
+// ld_sq, a multiple of 4; the last block clears the entries from the number of blocks to ld_sq).
+struct NormAhead {
+  const float* gain;
+  bf16_t* x;
+  float* sq;
+  int ldx, ld_sq;
+};
+
+// Sums of squares left by the product before (sq == nullptr: none): sq[m][0 .. 4 quads), row stride 4 quads,
+// 16-byte aligned; the results of row m are scaled by rsqrt(sum of the row / K + eps).
+struct RowSquares {
+  const float* sq;
+  int quads;
+};
+
+
 // Most waves per block for a tile shape,
 // bounded by the shared memory that holds a stage per wave (and later the waves' partials): at most 8
 // waves, so that several blocks fit a compute unit
@@ -47,12 +73,13 @@ __host__ __device__ constexpr int sk_max_waves(int mt, int nt) { return mt * nt 
 
 // The waves' partial results of a block are added in wave order through `red` and the sum goes where
 // EPI says.  acc[i][t][j] = partial C[m = 16 t + r][n0 + 16 i + 4 g + j].
-// With NORMX, sq[w][m] holds wave w's sum of squares of row m of X and the sums are scaled by
-// rsqrt(their total / K + eps) first.
-template <int MT, int NT, int EPI, typename TC, bool NORMX, typename RedT>
+// With `scaled`, sq[w][m] holds wave w's sum of squares of row m of X (or its share of the sums the product
+// before left) and the sums are scaled by rsqrt(their total / K + eps) first.
+template <int MT, int NT, int EPI, typename TC, typename RedT>
 __device__ __forceinline__ void skinny_finish(f32x4_t (&acc)[NT][MT], RedT& red, const float* __restrict__ bias,
                                               TC* __restrict__ C, float* __restrict__ R, int ldc, int M, int N, int n0,
-                                              const float (*sq)[16 * MT], int K, float eps) {
+                                              bool scaled, const float (*sq)[16 * MT], int K, float eps,
+                                              const NormAhead& ahead) {
   constexpr int OT = EPI == EPI_SILU ? NT / 2 : NT;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
   const int g = lane >> 4, r = lane & 15;
@@ -76,7 +103,7 @@ __device__ __forceinline__ void skinny_finish(f32x4_t (&acc)[NT][MT], RedT& red,
           acc[i][t][0] += o.x; acc[i][t][1] += o.y; acc[i][t][2] += o.z; acc[i][t][3] += o.w;
         }
   }
-  if (NORMX) {
+  if (scaled) {
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
       float total = 0.f;
@@ -87,6 +114,48 @@ __device__ __forceinline__ void skinny_finish(f32x4_t (&acc)[NT][MT], RedT& red,
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[i][t][j] *= rs;
     }
+  }
+  if (EPI == EPI_RESADD && ahead.gain) {
+    // the stream's new values, the same times the next norm's gain in bfloat16, and the block's share of
+    // the rows' sums of squares: a lane's columns in turn, then the four lanes of a row
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      const int m = 16 * t + r;
+      float q = 0.f;
+      if (m < M) {
+#pragma unroll
+        for (int i = 0; i < OT; ++i) {
+          const int nn = n0 + 16 * i + 4 * g;
+          float* rp = R + (size_t)m * ldc + nn;
+          bf16_t* xp = ahead.x + (size_t)m * ahead.ldx + nn;
+          if (nn + 3 < N) {
+            float4 o = *reinterpret_cast<float4*>(rp);
+            const float4 gn = *reinterpret_cast<const float4*>(ahead.gain + nn);
+            o.x += acc[i][t][0]; o.y += acc[i][t][1]; o.z += acc[i][t][2]; o.w += acc[i][t][3];
+            *reinterpret_cast<float4*>(rp) = o;
+            *reinterpret_cast<uint2*>(xp) = make_uint2(pack2_bf16(o.x * gn.x, o.y * gn.y), pack2_bf16(o.z * gn.z, o.w * gn.w));
+            q = fmaf(o.x, o.x, q); q = fmaf(o.y, o.y, q); q = fmaf(o.z, o.z, q); q = fmaf(o.w, o.w, q);
+          } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+              if (nn + j < N) {
+                const float o = rp[j] + acc[i][t][j];
+                rp[j] = o;
+                xp[j] = f32_to_bf16_bits(o * ahead.gain[nn + j]);
+                q = fmaf(o, o, q);
+              }
+          }
+        }
+      }
+      q += __shfl_xor(q, 16);
+      q += __shfl_xor(q, 32);
+      if (g == 0 && m < M) {
+        ahead.sq[(size_t)m * ahead.ld_sq + blockIdx.x] = q;
+        if (blockIdx.x == gridDim.x - 1)
+          for (int b = gridDim.x; b < ahead.ld_sq; ++b) ahead.sq[(size_t)m * ahead.ld_sq + b] = 0.f;
+      }
+    }
+    return;
   }
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
@@ -137,13 +206,14 @@ template <int MT, int NT, int EPI, typename TC, bool NORMX, int XH>
 __global__ void __launch_bounds__(64 * sk_max_waves(MT, NT))
 gemm_skinny_kernel(const void* __restrict__ Xv, int ldx, const bf16_t* __restrict__ W, int ldw,
                    const float* __restrict__ bias, const float* __restrict__ gain, float eps, TC* __restrict__ C,
-                   float* __restrict__ R, int ldc, int M, int N, int K, int k_per_wave, int rows_per_block) {
+                   float* __restrict__ R, int ldc, int M, int N, int K, int k_per_wave, int rows_per_block,
+                   NormAhead ahead, RowSquares before) {
   constexpr int MAXW = sk_max_waves(MT, NT);
   constexpr int TILE_BYTES = 16 * 128, STAGE_BYTES = (NT + MT) * TILE_BYTES;
   constexpr int RED_BYTES = (MAXW - 1) * NT * MT * 256 * 4;
   constexpr int LDS_BYTES = MAXW * STAGE_BYTES > RED_BYTES ? MAXW * STAGE_BYTES : RED_BYTES;
   __shared__ __attribute__((aligned(16))) unsigned char lds[LDS_BYTES];
-  __shared__ float sq[NORMX ? MAXW : 1][16 * MT];
+  __shared__ float sq[MAXW][16 * MT];
   using XT = typename std::conditional<NORMX, float, bf16_t>::type;
   constexpr int XV = NORMX ? 2 : 1;                       // 16-byte loads per 8 values of X
   const XT* const X = reinterpret_cast<const XT*>(Xv);
@@ -178,6 +248,24 @@ gemm_skinny_kernel(const void* __restrict__ Xv, int ldx, const bf16_t* __restric
         xrow[t][h] = 16 * t + row < M;
         xsrc[t][h] = X + (size_t)(xrow[t][h] ? 16 * t + row : M - 1) * ldx + 8 * lcol;
       }
+    }
+  }
+  // The sums of squares the product before left: the lanes of a wave that share a row (8 of them where the
+  // batch has up to 8 rows, else 4) take groups of four sums in turn, add theirs, and the waves' sums meet in `sq`.
+  // The loads go out before the first stage's (unconditional, with the index held in range) and are added while
+  // that stage is on its way, so nothing waits for them.
+  constexpr bool SQUARES = !NORMX && EPI != EPI_RESADD && MT == 1;      // one tile of rows: what a norm handed ahead covers
+  constexpr int SQ_LANES = XH == 1 ? 8 : 4, SQ_HELD = XH == 1 ? 1 : 2;
+  const bool scaled = NORMX || (SQUARES && before.sq != nullptr);
+  const int sq_row = lane & (64 / SQ_LANES - 1), sq_step = SQ_LANES * (blockDim.x >> 6),
+            sq_first = SQ_LANES * wave + lane / (64 / SQ_LANES);
+  const float* const sq_src = before.sq + (size_t)(sq_row < M ? sq_row : M - 1) * 4 * before.quads;
+  float4 held[SQ_HELD];
+  if (SQUARES && before.sq) {
+#pragma unroll
+    for (int i = 0; i < SQ_HELD; ++i) {
+      const int j = sq_first + i * sq_step;
+      held[i] = *reinterpret_cast<const float4*>(sq_src + 4 * (j < before.quads ? j : before.quads - 1));
     }
   }
   unsigned char* const mine = lds + wave * STAGE_BYTES;
@@ -261,6 +349,24 @@ gemm_skinny_kernel(const void* __restrict__ Xv, int ldx, const bf16_t* __restric
   if (k_begin < k_end) {
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) fetch(st[d], k_begin + 64 * d);
+  }
+  if (SQUARES && before.sq) {
+    float q = 0.f;
+#pragma unroll
+    for (int i = 0; i < SQ_HELD; ++i) {
+      const float4 v = held[i];
+      q += sq_first + i * sq_step < before.quads ? (v.x + v.y) + (v.z + v.w) : 0.f;
+    }
+    for (int j = sq_first + SQ_HELD * sq_step; j < before.quads; j += sq_step) {
+      const float4 v = *reinterpret_cast<const float4*>(sq_src + 4 * j);
+      q += (v.x + v.y) + (v.z + v.w);
+    }
+    if (SQ_LANES == 8) q += __shfl_xor(q, 8);
+    q += __shfl_xor(q, 16);
+    q += __shfl_xor(q, 32);
+    if (lane < 16) sq[wave][lane] = lane < 64 / SQ_LANES ? q : 0.f;
+  }
+  if (k_begin < k_end) {
     for (int k = k_begin; k < k_end; k += 64 * DEPTH) {
 #pragma unroll
       for (int d = 0; d < DEPTH; ++d) {
@@ -287,7 +393,7 @@ gemm_skinny_kernel(const void* __restrict__ Xv, int ldx, const bf16_t* __restric
   }
   __syncthreads();                                        // the partial sums take the place of the stages
   auto& red = *reinterpret_cast<float (*)[MAXW - 1][NT * MT][64 * 4]>(lds);
-  skinny_finish<MT, NT, EPI, TC, NORMX>(acc, red, bias, C, R, ldc, M, n_end, n0, sq, K, eps);
+  skinny_finish<MT, NT, EPI, TC>(acc, red, bias, C, R, ldc, M, n_end, n0, scaled, sq, K, eps, ahead);
 }
 
 template <int MT, int NT, int EPI, typename TC, bool NORMX, typename... Args>
@@ -336,20 +442,15 @@ extern "C" int ullm_gemm_skinny_supports(int M, int N, int K, int ldx, int ldw) 
   return M >= 1 && M <= 64 && N >= 1 && K >= 8 && K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0;
 }
 
-// X bfloat16 [M, K]; W bfloat16 [N, K] (with epi 2: [2 N, K]).  epi: 0 store to C (c_dtype, bias optional),
-// 1 add into R (float32 [M, N], row stride ldc), 2 silu(gate) * up to C (bfloat16 [M, N]).
-// With gain (float32 [K]): X is float32 [M <= 16, K] and its RMS norm with this gain and eps is what
-// is multiplied (epi 0 and 2).  force_nt / force_waves: 0 = chosen here.
-extern "C" int ullm_gemm_skinny(const void* X, int ldx, const void* W, int ldw, const float* bias, void* C,
-                                int ldc, int M, int N, int K, int epi, int c_dtype, int force_nt,
-                                int force_waves, const float* gain, float eps, int force_rows, hipStream_t stream) {
-  if (M <= 0 || N <= 0) return 0;
-  if (!ullm_gemm_skinny_supports(M, N, K, ldx, ldw) || ldc < N) return ULLM_ERR_SHAPE;
-  if (((uintptr_t)X & 15) || ((uintptr_t)W & 15)) return ULLM_ERR_SHAPE;
+struct SkinnyPlan {
+  int mt, nt, rows, tiles, waves, k_per_wave;
+};
+
+// The launch shape of a product: a function of the sizes, the epilogue and whether the norm is folded in.
+static int skinny_plan(int M, int N, int K, int ldx, int ldw, int epi, int force_nt, int force_waves, bool normed,
+                       int force_rows, SkinnyPlan* p) {
+  if (!ullm_gemm_skinny_supports(M, N, K, ldx, ldw)) return ULLM_ERR_SHAPE;
   if (epi < 0 || epi > 2) return ULLM_ERR_UNSUPPORTED;
-  if (gain && (M > 16 || epi == EPI_RESADD || ((uintptr_t)gain & 15))) return ULLM_ERR_UNSUPPORTED;
-  if (epi == EPI_RESADD && (((uintptr_t)C & 15) || ldc % 4 != 0 || bias)) return ULLM_ERR_SHAPE;
-  if (epi == EPI_SILU && (bias || c_dtype != ULLM_BF16)) return ULLM_ERR_UNSUPPORTED;
   int mt = (M + 15) / 16;
   if (mt == 3) mt = 4;                                  // instantiated for 1, 2 and 4 tiles of rows
   const int tiles16 = (N + 15) / 16;
@@ -358,7 +459,7 @@ extern "C" int ullm_gemm_skinny(const void* X, int ldx, const void* W, int ldw, 
   else if (tiles16 >= 4096) nt = mt >= 2 ? 4 : 2;
   else if (tiles16 >= 1024 && mt >= 2) nt = 2;
   // with the norm folded in, a tile of X costs a wave as much as a tile of W: two tiles of W per tile of X
-  if (gain && force_nt <= 0) nt = 2;
+  if (normed && force_nt <= 0) nt = 2;
   if (epi == EPI_SILU) nt = (force_nt == 4 || mt >= 4) ? 4 : 2;   // gate and up tiles come in pairs
   if (nt != 1 && nt != 2 && nt != 4) return ULLM_ERR_UNSUPPORTED;
   if (nt == 4 && mt == 1) nt = 2;                       // not instantiated
@@ -381,21 +482,65 @@ extern "C" int ullm_gemm_skinny(const void* X, int ldx, const void* W, int ldw, 
     if (force_rows > 16 * out_tiles || force_rows % 4) return ULLM_ERR_UNSUPPORTED;
     rows = force_rows;
   }
-  const int tiles = (N + rows - 1) / rows;
   // waves per block: 8 tiles of W in flight per block (8 waves with one tile each, 4 with two),
   // each wave with at least 128 values of K
   const int max_waves = sk_max_waves(mt, nt);
   int waves = 1;
-  const int in_flight = (gain && epi == EPI_STORE) || epi == EPI_SILU || nt == 4 ? 16 : 8;   // in 16-row tiles of W
+  const int in_flight = (normed && epi == EPI_STORE) || epi == EPI_SILU || nt == 4 ? 16 : 8;   // in 16-row tiles of W
   const int w_rows = rows * (nt / out_tiles);           // rows of W a block fetches
   while (waves < max_waves && waves * w_rows < 16 * in_flight && K / (waves * 2) >= 128) waves *= 2;
   if (force_waves > 0) waves = force_waves < max_waves ? force_waves : max_waves;
   int k_per_wave = (K + waves - 1) / waves;
   k_per_wave = (k_per_wave + 63) / 64 * 64;
+  *p = SkinnyPlan{mt, nt, rows, (N + rows - 1) / rows, waves, k_per_wave};
+  return 0;
+}
+
+// Blocks of the product that adds into the stream (epi 1) for these sizes: the number of partial sums of squares it
+// leaves per row when it hands the next norm ahead.  Negative: an error code.
+extern "C" int ullm_gemm_skinny_blocks(int M, int N, int K, int ldx, int ldw, int epi, int force_nt, int force_waves,
+                                       int force_rows) {
+  SkinnyPlan p;
+  const int err = skinny_plan(M, N, K, ldx, ldw, epi, force_nt, force_waves, false, force_rows, &p);
+  return err ? err : p.tiles;
+}
+
+// X bfloat16 [M, K]; W bfloat16 [N, K] (with epi 2: [2 N, K]).  epi: 0 store to C (c_dtype, bias optional),
+// 1 add into R (float32 [M, N], row stride ldc), 2 silu(gate) * up to C (bfloat16 [M, N]).
+// With gain (float32 [K]): X is float32 [M <= 16, K] and its RMS norm with this gain and eps is what
+// is multiplied (epi 0 and 2).  force_nt / force_waves: 0 = chosen here.
+// With next_gain (float32 [N], epi 1): the norm that follows is handed ahead: next_x (bfloat16 [M, N], row stride
+// ld_next) = the stream's new values * next_gain, next_sq (float32 [M, P], P = ullm_gemm_skinny_blocks(..) rounded
+// up to a multiple of 4) = every block's sum of squares of its columns of a row, zeros behind the last block's.
+// With row_sq (float32 [M, sq_parts], sq_parts a multiple of 4; epi 0 and 2, no gain): X is such a next_x and the
+// results of row m are scaled by rsqrt(sum of row_sq[m][.] / K + eps).
+extern "C" int ullm_gemm_skinny(const void* X, int ldx, const void* W, int ldw, const float* bias, void* C,
+                                int ldc, int M, int N, int K, int epi, int c_dtype, int force_nt,
+                                int force_waves, const float* gain, float eps, int force_rows,
+                                const float* next_gain, void* next_x, int ld_next, float* next_sq,
+                                const float* row_sq, int sq_parts, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (!ullm_gemm_skinny_supports(M, N, K, ldx, ldw) || ldc < N) return ULLM_ERR_SHAPE;
+  if (((uintptr_t)X & 15) || ((uintptr_t)W & 15)) return ULLM_ERR_SHAPE;
+  if (epi < 0 || epi > 2) return ULLM_ERR_UNSUPPORTED;
+  if (gain && (M > 16 || epi == EPI_RESADD || ((uintptr_t)gain & 15))) return ULLM_ERR_UNSUPPORTED;
+  if (epi == EPI_RESADD && (((uintptr_t)C & 15) || ldc % 4 != 0 || bias)) return ULLM_ERR_SHAPE;
+  if (epi == EPI_SILU && (bias || c_dtype != ULLM_BF16)) return ULLM_ERR_UNSUPPORTED;
+  if (next_gain && (epi != EPI_RESADD || !next_x || !next_sq || ld_next < N || ld_next % 4 != 0 ||
+                    ((uintptr_t)next_x & 7) || ((uintptr_t)next_gain & 15)))
+    return ULLM_ERR_UNSUPPORTED;
+  if (row_sq && (gain || M > 16 || epi == EPI_RESADD || sq_parts < 4 || sq_parts % 4 || ((uintptr_t)row_sq & 15))) return ULLM_ERR_UNSUPPORTED;
+  SkinnyPlan plan;
+  const int err = skinny_plan(M, N, K, ldx, ldw, epi, force_nt, force_waves, gain != nullptr, force_rows, &plan);
+  if (err) return err;
+  const int mt = plan.mt, nt = plan.nt, rows = plan.rows, tiles = plan.tiles, waves = plan.waves,
+            k_per_wave = plan.k_per_wave;
+  const NormAhead ahead{next_gain, (bf16_t*)next_x, next_sq, ld_next, (tiles + 3) / 4 * 4};
+  const RowSquares before{row_sq, sq_parts / 4};
   dim3 grid(tiles), block(64 * waves);
   float* R = (float*)C;
 #define GO_(MT, NT, EPI, TC, NORMX) skinny_launch<MT, NT, EPI, TC, NORMX>(grid, block, stream, X, ldx, \
-    (const bf16_t*)W, ldw, bias, gain, eps, (TC*)C, R, ldc, M, N, K, k_per_wave, rows)
+    (const bf16_t*)W, ldw, bias, gain, eps, (TC*)C, R, ldc, M, N, K, k_per_wave, rows, ahead, before)
 #define GO(MT, NT, EPI, TC) GO_(MT, NT, EPI, TC, false)
 #define GO_SHAPE(EPI, TC)                                              \
   switch (mt * 8 + nt) {                                               \

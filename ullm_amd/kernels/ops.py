@@ -303,20 +303,36 @@ def gemm_skinny_supports(a: torch.Tensor, w: torch.Tensor) -> bool:
     return a.dtype == torch.bfloat16 and _skinny_ok(a.shape[0], a.shape[1], a, w)
 
 
-def _gemm_skinny(x, w, bias, c, M, N, K, epi, c_dtype, nt=0, waves=0, gain=None, eps=0.0, rows=0) -> None:
+def _gemm_skinny(x, w, bias, c, M, N, K, epi, c_dtype, nt=0, waves=0, gain=None, eps=0.0, rows=0,
+                 ahead=None, squares=None) -> None:
+    """``ahead``: (next gain, next x, next squares) that an adding product leaves for the norm after it;
+    ``squares``: the [parts, M] sums such a product left, which scale this product's rows."""
     lib = build.load("gemm_skinny")
+    next_gain, next_x, next_sq = ahead if ahead is not None else (None, None, None)
     _check(lib.ullm_gemm_skinny(_p(x), _c_int(x.stride(0)), _p(w), _c_int(w.stride(0)), _p(bias),
                                 _p(c), _c_int(c.stride(0)), _c_int(M), _c_int(N), _c_int(K),
                                 _c_int(epi), _c_int(c_dtype), _c_int(nt), _c_int(waves), _p(gain),
-                                ctypes.c_float(eps), _c_int(rows), _stream()),
+                                ctypes.c_float(eps), _c_int(rows), _p(next_gain), _p(next_x),
+                                _c_int(next_x.stride(0) if next_x is not None else 0), _p(next_sq), _p(squares),
+                                _c_int(squares.shape[1] if squares is not None else 0), _stream()),
            "gemm_skinny")
+
+
+def _check_squares(squares: Optional[torch.Tensor], M: int) -> None:
+    if squares is not None:
+        _need(M <= 16 and squares.dtype == torch.float32 and squares.dim() == 2 and squares.shape[0] == M
+              and squares.shape[1] >= 4 and squares.shape[1] % 4 == 0 and squares.is_contiguous()
+              and squares.data_ptr() % 16 == 0, f"row squares must be float32 [{M} <= 16, a multiple of 4]")
 
 
 def gemm_skinny(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
                 out_dtype: Optional[torch.dtype] = None, out: Optional[torch.Tensor] = None,
-                nt: int = 0, waves: int = 0, rows: int = 0) -> torch.Tensor:
+                nt: int = 0, waves: int = 0, rows: int = 0, squares: Optional[torch.Tensor] = None,
+                eps: float = 0.0) -> torch.Tensor:
     """a [M <= 64, K] times w [N, K] transposed, bfloat16 operands streamed once through the matrix
-    cores, 32-bit accumulation; output bfloat16 or float32."""
+    cores, 32-bit accumulation; output bfloat16 or float32.  With ``squares`` (float32 [M <= 16, parts], see
+    :func:`gemm_skinny_add`) row m of the product is scaled by rsqrt(sum of squares[m] / K + eps) before
+    the bias: a is then a stream times a norm's gain and the result the product of the normed stream."""
     M, K = a.shape
     N, K2 = w.shape
     _need(K == K2, f"inner sizes differ: a is [{M}, {K}], w is [{N}, {K2}]")
@@ -326,31 +342,53 @@ def gemm_skinny(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] =
     _need(out.shape == (M, N) and out.stride(1) == 1, "bad gemm output")
     if bias is not None:
         _need(bias.dtype == torch.float32 and bias.numel() == N and bias.is_contiguous(), "bias must be float32 [N]")
-    _gemm_skinny(a, w, bias, out, M, N, K, 0, _dt(out), nt, waves, rows=rows)
+    _check_squares(squares, M)
+    _gemm_skinny(a, w, bias, out, M, N, K, 0, _dt(out), nt, waves, eps=float(eps), rows=rows, squares=squares)
     return out
 
 
 def gemm_skinny_add(a: torch.Tensor, w: torch.Tensor, residual: torch.Tensor, nt: int = 0, waves: int = 0,
-                    rows: int = 0) -> None:
-    """residual (float32 [M, N]) += a (bfloat16 [M, K]) times w transposed."""
+                    rows: int = 0, next_gain: Optional[torch.Tensor] = None):
+    """residual (float32 [M, N]) += a (bfloat16 [M, K]) times w transposed.
+    With ``next_gain`` (float32 [N], the gain of the RMS norm that is applied to the residual next) the kernel
+    also leaves what that norm needs and returns it: (scaled, squares) with scaled = residual * next_gain in
+    bfloat16 [M, N] and squares float32 [M, parts], every block's sum of the squares of its columns of a row
+    (zeros behind them up to a multiple of four).
+    The norm of row m is scaled[m] * rsqrt(squares[m].sum() / N + eps), which a product after it applies
+    to its own results (``squares=`` of :func:`gemm_skinny`, :func:`gemm_skinny_silu`, :func:`gemm_rows`)."""
     M = a.shape[0]
     N, K = w.shape
     _need(a.dtype == torch.bfloat16 and a.shape[1] == K and _skinny_ok(M, K, a, w),
           "gemm_skinny_add takes bfloat16 activations [M <= 64, K]")
     _need(residual.dtype == torch.float32 and residual.shape == (M, N) and residual.stride(1) == 1
           and residual.stride(0) % 4 == 0 and residual.data_ptr() % 16 == 0, "residual must be float32 [M, N]")
-    _gemm_skinny(a, w, None, residual, M, N, K, 1, F32, nt, waves, rows=rows)
+    if next_gain is None:
+        _gemm_skinny(a, w, None, residual, M, N, K, 1, F32, nt, waves, rows=rows)
+        return None
+    _need(next_gain.dtype == torch.float32 and next_gain.numel() == N and next_gain.is_contiguous()
+          and next_gain.data_ptr() % 16 == 0 and N % 4 == 0, "the next norm's gain must be float32 [N], N a multiple of 4")
+    blocks = int(build.load("gemm_skinny").ullm_gemm_skinny_blocks(
+        _c_int(M), _c_int(N), _c_int(K), _c_int(a.stride(0)), _c_int(w.stride(0)), _c_int(1), _c_int(nt), _c_int(waves),
+        _c_int(rows)))
+    _check(min(blocks, 0), "gemm_skinny_blocks")
+    scaled = torch.empty((M, N), dtype=torch.bfloat16, device=a.device)
+    squares = torch.empty((M, -(-blocks // 4) * 4), dtype=torch.float32, device=a.device)
+    _gemm_skinny(a, w, None, residual, M, N, K, 1, F32, nt, waves, rows=rows, ahead=(next_gain, scaled, squares))
+    return scaled, squares
 
 
-def gemm_skinny_silu(a: torch.Tensor, w_gate_up: torch.Tensor, nt: int = 0, waves: int = 0, rows: int = 0) -> torch.Tensor:
+def gemm_skinny_silu(a: torch.Tensor, w_gate_up: torch.Tensor, nt: int = 0, waves: int = 0, rows: int = 0,
+                     squares: Optional[torch.Tensor] = None, eps: float = 0.0) -> torch.Tensor:
     """silu(a g^T) * (a u^T) as bfloat16 [M, I] for a (bfloat16 [M, K]) and the stacked weights
-    g | u (bfloat16 [2 I, K]); the activation is applied to the 32-bit sums."""
+    g | u (bfloat16 [2 I, K]); the activation is applied to the 32-bit sums (with ``squares``: to the sums
+    scaled as in :func:`gemm_skinny`)."""
     M, K = a.shape
     two_i, K2 = w_gate_up.shape
     _need(K == K2 and two_i % 2 == 0, f"gate|up weights must be [2 I, {K}]")
     _need(a.dtype == torch.bfloat16 and _skinny_ok(M, K, a, w_gate_up), "gemm_skinny_silu takes bfloat16 [M <= 64, K]")
     out = torch.empty((M, two_i // 2), dtype=torch.bfloat16, device=a.device)
-    _gemm_skinny(a, w_gate_up, None, out, M, two_i // 2, K, 2, BF16, nt, waves, rows=rows)
+    _check_squares(squares, M)
+    _gemm_skinny(a, w_gate_up, None, out, M, two_i // 2, K, 2, BF16, nt, waves, eps=float(eps), rows=rows, squares=squares)
     return out
 
 
@@ -427,21 +465,26 @@ def gemm_rows_supports(a: torch.Tensor, w: torch.Tensor, silu: bool = False) -> 
                 _c_int(1 if silu else 0))))
 
 
-def gemm_rows(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, silu: bool = False) -> torch.Tensor:
+def gemm_rows(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, silu: bool = False,
+              squares: Optional[torch.Tensor] = None, eps: float = 0.0) -> torch.Tensor:
     """a (bfloat16 [M <= 64, K]) times w (bfloat16 [N, K]) transposed (+ bias float32 [N]) as bfloat16 [M, N];
     with ``silu``, w is gate | up [2 I, K] and the result silu(gate) * up [M, I] on the 32-bit sums.  The
     matrix is cut into one block per compute unit and every wave keeps several stages of its rows of w in
-    flight: for the row counts between the few-rows kernel and the library."""
+    flight: for the row counts between the few-rows kernel and the library.  ``squares``, ``eps``: as in
+    :func:`gemm_skinny`."""
     M, K = a.shape
     _need(gemm_rows_supports(a, w, silu), "gemm_rows takes bfloat16, M <= 64, K a multiple of 8, N a multiple of 4")
     n_out = w.shape[0] // 2 if silu else w.shape[0]
     if bias is not None:
         _need(not silu and bias.dtype == torch.float32 and bias.numel() == n_out and bias.is_contiguous(),
               "bias must be float32 [N] (and there is none with silu)")
+    _check_squares(squares, M)
     out = torch.empty((M, n_out), dtype=torch.bfloat16, device=a.device)
     _check(build.load("gemm_rows").ullm_gemm_rows(_p(a), _c_int(a.stride(0)), _p(w), _c_int(w.stride(0)), _p(bias), _p(out),
                                                   _c_int(n_out), _c_int(M), _c_int(n_out), _c_int(K),
-                                                  _c_int(1 if silu else 0), _stream()), "gemm_rows")
+                                                  _c_int(1 if silu else 0), _p(squares),
+                                                  _c_int(squares.shape[1] if squares is not None else 0),
+                                                  ctypes.c_float(float(eps)), _stream()), "gemm_rows")
     return out
 
 

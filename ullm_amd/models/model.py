@@ -145,7 +145,13 @@ class Model:
                 cache = LayerCache()
             elif self.cache_owner[cache_id] != idx:
                 cache = cache.reader()
-            residual, pending = self.blocks[layer].forward(residual, pending, ctx, cache)
+            block = self.blocks[layer]
+            if block.hands_norm_ahead and idx + 1 < len(self.run_order):
+                # a block whose last kernel can prepare the norm that follows is told which norm that is
+                after = self.blocks[self.run_order[idx + 1][0]].entry_norm()
+                residual, pending = block.forward(residual, pending, ctx, cache, next_norm=after)
+            else:
+                residual, pending = block.forward(residual, pending, ctx, cache)
         if logit_rows is None or logit_rows.numel() == 0:
             return None
         x = self.final_norm.add_norm(pending, residual, rows=logit_rows, out_dtype=ctx.dtype)

@@ -16,7 +16,7 @@ import torch
 from ..kernels import ops
 from .base import (KVNeed, LayerCache, Mixer, PartEnv, PositionEncoding, StepContext, StepPlan, StepShape, WeightDecl,
                    register_part)
-from .linear import can_fuse, linear, linear_into_stream, linear_of_norm
+from .linear import add_into_stream, can_fuse, linear, linear_into_stream, linear_of_norm
 
 
 # Up to this many single new tokens a step, the attention kernel norms, rotates and writes the new keys itself.
@@ -55,6 +55,7 @@ def plan_attention_step(shape: StepShape) -> StepPlan:
 @register_part("mixer", "gqa_attention")
 class GQAttention(Mixer):
     folds_norm = True
+    hands_norm_ahead = True
     step_planners = {"attention": plan_attention_step}
 
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, prefix: str,
@@ -111,9 +112,10 @@ class GQAttention(Mixer):
     def fusable(self, residual, ctx: StepContext) -> bool:
         return can_fuse(residual, ctx.dtype, self.w_qkv, self.w_o)
 
-    def forward_fused(self, x, residual, ctx: StepContext, cache: LayerCache) -> None:
+    def forward_fused(self, x, residual, ctx: StepContext, cache: LayerCache, then=None):
         qkv = linear_of_norm(x, self.w_qkv, self.b_qkv)                               # the norm before folded in
-        ops.gemm_skinny_add(self._attend(qkv, ctx, cache), self.w_o, residual)        # residual add folded behind
+        # the residual add, and the next norm's share of the work, folded behind
+        return add_into_stream(self._attend(qkv, ctx, cache), self.w_o, residual, then, ctx.dtype)
 
     def _attend(self, qkv: torch.Tensor, ctx: StepContext, cache: LayerCache) -> torch.Tensor:
         """Per-head norm, rotation, cache write and attention for a fused projection [T, (nq+2nkv)*hd];

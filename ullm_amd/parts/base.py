@@ -243,9 +243,13 @@ class Mixer(Part):
     A mixer may also offer ``forward_fused(x, residual, ctx, cache)``: add mixer(x) into the 32-bit
     residual in place, with the add folded into its last kernel.  It is called only when
     ``fusable(residual, ctx)`` says so.  With ``folds_norm`` its ``forward_fused`` also takes a
-    :class:`PendingNorm` for x: the norm before it, left to the mixer's first projection."""
+    :class:`PendingNorm` for x: the norm before it, left to the mixer's first projection.
+    With ``hands_norm_ahead`` its ``forward_fused`` also takes ``then=``, the norm that will be applied to the
+    stream next (or None), and may return that norm as a :class:`PendingNorm` that its last kernel prepared
+    (the stream times the gain, the rows' sums of squares); it returns None where it prepared nothing."""
     kind = "mixer"
     folds_norm = False
+    hands_norm_ahead = False
 
     def cache_need(self) -> CacheNeed:
         return None
@@ -262,9 +266,10 @@ class Mixer(Part):
 
 class FeedForward(Part):
     """``forward(x [T, hidden], ctx) -> [T, hidden]``; keeps nothing between steps.
-    ``fusable``, ``forward_fused(x, residual, ctx)`` and ``folds_norm`` as for mixers."""
+    ``fusable``, ``forward_fused(x, residual, ctx)``, ``folds_norm`` and ``hands_norm_ahead`` as for mixers."""
     kind = "ffn"
     folds_norm = False
+    hands_norm_ahead = False
 
     def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
         raise NotImplementedError
@@ -279,10 +284,15 @@ class FeedForward(Part):
 class PendingNorm:
     """A norm of the residual stream that has not been computed: what a consumer needs to fold it
     into its first projection (``stream`` float32 [T, hidden], ``gain`` float32 [hidden], ``eps``;
-    the scale is rsqrt(mean of squares + eps)), and ``apply()`` for a consumer that cannot after all."""
+    the scale is rsqrt(mean of squares + eps)), and ``apply()`` for a consumer that cannot after all.
+    Where the product that wrote the stream last prepared the norm, also ``scaled`` (stream * gain in the
+    compute dtype) and ``squares`` (float32 [T, parts]: a row's sum of squares in parts): the consumer then
+    multiplies ``scaled`` and scales row t of its results by rsqrt(squares[t].sum() / hidden + eps)."""
 
-    def __init__(self, norm: "Norm", stream: torch.Tensor, gain: torch.Tensor, eps: float, out_dtype: torch.dtype):
+    def __init__(self, norm: "Norm", stream: torch.Tensor, gain: torch.Tensor, eps: float, out_dtype: torch.dtype,
+                 scaled: Optional[torch.Tensor] = None, squares: Optional[torch.Tensor] = None):
         self.norm, self.stream, self.gain, self.eps, self.out_dtype = norm, stream, gain, eps, out_dtype
+        self.scaled, self.squares = scaled, squares
 
     def apply(self) -> torch.Tensor:
         return self.norm.add_norm(None, self.stream, out_dtype=self.out_dtype)
@@ -294,11 +304,17 @@ class Norm(Part):
     ``adds_stacks``: the branch may also be a stack [S, T, hidden] of float32 partial sums, which
     the norm adds in order.
     ``pending(residual, out_dtype)``: a :class:`PendingNorm` of a stream with nothing left to add, for
-    a consumer with ``folds_norm``, or None if this norm has no such form."""
+    a consumer with ``folds_norm``, or None if this norm has no such form; with ``scaled`` and ``squares``
+    where a product prepared them.  ``ahead_gain()``: the float32 gain [hidden] such a product multiplies
+    the stream by, or None if this norm is not a gain times rsqrt(mean of squares + eps)."""
     kind = "norm"
     adds_stacks = False
 
-    def pending(self, residual: torch.Tensor, out_dtype: torch.dtype) -> Optional["PendingNorm"]:
+    def pending(self, residual: torch.Tensor, out_dtype: torch.dtype, scaled: Optional[torch.Tensor] = None,
+                squares: Optional[torch.Tensor] = None) -> Optional["PendingNorm"]:
+        return None
+
+    def ahead_gain(self) -> Optional[torch.Tensor]:
         return None
 
     def add_norm(self, branch: Optional[torch.Tensor], residual: torch.Tensor,
@@ -320,8 +336,17 @@ class Block(Part):
     """Arrangement of norm, mixer and feed-forward around the residual stream.
 
     ``forward(residual, pending, ctx, cache) -> (residual, pending)`` where ``residual`` is the
-    32-bit stream [T, hidden] and ``pending`` a branch output not yet added to it."""
+    32-bit stream [T, hidden] and ``pending`` a branch output not yet added to it.
+
+    A block with ``hands_norm_ahead`` takes ``next_norm=`` in ``forward``: the norm that the next block of the
+    run order applies to the stream first (that block's ``entry_norm()``), or None.  It may then return a
+    :class:`PendingNorm` of that norm as its pending branch (nothing is left to add; the norm is half done),
+    which is only ever given to the block whose ``entry_norm()`` it is."""
     kind = "block"
+    hands_norm_ahead = False
+
+    def entry_norm(self) -> Optional["Norm"]:
+        return None
 
     def cache_need(self):
         """Nothing, one need (``KVNeed`` / ``StateNeed``) or a list of needs; with a list the block

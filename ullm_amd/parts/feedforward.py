@@ -10,12 +10,13 @@ import torch
 
 from ..kernels import ops
 from .base import FeedForward, PartEnv, StepContext, WeightDecl, register_part
-from .linear import can_fuse, gate_up, linear_into_stream, linear_of_norm
+from .linear import add_into_stream, can_fuse, gate_up, linear_into_stream, linear_of_norm
 
 
 @register_part("ffn", "swiglu")
 class SwiGLU(FeedForward):
     folds_norm = True
+    hands_norm_ahead = True
 
     def __init__(self, hidden_size: int, intermediate_size: int, prefix: str):
         self.hidden_size, self.intermediate_size, self.prefix = hidden_size, intermediate_size, prefix
@@ -40,6 +41,6 @@ class SwiGLU(FeedForward):
     def fusable(self, residual, ctx: StepContext) -> bool:
         return can_fuse(residual, ctx.dtype, self.w_gate_up, self.w_down)
 
-    def forward_fused(self, x, residual, ctx: StepContext) -> None:
+    def forward_fused(self, x, residual, ctx: StepContext, then=None):
         act = linear_of_norm(x, self.w_gate_up, silu=True)     # the norm before, silu(gate) * up behind the first product
-        ops.gemm_skinny_add(act, self.w_down, residual)        # residual add behind the second
+        return add_into_stream(act, self.w_down, residual, then, ctx.dtype)   # residual add (and the next norm's part) behind the second

@@ -26,6 +26,10 @@ def linear_of_norm(x, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
     kernel takes the shapes, and computed first where not.  With ``silu`` the weights are gate | up
     and the result silu(gate) * up."""
     from .base import PendingNorm
+    if isinstance(x, PendingNorm) and x.scaled is not None:
+        y = _linear_of_prepared_norm(x, weight, bias, silu)
+        if y is not None:
+            return y
     if isinstance(x, PendingNorm):
         # folding the norm into the product pays up to a row count that depends on the matrix: beyond, the 32-bit
         # rows of X cost every block more registers and loads than the saved launch is worth
@@ -37,6 +41,43 @@ def linear_of_norm(x, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
     if silu:
         return gate_up(x, weight)
     return linear(x, weight, bias)
+
+
+def _linear_of_prepared_norm(x, weight: torch.Tensor, bias: Optional[torch.Tensor], silu: bool) -> Optional[torch.Tensor]:
+    """The product of a norm that the product before prepared (``x.scaled`` = stream * gain, ``x.squares``): the
+    kernel the matrix's limits name for this row count multiplies ``x.scaled`` and scales its rows.  None where no
+    kernel takes the shapes."""
+    a, rows = x.scaled, x.scaled.shape[0]
+    if a.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 or rows > ops.NORMED_MAX_ROWS:
+        return None
+    lim = dispatch.limits(weight.shape[0], weight.shape[1])
+    few = ops.gemm_skinny_supports(a, weight)
+    if silu:
+        if few and rows <= lim.silu_skinny:
+            return ops.gemm_skinny_silu(a, weight, squares=x.squares, eps=x.eps)
+        if ops.gemm_rows_supports(a, weight, silu=True):
+            return ops.gemm_rows(a, weight, silu=True, squares=x.squares, eps=x.eps)
+        return ops.gemm_skinny_silu(a, weight, squares=x.squares, eps=x.eps) if few else None
+    if few and rows <= lim.skinny:
+        return ops.gemm_skinny(a, weight, bias, squares=x.squares, eps=x.eps)
+    if ops.gemm_rows_supports(a, weight):
+        return ops.gemm_rows(a, weight, bias, squares=x.squares, eps=x.eps)
+    return ops.gemm_skinny(a, weight, bias, squares=x.squares, eps=x.eps) if few else None
+
+
+def add_into_stream(x: torch.Tensor, weight: torch.Tensor, residual: torch.Tensor, then=None,
+                    out_dtype: Optional[torch.dtype] = None):
+    """residual += x W^T by the few-rows kernel (the caller has asked :func:`can_fuse`).  With ``then``, the norm
+    that is applied to the stream next, the same kernel also prepares that norm where it can (the stream times
+    the norm's gain, the rows' sums of squares) and the result is the norm's record for the part behind it;
+    otherwise None."""
+    gain = then.ahead_gain() if then is not None else None
+    if (gain is not None and residual.shape[0] <= ops.NORMED_MAX_ROWS and weight.shape[0] % 4 == 0
+            and gain.dtype == torch.float32 and gain.numel() == weight.shape[0] and gain.data_ptr() % 16 == 0):
+        scaled, squares = ops.gemm_skinny_add(x, weight, residual, next_gain=gain)
+        return then.pending(residual, out_dtype or x.dtype, scaled, squares)
+    ops.gemm_skinny_add(x, weight, residual)
+    return None
 
 
 def gate_up(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:

@@ -35,5 +35,8 @@ class RMSNorm(Norm):
             out_dtype = branch.dtype if branch is not None and branch.dim() == 2 else torch.float32
         return ops.add_rmsnorm(branch, residual, self.gain, self.eps, out_dtype, rows=rows)
 
-    def pending(self, residual, out_dtype):
-        return PendingNorm(self, residual, self.gain, self.eps, out_dtype)
+    def pending(self, residual, out_dtype, scaled=None, squares=None):
+        return PendingNorm(self, residual, self.gain, self.eps, out_dtype, scaled, squares)
+
+    def ahead_gain(self):
+        return self.gain
