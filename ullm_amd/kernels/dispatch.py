@@ -26,7 +26,8 @@ class Limits:
     # (0: never), then the library
     skinny: int = 16
     rows: int = 64
-    # the RMS norm before the product folded into the few-rows kernel up to this many rows
+    # the RMS norm before the product folded into the few-rows kernel up to this many rows (asked where the product
+    # before has not prepared the norm: a model's first layer, a part behind one that adds no result of its own)
     fold_norm: int = 8
     # silu(gate) * up on store: the few-rows kernel up to ``silu_skinny``, the rows kernel up to ``silu_rows``,
     # then the library product and the activation kernel
