@@ -198,10 +198,18 @@ __device__ __forceinline__ void skinny_finish(f32x4_t (&acc)[NT][MT], RedT& red,
 // groups on different banks.  No barrier in the loop: a wave only reads what it wrote.
 // (Loading the operands straight from memory in the matrix layout, 64 bytes of each of 16 rows per
 // instruction and of X as many rows as the batch has, was slower the more rows X had.)
+// The stages in flight are real: every load is issued without a condition, so the compiler waits for exactly the
+// stage it works on while the next is on its way (with loads under conditions it waited for all of them; the
+// output and down projections of few columns, one block a compute unit, then ran 0.8 to 2 us slower, gate|up
+// at 9 to 16 rows 6 us).  Three stages in flight cost a wave per SIMD and bring nothing.
 // NORMX: X is float32 and gain [K] float32, see above; else X is bfloat16.
 // XH: 8-row halves of a tile of X that are fetched: 1 for M <= 8 (then MT = 1), where the other half
 // stays zero in shared memory and costs neither loads nor the registers that hold them in flight
 // (with NORMX 75 against 116 registers, that is 6 against 4 waves per SIMD).
+#ifndef SK_DEPTH
+#define SK_DEPTH 2
+#endif
+
 template <int MT, int NT, int EPI, typename TC, bool NORMX, int XH>
 __global__ void __launch_bounds__(64 * sk_max_waves(MT, NT))
 gemm_skinny_kernel(const void* __restrict__ Xv, int ldx, const bf16_t* __restrict__ W, int ldw,
@@ -221,15 +229,19 @@ gemm_skinny_kernel(const void* __restrict__ Xv, int ldx, const bf16_t* __restric
   const int g = lane >> 4, r = lane & 15, lrow = lane >> 3, lcol = lane & 7;
   constexpr int OT = EPI == EPI_SILU ? NT / 2 : NT;
   // a block's columns of the result: rows_per_block <= 16 OT of them (the host picks the number that spreads
-  // the matrix evenly over the compute units); rows of W past them are neither fetched nor stored
+  // the matrix evenly over the compute units); rows of W past them are not stored
   const int n0 = blockIdx.x * rows_per_block;
   const int n_end = n0 + rows_per_block < N ? n0 + rows_per_block : N;
+  // No load stands under a condition (a load under one makes the compiler wait for every load in flight at
+  // the next use of any, which would undo the stages in flight).  Nothing needs one: a row of W past the block's
+  // columns reads the block's last row again and only feeds result columns that are never stored; a row of X past M
+  // reads row M - 1 and only feeds result rows that are never stored; a piece past the end of K reads the row's last
+  // piece again, and the piece of X is then replaced by zeros on its way into shared memory.
   const bf16_t* wsrc[NT][2];
-  bool wrow[NT][2];
   static_assert(XH == 2 || MT == 1, "half a tile of X only where it is the only tile");
   const XT* xsrc[MT][XH];
-  bool xrow[MT][XH];                                      // rows of X past M are zeros and cost no load
   int put[2], get[2];
+  const int last_piece = K / 8 - 1;
 #pragma unroll
   for (int h = 0; h < 2; ++h) {
     const int row = 8 * h + lrow;
@@ -238,15 +250,13 @@ gemm_skinny_kernel(const void* __restrict__ Xv, int ldx, const bf16_t* __restric
 #pragma unroll
     for (int i = 0; i < NT; ++i) {
       const int col = n0 + 16 * (i % OT) + row;
-      wrow[i][h] = col < n_end;
-      const int n = (wrow[i][h] ? col : n_end - 1) + (i / OT) * N;
-      wsrc[i][h] = W + (size_t)n * ldw + 8 * lcol;
+      const int n = (col < n_end ? col : n_end - 1) + (i / OT) * N;
+      wsrc[i][h] = W + (size_t)n * ldw;
     }
     if (h < XH) {
 #pragma unroll
       for (int t = 0; t < MT; ++t) {
-        xrow[t][h] = 16 * t + row < M;
-        xsrc[t][h] = X + (size_t)(xrow[t][h] ? 16 * t + row : M - 1) * ldx + 8 * lcol;
+        xsrc[t][h] = X + (size_t)(16 * t + row < M ? 16 * t + row : M - 1) * ldx;
       }
     }
   }
@@ -282,31 +292,28 @@ gemm_skinny_kernel(const void* __restrict__ Xv, int ldx, const bf16_t* __restric
   float ss[MT][XH];                                        // squares of rows 16 t + 8 h + lrow, this lane's pieces
 #pragma unroll
   for (int t = 0; t < MT; ++t) ss[t][0] = ss[t][XH - 1] = 0.f;
-  constexpr int DEPTH = 2;                                // stages of 64 values of K on their way (3 and 4 were slower)
+  constexpr int DEPTH = SK_DEPTH;                         // stages of 64 values of K on their way
   Stage st[DEPTH];
-  auto fetch = [&](Stage& st, int k0) {
-    const bool in = k0 + 8 * lcol < k_end;                        // K is a multiple of 8
+  auto fetch = [&](Stage& st, int k0) __attribute__((always_inline)) {
+    const int piece = k0 / 8 + lcol, at = 8 * (piece < last_piece ? piece : last_piece);
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
 #pragma unroll
-      for (int i = 0; i < NT; ++i)
-        st.w[i][h] = in && wrow[i][h] ? ld_stream16(wsrc[i][h] + k0) : make_uint4(0, 0, 0, 0);
+      for (int i = 0; i < NT; ++i) st.w[i][h] = ld_stream16(wsrc[i][h] + at);
       if (h < XH) {
 #pragma unroll
         for (int t = 0; t < MT; ++t)
 #pragma unroll
-          for (int v = 0; v < XV; ++v)
-            st.x[t][h][v] = in && xrow[t][h] ? *reinterpret_cast<const uint4*>(xsrc[t][h] + k0 + 4 * v)
-                                             : make_uint4(0, 0, 0, 0);
+          for (int v = 0; v < XV; ++v) st.x[t][h][v] = ld16(xsrc[t][h] + at + 4 * v);
       }
     }
     if (NORMX) {
 #pragma unroll
-      for (int v = 0; v < XV; ++v)
-        st.gm[v] = in ? *reinterpret_cast<const uint4*>(gain + k0 + 8 * lcol + 4 * v) : make_uint4(0, 0, 0, 0);
+      for (int v = 0; v < XV; ++v) st.gm[v] = ld16(gain + at + 4 * v);
     }
   };
-  auto work = [&](const Stage& st) {
+  auto work = [&](const Stage& st, int k0) __attribute__((always_inline)) {
+    const bool in = k0 + 8 * lcol < k_end;                        // K is a multiple of 8
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
 #pragma unroll
@@ -321,12 +328,13 @@ gemm_skinny_kernel(const void* __restrict__ Xv, int ldx, const bf16_t* __restric
           float q = ss[t][h];
           q = fmaf(a.x, a.x, q); q = fmaf(a.y, a.y, q); q = fmaf(a.z, a.z, q); q = fmaf(a.w, a.w, q);
           q = fmaf(b.x, b.x, q); q = fmaf(b.y, b.y, q); q = fmaf(b.z, b.z, q); q = fmaf(b.w, b.w, q);
-          ss[t][h] = q;
+          ss[t][h] = in ? q : ss[t][h];
           piece = make_uint4(pack2_bf16(a.x * ga.x, a.y * ga.y), pack2_bf16(a.z * ga.z, a.w * ga.w),
                              pack2_bf16(b.x * gb.x, b.y * gb.y), pack2_bf16(b.z * gb.z, b.w * gb.w));
         } else {
           piece = st.x[t][h][0];
         }
+        if (!in) piece = make_uint4(0, 0, 0, 0);                     // past the end of K: zeros, whatever was read
         *reinterpret_cast<uint4*>(mine + (NT + t) * TILE_BYTES + put[h]) = piece;
       }
     }
@@ -346,10 +354,8 @@ gemm_skinny_kernel(const void* __restrict__ Xv, int ldx, const bf16_t* __restric
     }
     __builtin_amdgcn_wave_barrier();       // and the reads before the next stage's writes
   };
-  if (k_begin < k_end) {
 #pragma unroll
-    for (int d = 0; d < DEPTH; ++d) fetch(st[d], k_begin + 64 * d);
-  }
+  for (int d = 0; d < DEPTH; ++d) fetch(st[d], k_begin + 64 * d);
   if (SQUARES && before.sq) {
     float q = 0.f;
 #pragma unroll
@@ -366,15 +372,22 @@ gemm_skinny_kernel(const void* __restrict__ Xv, int ldx, const bf16_t* __restric
     q += __shfl_xor(q, 32);
     if (lane < 16) sq[wave][lane] = lane < 64 / SQ_LANES ? q : 0.f;
   }
-  if (k_begin < k_end) {
-    for (int k = k_begin; k < k_end; k += 64 * DEPTH) {
+  // DEPTH stages in flight: registers st[d] hold the stages s = d (mod DEPTH).  Whole rounds whose fetches all lie
+  // in the wave's share run without a condition; the last rounds fetch only what the share still holds.
+  const int stages = k_begin < k_end ? (k_end - k_begin + 63) / 64 : 0;
+  int sn = 0;
+  for (; sn + 2 * DEPTH <= stages; sn += DEPTH) {
 #pragma unroll
-      for (int d = 0; d < DEPTH; ++d) {
-        if (k + 64 * d < k_end) {
-          work(st[d]);
-          fetch(st[d], k + 64 * (d + DEPTH));
-        }
-      }
+    for (int d = 0; d < DEPTH; ++d) {
+      work(st[d], k_begin + 64 * (sn + d));
+      fetch(st[d], k_begin + 64 * (sn + d + DEPTH));
+    }
+  }
+  for (; sn < stages; sn += DEPTH) {
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+      if (sn + d < stages) work(st[d], k_begin + 64 * (sn + d));
+      if (sn + d + DEPTH < stages) fetch(st[d], k_begin + 64 * (sn + d + DEPTH));
     }
   }
   if (NORMX) {
