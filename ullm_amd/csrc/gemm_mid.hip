@@ -5,6 +5,9 @@
 // rows of X: a stage of 64 values of K of all rows of X goes through shared memory once per block
 // (every thread fetches one 16-byte piece of it), the waves' own tiles of W through wave-private
 // shared memory, both in whole 128-byte lines, two stages ahead in registers, one barrier a stage.
+// No load stands under a condition, so the compiler waits for the stage it works on and not for the one
+// on its way: a row of W past N reads the last row and a row of X past M row M - 1 (never stored), a piece
+// past the end of K reads the row's last piece and the piece of X is replaced by zeros.
 // So a block reads X once per 128 rows of W.  The matrices this is for (the output and down
 // projections, 4096 to 8192 rows) then give 32 to 64 blocks, too few for the chip; K is therefore
 // cut into S slices, one per blockIdx.y, and every slice stores its own partial sum.  Who adds the
@@ -36,7 +39,7 @@ gemm_partial_sums_kernel(const bf16_t* __restrict__ X, int ldx, const bf16_t* __
                          float* __restrict__ P, int M, int N, int K, int k_per_slice) {
   constexpr int TILE = 16 * 128;                        // 16 rows x 64 values
   constexpr int XB = MT * TILE;                         // a stage of X
-  __shared__ __attribute__((aligned(16))) unsigned char xs[2 * XB];
+  __shared__ __attribute__((aligned(16))) unsigned char xs[2 * XB + 64 * 16];   // two stages, then a spare place per lane
   __shared__ __attribute__((aligned(16))) unsigned char ws[MID_WAVES * TILE];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int g = lane >> 4, r = lane & 15, lrow = lane >> 3, lcol = lane & 7;
@@ -52,20 +55,24 @@ gemm_partial_sums_kernel(const bf16_t* __restrict__ X, int ldx, const bf16_t* __
     const int row = 8 * h + lrow, n = n0 + row;
     put[h] = row * 128 + ((lcol ^ ((row >> 1) & 7)) << 4);
     get[h] = r * 128 + (((4 * h + g) ^ ((r >> 1) & 7)) << 4);       // h here: the step of 32 inside the stage
-    wsrc[h] = W + (size_t)(n < N ? n : N - 1) * ldw + 8 * lcol;     // rows past N repeat the last row; never stored
+    wsrc[h] = W + (size_t)(n < N ? n : N - 1) * ldw;                // rows past N repeat the last row; never stored
   }
   // X: piece p = tid + 512 q of the stage is row p / 8, piece p % 8
   constexpr int XPIECES = MT * 16 * 8;
   constexpr int XQ = (XPIECES + 64 * MID_WAVES - 1) / (64 * MID_WAVES);
+  // a thread whose piece lies past the stage reads piece 0 and stores to the spare place instead of skipping either
+  // (a store of a loaded value under a condition would again wait for every load in flight)
   const bf16_t* xsrc[XQ];
-  int xput[XQ];
-  bool xok[XQ];
+  int xput[XQ], xstep[XQ];
+  const int last_piece = K / 8 - 1, xcol = tid & 7;               // 64 MID_WAVES is a multiple of 8: the same for every q
 #pragma unroll
   for (int q = 0; q < XQ; ++q) {
-    const int p = tid + 64 * MID_WAVES * q, row = p >> 3, col = p & 7;
-    xok[q] = p < XPIECES;
-    xsrc[q] = X + (size_t)(row < M ? row : M - 1) * ldx + 8 * col;
-    xput[q] = (row >> 4) * TILE + (row & 15) * 128 + ((col ^ (((row & 15) >> 1) & 7)) << 4);
+    const int p = tid + 64 * MID_WAVES * q;
+    const bool ok = p < XPIECES;
+    const int row = ok ? p >> 3 : 0;
+    xsrc[q] = X + (size_t)(row < M ? row : M - 1) * ldx;
+    xput[q] = ok ? (row >> 4) * TILE + (row & 15) * 128 + ((xcol ^ (((row & 15) >> 1) & 7)) << 4) : 2 * XB + 16 * lane;
+    xstep[q] = ok ? XB : 0;
   }
   unsigned char* const mine = ws + wave * TILE;
   f32x4_t acc[MT];
@@ -73,46 +80,48 @@ gemm_partial_sums_kernel(const bf16_t* __restrict__ X, int ldx, const bf16_t* __
   for (int t = 0; t < MT; ++t) acc[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   struct Stage { uint4 w[2]; uint4 x[XQ]; };
   Stage st[2];
-  auto fetch = [&](Stage& s, int k0) {
-    const bool in = k0 + 8 * lcol < k_end;                          // K is a multiple of 8
+  auto fetch = [&](Stage& s, int k0) __attribute__((always_inline)) {
+    const int wp = k0 / 8 + lcol, xp = k0 / 8 + xcol;
+    const int wat = 8 * (wp < last_piece ? wp : last_piece), xat = 8 * (xp < last_piece ? xp : last_piece);
 #pragma unroll
-    for (int h = 0; h < 2; ++h) s.w[h] = in ? ld_stream16(wsrc[h] + k0) : make_uint4(0, 0, 0, 0);
+    for (int h = 0; h < 2; ++h) s.w[h] = ld_stream16(wsrc[h] + wat);
 #pragma unroll
-    for (int q = 0; q < XQ; ++q) {
-      const bool xin = xok[q] && k0 + 8 * ((tid + 64 * MID_WAVES * q) & 7) < k_end;
-      s.x[q] = xin ? *reinterpret_cast<const uint4*>(xsrc[q] + k0) : make_uint4(0, 0, 0, 0);
+    for (int q = 0; q < XQ; ++q) s.x[q] = ld16(xsrc[q] + xat);
+  };
+  // One stage: the registers that hold stage s go to shared memory (stage s to the X buffer that was last read two
+  // stages ago, before the previous barrier) and are refilled with stage s + 2 if the slice holds one; a barrier;
+  // the products.
+  auto stage = [&](Stage& sr, int s, bool more) __attribute__((always_inline)) {
+    const int k0 = k_begin + 64 * s;
+    unsigned char* xb = xs + (s & 1) * XB;
+    const bool xin = k0 + 8 * xcol < k_end;                         // K is a multiple of 8
+#pragma unroll
+    for (int q = 0; q < XQ; ++q) st16(xs + xput[q] + (s & 1) * xstep[q], xin ? sr.x[q] : make_uint4(0, 0, 0, 0));
+#pragma unroll
+    for (int h = 0; h < 2; ++h) st16(mine + put[h], sr.w[h]);
+    if (more) fetch(sr, k0 + 128);
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      Pack8 wf, xf[MT];
+      wf.u4 = *reinterpret_cast<const uint4*>(mine + get[j]);
+#pragma unroll
+      for (int t = 0; t < MT; ++t) xf[t].u4 = *reinterpret_cast<const uint4*>(xb + t * TILE + get[j]);
+#pragma unroll
+      for (int t = 0; t < MT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf.v, xf[t].v, acc[t], 0, 0, 0);
     }
   };
   const int stages = k_begin < k_end ? (k_end - k_begin + 63) / 64 : 0;   // the same for every wave of the block
-  if (stages > 0) {
-    fetch(st[0], k_begin);
-    fetch(st[1], k_begin + 64);
+  fetch(st[0], k_begin);
+  fetch(st[1], k_begin + 64);
+  int s0 = 0;
+  for (; s0 + 4 <= stages; s0 += 2) {                              // whole rounds whose fetches lie in the slice
+    stage(st[0], s0, true);
+    stage(st[1], s0 + 1, true);
   }
-  for (int s0 = 0; s0 < stages; s0 += 2) {
-#pragma unroll
-    for (int d = 0; d < 2; ++d) {
-      const int s = s0 + d;
-      if (s < stages) {
-        // stage s goes to the X buffer that was last read two stages ago, before the previous barrier
-        unsigned char* xb = xs + (s & 1) * XB;
-#pragma unroll
-        for (int q = 0; q < XQ; ++q)
-          if (xok[q]) *reinterpret_cast<uint4*>(xb + xput[q]) = st[d].x[q];
-#pragma unroll
-        for (int h = 0; h < 2; ++h) *reinterpret_cast<uint4*>(mine + put[h]) = st[d].w[h];
-        fetch(st[d], k_begin + 64 * (s + 2));
-        __syncthreads();
-#pragma unroll
-        for (int j = 0; j < 2; ++j) {
-          Pack8 wf, xf[MT];
-          wf.u4 = *reinterpret_cast<const uint4*>(mine + get[j]);
-#pragma unroll
-          for (int t = 0; t < MT; ++t) xf[t].u4 = *reinterpret_cast<const uint4*>(xb + t * TILE + get[j]);
-#pragma unroll
-          for (int t = 0; t < MT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf.v, xf[t].v, acc[t], 0, 0, 0);
-        }
-      }
-    }
+  for (; s0 < stages; s0 += 2) {
+    stage(st[0], s0, s0 + 2 < stages);
+    if (s0 + 1 < stages) stage(st[1], s0 + 1, s0 + 3 < stages);
   }
   // acc[t][j] = P[slice][m = 16 t + r][n0 + 4 g + j]
   float* out = P + (size_t)blockIdx.y * M * N;
