@@ -257,15 +257,36 @@ __global__ void add_rmsnorm_vec_kernel(const TB* __restrict__ branch, float* __r
   const int i = rows ? rows[r] : r;
   float* res = residual + (size_t)i * H;
   const TB* br = branch ? branch + (size_t)i * H : nullptr;
-  float4 v[NORM_VEC_MAX];
+  float4 v[NORM_VEC_MAX], gn[NORM_VEC_MAX];
   float ss = 0.f;
 #pragma unroll
   for (int j = 0; j < NORM_VEC_MAX; ++j) {
     const int c = 4 * (threadIdx.x + j * blockDim.x);
     if (c < H) {
       float4 s = ld4_f32(res + c);
+      gn[j] = ld4_f32(gain + c);                     // on its way during the reduction
       if (br) {
-        for (int p = 0; p < n_branch; ++p) {
+        // a stack is added in order, eight of its arrays fetched at a time (a load per turn of the loop would
+        // wait for each before the next goes out)
+        // a stack is added in order, eight (then four) of its arrays fetched at a time: a load per turn of
+        // the loop would wait for each before the next goes out
+        int p = 0;
+        for (; p + 8 <= n_branch; p += 8) {
+          float4 b[8];
+#pragma unroll
+          for (int u = 0; u < 8; ++u) b[u] = ld4_f32_stream(br + (size_t)(p + u) * branch_stride + c);
+#pragma unroll
+          for (int u = 0; u < 8; ++u) { s.x += b[u].x; s.y += b[u].y; s.z += b[u].z; s.w += b[u].w; }
+        }
+        if (p + 4 <= n_branch) {
+          float4 b[4];
+#pragma unroll
+          for (int u = 0; u < 4; ++u) b[u] = ld4_f32_stream(br + (size_t)(p + u) * branch_stride + c);
+#pragma unroll
+          for (int u = 0; u < 4; ++u) { s.x += b[u].x; s.y += b[u].y; s.z += b[u].z; s.w += b[u].w; }
+          p += 4;
+        }
+        for (; p < n_branch; ++p) {
           const float4 b = ld4_f32_stream(br + (size_t)p * branch_stride + c);
           s.x += b.x; s.y += b.y; s.z += b.z; s.w += b.w;
         }
@@ -281,7 +302,7 @@ __global__ void add_rmsnorm_vec_kernel(const TB* __restrict__ branch, float* __r
   for (int j = 0; j < NORM_VEC_MAX; ++j) {
     const int c = 4 * (threadIdx.x + j * blockDim.x);
     if (c < H) {
-      const float4 g = ld4_f32(gain + c);
+      const float4 g = gn[j];
       st4_f32(out + c, make_float4((v[j].x * rs) * g.x, (v[j].y * rs) * g.y, (v[j].z * rs) * g.z, (v[j].w * rs) * g.w));
     }
   }
