@@ -581,28 +581,38 @@ attention_reduce_kernel(const float* __restrict__ part, bf16_t* __restrict__ out
   const int t = token_list ? token_list[item] : item;
   const int row = hd + 4;
   const float* pp = part + ((size_t)item * nq + head) * num_splits * row;
+  // Eight splits at a time: their loads are all queued before the first is used, and those of the first eight go
+  // out before anything else (no load under a condition: an index past the end reads the last element), so that
+  // the splits' maxima and their values come back in one round trip instead of two.
+  float v[8][4];
+  int dim[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) dim[r] = lane + 64 * r < hd ? lane + 64 * r : hd - 1;
+  auto fetch = [&](int s0, int j0, int n) __attribute__((always_inline)) {
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const float* pj = pp + (size_t)(s0 + (j0 + u < n ? j0 + u : n - 1)) * row;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) v[u][r] = pj[dim[r]];
+    }
+  };
+  fetch(0, 0, num_splits < 64 ? num_splits : 64);
   float M = NEG_BIG;
   for (int s0 = 0; s0 < num_splits; s0 += 64) {
     const int sp = s0 + lane;
-    M = fmaxf(M, wave_max(sp < num_splits ? pp[sp * row + hd] : NEG_BIG));
+    M = fmaxf(M, wave_max(pp[(sp < num_splits ? sp : num_splits - 1) * row + hd]));
   }
   float acc[4] = {0.f, 0.f, 0.f, 0.f};       // head_dim <= 256: dims lane, lane + 64, ...
   float L = 0.f;
   for (int s0 = 0; s0 < num_splits; s0 += 64) {
     const int sp = s0 + lane;
     const bool ok = sp < num_splits;
-    const float f = ok ? fast_exp2(pp[sp * row + hd] - M) : 0.f;
-    L += wave_sum(ok ? pp[sp * row + hd + 1] * f : 0.f);
+    const float* mine = pp + (ok ? sp : num_splits - 1) * row + hd;
+    const float f = ok ? fast_exp2(mine[0] - M) : 0.f;
+    L += wave_sum(ok ? mine[1] * f : 0.f);
     const int n = num_splits - s0 < 64 ? num_splits - s0 : 64;
-    // eight splits at a time: their loads are all queued before the first is used
     for (int j0 = 0; j0 < n; j0 += 8) {
-      float v[8][4];
-#pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        const float* pj = pp + (size_t)(s0 + (j0 + u < n ? j0 + u : n - 1)) * row;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) v[u][r] = lane + 64 * r < hd ? pj[lane + 64 * r] : 0.f;
-      }
+      if (s0 + j0 > 0) fetch(s0, j0, n);
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
         const float fj = j0 + u < n ? __shfl(f, j0 + u, 64) : 0.f;
