@@ -452,6 +452,45 @@ def test_trace_run_program(trace_run, model_dirs, plain_models):
         close(c, want[31:], dtype)
 
 
+@pytest.mark.parametrize("name", ["B", "C", "D"])
+def test_steps_of_few_tokens_hand_the_norms_from_product_to_product(model_dirs, plain_models, name, monkeypatch):
+    """In a bfloat16 step of up to 16 tokens every product that ends in the stream prepares the norm behind it, so
+    between the first layer's norm and the last one no norm kernel runs and no product takes 32-bit rows to fold a
+    norm in; with the hand-over switched off the same step folds or runs a norm per part and gives the same logits
+    up to rounding.  Both against the plain model."""
+    from ullm_amd.kernels import ops
+    from ullm_amd.parts.attention import GQAttention
+    from ullm_amd.parts.feedforward import SwiGLU
+    from ullm_amd.replay import Replayer
+    cfg = plain_models[name][0]
+    layers, vocab = cfg["num_hidden_layers"], cfg["vocab_size"]
+    toks = make_tokens(vocab, 40, 77)
+    want = oracle(plain_models, name, toks)
+    calls, inner, inner_folded = [], ops.add_rmsnorm, ops.gemm_skinny_normed
+    monkeypatch.setattr(ops, "add_rmsnorm", lambda *a, **k: calls.append(1) or inner(*a, **k))
+    monkeypatch.setattr(ops, "gemm_skinny_normed", lambda *a, **k: calls.append(1) or inner_folded(*a, **k))
+    results = {}
+    for ahead in (True, False):
+        monkeypatch.setattr(GQAttention, "hands_norm_ahead", ahead)
+        monkeypatch.setattr(SwiGLU, "hands_norm_ahead", ahead)
+        rep = Replayer(model_dirs[name], "bfloat16", 256, 16, DEV, use_graphs=False)
+        rows = [rep.step({"step": 0, "entries": [{"id": "r", "tokens": toks[:24], "want": list(range(24))}], "end": []})]
+        counts = []
+        for i, n in enumerate((1, 7, 8)):                  # 24 + 1 + 7 + 8 = 40 tokens
+            at = 24 + sum((1, 7, 8)[:i])
+            calls.clear()
+            rows.append(rep.step({"step": 1 + i, "entries": [{"id": "r", "tokens": toks[at:at + n], "want": list(range(n))}],
+                                  "end": ["r"] if at + n == 40 else []}))
+            counts.append(len(calls))
+        results[ahead] = np.concatenate(rows)
+        close(results[ahead], want, "bfloat16")
+        if ahead:
+            assert all(c == 2 for c in counts), counts      # the first layer's norm and the last
+        else:
+            assert all(c == 2 * layers + 1 for c in counts), counts
+    close(results[True], results[False], "bfloat16")
+
+
 @pytest.mark.parametrize("name,dtype", [("B", "float32"), ("B", "bfloat16"), ("C", "bfloat16")])
 def test_graph_replays_equal_eager_steps(model_dirs, plain_models, name, dtype):
     """Decode steps replayed from HIP graphs: every replay is checked against the same step run
