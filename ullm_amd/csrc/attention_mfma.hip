@@ -18,6 +18,7 @@
 // Semantics as in the general kernel: causal with the queries at the end of the keys, optional
 // window, query head h reads kv head h / (nq / nkv) (ullm/layers/attention.py:76-104,271,298-309).
 #include "common.h"
+#include <type_traits>
 #include "no_alloc.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
@@ -100,14 +101,16 @@ __device__ __forceinline__ void load_tile(KVTile<NQK>& t, int key0, const PageWi
 // `own` (or null): the key (head_dim values) and value (head_dim values) of the token itself, at
 // position max_hi, in shared memory.  The tile that holds that position takes them from there instead
 // of from the cache, where the same kernel is only just writing them.
-template <int NQK, int NG, bool OWN>
+// INNER: every key of the tile is written data that every column may see (no key before a window's start, none
+// past the newest): no test per score, no zeroing of values, and the token's own key is not in it.
+template <int NQK, int NG, bool OWN, bool INNER>
 __device__ __forceinline__ void process_tile(const KVTile<NQK>& cur, int key0, const Pack8 (&qreg)[NG][NQK],
                                              const int (&col_lo)[NG], const int (&col_hi)[NG], int max_hi,
                                              float scale_log2e, f32x4_t (&acc)[NG][2 * NQK], float (&m)[NG],
                                              float (&l)[NG], const bf16_t* own) {
   constexpr int HD = 32 * NQK;
   const int lane = threadIdx.x & 63, g = lane >> 4;
-  const bool edge = key0 + 32 > max_hi + 1;     // some keys of the tile hold no written data
+  const bool edge = !INNER && key0 + 32 > max_hi + 1;     // some keys of the tile hold no written data
   Pack8 vals[2 * NQK], keys[2][NQK];
 #pragma unroll
   for (int n = 0; n < 2 * NQK; ++n) {
@@ -120,14 +123,14 @@ __device__ __forceinline__ void process_tile(const KVTile<NQK>& cur, int key0, c
     }
   }
   const Pack8 (*kp)[NQK] = cur.k;
-  if constexpr (OWN) {
+  if constexpr (OWN && !INNER) {
 #pragma unroll
     for (int sb = 0; sb < 2; ++sb)
 #pragma unroll
       for (int ch = 0; ch < NQK; ++ch) keys[sb][ch] = cur.k[sb][ch];
     kp = keys;
   }
-  if (OWN && own && key0 + 32 > max_hi) {
+  if (OWN && !INNER && own && key0 + 32 > max_hi) {
     const int c = lane & 15;
     const int at = max_hi - key0;               // 0 .. 31: sub-block at >> 4, row at & 15, which lane group at >> 2 & 3 holds
     if (c == (at & 15)) {
@@ -165,13 +168,12 @@ __device__ __forceinline__ void process_tile(const KVTile<NQK>& cur, int key0, c
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int kk = key0 + 16 * sb + 4 * g + r;
-        const bool ok = cur.ok[sb] && kk >= col_lo[q] && kk <= col_hi[q];
+        const bool ok = INNER || (cur.ok[sb] && kk >= col_lo[q] && kk <= col_hi[q]);
         const float v = ok ? s[sb][r] * scale_log2e : NEG_BIG;
         s[sb][r] = v;
         tile_max = fmaxf(tile_max, v);
       }
-    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, 64));
-    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, 64));
+    tile_max = max_with_lane_xor32(max_with_lane_xor16(tile_max));     // over the four lanes of the column
     const float m_new = fmaxf(m[q], tile_max);
     const float alpha = fast_exp2(m[q] - m_new);
     Pack8 p;
@@ -182,7 +184,7 @@ __device__ __forceinline__ void process_tile(const KVTile<NQK>& cur, int key0, c
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         // a masked score stays at NEG_BIG: its weight is zero even while m_new is still NEG_BIG
-        e[r] = s[sb][r] > 0.5f * NEG_BIG ? fast_exp2(s[sb][r] - m_new) : 0.f;
+        e[r] = INNER || s[sb][r] > 0.5f * NEG_BIG ? fast_exp2(s[sb][r] - m_new) : 0.f;
         psum += e[r];
       }
       p.w[2 * sb] = pack2_bf16(e[0], e[1]);
@@ -209,13 +211,16 @@ __device__ __forceinline__ void process_tile(const KVTile<NQK>& cur, int key0, c
 //   max_hi     : largest key position that holds written data for this request
 // Results per group: acc[q][n][r] = O^T[16n + 4g + r][col] (unnormalised), m (log2 domain), l (this
 // lane's share of the sum; the four lanes of a column add up to the column's sum).
-// Page ids are fetched 1024 keys at a time; the loads of the next DEPTH (1 or 2) tiles are in flight
-// while the current one is worked on.
-template <int NQK, int NG, int DEPTH, bool OWN, class Queries>
+// Page ids are fetched 1024 keys at a time; the loads of the next tile are in flight while the current one
+// is worked on (two tiles ahead, in three sets of registers, was slower at every batch size and context: the
+// third set costs moves between the two halves of the register file, and a wave's products are the longer
+// part of a tile's time).
+template <int NQK, int NG, bool OWN, class Queries>
 __device__ __forceinline__ void attend_range(
     Queries& queries, const int (&col_lo)[NG], const int (&col_hi)[NG], int key_begin, int key_end,
-    int max_hi, const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool, const int* __restrict__ bt,
-    int page_size, int nkv, int kvh, float scale_log2e, f32x4_t (&acc)[NG][2 * NQK], float (&m)[NG], float (&l)[NG]) {
+    int max_hi, int all_lo, const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
+    const int* __restrict__ bt, int page_size, int nkv, int kvh, float scale_log2e, f32x4_t (&acc)[NG][2 * NQK],
+    float (&m)[NG], float (&l)[NG]) {
 #pragma unroll
   for (int q = 0; q < NG; ++q) {
 #pragma unroll
@@ -229,40 +234,33 @@ __device__ __forceinline__ void attend_range(
   Pack8 qreg[NG][NQK];
   const bf16_t* own = nullptr;
 #define TILE_LOAD(T, K0) load_tile<NQK>(T, K0, pw, k_pool, v_pool, page_size, nkv, kvh)
-#define TILE_WORK(T, K0) process_tile<NQK, NG, OWN>(T, K0, qreg, col_lo, col_hi, max_hi, scale_log2e, acc, m, l, own)
-  KVTile<NQK> t0, t1, t2;                                 // DEPTH 1 takes two of them in turns, DEPTH 2 all three
+  // a tile all of whose keys every column of the wave sees (all_lo: the columns' common first key, or a value no
+  // tile reaches where they have none in common) takes the variant without tests; with OWN not the tile of the
+  // newest key, which comes from shared memory
+#define TILE_WORK(T, K0)                                                                                          \
+  do {                                                                                                            \
+    if ((K0) >= all_lo && (K0) + 31 < max_hi + (OWN ? 0 : 1) && T.ok[0] && T.ok[1])                               \
+      process_tile<NQK, NG, OWN, true>(T, K0, qreg, col_lo, col_hi, max_hi, scale_log2e, acc, m, l, own);         \
+    else                                                                                                          \
+      process_tile<NQK, NG, OWN, false>(T, K0, qreg, col_lo, col_hi, max_hi, scale_log2e, acc, m, l, own);        \
+  } while (0)
+  KVTile<NQK> t0, t1;                                     // in turns: one is worked on while the other loads
   int base = key_begin, stop = base + 1024 < key_end ? base + 1024 : key_end;
   TILE_LOAD(t0, base);
-  if (DEPTH == 2 && base + 32 < stop) TILE_LOAD(t1, base + 32);
   own = queries.finish(qreg);
   for (;;) {
-    if (DEPTH == 1) {
-      for (int key0 = base; key0 < stop; key0 += 64) {
-        if (key0 + 32 < stop) TILE_LOAD(t1, key0 + 32);
-        TILE_WORK(t0, key0);
-        if (key0 + 32 >= stop) break;
-        if (key0 + 64 < stop) TILE_LOAD(t0, key0 + 64);
-        TILE_WORK(t1, key0 + 32);
-      }
-    } else {
-      // three buffers in rotation: while tile i is worked on, tiles i+1 and i+2 are loading
-      for (int key0 = base; key0 < stop; key0 += 96) {
-        if (key0 + 64 < stop) TILE_LOAD(t2, key0 + 64);
-        TILE_WORK(t0, key0);
-        if (key0 + 32 >= stop) break;
-        if (key0 + 96 < stop) TILE_LOAD(t0, key0 + 96);
-        TILE_WORK(t1, key0 + 32);
-        if (key0 + 64 >= stop) break;
-        if (key0 + 128 < stop) TILE_LOAD(t1, key0 + 128);
-        TILE_WORK(t2, key0 + 64);
-      }
+    for (int key0 = base; key0 < stop; key0 += 64) {
+      if (key0 + 32 < stop) TILE_LOAD(t1, key0 + 32);
+      TILE_WORK(t0, key0);
+      if (key0 + 32 >= stop) break;
+      if (key0 + 64 < stop) TILE_LOAD(t0, key0 + 64);
+      TILE_WORK(t1, key0 + 32);
     }
     base += 1024;
     if (base >= key_end) break;
     pw = load_pages(base, key_end, bt, page_size);        // the next 1024 keys' page ids
     stop = base + 1024 < key_end ? base + 1024 : key_end;
     TILE_LOAD(t0, base);
-    if (DEPTH == 2 && base + 32 < stop) TILE_LOAD(t1, base + 32);
   }
 #undef TILE_LOAD
 #undef TILE_WORK
@@ -342,13 +340,14 @@ struct ReadyQueries {
   const bf16_t* row;                    // the column's head, or null for a padding column
   int g;
   Pack8 raw[NQK];
-  __device__ __forceinline__ void fetch() {
+  __device__ __forceinline__ void fetch_early() {       // needs the token alone, not its position
 #pragma unroll
     for (int ch = 0; ch < NQK; ++ch) {
       if (row) raw[ch].u4 = *reinterpret_cast<const uint4*>(row + 32 * ch + 8 * g);
       else raw[ch].u4 = make_uint4(0, 0, 0, 0);
     }
   }
+  __device__ __forceinline__ void fetch() {}
   __device__ __forceinline__ const bf16_t* finish(Pack8 (&qreg)[1][NQK]) {
 #pragma unroll
     for (int ch = 0; ch < NQK; ++ch) qreg[0][ch] = raw[ch];
@@ -377,9 +376,22 @@ struct RawQueries {
     const float4 a = *reinterpret_cast<const float4*>(from), b = *reinterpret_cast<const float4*>(from + 4);
     to[0] = a.x; to[1] = a.y; to[2] = a.z; to[3] = a.w; to[4] = b.x; to[5] = b.y; to[6] = b.z; to[7] = b.w;
   }
-  __device__ __forceinline__ void fetch() {
+  // What needs neither the token's position nor its pages goes out first, while those are still on their way:
+  // the query head's row of the projection and the norms' gains.
+  __device__ __forceinline__ void fetch_early() {
 #pragma unroll
     for (int ch = 0; ch < NQK; ++ch) q_raw[ch].u4 = ld16(q_head + 32 * ch + 8 * g);
+    if (fuse.q_gain) {
+#pragma unroll
+      for (int ch = 0; ch < NQK; ++ch) load8(q_gain[ch], fuse.q_gain + 32 * ch + 8 * g);
+    }
+    if (fuse.k_gain) {
+#pragma unroll
+      for (int ch = 0; ch < NQK; ++ch) load8(k_gain[ch], fuse.k_gain + 32 * ch + 8 * g);
+    }
+  }
+  // The rest, once the position is known: the table's row, and the token's key and value where this wave has them.
+  __device__ __forceinline__ void fetch() {
     if (k_head) {
 #pragma unroll
       for (int ch = 0; ch < NQK; ++ch) k_raw[ch].u4 = ld16(k_head + 32 * ch + 8 * g);
@@ -392,14 +404,6 @@ struct RawQueries {
         load8(cos_[ch], cs + 32 * ch + 8 * g);
         load8(sin_[ch], cs + HD / 2 + 32 * ch + 8 * g);
       }
-    }
-    if (fuse.q_gain) {
-#pragma unroll
-      for (int ch = 0; ch < NQK; ++ch) load8(q_gain[ch], fuse.q_gain + 32 * ch + 8 * g);
-    }
-    if (fuse.k_gain && k_head) {
-#pragma unroll
-      for (int ch = 0; ch < NQK; ++ch) load8(k_gain[ch], fuse.k_gain + 32 * ch + 8 * g);
     }
   }
   // Per-head norm and half-split rotation of a head held by the four lanes of a column: chunk ch,
@@ -504,6 +508,20 @@ attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __re
   const int kvh = blockIdx.y / groups, cg = blockIdx.y % groups;
   const int item = blockIdx.z;
   const int t = token_list ? token_list[item] : item;
+  const int head_in_group = cg * 16 + c;
+  const bool col_ok = head_in_group < G;
+  const int head = kvh * G + head_in_group;
+  const bf16_t* const row = q + (size_t)t * q_stride;
+  // the queries' loads that need the token alone go out before its position is asked for
+  using Queries = typename std::conditional<FUSE, RawQueries<NQK>, ReadyQueries<NQK>>::type;
+  Queries queries = [&]() {
+    if constexpr (FUSE)       // a padding column takes the group's first head: never stored
+      return RawQueries<NQK>{fuse, row + (size_t)(col_ok ? head : kvh * G) * HD, nullptr, nullptr, nullptr, nullptr, nullptr,
+                             page_size, g, c, own_kv};
+    else
+      return ReadyQueries<NQK>{col_ok ? row + (size_t)head * HD : nullptr, g};
+  }();
+  queries.fetch_early();
   const int pos = positions[t];
   const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
   const int first = lo & ~31;
@@ -511,37 +529,28 @@ attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __re
   const int share = 32 * ((tiles + num_splits * WAVES - 1) / (num_splits * WAVES));
   int begin = first + (split * WAVES + wave) * share, end = begin + share;
   if (end > pos + 1) end = pos + 1;
-  const int head_in_group = cg * 16 + c;
-  const bool col_ok = head_in_group < G;
-  const int head = kvh * G + head_in_group;
   f32x4_t accs[1][2 * NQK];
   float ms[1], ls[1];
   {
     const int* const bt = block_table + (size_t)token_entry[t] * bt_stride;
-    const bf16_t* const row = q + (size_t)t * q_stride;
     const int clo[1] = {lo}, chi[1] = {col_ok ? pos : -1};
-    constexpr int DEPTH = WAVES > 4 || NQK >= 8 ? 1 : 2;
     if constexpr (FUSE) {
       const bool has_own = fuse.k_pool && begin < end && end == pos + 1;
       // no page (a padding entry), no write, as in the kernel for prompt portions; one block per kv head writes
       const int page = has_own && cg == 0 ? bt[pos / page_size] : -1;
       const int off = pos % page_size;
-      RawQueries<NQK> queries{
-          fuse,
-          row + (size_t)(col_ok ? head : kvh * G) * HD,      // a padding column takes the group's first head: never stored
-          has_own ? row + (size_t)(nq + kvh) * HD : nullptr,
-          has_own ? row + (size_t)(nq + nkv + kvh) * HD : nullptr,
-          fuse.cos_sin ? fuse.cos_sin + (size_t)(pos < fuse.table_rows ? pos : fuse.table_rows - 1) * HD : nullptr,
-          page >= 0 ? fuse.k_pool + (((size_t)page * nkv + kvh) * page_size + off) * HD : nullptr,
-          page >= 0 ? fuse.v_pool + ((size_t)page * nkv + kvh) * HD * page_size + off : nullptr,
-          page_size, g, c, own_kv};
-      attend_range<NQK, 1, DEPTH, true>(queries, clo, chi, begin, end, pos, k_pool, v_pool, bt, page_size, nkv, kvh,
-                                        scale_log2e, accs, ms, ls);
-    } else {
-      ReadyQueries<NQK> queries{col_ok ? row + (size_t)head * HD : nullptr, g};
-      attend_range<NQK, 1, DEPTH, false>(queries, clo, chi, begin, end, pos, k_pool, v_pool, bt, page_size, nkv, kvh,
-                                         scale_log2e, accs, ms, ls);
+      if (has_own) {
+        queries.k_head = row + (size_t)(nq + kvh) * HD;
+        queries.v_head = row + (size_t)(nq + nkv + kvh) * HD;
+      }
+      if (fuse.cos_sin) queries.cs = fuse.cos_sin + (size_t)(pos < fuse.table_rows ? pos : fuse.table_rows - 1) * HD;
+      if (page >= 0) {
+        queries.k_dst = fuse.k_pool + (((size_t)page * nkv + kvh) * page_size + off) * HD;
+        queries.v_dst = fuse.v_pool + ((size_t)page * nkv + kvh) * HD * page_size + off;
+      }
     }
+    attend_range<NQK, 1, FUSE>(queries, clo, chi, begin, end, pos, lo, k_pool, v_pool, bt, page_size, nkv, kvh,
+                               scale_log2e, accs, ms, ls);
   }
   merge_waves<NQK, 1, WAVES>(accs, ms, ls, merge);
   f32x4_t (&acc)[2 * NQK] = accs[0];

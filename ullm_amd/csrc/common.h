@@ -66,6 +66,28 @@ __device__ __forceinline__ uint2 ld_stream8(const void* p) {
   return make_uint2(v.x, v.y);
 }
 
+// max(v, v of the lane 16 (32) further on or back): the two values change places between rows of 16 (32) lanes
+// inside the vector unit (v_permlane16_swap / v_permlane32_swap), without a trip through the LDS crossbar that
+// a general lane permutation takes.
+__device__ __forceinline__ float max_with_lane_xor16(float v) {
+#ifdef __HIP_DEVICE_COMPILE__
+  const unsigned u = __float_as_uint(v);
+  const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+#else
+  return v;
+#endif
+}
+__device__ __forceinline__ float max_with_lane_xor32(float v) {
+#ifdef __HIP_DEVICE_COMPILE__
+  const unsigned u = __float_as_uint(v);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+#else
+  return v;
+#endif
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int m = WAVE / 2; m > 0; m >>= 1) v += __shfl_xor(v, m, WAVE);
