@@ -44,29 +44,31 @@ __device__ __forceinline__ float uniform_from_seed(uint64_t seed, uint32_t posit
 // Visits the elements [wbeg, wend) of a wave's range, lane-strided, with several independent loads
 // in flight per lane.  VEC: 16-byte loads (the row must be 16-byte aligned and wbeg, wend multiples
 // of 4): a lane gets 4 consecutive values, the wave 256 consecutive values per access.
-template <bool VEC, typename F>
+// U: loads a lane has in flight.  The passes that every sampled row takes (maximum, sum) run with 8: a wave's
+// share of 150 K values is then five round trips to memory instead of ten.
+template <bool VEC, int U = 4, typename F>
 __device__ __forceinline__ void for_range(const float* __restrict__ x, int wbeg, int wend, int lane, F f) {
   if (VEC) {
-    for (int i0 = wbeg + 4 * lane; i0 < wend; i0 += 4 * 4 * WAVE) {
-      float4 v[4];
+    for (int i0 = wbeg + 4 * lane; i0 < wend; i0 += U * 4 * WAVE) {
+      float4 v[U];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
+      for (int u = 0; u < U; ++u) {
         const int ii = i0 + u * 4 * WAVE;
         v[u] = ii < wend ? *reinterpret_cast<const float4*>(x + ii) : make_float4(0.f, 0.f, 0.f, 0.f);
       }
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
+      for (int u = 0; u < U; ++u) {
         const int ii = i0 + u * 4 * WAVE;
         if (ii < wend) { f(ii, v[u].x); f(ii + 1, v[u].y); f(ii + 2, v[u].z); f(ii + 3, v[u].w); }
       }
     }
   } else {
-    for (int i0 = wbeg + lane; i0 < wend; i0 += 4 * WAVE) {
-      float v[4];
+    for (int i0 = wbeg + lane; i0 < wend; i0 += U * WAVE) {
+      float v[U];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) v[u] = i0 + u * WAVE < wend ? x[i0 + u * WAVE] : 0.f;
+      for (int u = 0; u < U; ++u) v[u] = i0 + u * WAVE < wend ? x[i0 + u * WAVE] : 0.f;
 #pragma unroll
-      for (int u = 0; u < 4; ++u)
+      for (int u = 0; u < U; ++u)
         if (i0 + u * WAVE < wend) f(i0 + u * WAVE, v[u]);
     }
   }
@@ -291,7 +293,9 @@ sample_kernel(const float* __restrict__ logits, int V, int ld, const float* __re
   __shared__ float fscratch[16];
   __shared__ int iscratch[16];
   __shared__ float wave_tot[16];
-  __shared__ int chosen;
+  __shared__ int chosen, range_of;
+  __shared__ float step_sum[WAVE];
+  __shared__ int step_kept[WAVE];
   __shared__ Candidates cand;
   constexpr int STEP = VEC ? 4 * WAVE : WAVE;        // values a wave reads per access
   const int row = blockIdx.x, tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
@@ -327,7 +331,7 @@ sample_kernel(const float* __restrict__ logits, int V, int ld, const float* __re
   const float inv_t = 1.f / (t < 0.f ? 1.f : t);  // the reference maps T <= 0 to 1 (sampler.py:41)
   const float L2E = 1.4426950408889634f;
   float mloc = -INFINITY;
-  for_range<VEC>(x, wbeg, wend, lane, [&](int, float v) { mloc = fmaxf(mloc, v); });   // 1 / T is positive
+  for_range<VEC, 8>(x, wbeg, wend, lane, [&](int, float v) { mloc = fmaxf(mloc, v); });   // 1 / T is positive
   const float m = block_max(mloc, fscratch) * inv_t;
   const uint32_t key_max = order_key(m);
   uint32_t kmin = 0;
@@ -380,7 +384,7 @@ sample_kernel(const float* __restrict__ logits, int V, int ld, const float* __re
   const float mp = min_p[row];
   float s = 0.f;
   if (kmin == 0 && !(mp > 0.f)) {          // nothing filtered: every value counts (3 instructions a value)
-    for_range<VEC>(x, wbeg, wend, lane, [&](int, float v) { s += E_OF(v * inv_t); });
+    for_range<VEC, 8>(x, wbeg, wend, lane, [&](int, float v) { s += E_OF(v * inv_t); });
   } else {
     for_range<VEC>(x, wbeg, wend, lane, [&](int, float v) {
       const float z = v * inv_t;
@@ -389,7 +393,7 @@ sample_kernel(const float* __restrict__ logits, int V, int ld, const float* __re
     });
   }
   s = wave_sum(s);
-  if (tid == 0) chosen = -1;
+  if (tid == 0) { chosen = -1; range_of = -1; }
   if (lane == 0) wave_tot[wave] = s;
   __syncthreads();
   float base = 0.f, total = 0.f;
@@ -400,56 +404,91 @@ sample_kernel(const float* __restrict__ logits, int V, int ld, const float* __re
   const uint64_t seed = ((uint64_t)seed_hi[row] << 32) | (uint64_t)seed_lo[row];
   const float target = uniform_from_seed(seed, (uint32_t)position[row]) * total;
   const bool mine = s > 0.f && base + s > target && !(base > target);   // exactly one wave
-  if (mine) {
-    // walk this wave's range in index order, STEP values at a time (the next ones already loading)
+  if (mine && lane == 0) range_of = wave;
+  __syncthreads();
+  const int rw = range_of;
+  if (rw >= 0) {
+    // The draw lies in wave rw's range.  The walk over it in index order, STEP values at a time, is a chain
+    // of sums; the sums of the steps are not: the block's waves take the steps of the range in turn, then
+    // every thread adds the steps' sums in order until one crosses the target, and adds that step's values
+    // one by one.  The additions and their order are those of a walk by one wave.
     constexpr int PER = VEC ? 4 : 1;
-    float run = base;
+    constexpr int HELD = 4;                 // steps a wave takes per round
+    const int rbeg = rw * per < V ? rw * per : V;
+    const int rend = rbeg + per < V ? rbeg + per : V;
+    float run = 0.f;
+    for (int w = 0; w < rw; ++w) run += wave_tot[w];
     int pick = -1, last_kept = -1;
-    float nxt[PER];
-    auto fetch = [&](int i0, float (&dst)[PER]) {
-      if (VEC) {
-        const int ii = i0 + 4 * lane;
-        const float4 v = ii < wend ? *reinterpret_cast<const float4*>(x + ii) : make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
-        dst[0] = v.x; if (PER > 1) { dst[1] = v.y; dst[2] = v.z; dst[3] = v.w; }
-      } else {
-        dst[0] = i0 + lane < wend ? x[i0 + lane] : -INFINITY;
-      }
-    };
-    fetch(wbeg, nxt);
-    for (int i0 = wbeg; i0 < wend && pick < 0; i0 += STEP) {
-      float cur[PER];
-#pragma unroll
-      for (int c = 0; c < PER; ++c) cur[c] = nxt[c];
-      if (i0 + STEP < wend) fetch(i0 + STEP, nxt);
-      float e[PER], esum = 0.f;
-      int kept_hi = -1;
+    // the values of the step at i0 that count, as a lane holds them; the highest index among them that counts
+    auto weights_of = [&](const float (&cur)[PER], int i0, float (&e)[PER], int& kept_hi) {
+      kept_hi = -1;
 #pragma unroll
       for (int c = 0; c < PER; ++c) {
         const int i = i0 + PER * lane + c;
         const float z = cur[c] * inv_t;
         const float ev = E_OF(z);
-        e[c] = (i < wend && order_key(z) >= kmin && ev >= mp) ? ev : 0.f;
+        e[c] = (i < rend && order_key(z) >= kmin && ev >= mp) ? ev : 0.f;
         if (e[c] > 0.f) kept_hi = i;
-        esum += e[c];
       }
 #pragma unroll
       for (int sft = WAVE / 2; sft > 0; sft >>= 1) { const int o = __shfl_xor(kept_hi, sft, WAVE); kept_hi = o > kept_hi ? o : kept_hi; }
-      if (kept_hi >= 0) last_kept = kept_hi;
-      const float step = wave_sum(esum);
-      if (run + step > target) {            // the crossing is among these: add them one by one
-        for (int j = 0; j < WAVE && pick < 0; ++j) {
-#pragma unroll
-          for (int c = 0; c < PER; ++c) {
-            const float ej = __shfl(e[c], j, WAVE);
-            run += ej;
-            if (pick < 0 && ej > 0.f && run > target) pick = i0 + PER * j + c;
-          }
-        }
+    };
+    auto fetch = [&](int i0, float (&dst)[PER]) {
+      const int last = rend - PER;          // rend - rbeg is a multiple of PER, and the range is not empty
+      if (VEC) {
+        const int ii = i0 + 4 * lane;
+        const float4 v = *reinterpret_cast<const float4*>(x + (ii < last ? ii : last));
+        dst[0] = v.x; if (PER > 1) { dst[1] = v.y; dst[2] = v.z; dst[3] = v.w; }
       } else {
-        run += step;
+        const int ii = i0 + lane;
+        dst[0] = x[ii < last ? ii : last];
       }
+    };
+    const int round_span = HELD * nwaves * STEP;
+    for (int r0 = rbeg; r0 < rend && pick < 0; r0 += round_span) {
+      float cur[HELD][PER];
+#pragma unroll
+      for (int j = 0; j < HELD; ++j) fetch(r0 + (wave + nwaves * j) * STEP, cur[j]);
+#pragma unroll
+      for (int j = 0; j < HELD; ++j) {
+        const int i0 = r0 + (wave + nwaves * j) * STEP;
+        float e[PER], esum = 0.f;
+        int kept_hi;
+        weights_of(cur[j], i0, e, kept_hi);
+#pragma unroll
+        for (int c = 0; c < PER; ++c) esum += e[c];
+        const float step = wave_sum(esum);
+        if (lane == 0) { step_sum[wave + nwaves * j] = step; step_kept[wave + nwaves * j] = kept_hi; }
+      }
+      __syncthreads();
+      const float my_step = step_sum[lane];
+      const int my_kept = step_kept[lane];
+      const int steps_here = (rend - r0 + STEP - 1) / STEP < HELD * nwaves ? (rend - r0 + STEP - 1) / STEP : HELD * nwaves;
+      for (int c = 0; c < steps_here && pick < 0; ++c) {
+        const float step = __shfl(my_step, c, WAVE);
+        const int kept_hi = __shfl(my_kept, c, WAVE);
+        if (kept_hi >= 0) last_kept = kept_hi;
+        if (run + step > target) {            // the crossing is among these: add them one by one
+          const int i0 = r0 + c * STEP;
+          float one[PER], e[PER];
+          int unused;
+          fetch(i0, one);
+          weights_of(one, i0, e, unused);
+          for (int j = 0; j < WAVE && pick < 0; ++j) {
+#pragma unroll
+            for (int cc = 0; cc < PER; ++cc) {
+              const float ej = __shfl(e[cc], j, WAVE);
+              run += ej;
+              if (pick < 0 && ej > 0.f && run > target) pick = i0 + PER * j + cc;
+            }
+          }
+        } else {
+          run += step;
+        }
+      }
+      __syncthreads();                        // the next round writes the steps' sums again
     }
-    if (lane == 0) chosen = pick >= 0 ? pick : last_kept;
+    if (tid == 0) chosen = pick >= 0 ? pick : last_kept;
   }
   __syncthreads();
   if (chosen < 0) {  // rounding pushed the target past the total: take the last kept index
