@@ -366,8 +366,13 @@ def test_sampler_with_a_small_top_k_over_a_large_vocabulary(ops):
     configs = [(0.6, 20, 0.95, 0.0), (1.0, 5, 1.0, 0.0), (0.8, 50, 0.9, 0.02), (1.0, 1000, 1.0, 0.0), (1.2, 1, 1.0, 0.0),
                (0.7, 20, 0.5, 0.0), (1.0, 1024, 0.99, 0.0), (1.0, 1025, 1.0, 0.0),
                (0.7, -1, 0.9, 0.0), (1.0, 0, 0.5, 0.02), (0.5, -1, 0.99, 0.0)]        # top-p alone
+    whole_rows = Sampler(torch.device(DEV), cut_rows=False)    # one block per row, no parts
     for V in (32000, 151936, 50257):       # 50257: rows not aligned for 16-byte loads
+        masked = torch.randn(len(configs), V) * 3
+        masked[:, 5000:27000] = float("-inf")                            # whole parts of a row without weight
+        masked[:, -2000:] = float("-inf")
         kinds = {
+            "masked": masked,
             "spread": torch.randn(len(configs), V) * 3,
             "peaked": torch.randn(len(configs), V) * 8,
             "flat": torch.randn(len(configs), V) * 0.01,                     # all within a hair of the maximum
@@ -386,6 +391,45 @@ def test_sampler_with_a_small_top_k_over_a_large_vocabulary(ops):
                 assert got[i] in plain.sample_token_set(logits[i], *c, seeds[i], pos[i]), (V, name, c, got[i])
             again = sampler.sample(logits.flip(0).contiguous().to(DEV), ps[::-1], seeds[::-1], pos[::-1])
             assert again[::-1] == got
+            whole = whole_rows.sample(logits.to(DEV), ps, seeds, pos)
+            for i, c in enumerate(configs):
+                if name == "ties" and c[2] < 1.0:
+                    continue
+                assert whole[i] in plain.sample_token_set(logits[i], *c, seeds[i], pos[i]), (V, name, c, whole[i])
+
+
+def test_sampler_rows_cut_into_parts(ops):
+    """Temperature alone and top-k up to 64 take sums and candidates from parts of the row that a first kernel
+    makes; the token is one the plain sampler may draw, whatever the row looks like and wherever in it the
+    weight lies, and the same as in another batch position."""
+    from ullm_amd.sampling import Sampler, SamplingParams
+    torch.manual_seed(23)
+    sampler = Sampler(torch.device(DEV))
+    configs = [(0.7, -1, 1.0, 0.0), (1.0, 0, 1.0, 0.0), (1.5, -1, 1.0, 0.0), (0.6, 20, 0.95, 0.0), (1.0, 64, 1.0, 0.0),
+               (0.8, 50, 0.9, 0.02), (1.0, 1, 1.0, 0.0), (0.3, 3, 1.0, 0.1), (1.0, 65, 1.0, 0.0)]
+    for V in (10240, 10244, 40960, 151936, 327680, 327684):      # one part exactly, one value into the next, the most parts, too many
+        rows = {
+            "spread": torch.randn(len(configs), V) * 3,
+            "weight at the end": torch.cat([torch.randn(len(configs), V - 8) - 30.0, torch.randn(len(configs), 8) * 2], 1),
+            "weight at a part's edge": torch.full((len(configs), V), -40.0),
+            "equal values": torch.zeros(len(configs), V),
+            "the largest all in one part": torch.randn(len(configs), V),
+        }
+        edge = min(10236, V - 8)
+        rows["weight at a part's edge"][:, edge:edge + 8] = torch.randn(len(configs), 8)
+        rows["the largest all in one part"][:, 3000:3100] += 20.0
+        for name, logits in rows.items():
+            ps = [SamplingParams(temperature=c[0], top_k=c[1], top_p=c[2], min_p=c[3]) for c in configs]
+            seeds = [11 + i for i in range(len(configs))]
+            for trial in range(3):
+                pos = [trial * 5 + i for i in range(len(configs))]
+                got = sampler.sample(logits.to(DEV), ps, seeds, pos)
+                for i, c in enumerate(configs):
+                    if name == "equal values" and c[2] < 1.0:
+                        continue   # which of several equal values top-p drops follows the reference's sort; here all or none
+                    assert got[i] in plain.sample_token_set(logits[i], *c, seeds[i], pos[i]), (V, name, c, got[i])
+                again = sampler.sample(logits.flip(0).contiguous().to(DEV), ps[::-1], seeds[::-1], pos[::-1])
+                assert again[::-1] == got
 
 
 MFMA_CASES = [dict(nq=8, nkv=2, hd=32, P=16, lens=[(1, 1), (1, 37), (1, 300), (1, 64)], window=0),

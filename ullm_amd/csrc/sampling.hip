@@ -1,4 +1,5 @@
-// Next-token choice on the device, one block per row of 32-bit logits.
+// Next-token choice on the device from rows of 32-bit logits: one block per row, after a first kernel that
+// cuts the rows into parts over many blocks for the settings it serves (temperature alone, a small top-k).
 //
 // What is computed follows the reference's sampler (ullm/layers/sampler.py:39-56): logits / T, top-k
 // (keep values >= the k-th largest, ties kept, sampler.py:67-76), top-p on the softmax of what top-k
@@ -96,6 +97,166 @@ struct Candidates {
   int lidx[16 * SEG];
   int result;
 };
+
+// draw_from_list for up to 4 * 64 candidates: a lane keeps its four in registers, counts are ballots, and
+// top-p needs no search: a candidate stays if the weight of the larger ones (of those top-k left) is below
+// the bound, which every lane adds up for its own candidates in index order.
+__device__ int draw_from_short_list(const Candidates& cand, int n_all, bool by_count, int k, float p, float mp,
+                                    float all_weight, uint32_t key_thr, uint32_t key_max, float uniform, int lane) {
+  constexpr int H = 4;
+  float zr[H], er[H];
+  uint32_t kr[H];
+  bool have[H];
+#pragma unroll
+  for (int i = 0; i < H; ++i) {
+    const int j = lane + i * WAVE;
+    have[i] = j < n_all;
+    zr[i] = cand.lz[have[i] ? j : 0];
+    er[i] = have[i] ? cand.le[j] : 0.f;
+    kr[i] = order_key(zr[i]);
+  }
+  uint32_t kmin = key_thr;
+  if (by_count) {                           // the largest key v with #{key >= v} >= k
+    uint32_t lo = key_thr, hi = key_max;
+    while (lo < hi) {
+      const uint32_t mid = lo + (hi - lo + 1) / 2;
+      int c = 0;
+#pragma unroll
+      for (int i = 0; i < H; ++i) c += __popcll(__ballot(have[i] && kr[i] >= mid));
+      if (c >= k) lo = mid; else hi = mid - 1;
+    }
+    kmin = lo;
+  }
+  if (p > 0.f && p < 1.f) {
+    float a = 0.f;
+#pragma unroll
+    for (int i = 0; i < H; ++i) a += (have[i] && kr[i] >= kmin) ? er[i] : 0.f;
+    const float listed = wave_sum(a);
+    const float bound = p * (by_count ? listed : all_weight);
+    if (!by_count && listed < bound) return -1;
+    float above[H] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int src = 0; src < H; ++src) {
+      const int n_here = n_all - src * WAVE < WAVE ? n_all - src * WAVE : WAVE;
+      const float e_src = kr[src] >= kmin ? er[src] : 0.f;
+      for (int j = 0; j < n_here; ++j) {
+        const float zj = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(zr[src]), j));
+        const float ej = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(e_src), j));
+#pragma unroll
+        for (int i = 0; i < H; ++i) above[i] += zj > zr[i] ? ej : 0.f;
+      }
+    }
+    uint32_t least = 0xffffffffu;           // the smallest key that stays
+#pragma unroll
+    for (int i = 0; i < H; ++i)
+      if (have[i] && kr[i] >= kmin && above[i] < bound) least = kr[i] < least ? kr[i] : least;
+#pragma unroll
+    for (int d = WAVE / 2; d > 0; d >>= 1) { const uint32_t o = __shfl_xor(least, d, WAVE); least = o < least ? o : least; }
+    if (least != 0xffffffffu) kmin = least;
+  }
+  // min-p and the draw
+  float w[H], total = 0.f;
+#pragma unroll
+  for (int i = 0; i < H; ++i) {
+    w[i] = (have[i] && kr[i] >= kmin && er[i] >= mp) ? er[i] : 0.f;
+    total += w[i];
+  }
+  total = wave_sum(total);
+  const float target = uniform * total;
+  float run = 0.f;
+  int token = -1, last_kept = -1;
+#pragma unroll
+  for (int i = 0; i < H; ++i) {
+    if (i * WAVE >= n_all || token >= 0) continue;
+    float incl = w[i];
+#pragma unroll
+    for (int d = 1; d < WAVE; d <<= 1) {
+      const float o = __shfl_up(incl, d, WAVE);
+      if (lane >= d) incl += o;
+    }
+    const unsigned long long kept = __ballot(w[i] > 0.f);
+    const unsigned long long crossed = __ballot(w[i] > 0.f && run + incl > target);
+    if (crossed) token = cand.lidx[i * WAVE + __ffsll((long long)crossed) - 1];
+    if (kept) last_kept = cand.lidx[i * WAVE + 63 - __clzll((long long)kept)];
+    run += __shfl(incl, WAVE - 1, WAVE);
+  }
+  if (token < 0) token = last_kept < 0 ? 0 : last_kept;
+  return token;
+}
+
+// Top-k, top-p, min-p and the draw over a list of candidates in index order (lz: values / T, le: weights
+// exp(z - max), lidx: vocabulary indices), the work of one wave.  by_count: top-k is at work and every value
+// >= the k-th largest is in the list; else the list holds the nucleus of all weight `all_weight`.  key_thr: a key
+// with at least k candidates at or above it (by_count) / the key all candidates reach.  -1: the list does not
+// hold the nucleus (take the long way); else the token.
+__device__ int draw_from_list(const Candidates& cand, int n_all, bool by_count, int k, float p, float mp,
+                              float all_weight, uint32_t key_thr, uint32_t key_max, float uniform, int lane) {
+  if (n_all <= 4 * WAVE)
+    return draw_from_short_list(cand, n_all, by_count, k, p, mp, all_weight, key_thr, key_max, uniform, lane);
+  auto count_if = [&](auto pred) {
+    int c = 0;
+    for (int j0 = 0; j0 < n_all; j0 += WAVE)
+      c += __popcll(__ballot(j0 + lane < n_all && pred(cand.lz[j0 + lane < n_all ? j0 + lane : 0])));
+    return c;
+  };
+  auto mass_if = [&](auto pred) {
+    float a = 0.f;
+    for (int j = lane; j < n_all; j += WAVE) {
+      if (pred(cand.lz[j])) a += cand.le[j];
+    }
+    return wave_sum(a);
+  };
+  // 3. top-k: the largest key v with #{key >= v} >= k; all such keys are candidates
+  uint32_t kmin = key_thr;
+  if (by_count) {
+    uint32_t lo = key_thr, hi = key_max;
+    while (lo < hi) {
+      const uint32_t mid = lo + (hi - lo + 1) / 2;
+      if (count_if([&](float zz) { return order_key(zz) >= mid; }) >= k) lo = mid; else hi = mid - 1;
+    }
+    kmin = lo;
+  }
+  // 4. top-p on what top-k left (without top-k: on everything, and the candidates must hold the nucleus)
+  if (p > 0.f && p < 1.f) {
+    const float listed = mass_if([&](float zz) { return order_key(zz) >= kmin; });
+    const float bound = p * (by_count ? listed : all_weight);
+    if (!by_count && listed < bound) return -1;
+    uint32_t lo = kmin, hi = key_max;
+    while (lo < hi) {
+      const uint32_t mid = lo + (hi - lo) / 2;
+      if (mass_if([&](float zz) { return order_key(zz) > mid; }) < bound) hi = mid; else lo = mid + 1;
+    }
+    kmin = lo;
+  }
+  // 5. min-p and the draw: a walk along the list, 64 candidates at a time
+  auto weight = [&](int j) {
+    if (j >= n_all) return 0.f;
+    const float e = cand.le[j];
+    return (order_key(cand.lz[j]) >= kmin && e >= mp) ? e : 0.f;
+  };
+  float total = 0.f;
+  for (int j = lane; j < n_all; j += WAVE) total += weight(j);
+  total = wave_sum(total);
+  const float target = uniform * total;
+  float run = 0.f;
+  int token = -1, last_kept = -1;
+  for (int j0 = 0; j0 < n_all && token < 0; j0 += WAVE) {
+    const float e = weight(j0 + lane);
+    float incl = e;
+#pragma unroll
+    for (int d = 1; d < WAVE; d <<= 1) {
+      const float o = __shfl_up(incl, d, WAVE);
+      if (lane >= d) incl += o;
+    }
+    const unsigned long long kept = __ballot(e > 0.f);
+    const unsigned long long crossed = __ballot(e > 0.f && run + incl > target);
+    if (crossed) token = cand.lidx[j0 + __ffsll((long long)crossed) - 1];
+    if (kept) last_kept = cand.lidx[j0 + 63 - __clzll((long long)kept)];
+    run += __shfl(incl, WAVE - 1, WAVE);
+  }
+  if (token < 0) token = last_kept < 0 ? 0 : last_kept;   // rounding pushed the target past the total: the last index kept
+  return token;
+}
 
 // -1: take the long way.  Otherwise the token.  Every thread of the block returns the same value.
 template <bool VEC>
@@ -206,74 +367,8 @@ __device__ int sample_small_k(const float* __restrict__ x, int wbeg, int wend, f
     }
   }
   __syncthreads();
-  auto list_phase = [&]() -> int {
-  auto count_if = [&](auto pred) {
-    int c = 0;
-    for (int j = lane; j < n_all; j += WAVE) c += pred(cand.lz[j]);
-#pragma unroll
-    for (int d = WAVE / 2; d > 0; d >>= 1) c += __shfl_xor(c, d, WAVE);
-    return c;
-  };
-  auto mass_if = [&](auto pred) {
-    float a = 0.f;
-    for (int j = lane; j < n_all; j += WAVE) {
-      if (pred(cand.lz[j])) a += cand.le[j];
-    }
-    return wave_sum(a);
-  };
-  // 3. top-k: the largest key v with #{key >= v} >= k; all such keys are candidates
-  uint32_t kmin = key_thr;
-  if (by_count) {
-    uint32_t lo = key_thr, hi = key_max;
-    while (lo < hi) {
-      const uint32_t mid = lo + (hi - lo + 1) / 2;
-      if (count_if([&](float zz) { return order_key(zz) >= mid; }) >= k) lo = mid; else hi = mid - 1;
-    }
-    kmin = lo;
-  }
-  // 4. top-p on what top-k left (without top-k: on everything, and the candidates must hold the nucleus)
-  if (p > 0.f && p < 1.f) {
-    const float listed = mass_if([&](float zz) { return order_key(zz) >= kmin; });
-    const float bound = p * (by_count ? listed : all_weight);
-    if (!by_count && listed < bound) return -1;
-    uint32_t lo = kmin, hi = key_max;
-    while (lo < hi) {
-      const uint32_t mid = lo + (hi - lo) / 2;
-      if (mass_if([&](float zz) { return order_key(zz) > mid; }) < bound) hi = mid; else lo = mid + 1;
-    }
-    kmin = lo;
-  }
-  // 5. min-p and the draw: a walk along the list, 64 candidates at a time
-  auto weight = [&](int j) {
-    if (j >= n_all) return 0.f;
-    const float e = cand.le[j];
-    return (order_key(cand.lz[j]) >= kmin && e >= mp) ? e : 0.f;
-  };
-  float total = 0.f;
-  for (int j = lane; j < n_all; j += WAVE) total += weight(j);
-  total = wave_sum(total);
-  const float target = uniform * total;
-  float run = 0.f;
-  int token = -1, last_kept = -1;
-  for (int j0 = 0; j0 < n_all && token < 0; j0 += WAVE) {
-    const float e = weight(j0 + lane);
-    float incl = e;
-#pragma unroll
-    for (int d = 1; d < WAVE; d <<= 1) {
-      const float o = __shfl_up(incl, d, WAVE);
-      if (lane >= d) incl += o;
-    }
-    const unsigned long long kept = __ballot(e > 0.f);
-    const unsigned long long crossed = __ballot(e > 0.f && run + incl > target);
-    if (crossed) token = cand.lidx[j0 + __ffsll((long long)crossed) - 1];
-    if (kept) last_kept = cand.lidx[j0 + 63 - __clzll((long long)kept)];
-    run += __shfl(incl, WAVE - 1, WAVE);
-  }
-  if (token < 0) token = last_kept < 0 ? 0 : last_kept;   // rounding pushed the target past the total: the last index kept
-  return token;
-  };
   if (wave == 0) {
-    const int token = list_phase();
+    const int token = draw_from_list(cand, n_all, by_count, k, p, mp, all_weight, key_thr, key_max, uniform, lane);
     if (lane == 0) cand.result = token;
   }
   __syncthreads();
@@ -281,19 +376,289 @@ __device__ int sample_small_k(const float* __restrict__ x, int wbeg, int wend, f
   return cand.result;
 }
 
+// The draw inside [rbeg, rend) (not empty; with VEC a multiple of 4 long, from a multiple of 4), by the whole
+// block: `run` is the weight before the range, the token is the first index at which the running sum passes
+// `target`.  The walk over the range in index order, STEP values at a time, is a chain of sums; the sums of the
+// steps are not: the block's waves take the steps of the range in turn, then every thread adds the steps' sums
+// in order until one crosses the target, and takes running sums inside that step (a lane's values in order,
+// the lanes by a scan).  Returns the token, or the last index of the range that counts if
+// rounding kept the running sum from passing the target (-1: none counts).  Every thread gets the same value.
+template <bool VEC>
+__device__ int walk_range(const float* __restrict__ x, int rbeg, int rend, float run, float target, float inv_t,
+                          float m, uint32_t kmin, float mp, float* step_sum, int* step_kept) {
+  constexpr int PER = VEC ? 4 : 1;
+  constexpr int STEP = PER * WAVE;
+  constexpr int HELD = 4;                 // steps a wave takes per round
+  const float L2E = 1.4426950408889634f;
+  const int tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE, nwaves = blockDim.x / WAVE;
+  int pick = -1, last_kept = -1;
+  // the values of the step at i0 that count, as a lane holds them; the highest index among them that counts
+  auto weights_of = [&](const float (&cur)[PER], int i0, float (&e)[PER], int& kept_hi) {
+    kept_hi = -1;
+#pragma unroll
+    for (int c = 0; c < PER; ++c) {
+      const int i = i0 + PER * lane + c;
+      const float z = cur[c] * inv_t;
+      const float ev = __builtin_amdgcn_exp2f((z - m) * L2E);
+      e[c] = (i < rend && order_key(z) >= kmin && ev >= mp) ? ev : 0.f;
+      if (e[c] > 0.f) kept_hi = i;
+    }
+#pragma unroll
+    for (int sft = WAVE / 2; sft > 0; sft >>= 1) { const int o = __shfl_xor(kept_hi, sft, WAVE); kept_hi = o > kept_hi ? o : kept_hi; }
+  };
+  auto fetch = [&](int i0, float (&dst)[PER]) {
+    const int last = rend - PER;
+    if (VEC) {
+      const int ii = i0 + 4 * lane;
+      const float4 v = *reinterpret_cast<const float4*>(x + (ii < last ? ii : last));
+      dst[0] = v.x; if (PER > 1) { dst[1] = v.y; dst[2] = v.z; dst[3] = v.w; }
+    } else {
+      const int ii = i0 + lane;
+      dst[0] = x[ii < last ? ii : last];
+    }
+  };
+  const int round_span = HELD * nwaves * STEP;
+  for (int r0 = rbeg; r0 < rend && pick < 0; r0 += round_span) {
+    float cur[HELD][PER];
+#pragma unroll
+    for (int j = 0; j < HELD; ++j) fetch(r0 + (wave + nwaves * j) * STEP, cur[j]);
+#pragma unroll
+    for (int j = 0; j < HELD; ++j) {
+      const int i0 = r0 + (wave + nwaves * j) * STEP;
+      float e[PER], esum = 0.f;
+      int kept_hi;
+      weights_of(cur[j], i0, e, kept_hi);
+#pragma unroll
+      for (int c = 0; c < PER; ++c) esum += e[c];
+      const float step = wave_sum(esum);
+      if (lane == 0) { step_sum[wave + nwaves * j] = step; step_kept[wave + nwaves * j] = kept_hi; }
+    }
+    __syncthreads();
+    const float my_step = step_sum[lane];
+    const int my_kept = step_kept[lane];
+    const int steps_here = (rend - r0 + STEP - 1) / STEP < HELD * nwaves ? (rend - r0 + STEP - 1) / STEP : HELD * nwaves;
+    for (int c = 0; c < steps_here && pick < 0; ++c) {
+      const float step = __shfl(my_step, c, WAVE);
+      const int kept_hi = __shfl(my_kept, c, WAVE);
+      if (kept_hi >= 0) last_kept = kept_hi;
+      if (run + step > target) {            // the crossing is among these: running sums inside the step
+        const int i0 = r0 + c * STEP;
+        float one[PER], e[PER];
+        int unused;
+        fetch(i0, one);
+        weights_of(one, i0, e, unused);
+        float upto[PER];                      // a lane's values, added in order
+        upto[0] = e[0];
+#pragma unroll
+        for (int cc = 1; cc < PER; ++cc) upto[cc] = upto[cc - 1] + e[cc];
+        float incl = upto[PER - 1];           // then the lanes, by a scan
+#pragma unroll
+        for (int d = 1; d < WAVE; d <<= 1) {
+          const float o = __shfl_up(incl, d, WAVE);
+          if (lane >= d) incl += o;
+        }
+        float before = __shfl_up(incl, 1, WAVE);
+        if (lane == 0) before = 0.f;
+        int first = PER;                      // the lane's first value at which the sum has passed the target
+#pragma unroll
+        for (int cc = PER - 1; cc >= 0; --cc)
+          if (e[cc] > 0.f && run + (before + upto[cc]) > target) first = cc;
+        const unsigned long long crossed = __ballot(first < PER);
+        if (crossed) {
+          const int at = __ffsll((long long)crossed) - 1;
+          pick = i0 + PER * at + __shfl(first, at, WAVE);
+        }
+        run += __shfl(incl, WAVE - 1, WAVE);
+      } else {
+        run += step;
+      }
+    }
+    __syncthreads();                        // the next round writes the steps' sums again
+  }
+  return pick >= 0 ? pick : last_kept;
+}
+
+// ------------------------------------------------------------------------------ parts of a row
+// One block per row reads 150 K values with one compute unit, pass after pass.  For the two common settings
+// (temperature alone; top-k with a small k, with or without top-p and min-p) a first kernel cuts every row
+// into parts of PART_VALUES values, one block each, which hold their values in registers and leave per part:
+// the maximum, the sum of exp(z - that maximum) and, with top-k, the candidates: every value of the part at
+// or above a threshold that at least k of its values reach (so the k largest of the row, ties included, are
+// among the parts' candidates), in index order, and that threshold (the row's k-th largest value is at or
+// above every part's).  The row's block then only scales and adds the parts' sums and walks the one part
+// the draw falls into, or runs the list phase over the candidates at or above the highest threshold.  A
+// part with more candidates than it can pass on (many equal values) says so, and the row's block takes the
+// way over the whole vocabulary.
+#define PART_THREADS 256
+#define PART_HOLD 10                                         // 16-byte pieces a thread holds
+#define PART_WAVE_VALUES (4 * WAVE * PART_HOLD)              // a wave's consecutive values
+#define PART_VALUES (PART_THREADS / WAVE * PART_WAVE_VALUES)
+#define PART_CAND 128                                        // candidates a part can pass on
+#define PART_K_MAX 64
+#define PART_WORDS (4 + 2 * PART_CAND)                       // maximum, sum, candidates (-1: unbounded), their threshold; values; indices
+#define MAX_PARTS 32
+#define TOP_K_PARTS 16                                       // with top-k: one wave holds all candidates, two per lane and part
+
+enum { PARTS_NONE = 0, PARTS_SUMS = 1, PARTS_TOP_K = 2 };
+__device__ __forceinline__ int parts_mode(float t, int k, int V, float p, float mp) {
+  if (t == 0.f) return PARTS_NONE;
+  if (k > 0 && k < V) return (k <= PART_K_MAX && V <= TOP_K_PARTS * PART_VALUES) ? PARTS_TOP_K : PARTS_NONE;
+  return (!(p > 0.f && p < 1.f) && !(mp > 0.f)) ? PARTS_SUMS : PARTS_NONE;
+}
+
+// grid (parts, rows); V a multiple of 4 and rows 16-byte aligned
+__global__ void __launch_bounds__(PART_THREADS)
+sample_parts_kernel(const float* __restrict__ logits, int V, int ld, const float* __restrict__ temperature,
+                    const int* __restrict__ top_k, const float* __restrict__ top_p, const float* __restrict__ min_p,
+                    float* __restrict__ parts, int n_parts) {
+  constexpr int NW = PART_THREADS / WAVE;
+  __shared__ float fscratch[16];
+  __shared__ float lane_max[PART_THREADS];
+  __shared__ float seg_z[NW][PART_CAND];
+  __shared__ int seg_i[NW][PART_CAND];
+  __shared__ int seg_n[NW];
+  const int part = blockIdx.x, row = blockIdx.y, tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
+  const float t = temperature[row];
+  const int k = top_k[row];
+  const int mode = parts_mode(t, k, V, top_p[row], min_p[row]);
+  if (mode == PARTS_NONE) return;
+  const float* x = logits + (size_t)row * ld;
+  float* const mine = parts + ((size_t)row * n_parts + part) * PART_WORDS;
+  const int pbeg = part * PART_VALUES;
+  const int pend = pbeg + PART_VALUES < V ? pbeg + PART_VALUES : V;
+  const int wbeg = pbeg + wave * PART_WAVE_VALUES;
+  const float inv_t = 1.f / (t < 0.f ? 1.f : t);
+  const float L2E = 1.4426950408889634f;
+  // piece j of a lane: values wbeg + (64 j + lane) * 4 ..; past the part the part's last piece, which then does not count
+  float z[PART_HOLD][4];
+  bool in[PART_HOLD];
+#pragma unroll
+  for (int j = 0; j < PART_HOLD; ++j) {
+    const int ii = wbeg + (j * WAVE + lane) * 4;
+    in[j] = ii < pend;
+    const float4 v = *reinterpret_cast<const float4*>(x + (in[j] ? ii : pend - 4));
+    z[j][0] = v.x * inv_t; z[j][1] = v.y * inv_t; z[j][2] = v.z * inv_t; z[j][3] = v.w * inv_t;
+  }
+  float mloc = -INFINITY;
+#pragma unroll
+  for (int j = 0; j < PART_HOLD; ++j)
+#pragma unroll
+    for (int c = 0; c < 4; ++c) mloc = in[j] ? fmaxf(mloc, z[j][c]) : mloc;
+  const float m = block_max(mloc, fscratch);
+  float s = 0.f;
+  if (m > -INFINITY) {
+#pragma unroll
+    for (int j = 0; j < PART_HOLD; ++j)
+#pragma unroll
+      for (int c = 0; c < 4; ++c) s += in[j] ? __builtin_amdgcn_exp2f((z[j][c] - m) * L2E) : 0.f;
+  }
+  s = wave_sum(s);
+  __syncthreads();
+  if (lane == 0) fscratch[wave] = s;
+  __syncthreads();
+  if (tid == 0) {
+    float total = 0.f;
+    for (int w = 0; w < NW; ++w) total += fscratch[w];
+    mine[0] = m;
+    mine[1] = total;
+    reinterpret_cast<int*>(mine)[2] = 0;
+  }
+  if (mode != PARTS_TOP_K) return;
+  // A threshold that at least kk of the part's values reach, and not many more: one that kk of the threads'
+  // own maxima reach (the largest values of a part mostly lie with different threads).  Every wave looks
+  // for it by itself, halving the span of the maxima twelve times, with counts by ballot.
+  const int kk = k < pend - pbeg ? k : pend - pbeg;
+  lane_max[tid] = mloc;
+  __syncthreads();
+  float lm[NW];
+  float lowest = INFINITY;
+  int with_values = 0;
+#pragma unroll
+  for (int i = 0; i < NW; ++i) {
+    lm[i] = lane_max[lane + i * WAVE];
+    lowest = lm[i] > -INFINITY ? fminf(lowest, lm[i]) : lowest;
+    with_values += __popcll(__ballot(lm[i] > -INFINITY));
+  }
+#pragma unroll
+  for (int d = WAVE / 2; d > 0; d >>= 1) lowest = fminf(lowest, __shfl_xor(lowest, d, WAVE));
+  float wide = -INFINITY;                   // fewer threads with values than kk: everything is a candidate
+  if (with_values >= kk) {
+    float lo = lowest, hi = m;
+    for (int it = 0; it < 12; ++it) {
+      const float mid = 0.5f * (lo + hi);
+      if (!(mid > lo && mid < hi)) break;
+      int c = 0;
+#pragma unroll
+      for (int i = 0; i < NW; ++i) c += __popcll(__ballot(lm[i] >= mid));
+      if (c >= kk) lo = mid; else hi = mid;
+    }
+    wide = lo;
+  }
+  // the candidates, in index order: a wave appends what it keeps to its segment
+  int pos = 0;
+  bool overflow = false;
+#pragma unroll
+  for (int j = 0; j < PART_HOLD; ++j) {
+    unsigned long long kept[4];
+    int total = 0;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      kept[c] = __ballot(in[j] && z[j][c] >= wide);
+      total += __popcll(kept[c]);
+    }
+    if (overflow || total == 0) continue;
+    if (pos + total > PART_CAND) { overflow = true; continue; }
+    const unsigned long long below = (1ull << lane) - 1ull;
+    int o = pos;                            // values of lower lanes first, then this lane's own in order
+#pragma unroll
+    for (int c = 0; c < 4; ++c) o += __popcll(kept[c] & below);
+    const int ii = wbeg + (j * WAVE + lane) * 4;
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+      if ((kept[c] >> lane) & 1ull) { seg_z[wave][o] = z[j][c]; seg_i[wave][o] = ii + c; ++o; }
+    pos += total;
+  }
+  if (lane == 0) seg_n[wave] = overflow ? -1 : pos;
+  __syncthreads();
+  int n_all = 0, off = 0;
+  bool bad = false;
+  for (int w = 0; w < NW; ++w) {
+    bad = bad || seg_n[w] < 0;
+    if (w < wave) off += seg_n[w];
+    n_all += seg_n[w];
+  }
+  if (bad || n_all > PART_CAND || n_all < kk) {
+    if (tid == 0) reinterpret_cast<int*>(mine)[2] = -1;
+    return;
+  }
+  for (int j = lane; j < seg_n[wave]; j += WAVE) {
+    mine[4 + off + j] = seg_z[wave][j];
+    reinterpret_cast<int*>(mine)[4 + PART_CAND + off + j] = seg_i[wave][j];
+  }
+  if (tid == 0) {
+    reinterpret_cast<int*>(mine)[2] = n_all;
+    mine[3] = kk == k ? wide : -INFINITY;   // k values of the row are at or above it: so is the row's k-th largest
+  }
+}
+
 // Each wave owns a contiguous range of the vocabulary, so sums over a wave's range are sums over
 // consecutive indices and the draw can walk the index order wave by wave.
+// With `parts` (what sample_parts_kernel left for each row, n_parts parts a row) the two settings it serves take
+// their sums or candidates from there.
 template <bool VEC>
 __global__ void __launch_bounds__(SAMPLE_THREADS)
 sample_kernel(const float* __restrict__ logits, int V, int ld, const float* __restrict__ temperature,
               const int* __restrict__ top_k, const float* __restrict__ top_p,
               const float* __restrict__ min_p, const unsigned* __restrict__ seed_lo,
               const unsigned* __restrict__ seed_hi, const int* __restrict__ position,
-              int* __restrict__ out) {
+              int* __restrict__ out, const float* __restrict__ parts, int n_parts) {
   __shared__ float fscratch[16];
   __shared__ int iscratch[16];
   __shared__ float wave_tot[16];
   __shared__ int chosen, range_of;
+  __shared__ float part_m[MAX_PARTS], part_s[MAX_PARTS];
+  __shared__ int part_n[MAX_PARTS];
+  __shared__ float part_w[MAX_PARTS];
   __shared__ float step_sum[WAVE];
   __shared__ int step_kept[WAVE];
   __shared__ Candidates cand;
@@ -301,10 +666,118 @@ sample_kernel(const float* __restrict__ logits, int V, int ld, const float* __re
   const int row = blockIdx.x, tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
   const int nwaves = blockDim.x / WAVE;
   const float* x = logits + (size_t)row * ld;
+  // every per-row number, and this thread's part of what the first kernel left, asked for at once
   const float t = temperature[row];
+  const int k_row = top_k[row];
+  const float p_row = top_p[row], mp_row = min_p[row];
+  const uint64_t seed = ((uint64_t)seed_hi[row] << 32) | (uint64_t)seed_lo[row];
+  const uint32_t position_row = (uint32_t)position[row];
+  float4 header = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (parts && tid < n_parts) header = *reinterpret_cast<const float4*>(parts + ((size_t)row * n_parts + tid) * PART_WORDS);
   const int per = ((V + nwaves - 1) / nwaves + STEP - 1) / STEP * STEP;
   const int wbeg = wave * per < V ? wave * per : V;
   const int wend = wbeg + per < V ? wbeg + per : V;
+
+  const int mode = parts ? parts_mode(t, k_row, V, p_row, mp_row) : PARTS_NONE;
+  if (mode != PARTS_NONE) {
+    const float* const mine = parts + (size_t)row * n_parts * PART_WORDS;
+    const int* const mine_i = reinterpret_cast<const int*>(mine);
+    const float inv_t = 1.f / (t < 0.f ? 1.f : t);
+    const float L2E = 1.4426950408889634f;
+    // the parts' maxima, sums and numbers of candidates: one load each, side by side, then shared
+    if (tid < n_parts) {
+      part_m[tid] = header.x;
+      part_s[tid] = header.y;
+      part_n[tid] = __float_as_int(header.z);
+      part_w[tid] = header.w;
+    }
+    __syncthreads();
+    float m = -INFINITY;
+    for (int p = 0; p < n_parts; ++p) m = fmaxf(m, part_m[p]);
+    const float uniform = uniform_from_seed(seed, position_row);
+    if (mode == PARTS_TOP_K) {
+      bool bad = false;
+      float bound = -INFINITY;              // the row's k-th largest value is at or above every part's threshold
+      for (int p = 0; p < n_parts; ++p) {
+        bad = bad || part_n[p] < 0;
+        bound = fmaxf(bound, part_w[p]);
+      }
+      if (!bad) {
+        // One wave does the rest.  It holds all candidates (two per lane and part), raises the bound towards
+        // the row's k-th largest value by halving the span to the maximum twelve times (counts by ballot; at
+        // least k candidates stay at or above it), puts what is at or above it side by side, still in index
+        // order, and runs the list phase on that short list.
+        if (wave == 0) {
+          constexpr int HELD = 2 * TOP_K_PARTS;
+          float held[HELD];
+#pragma unroll
+          for (int i = 0; i < HELD; ++i) {
+            const int pp = i >> 1, j = lane + (i & 1) * WAVE;
+            held[i] = (pp < n_parts && j < part_n[pp]) ? mine[pp * PART_WORDS + 4 + j] : -INFINITY;
+          }
+          float lo = bound, hi = m;
+          if (lo > -INFINITY) {
+            for (int it = 0; it < 12; ++it) {
+              const float mid = 0.5f * (lo + hi);
+              if (!(mid > lo && mid < hi)) break;
+              int c = 0;
+#pragma unroll
+              for (int i = 0; i < HELD; ++i) c += __popcll(__ballot(held[i] >= mid));
+              if (c >= k_row) lo = mid; else hi = mid;
+            }
+          }
+          int n_all = 0;
+#pragma unroll
+          for (int i = 0; i < HELD; ++i) {
+            const int pp = i >> 1, j = lane + (i & 1) * WAVE;
+            const bool keep = pp < n_parts && j < part_n[pp] && held[i] >= lo;
+            const unsigned long long kept = __ballot(keep);
+            const int o = n_all + __popcll(kept & ((1ull << lane) - 1ull));
+            if (keep && o < 4 * WAVE) {
+              cand.lz[o] = held[i];
+              cand.le[o] = __builtin_amdgcn_exp2f((held[i] - m) * L2E);
+              cand.lidx[o] = mine_i[pp * PART_WORDS + 4 + PART_CAND + j];
+            }
+            n_all += __popcll(kept);
+          }
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+          __builtin_amdgcn_wave_barrier();
+          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+          if (n_all <= 4 * WAVE) {
+            const int token = draw_from_short_list(cand, n_all, true, k_row, p_row, mp_row, 0.f, order_key(lo), order_key(m),
+                                                   uniform, lane);
+            if (lane == 0) { out[row] = token; chosen = 0; }
+          } else if (lane == 0) {
+            chosen = -1;                    // many equal values around the k-th largest: the long way
+          }
+        }
+        __syncthreads();
+        if (chosen >= 0) return;
+      }
+    } else {
+      // every part's sum, brought to the row's maximum, in order; the part in which the running sum passes the target
+      float total = 0.f;
+      for (int p = 0; p < n_parts; ++p) total += part_s[p] * __builtin_amdgcn_exp2f((part_m[p] - m) * L2E);
+      const float target = uniform * total;
+      float run = 0.f;
+      int in_part = -1;
+      for (int p = 0; p < n_parts && in_part < 0; ++p) {
+        const float w = part_s[p] * __builtin_amdgcn_exp2f((part_m[p] - m) * L2E);
+        if (w > 0.f && run + w > target) in_part = p;
+        else run += w;
+      }
+      if (in_part >= 0) {
+        const int rbeg = in_part * PART_VALUES;
+        const int picked = walk_range<VEC>(x, rbeg, rbeg + PART_VALUES < V ? rbeg + PART_VALUES : V, run, target, inv_t, m,
+                                           0u, 0.f, step_sum, step_kept);
+        if (picked >= 0) {
+          if (tid == 0) out[row] = picked;
+          return;
+        }
+      }
+    }
+    __syncthreads();                        // the way over the whole vocabulary
+  }
 
   if (t == 0.f) {  // greedy: first index of the maximum
     float best = -INFINITY;
@@ -337,12 +810,11 @@ sample_kernel(const float* __restrict__ logits, int V, int ld, const float* __re
   uint32_t kmin = 0;
 #define E_OF(z) __builtin_amdgcn_exp2f(((z) - m) * L2E)
 
-  const int k = top_k[row];
-  const bool top_k_on = k > 0 && k < V, top_p_on = top_p[row] > 0.f && top_p[row] < 1.f;
+  const int k = k_row;
+  const bool top_k_on = k > 0 && k < V, top_p_on = p_row > 0.f && p_row < 1.f;
   if (((top_k_on && k <= SMALL_K_MAX) || (!top_k_on && top_p_on)) && blockDim.x == SAMPLE_THREADS) {
-    const uint64_t seed = ((uint64_t)seed_hi[row] << 32) | (uint64_t)seed_lo[row];
-    const int token = sample_small_k<VEC>(x, wbeg, wend, inv_t, m, top_k_on ? k : 0, top_p[row], min_p[row],
-                                          uniform_from_seed(seed, (uint32_t)position[row]), cand, fscratch, iscratch);
+    const int token = sample_small_k<VEC>(x, wbeg, wend, inv_t, m, top_k_on ? k : 0, p_row, mp_row,
+                                          uniform_from_seed(seed, position_row), cand, fscratch, iscratch);
     if (token >= 0) {
       if (tid == 0) out[row] = token;
       return;
@@ -360,7 +832,7 @@ sample_kernel(const float* __restrict__ logits, int V, int ld, const float* __re
     kmin = lo;
   }
 
-  const float p = top_p[row];
+  const float p = p_row;
   if (p > 0.f && p < 1.f) {  // smallest key v with (mass of keys > v) < p * (mass kept so far)
     float s = 0.f;
     for_range<VEC>(x, wbeg, wend, lane, [&](int, float v) {
@@ -381,7 +853,7 @@ sample_kernel(const float* __restrict__ logits, int V, int ld, const float* __re
     kmin = lo;
   }
 
-  const float mp = min_p[row];
+  const float mp = mp_row;
   float s = 0.f;
   if (kmin == 0 && !(mp > 0.f)) {          // nothing filtered: every value counts (3 instructions a value)
     for_range<VEC, 8>(x, wbeg, wend, lane, [&](int, float v) { s += E_OF(v * inv_t); });
@@ -401,94 +873,18 @@ sample_kernel(const float* __restrict__ logits, int V, int ld, const float* __re
     if (w == wave) base = total;
     total += wave_tot[w];
   }
-  const uint64_t seed = ((uint64_t)seed_hi[row] << 32) | (uint64_t)seed_lo[row];
-  const float target = uniform_from_seed(seed, (uint32_t)position[row]) * total;
+  const float target = uniform_from_seed(seed, position_row) * total;
   const bool mine = s > 0.f && base + s > target && !(base > target);   // exactly one wave
   if (mine && lane == 0) range_of = wave;
   __syncthreads();
   const int rw = range_of;
   if (rw >= 0) {
-    // The draw lies in wave rw's range.  The walk over it in index order, STEP values at a time, is a chain
-    // of sums; the sums of the steps are not: the block's waves take the steps of the range in turn, then
-    // every thread adds the steps' sums in order until one crosses the target, and adds that step's values
-    // one by one.  The additions and their order are those of a walk by one wave.
-    constexpr int PER = VEC ? 4 : 1;
-    constexpr int HELD = 4;                 // steps a wave takes per round
-    const int rbeg = rw * per < V ? rw * per : V;
-    const int rend = rbeg + per < V ? rbeg + per : V;
     float run = 0.f;
     for (int w = 0; w < rw; ++w) run += wave_tot[w];
-    int pick = -1, last_kept = -1;
-    // the values of the step at i0 that count, as a lane holds them; the highest index among them that counts
-    auto weights_of = [&](const float (&cur)[PER], int i0, float (&e)[PER], int& kept_hi) {
-      kept_hi = -1;
-#pragma unroll
-      for (int c = 0; c < PER; ++c) {
-        const int i = i0 + PER * lane + c;
-        const float z = cur[c] * inv_t;
-        const float ev = E_OF(z);
-        e[c] = (i < rend && order_key(z) >= kmin && ev >= mp) ? ev : 0.f;
-        if (e[c] > 0.f) kept_hi = i;
-      }
-#pragma unroll
-      for (int sft = WAVE / 2; sft > 0; sft >>= 1) { const int o = __shfl_xor(kept_hi, sft, WAVE); kept_hi = o > kept_hi ? o : kept_hi; }
-    };
-    auto fetch = [&](int i0, float (&dst)[PER]) {
-      const int last = rend - PER;          // rend - rbeg is a multiple of PER, and the range is not empty
-      if (VEC) {
-        const int ii = i0 + 4 * lane;
-        const float4 v = *reinterpret_cast<const float4*>(x + (ii < last ? ii : last));
-        dst[0] = v.x; if (PER > 1) { dst[1] = v.y; dst[2] = v.z; dst[3] = v.w; }
-      } else {
-        const int ii = i0 + lane;
-        dst[0] = x[ii < last ? ii : last];
-      }
-    };
-    const int round_span = HELD * nwaves * STEP;
-    for (int r0 = rbeg; r0 < rend && pick < 0; r0 += round_span) {
-      float cur[HELD][PER];
-#pragma unroll
-      for (int j = 0; j < HELD; ++j) fetch(r0 + (wave + nwaves * j) * STEP, cur[j]);
-#pragma unroll
-      for (int j = 0; j < HELD; ++j) {
-        const int i0 = r0 + (wave + nwaves * j) * STEP;
-        float e[PER], esum = 0.f;
-        int kept_hi;
-        weights_of(cur[j], i0, e, kept_hi);
-#pragma unroll
-        for (int c = 0; c < PER; ++c) esum += e[c];
-        const float step = wave_sum(esum);
-        if (lane == 0) { step_sum[wave + nwaves * j] = step; step_kept[wave + nwaves * j] = kept_hi; }
-      }
-      __syncthreads();
-      const float my_step = step_sum[lane];
-      const int my_kept = step_kept[lane];
-      const int steps_here = (rend - r0 + STEP - 1) / STEP < HELD * nwaves ? (rend - r0 + STEP - 1) / STEP : HELD * nwaves;
-      for (int c = 0; c < steps_here && pick < 0; ++c) {
-        const float step = __shfl(my_step, c, WAVE);
-        const int kept_hi = __shfl(my_kept, c, WAVE);
-        if (kept_hi >= 0) last_kept = kept_hi;
-        if (run + step > target) {            // the crossing is among these: add them one by one
-          const int i0 = r0 + c * STEP;
-          float one[PER], e[PER];
-          int unused;
-          fetch(i0, one);
-          weights_of(one, i0, e, unused);
-          for (int j = 0; j < WAVE && pick < 0; ++j) {
-#pragma unroll
-            for (int cc = 0; cc < PER; ++cc) {
-              const float ej = __shfl(e[cc], j, WAVE);
-              run += ej;
-              if (pick < 0 && ej > 0.f && run > target) pick = i0 + PER * j + cc;
-            }
-          }
-        } else {
-          run += step;
-        }
-      }
-      __syncthreads();                        // the next round writes the steps' sums again
-    }
-    if (tid == 0) chosen = pick >= 0 ? pick : last_kept;
+    const int rbeg = rw * per < V ? rw * per : V;
+    const int picked = walk_range<VEC>(x, rbeg, rbeg + per < V ? rbeg + per : V, run, target, inv_t, m, kmin, mp,
+                                       step_sum, step_kept);
+    if (tid == 0) chosen = picked;
   }
   __syncthreads();
   if (chosen < 0) {  // rounding pushed the target past the total: take the last kept index
@@ -513,18 +909,36 @@ sample_kernel(const float* __restrict__ logits, int V, int ld, const float* __re
 #undef E_OF
 }
 
+// Floats of workspace with which ullm_sample cuts the rows into parts (0: it would not: rows that are not
+// 16-byte aligned, or a vocabulary of more than MAX_PARTS parts).
+extern "C" long long ullm_sample_workspace(int n_rows, int V, int ld) {
+  if (n_rows <= 0 || V <= 0 || V % 4 || ld % 4 || n_rows > 65535) return 0;
+  const int n_parts = (V + PART_VALUES - 1) / PART_VALUES;
+  return n_parts > MAX_PARTS ? 0 : (long long)n_rows * n_parts * PART_WORDS;
+}
+
+// `workspace`: null, or ullm_sample_workspace(n_rows, V, ld) floats (then, if that is not 0, the rows are cut into
+// parts by a first kernel).
 extern "C" int ullm_sample(const float* logits, int n_rows, int V, int ld, const float* temperature,
                            const int* top_k, const float* top_p, const float* min_p,
                            const unsigned* seed_lo, const unsigned* seed_hi, const int* position,
-                           int* out, hipStream_t stream) {
+                           int* out, float* workspace, hipStream_t stream) {
   if (n_rows <= 0) return 0;
   if (V <= 0 || ld < V) return ULLM_ERR_SHAPE;
   const bool vec = V % 4 == 0 && ld % 4 == 0 && !((uintptr_t)logits & 15);
+  const int n_parts = (V + PART_VALUES - 1) / PART_VALUES;
+  float* const parts = vec && workspace && ullm_sample_workspace(n_rows, V, ld) > 0 ? workspace : nullptr;
+  if (parts) {
+    hipLaunchKernelGGL(sample_parts_kernel, dim3(n_parts, n_rows), dim3(PART_THREADS), 0, stream, logits, V, ld,
+                       temperature, top_k, top_p, min_p, parts, n_parts);
+    const int rc = (int)hipGetLastError();
+    if (rc != 0) return rc;
+  }
   if (vec)
     hipLaunchKernelGGL(sample_kernel<true>, dim3(n_rows), dim3(SAMPLE_THREADS), 0, stream, logits, V, ld,
-                       temperature, top_k, top_p, min_p, seed_lo, seed_hi, position, out);
+                       temperature, top_k, top_p, min_p, seed_lo, seed_hi, position, out, parts, n_parts);
   else
     hipLaunchKernelGGL(sample_kernel<false>, dim3(n_rows), dim3(SAMPLE_THREADS), 0, stream, logits, V, ld,
-                       temperature, top_k, top_p, min_p, seed_lo, seed_hi, position, out);
+                       temperature, top_k, top_p, min_p, seed_lo, seed_hi, position, out, nullptr, 0);
   ULLM_LAUNCH_CHECK();
 }

@@ -741,11 +741,16 @@ def paged_attention(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
 
 # ---------------------------------------------------------------------------------- sampling
 
+SAMPLE_PARTS_TOP_K = 64     # the largest top-k that the sampling kernels serve from parts of a row (PART_K_MAX)
+
+
 def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
            min_p: torch.Tensor, seed_lo: torch.Tensor, seed_hi: torch.Tensor, position: torch.Tensor,
-           out: Optional[torch.Tensor] = None) -> torch.Tensor:
+           out: Optional[torch.Tensor] = None, parts: bool = True) -> torch.Tensor:
     """One token id per row of float32 ``logits`` [n, V].  Per-row parameters: temperature (0 =
-    greedy), top_k (<= 0 = all), top_p, min_p (float32), seed halves and position (int32)."""
+    greedy), top_k (<= 0 = all), top_p, min_p (float32), seed halves and position (int32).  ``parts``: a first
+    kernel cuts the rows into parts over many blocks where the settings allow (False: one block per row does
+    everything)."""
     n, V = logits.shape
     _need(logits.dtype == torch.float32 and logits.stride(1) == 1, "logits must be float32 with unit stride")
     for t, nm, dt in ((temperature, "temperature", torch.float32), (top_k, "top_k", torch.int32),
@@ -757,7 +762,10 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
         out = torch.empty((n,), dtype=torch.int32, device=logits.device)
     _need(out.dtype == torch.int32 and out.numel() >= n and out.is_contiguous(), "bad sample output")
     lib = build.load("sampling")
+    lib.ullm_sample_workspace.restype = ctypes.c_longlong
+    need = int(lib.ullm_sample_workspace(_c_int(n), _c_int(V), _c_int(logits.stride(0)))) if parts else 0
+    ws = torch.empty(need, dtype=torch.float32, device=logits.device) if need > 0 else None
     _check(lib.ullm_sample(_p(logits), _c_int(n), _c_int(V), _c_int(logits.stride(0)), _p(temperature), _p(top_k),
-                           _p(top_p), _p(min_p), _p(seed_lo), _p(seed_hi), _p(position), _p(out), _stream()),
+                           _p(top_p), _p(min_p), _p(seed_lo), _p(seed_hi), _p(position), _p(out), _p(ws), _stream()),
            "sample")
     return out

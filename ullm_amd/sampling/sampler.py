@@ -20,11 +20,13 @@ class SamplerInputs:
     """Per-row parameters on the device: rows of one int32 buffer (the float ones bit-cast)."""
     n: int
     packed: torch.Tensor      # int32 [7, n]: temperature, top_p, min_p (float bits), top_k, seed low, seed high, position
+    cut_rows: bool = True     # some row has settings for which the kernels cut rows into parts (ops.sample)
 
 
 class Sampler:
-    def __init__(self, device: torch.device):
+    def __init__(self, device: torch.device, cut_rows: bool = True):
         self.device = device
+        self.cut_rows = cut_rows      # False: one block per row does all the work (ops.sample)
         self._upload = StagedUpload(device)
 
     def stage(self, params: Sequence[SamplingParams], seeds: Sequence[int], positions: Sequence[int]) -> torch.Tensor:
@@ -34,7 +36,8 @@ class Sampler:
         n = len(params)
         if not (len(seeds) == len(positions) == n):
             raise ValueError("one parameter set, seed and position per logits row is needed")
-        host = np.empty((7, n), dtype=np.int32)
+        flat = np.empty(7 * n + 1, dtype=np.int32)
+        host = flat[:7 * n].reshape(7, n)
         host[0:3].view(np.float32)[:] = [[p.temperature for p in params], [p.top_p for p in params],
                                          [p.min_p for p in params]]
         host[3] = [p.top_k for p in params]
@@ -42,13 +45,18 @@ class Sampler:
         host[4] = (s64 & np.uint64(0xFFFFFFFF)).astype(np.uint32).view(np.int32)
         host[5] = (s64 >> np.uint64(32)).astype(np.uint32).view(np.int32)
         host[6] = positions
-        return self._upload.stage(host.reshape(-1))
+        # one more word, for the host alone: whether any row has settings that the kernels serve by cutting rows
+        # into parts (temperature alone, or top-k up to ops.SAMPLE_PARTS_TOP_K); without one, that kernel is not launched
+        flat[-1] = int(any(p.temperature != 0 and (0 < p.top_k <= ops.SAMPLE_PARTS_TOP_K or
+                                                   (p.top_k <= 0 and not 0 < p.top_p < 1 and not p.min_p > 0))
+                           for p in params))
+        return self._upload.stage(flat)
 
     def send(self, staged: torch.Tensor) -> SamplerInputs:
         """Queue the upload of staged parameters.  Called before the model step is launched, the copy
         does not wait for the step, and sampling can follow it without the host in between."""
         n = staged.numel() // 7
-        return SamplerInputs(n, self._upload.send(staged).view(7, n))
+        return SamplerInputs(n, self._upload.send(staged)[:7 * n].view(7, n), bool(int(staged[-1])))
 
     def prepare(self, params: Sequence[SamplingParams], seeds: Sequence[int], positions: Sequence[int]) -> SamplerInputs:
         return self.send(self.stage(params, seeds, positions))
@@ -60,7 +68,8 @@ class Sampler:
             raise ValueError("one parameter set, seed and position per logits row is needed")
         f = prepared.packed[0:3].view(torch.float32)
         i = prepared.packed
-        return ops.sample(logits, f[0], i[3], f[1], f[2], i[4], i[5], i[6], out=out)[:prepared.n]
+        return ops.sample(logits, f[0], i[3], f[1], f[2], i[4], i[5], i[6], out=out,
+                          parts=self.cut_rows and prepared.cut_rows)[:prepared.n]
 
     def sample(self, logits: torch.Tensor, params: Optional[Sequence[SamplingParams]] = None,
                seeds: Optional[Sequence[int]] = None, positions: Optional[Sequence[int]] = None,
