@@ -187,6 +187,43 @@ def test_qk_norm_rope_write(ops, dtype, cfg):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("cfg", [dict(nq=32, nkv=8, hd=128, P=16, rot=128, style=1),    # 48 heads: three in turn per thread
+                                 dict(nq=70, nkv=2, hd=32, P=8, rot=32, style=2),       # 74 heads of 4 lanes: two in turn
+                                 dict(nq=5, nkv=1, hd=128, P=16, rot=64, style=2),      # 7 heads: one block, one turn
+                                 dict(nq=40, nkv=40, hd=64, P=16, rot=32, style=1)])    # 120 heads: four in turn, a spare turn
+def test_qk_norm_rope_write_of_a_long_prompt(ops, dtype, cfg):
+    """From 1 024 tokens on a thread takes several heads in turn with one fetch of its cosines and sines; what it
+    writes is, bit for bit, what the same tokens give in portions below that length (which the test above
+    checks against the plain formulas)."""
+    torch.manual_seed(41)
+    nq, nkv, hd, P, rot, style = (cfg[k] for k in ("nq", "nkv", "hd", "P", "rot", "style"))
+    T = 1100
+    positions = torch.arange(T, dtype=torch.int32, device=DEV)
+    entry = torch.zeros(T, dtype=torch.int32, device=DEV)
+    n_pages = -(-T // P)
+    bt = table_tensor([torch.randperm(n_pages).tolist()], DEV)
+    qkv = torch.randn(T, (nq + 2 * nkv) * hd).to(dtype).to(DEV)
+    qg, kg = (1 + 0.2 * torch.randn(hd)).to(DEV), (1 + 0.2 * torch.randn(hd)).to(DEV)
+    inv = 1.0 / (10000.0 ** (torch.arange(0, rot, 2, dtype=torch.float32) / rot))
+    ang = torch.arange(T + 5, dtype=torch.float32)[:, None] * inv[None]
+    table = torch.cat((ang.cos(), ang.sin()), -1).contiguous().to(DEV)
+    results = []
+    for portions in ([T], [500, 400, 200]):
+        k_pool = torch.zeros(n_pages, nkv, P, hd, dtype=dtype, device=DEV)
+        v_pool = torch.zeros(n_pages, nkv, hd, P, dtype=dtype, device=DEV)
+        q_out = torch.zeros(T, nq * hd, dtype=dtype, device=DEV)
+        at = 0
+        for n in portions:
+            ops.qk_norm_rope_write(qkv[at:at + n], q_out[at:at + n], qg, kg, 1e-6, table, rot, style, positions[at:at + n],
+                                   entry[at:at + n], bt, k_pool, v_pool, P, nq, nkv, hd, write_kv=True)
+            at += n
+        results.append((q_out, k_pool, v_pool))
+    for whole, cut in zip(*results):
+        assert torch.equal(whole, cut)
+    assert float(results[0][0].float().abs().sum()) > 0 and float(results[0][1].float().abs().sum()) > 0
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("cfg", [dict(nq=8, nkv=2, hd=128, P=16), dict(nq=4, nkv=4, hd=64, P=8),
                                  dict(nq=2, nkv=1, hd=256, P=32), dict(nq=4, nkv=2, hd=32, P=24),
                                  dict(nq=4, nkv=2, hd=64, P=12),      # pages that do not hold whole groups of 8

@@ -571,7 +571,7 @@ __device__ __forceinline__ void value_runs_block(
 
 // The same for head sizes of 8 * (a power of two): a head is held by head_dim / 8 neighbouring lanes
 // with 8 consecutive dims each (16-byte loads and stores for bfloat16), a block of 256 threads takes
-// 2048 / head_dim heads of one token.  For half-split pairs the partner dims come from the lane
+// 2048 / head_dim heads of one token at a time, heads_per_thread times in turn.  For half-split pairs the partner dims come from the lane
 // rot / 16 further on (or back) by shuffles, which needs rot to be a multiple of 16.
 template <typename T>
 __global__ void __launch_bounds__(256)
@@ -581,7 +581,7 @@ qk_norm_rope_write_vec_kernel(
     const float* __restrict__ cos_sin, int table_rows, int rot, int style,
     const int* __restrict__ positions, const int* __restrict__ token_entry,
     const int* __restrict__ block_table, int bt_stride, T* __restrict__ k_pool, T* __restrict__ v_pool,
-    int page_size, int nq, int nkv, int hd, int write_kv, int n_tokens, int blocks_per_token) {
+    int page_size, int nq, int nkv, int hd, int write_kv, int n_tokens, int blocks_per_token, int heads_per_thread) {
   if (blockIdx.x >= (unsigned)(n_tokens * blocks_per_token)) {
     value_runs_block<T>(qkv, qkv_stride, positions, token_entry, block_table, bt_stride, v_pool, page_size, nq, nkv,
                         hd, n_tokens, (int)blockIdx.x - n_tokens * blocks_per_token);
@@ -589,87 +589,98 @@ qk_norm_rope_write_vec_kernel(
   }
   const int lph = hd >> 3;                                  // lanes per head
   const int t = blockIdx.x / blocks_per_token;
-  const int head = (blockIdx.x % blocks_per_token) * (256 / lph) + threadIdx.x / lph, part = threadIdx.x % lph, d0 = 8 * part;
-  const bool live = head < nq + 2 * nkv;
+  const int part = threadIdx.x % lph, d0 = 8 * part;
   const int pos = positions[t];
-  const bool is_q = head < nq, is_k = !is_q && head < nq + nkv;
-  float x[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  if (live) {
-    const T* src = qkv + (size_t)t * qkv_stride + (size_t)head * hd + d0;
-    const float4 lo = ld4_f32_stream(src), hi = ld4_f32_stream(src + 4);     // the projection row is read once
-    x[0] = lo.x; x[1] = lo.y; x[2] = lo.z; x[3] = lo.w; x[4] = hi.x; x[5] = hi.y; x[6] = hi.z; x[7] = hi.w;
-  }
-  int page = -1;
-  if (live && !is_q && (write_kv & (is_k ? 1 : 2)))
-    page = block_table[(size_t)token_entry[t] * bt_stride + pos / page_size];
   const int off = pos % page_size;
-  if (live && !is_q && !is_k) {                             // v: transposed copy, no arithmetic
-    if (page >= 0) {
-      const int kvh = head - nq - nkv;
-      T* vdst = v_pool + ((size_t)page * nkv + kvh) * hd * page_size + (size_t)d0 * page_size + off;
-#pragma unroll
-      for (int j = 0; j < 8; ++j) st_f32(vdst + (size_t)j * page_size, x[j]);
-    }
-  }
-  // every lane takes part in the shuffles below; lanes of value heads and dead lanes carry zeros
-  const float* gain = is_q ? q_gain : k_gain;
-  const bool arith = live && (is_q || is_k);
-  if (gain) {
-    float ss = 0.f;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) ss = fmaf(x[j], x[j], ss);
-    // pairwise, the most distant lanes of a head first: the decode attention kernel, which does this
-    // norm itself for single new tokens, adds in the same order (multiply-adds spelled out in both)
-    for (int m = lph >> 1; m > 0; m >>= 1) ss += __shfl_xor(ss, m, WAVE);
-    const float rs = rsqrtf(ss / (float)hd + eps);
-    if (arith) {
-      const float4 g0 = *reinterpret_cast<const float4*>(gain + d0), g1 = *reinterpret_cast<const float4*>(gain + d0 + 4);
-      const float gg[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
-#pragma unroll
-      for (int j = 0; j < 8; ++j) x[j] = (x[j] * rs) * gg[j];
-    }
-  }
-  if (style != 0 && rot > 0) {
-    const int half = rot / 2;
+  // what depends on the token and the lane's dims alone is fetched once for all the heads the thread takes
+  const bool rotates = style != 0 && rot > 0;
+  const int half = rot / 2;
+  const bool first = d0 < half, in = d0 < rot;              // rot and half are multiples of 8: a lane is on one side
+  float c[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, sn[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  const float* cs = nullptr;
+  if (rotates) {
     const int p = pos < table_rows ? pos : table_rows - 1;  // host rejects positions past the table
-    const float* cs = cos_sin + (size_t)p * rot;
-    if (style == 1) {
-      const bool first = d0 < half, in = d0 < rot;         // rot and half are multiples of 8: a lane is on one side
-      const int src_lane = (int)(threadIdx.x & (WAVE - 1)) + (first ? half / 8 : -(half / 8));
-      float y[8];
+    cs = cos_sin + (size_t)p * rot;
+    if (style == 1 && in) {
+      const int i0 = first ? d0 : d0 - half;
+      const float4 c0 = *reinterpret_cast<const float4*>(cs + i0), c1 = *reinterpret_cast<const float4*>(cs + i0 + 4);
+      const float4 s0 = *reinterpret_cast<const float4*>(cs + half + i0), s1 = *reinterpret_cast<const float4*>(cs + half + i0 + 4);
+      c[0] = c0.x; c[1] = c0.y; c[2] = c0.z; c[3] = c0.w; c[4] = c1.x; c[5] = c1.y; c[6] = c1.z; c[7] = c1.w;
+      sn[0] = s0.x; sn[1] = s0.y; sn[2] = s0.z; sn[3] = s0.w; sn[4] = s1.x; sn[5] = s1.y; sn[6] = s1.z; sn[7] = s1.w;
+    }
+  }
+  for (int pass = 0; pass < heads_per_thread; ++pass) {
+    const int head = ((blockIdx.x % blocks_per_token) * heads_per_thread + pass) * (256 / lph) + threadIdx.x / lph;
+    const bool live = head < nq + 2 * nkv;
+    const bool is_q = head < nq, is_k = !is_q && head < nq + nkv;
+    float x[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if (live) {
+      const T* src = qkv + (size_t)t * qkv_stride + (size_t)head * hd + d0;
+      const float4 lo = ld4_f32_stream(src), hi = ld4_f32_stream(src + 4);     // the projection row is read once
+      x[0] = lo.x; x[1] = lo.y; x[2] = lo.z; x[3] = lo.w; x[4] = hi.x; x[5] = hi.y; x[6] = hi.z; x[7] = hi.w;
+    }
+    int page = -1;
+    if (live && !is_q && (write_kv & (is_k ? 1 : 2)))
+      page = block_table[(size_t)token_entry[t] * bt_stride + pos / page_size];
+    if (live && !is_q && !is_k) {                             // v: transposed copy, no arithmetic
+      if (page >= 0) {
+        const int kvh = head - nq - nkv;
+        T* vdst = v_pool + ((size_t)page * nkv + kvh) * hd * page_size + (size_t)d0 * page_size + off;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) y[j] = __shfl(x[j], in ? src_lane : (int)(threadIdx.x & (WAVE - 1)), WAVE);
-      if (in && arith) {
-        const int i0 = first ? d0 : d0 - half;
-        const float4 c0 = *reinterpret_cast<const float4*>(cs + i0), c1 = *reinterpret_cast<const float4*>(cs + i0 + 4);
-        const float4 s0 = *reinterpret_cast<const float4*>(cs + half + i0), s1 = *reinterpret_cast<const float4*>(cs + half + i0 + 4);
-        const float c[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
-        const float sn[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
-#pragma unroll
-        for (int j = 0; j < 8; ++j) x[j] = first ? fmaf(x[j], c[j], -(y[j] * sn[j])) : fmaf(x[j], c[j], y[j] * sn[j]);
+        for (int j = 0; j < 8; ++j) st_f32(vdst + (size_t)j * page_size, x[j]);
       }
-    } else if (arith) {
+    }
+    // every lane takes part in the shuffles below; lanes of value heads and dead lanes carry zeros
+    const float* gain = is_q ? q_gain : k_gain;
+    const bool arith = live && (is_q || is_k);
+    if (gain) {
+      float ss = 0.f;
 #pragma unroll
-      for (int j = 0; j < 8; j += 2) {
-        if (d0 + j < rot) {
-          const int i = (d0 + j) >> 1;
-          const float c = cs[i], sn = cs[half + i], a = x[j], b = x[j + 1];
-          x[j] = a * c - b * sn;
-          x[j + 1] = b * c + a * sn;
+      for (int j = 0; j < 8; ++j) ss = fmaf(x[j], x[j], ss);
+      // pairwise, the most distant lanes of a head first: the decode attention kernel, which does this
+      // norm itself for single new tokens, adds in the same order (multiply-adds spelled out in both)
+      for (int m = lph >> 1; m > 0; m >>= 1) ss += __shfl_xor(ss, m, WAVE);
+      const float rs = rsqrtf(ss / (float)hd + eps);
+      if (arith) {
+        const float4 g0 = *reinterpret_cast<const float4*>(gain + d0), g1 = *reinterpret_cast<const float4*>(gain + d0 + 4);
+        const float gg[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
+#pragma unroll
+        for (int j = 0; j < 8; ++j) x[j] = (x[j] * rs) * gg[j];
+      }
+    }
+    if (rotates) {
+      if (style == 1) {
+        const int src_lane = (int)(threadIdx.x & (WAVE - 1)) + (first ? half / 8 : -(half / 8));
+        float y[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) y[j] = __shfl(x[j], in ? src_lane : (int)(threadIdx.x & (WAVE - 1)), WAVE);
+        if (in && arith) {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) x[j] = first ? fmaf(x[j], c[j], -(y[j] * sn[j])) : fmaf(x[j], c[j], y[j] * sn[j]);
+        }
+      } else if (arith) {
+#pragma unroll
+        for (int j = 0; j < 8; j += 2) {
+          if (d0 + j < rot) {
+            const int i = (d0 + j) >> 1;
+            const float cc = cs[i], ss2 = cs[half + i], a = x[j], b2 = x[j + 1];
+            x[j] = a * cc - b2 * ss2;
+            x[j + 1] = b2 * cc + a * ss2;
+          }
         }
       }
     }
+    if (!arith) continue;
+    T* dst;
+    if (is_q) {
+      dst = q_out + (size_t)t * q_out_stride + (size_t)head * hd + d0;
+    } else {
+      if (page < 0) continue;
+      dst = k_pool + (((size_t)page * nkv + (head - nq)) * page_size + off) * hd + d0;
+    }
+    st4_f32(dst, make_float4(x[0], x[1], x[2], x[3]));
+    st4_f32(dst + 4, make_float4(x[4], x[5], x[6], x[7]));
   }
-  if (!arith) return;
-  T* dst;
-  if (is_q) {
-    dst = q_out + (size_t)t * q_out_stride + (size_t)head * hd + d0;
-  } else {
-    if (page < 0) return;
-    dst = k_pool + (((size_t)page * nkv + (head - nq)) * page_size + off) * hd + d0;
-  }
-  st4_f32(dst, make_float4(x[0], x[1], x[2], x[3]));
-  st4_f32(dst + 4, make_float4(x[4], x[5], x[6], x[7]));
 }
 
 extern "C" int ullm_qk_norm_rope_write(
@@ -689,8 +700,15 @@ extern "C" int ullm_qk_norm_rope_write(
                    (!cos_sin || ((uintptr_t)cos_sin & 15) == 0) && (!q_gain || ((uintptr_t)q_gain & 15) == 0) &&
                    (!k_gain || ((uintptr_t)k_gain & 15) == 0) && rot % 8 == 0;
   if (vec) {
+    // with few tokens a thread takes one head, so that many blocks are under way; with many it takes up to four
+    // in turn, for which it fetches its cosines and sines once
     const int heads_per_block = 256 / lph;
-    const int blocks_per_token = (nq + 2 * nkv + heads_per_block - 1) / heads_per_block;
+    int blocks_per_token = (nq + 2 * nkv + heads_per_block - 1) / heads_per_block;
+    int heads_per_thread = 1;
+    if (T_ >= 1024) {
+      heads_per_thread = blocks_per_token < 4 ? blocks_per_token : 4;
+      blocks_per_token = (blocks_per_token + heads_per_thread - 1) / heads_per_thread;
+    }
     // with many tokens the values go through blocks of their own that write runs of eight at once
     const bool runs = write_kv && T_ >= 128 && page_size % 8 == 0 && hd <= VALUE_RUN_MAX_HD &&
                       ((uintptr_t)v_pool & 15) == 0;
@@ -702,7 +720,7 @@ extern "C" int ullm_qk_norm_rope_write(
 #define GOV(TT) hipLaunchKernelGGL(qk_norm_rope_write_vec_kernel<TT>, vgrid, vblock, 0, stream, \
     (const TT*)qkv, qkv_stride, (TT*)q_out, q_out_stride, q_gain, k_gain, eps, cos_sin, table_rows, \
     rot, style, positions, token_entry, block_table, bt_stride, (TT*)k_pool, (TT*)v_pool, page_size, \
-    nq, nkv, hd, kv_flags, T_, blocks_per_token)
+    nq, nkv, hd, kv_flags, T_, blocks_per_token, heads_per_thread)
     if (dtype == ULLM_F32) GOV(float);
     else if (dtype == ULLM_BF16) GOV(bf16_t);
     else return ULLM_ERR_DTYPE;
