@@ -70,7 +70,10 @@ class EngineConfig:
     profile_dir: str = "./profiles"             # where those traces are written
     # -- beyond the reference ------------------------------------------------------
     dtype: str = "bfloat16"                     # "bfloat16" | "float32" (whole model in true 32-bit)
-    page_size: int = 16                         # tokens per cache page
+    page_size: int = 16                         # tokens per cache page.  16 is what the decode attention kernel reads in one
+                                                # piece: values lie transposed in a page, [head_dim, page_size], and a
+                                                # wave takes 16 keys of 16 dims per load, so with longer pages it uses a
+                                                # part of every line it fetches (measured 1.2x slower at 32, 2x at 64)
     num_pages: Optional[int] = None             # pages of every cache group; None: from memory
     max_num_batched_tokens: int = 2048          # token budget of one step
     max_prefill_chunk: int = 2048               # longest prompt portion given to one request per step
