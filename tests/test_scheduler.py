@@ -176,3 +176,25 @@ def test_batch_buckets_of_the_captured_decode_graphs():
     for n in range(1, 600):
         b = batch_bucket(n)
         assert b >= n and batch_bucket(b) == b and (n <= 32 or 2 * b < 3 * n)
+
+
+def test_sampler_stages_one_word_for_the_host_beside_the_rows():
+    """The staged parameters are seven words a row and one more that only the host reads: whether any row has
+    settings that the sampling kernels serve by cutting rows into parts (temperature alone, a small top-k)."""
+    import torch
+    from ullm_amd.sampling import Sampler, SamplingParams
+    sampler = Sampler(torch.device("cpu"))
+    cases = [([SamplingParams(temperature=0.0)] * 3, False),
+             ([SamplingParams(temperature=0.0), SamplingParams(temperature=0.7)], True),
+             ([SamplingParams(temperature=0.7, top_p=0.9)], False),
+             ([SamplingParams(temperature=0.7, top_k=20, top_p=0.9, min_p=0.05)], True),
+             ([SamplingParams(temperature=0.7, top_k=100)], False),
+             ([SamplingParams(temperature=0.7, min_p=0.1)], False)]
+    for params, cut in cases:
+        n = len(params)
+        staged = sampler.stage(params, list(range(n)), [5] * n)
+        assert staged.numel() == 7 * n + 1
+        inputs = sampler.send(staged)
+        assert inputs.n == n and inputs.packed.shape == (7, n) and inputs.cut_rows is cut
+        assert inputs.packed[3].tolist() == [p.top_k for p in params]
+        assert inputs.packed[6].tolist() == [5] * n
