@@ -1,6 +1,6 @@
 """Chooses next tokens from a step's logits on the device (reference: ullm/layers/sampler.py).
 
-One kernel launch per step for all rows; each row carries its own parameters and its own
+One or two kernel launches per step for all rows; each row carries its own parameters and its own
 (seed, position), so what a request draws does not depend on the rest of the batch."""
 from __future__ import annotations
 
