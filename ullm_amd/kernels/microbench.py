@@ -10,6 +10,8 @@ cache: the figures are those of a cold read from HBM, as in a model whose weight
   projection         a [rows, K] x [N, K]^T product by each kernel that can take it, and the library
   tune               the same for one matrix in the roles it has in a model; writes the row limits up to which
                      each kernel is ahead into the table that ullm_amd.kernels.dispatch reads
+  sampling           the sampling kernels on rows of logits, per setting, with and without the kernel that cuts rows
+                     into parts
 """
 from __future__ import annotations
 
@@ -274,6 +276,29 @@ def tune(args) -> None:
         print(f"written to {dispatch.TABLE_PATH}", flush=True)
 
 
+def sampling(args) -> None:
+    """The sampling kernels on rows of normal logits (scale 3), per setting, both ways: rows cut into parts by a
+    first kernel, and one block per row alone."""
+    V = args.vocab
+    settings = (("greedy", 0.0, -1, 1.0, 0.0), ("temperature 0.6", 0.6, -1, 1.0, 0.0),
+                ("top-k 20, top-p 0.95", 0.6, 20, 0.95, 0.0), ("top-k 50", 0.8, 50, 1.0, 0.0),
+                ("top-k 50, top-p 0.9, min-p 0.02", 0.8, 50, 0.9, 0.02), ("min-p 0.05", 0.8, -1, 1.0, 0.05),
+                ("top-p 0.9 (these rows are flat: the long way)", 0.8, -1, 0.9, 0.0))
+    for B in args.rows:
+        torch.manual_seed(0)
+        logits = torch.randn(B, V, device=DEV) * 3
+        lo, hi = torch.arange(B, dtype=torch.int32, device=DEV), torch.zeros(B, dtype=torch.int32, device=DEV)
+        pos = torch.arange(B, dtype=torch.int32, device=DEV)
+        out = torch.empty(B, dtype=torch.int32, device=DEV)
+        for name, t, k, p, mp in settings:
+            T, K = torch.full((B,), t, device=DEV), torch.full((B,), k, dtype=torch.int32, device=DEV)
+            P, MP = torch.full((B,), p, device=DEV), torch.full((B,), mp, device=DEV)
+            cut = graph_time([lambda: ops.sample(logits, T, K, P, MP, lo, hi, pos, out, parts=True)])
+            whole = graph_time([lambda: ops.sample(logits, T, K, P, MP, lo, hi, pos, out, parts=False)])
+            print(f"sampling, {B} rows of {V} logits, {name}: rows cut into parts {cut:.1f} us, one block per row {whole:.1f} us",
+                  flush=True)
+
+
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(prog="ullm_amd.kernels.microbench", description=__doc__.split("\n\n")[0])
     sub = ap.add_subparsers(dest="what", required=True)
@@ -296,9 +321,12 @@ def main(argv=None) -> int:
     p.add_argument("--roles", type=lambda s: s.split(","), required=True,
                    help="comma-separated roles of the matrix: store, silu, stream, logits")
     p.add_argument("--dry-run", action="store_true", help="measure and print, leave the table as it is")
+    p = sub.add_parser("sampling")
+    p.add_argument("--vocab", type=int, default=151936)
+    p.add_argument("--rows", type=ints, default=[1, 8, 64, 256], help="comma-separated numbers of rows of logits")
     args = ap.parse_args(argv)
     {"decode-attention": decode_attention, "prefill-attention": prefill_attention, "projection": projection,
-     "tune": tune}[args.what](args)
+     "tune": tune, "sampling": sampling}[args.what](args)
     return 0
 
 
