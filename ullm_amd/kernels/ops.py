@@ -563,8 +563,9 @@ def decode_split(n_items: int, nkv: int, groups: int, max_kv: int, hd: int = 128
     if pairs == units:
         return (4 if tiles > 16 else 1), 1
     # up to 16 blocks a pair; up to 32 where very few pairs have very many keys (one request at 4 096 keys and
-    # more: 134 MB of cache at 32 768 keys in 34 us against 49 us with 16)
-    most = 32 if (pairs * 128 <= simds and tiles >= 128) else 16
+    # more: 134 MB of cache at 32 768 keys in 34 us against 49 us with 16; three or four requests at 32 000 keys:
+    # 70 and 89 us against 89 and 93 us; two requests are better off with 16 blocks of four waves)
+    most = 32 if ((pairs * 128 <= simds and tiles >= 128) or (16 < pairs <= simds // 32 and tiles >= 512)) else 16
     splits = min(most, max(1, 2 * units // pairs), tiles)
     if tiles > 8 * splits:
         splits = min(most, max(1, simds // pairs), tiles)
