@@ -436,14 +436,15 @@ def test_sampler_with_a_small_top_k_over_a_large_vocabulary(ops):
 
 
 def test_sampler_rows_cut_into_parts(ops):
-    """Temperature alone and top-k up to 64 take sums and candidates from parts of the row that a first kernel
-    makes; the token is one the plain sampler may draw, whatever the row looks like and wherever in it the
+    """Temperature alone, top-k up to 64 and top-p without top-k take sums and candidates from parts of the row that
+    a first kernel makes (top-p where the nucleus lies within the 64 largest values of every part); the token is one the plain sampler may draw, whatever the row looks like and wherever in it the
     weight lies, and the same as in another batch position."""
     from ullm_amd.sampling import Sampler, SamplingParams
     torch.manual_seed(23)
     sampler = Sampler(torch.device(DEV))
     configs = [(0.7, -1, 1.0, 0.0), (1.0, 0, 1.0, 0.0), (1.5, -1, 1.0, 0.0), (0.6, 20, 0.95, 0.0), (1.0, 64, 1.0, 0.0),
-               (0.8, 50, 0.9, 0.02), (1.0, 1, 1.0, 0.0), (0.3, 3, 1.0, 0.1), (1.0, 65, 1.0, 0.0)]
+               (0.8, 50, 0.9, 0.02), (1.0, 1, 1.0, 0.0), (0.3, 3, 1.0, 0.1), (1.0, 65, 1.0, 0.0),
+               (0.7, -1, 0.9, 0.0), (0.25, 0, 0.5, 0.02), (1.0, -1, 0.999, 0.0)]        # top-p without top-k
     for V in (10240, 10244, 40960, 151936, 327680, 327684):      # one part exactly, one value into the next, the most parts, too many
         rows = {
             "spread": torch.randn(len(configs), V) * 3,
@@ -451,6 +452,7 @@ def test_sampler_rows_cut_into_parts(ops):
             "weight at a part's edge": torch.full((len(configs), V), -40.0),
             "equal values": torch.zeros(len(configs), V),
             "the largest all in one part": torch.randn(len(configs), V),
+            "peaked": torch.randn(len(configs), V) * 12,                     # a nucleus of few values
         }
         edge = min(10236, V - 8)
         rows["weight at a part's edge"][:, edge:edge + 8] = torch.randn(len(configs), 8)

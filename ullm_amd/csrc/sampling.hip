@@ -479,16 +479,18 @@ __device__ int walk_range(const float* __restrict__ x, int rbeg, int rend, float
 }
 
 // ------------------------------------------------------------------------------ parts of a row
-// One block per row reads 150 K values with one compute unit, pass after pass.  For the two common settings
-// (temperature alone; top-k with a small k, with or without top-p and min-p) a first kernel cuts every row
-// into parts of PART_VALUES values, one block each, which hold their values in registers and leave per part:
-// the maximum, the sum of exp(z - that maximum) and, with top-k, the candidates: every value of the part at
-// or above a threshold that at least k of its values reach (so the k largest of the row, ties included, are
-// among the parts' candidates), in index order, and that threshold (the row's k-th largest value is at or
-// above every part's).  The row's block then only scales and adds the parts' sums and walks the one part
-// the draw falls into, or runs the list phase over the candidates at or above the highest threshold.  A
-// part with more candidates than it can pass on (many equal values) says so, and the row's block takes the
-// way over the whole vocabulary.
+// One block per row reads 150 K values with one compute unit, pass after pass.  For the common settings
+// (temperature alone; top-k with a small k, with or without top-p and min-p; top-p without top-k) a first
+// kernel cuts every row into parts of PART_VALUES values, one block each, which hold their values in
+// registers and leave per part: the maximum, the sum of exp(z - that maximum) and, unless temperature stands
+// alone, the candidates: every value of the part at or above a threshold that at least k of its values reach
+// (k = PART_K_MAX with top-p alone), in index order, and that threshold.  With top-k the k largest values of
+// the row, ties included, are then among the parts' candidates, and the row's k-th largest value is at or
+// above every part's threshold; with top-p alone every value of the row at or above the highest threshold is
+// a candidate.  The row's block then only scales and adds the parts' sums and walks the one part the draw
+// falls into, or runs the list phase over the candidates at or above a bound it raises from the highest
+// threshold.  A part with more candidates than it can pass on (many equal values) says so, a nucleus may
+// reach below the highest threshold: the row's block then takes the way over the whole vocabulary.
 #define PART_THREADS 256
 #define PART_HOLD 10                                         // 16-byte pieces a thread holds
 #define PART_WAVE_VALUES (4 * WAVE * PART_HOLD)              // a wave's consecutive values
@@ -499,11 +501,16 @@ __device__ int walk_range(const float* __restrict__ x, int rbeg, int rend, float
 #define MAX_PARTS 32
 #define TOP_K_PARTS 16                                       // with top-k: one wave holds all candidates, two per lane and part
 
-enum { PARTS_NONE = 0, PARTS_SUMS = 1, PARTS_TOP_K = 2 };
+// What the parts leave for a row: nothing (greedy, a large top-k, min-p alone: the row's block does it all),
+// maxima and sums (temperature alone), or also candidates: the largest k values of every part with top-k, the
+// largest PART_K_MAX of every part with top-p and no top-k (a nucleus that lies within them is served from them).
+enum { PARTS_NONE = 0, PARTS_SUMS = 1, PARTS_TOP_K = 2, PARTS_TOP_P = 3 };
 __device__ __forceinline__ int parts_mode(float t, int k, int V, float p, float mp) {
   if (t == 0.f) return PARTS_NONE;
-  if (k > 0 && k < V) return (k <= PART_K_MAX && V <= TOP_K_PARTS * PART_VALUES) ? PARTS_TOP_K : PARTS_NONE;
-  return (!(p > 0.f && p < 1.f) && !(mp > 0.f)) ? PARTS_SUMS : PARTS_NONE;
+  const bool lists_fit = V <= TOP_K_PARTS * PART_VALUES;
+  if (k > 0 && k < V) return (k <= PART_K_MAX && lists_fit) ? PARTS_TOP_K : PARTS_NONE;
+  if (p > 0.f && p < 1.f) return lists_fit ? PARTS_TOP_P : PARTS_NONE;
+  return !(mp > 0.f) ? PARTS_SUMS : PARTS_NONE;
 }
 
 // grid (parts, rows); V a multiple of 4 and rows 16-byte aligned
@@ -563,11 +570,12 @@ sample_parts_kernel(const float* __restrict__ logits, int V, int ld, const float
     mine[1] = total;
     reinterpret_cast<int*>(mine)[2] = 0;
   }
-  if (mode != PARTS_TOP_K) return;
+  if (mode == PARTS_SUMS) return;
   // A threshold that at least kk of the part's values reach, and not many more: one that kk of the threads'
   // own maxima reach (the largest values of a part mostly lie with different threads).  Every wave looks
   // for it by itself, halving the span of the maxima twelve times, with counts by ballot.
-  const int kk = k < pend - pbeg ? k : pend - pbeg;
+  const int asked = mode == PARTS_TOP_K ? k : PART_K_MAX;
+  const int kk = asked < pend - pbeg ? asked : pend - pbeg;
   lane_max[tid] = mloc;
   __syncthreads();
   float lm[NW];
@@ -637,7 +645,9 @@ sample_parts_kernel(const float* __restrict__ logits, int V, int ld, const float
   }
   if (tid == 0) {
     reinterpret_cast<int*>(mine)[2] = n_all;
-    mine[3] = kk == k ? wide : -INFINITY;   // k values of the row are at or above it: so is the row's k-th largest
+    // With top-k: k values of the row are at or above it, so the row's k-th largest is.  With top-p: every
+    // value of the part at or above it is listed.  A part that lists all it has sets no bound (-inf).
+    mine[3] = kk == asked ? wide : -INFINITY;
   }
 }
 
@@ -695,18 +705,22 @@ sample_kernel(const float* __restrict__ logits, int V, int ld, const float* __re
     float m = -INFINITY;
     for (int p = 0; p < n_parts; ++p) m = fmaxf(m, part_m[p]);
     const float uniform = uniform_from_seed(seed, position_row);
-    if (mode == PARTS_TOP_K) {
+    if (mode == PARTS_TOP_K || mode == PARTS_TOP_P) {
       bool bad = false;
-      float bound = -INFINITY;              // the row's k-th largest value is at or above every part's threshold
+      float bound = -INFINITY;              // the highest of the parts' thresholds
+      float all_weight = 0.f;               // every part's sum, brought to the row's maximum, in order
       for (int p = 0; p < n_parts; ++p) {
         bad = bad || part_n[p] < 0;
         bound = fmaxf(bound, part_w[p]);
+        all_weight += part_s[p] * __builtin_amdgcn_exp2f((part_m[p] - m) * L2E);
       }
       if (!bad) {
-        // One wave does the rest.  It holds all candidates (two per lane and part), raises the bound towards
-        // the row's k-th largest value by halving the span to the maximum twelve times (counts by ballot; at
-        // least k candidates stay at or above it), puts what is at or above it side by side, still in index
-        // order, and runs the list phase on that short list.
+        // One wave does the rest.  It holds all candidates (two per lane and part).  With top-k the row's k-th
+        // largest value is at or above every part's threshold; with top-p alone every value of the row at or
+        // above the highest threshold is a candidate, so a nucleus that ends above it is among them.  The wave
+        // raises that bound by halving the span to the maximum twelve times, as long as k candidates (counts by
+        // ballot), or a little more than the share p of all weight, stay at or above it, puts what does side
+        // by side, still in index order, and runs the list phase on that short list.
         if (wave == 0) {
           constexpr int HELD = 2 * TOP_K_PARTS;
           float held[HELD];
@@ -716,14 +730,31 @@ sample_kernel(const float* __restrict__ logits, int V, int ld, const float* __re
             held[i] = (pp < n_parts && j < part_n[pp]) ? mine[pp * PART_WORDS + 4 + j] : -INFINITY;
           }
           float lo = bound, hi = m;
-          if (lo > -INFINITY) {
-            for (int it = 0; it < 12; ++it) {
+          bool served = true;
+          if (mode == PARTS_TOP_K) {
+            if (lo > -INFINITY) {
+              for (int it = 0; it < 12; ++it) {
+                const float mid = 0.5f * (lo + hi);
+                if (!(mid > lo && mid < hi)) break;
+                int c = 0;
+#pragma unroll
+                for (int i = 0; i < HELD; ++i) c += __popcll(__ballot(held[i] >= mid));
+                if (c >= k_row) lo = mid; else hi = mid;
+              }
+            }
+          } else if (lo > -INFINITY) {
+            auto weight_from = [&](float from) {
+              float a = 0.f;
+#pragma unroll
+              for (int i = 0; i < HELD; ++i) a += held[i] >= from ? __builtin_amdgcn_exp2f((held[i] - m) * L2E) : 0.f;
+              return wave_sum(a);
+            };
+            const float need = p_row * all_weight * 1.001f;
+            served = weight_from(lo) >= need;
+            for (int it = 0; it < 12 && served; ++it) {
               const float mid = 0.5f * (lo + hi);
               if (!(mid > lo && mid < hi)) break;
-              int c = 0;
-#pragma unroll
-              for (int i = 0; i < HELD; ++i) c += __popcll(__ballot(held[i] >= mid));
-              if (c >= k_row) lo = mid; else hi = mid;
+              if (weight_from(mid) >= need) lo = mid; else hi = mid;
             }
           }
           int n_all = 0;
@@ -743,12 +774,13 @@ sample_kernel(const float* __restrict__ logits, int V, int ld, const float* __re
           __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
           __builtin_amdgcn_wave_barrier();
           __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-          if (n_all <= 4 * WAVE) {
-            const int token = draw_from_short_list(cand, n_all, true, k_row, p_row, mp_row, 0.f, order_key(lo), order_key(m),
-                                                   uniform, lane);
-            if (lane == 0) { out[row] = token; chosen = 0; }
-          } else if (lane == 0) {
-            chosen = -1;                    // many equal values around the k-th largest: the long way
+          int token = -1;                   // stays so where the short list cannot serve the row: the long way
+          if (served && n_all <= 4 * WAVE)
+            token = draw_from_short_list(cand, n_all, mode == PARTS_TOP_K, k_row, p_row, mp_row, all_weight, order_key(lo),
+                                         order_key(m), uniform, lane);
+          if (lane == 0) {
+            if (token >= 0) out[row] = token;
+            chosen = token >= 0 ? 0 : -1;
           }
         }
         __syncthreads();

@@ -283,14 +283,16 @@ def sampling(args) -> None:
     settings = (("greedy", 0.0, -1, 1.0, 0.0), ("temperature 0.6", 0.6, -1, 1.0, 0.0),
                 ("top-k 20, top-p 0.95", 0.6, 20, 0.95, 0.0), ("top-k 50", 0.8, 50, 1.0, 0.0),
                 ("top-k 50, top-p 0.9, min-p 0.02", 0.8, 50, 0.9, 0.02), ("min-p 0.05", 0.8, -1, 1.0, 0.05),
-                ("top-p 0.9 (these rows are flat: the long way)", 0.8, -1, 0.9, 0.0))
+                ("top-p 0.9 (these rows are flat: the long way)", 0.8, -1, 0.9, 0.0),
+                ("top-p 0.9, rows of scale 12 (a nucleus of few values)", 0.8, -1, 0.9, 0.0))
     for B in args.rows:
         torch.manual_seed(0)
-        logits = torch.randn(B, V, device=DEV) * 3
+        flat_rows = torch.randn(B, V, device=DEV)
         lo, hi = torch.arange(B, dtype=torch.int32, device=DEV), torch.zeros(B, dtype=torch.int32, device=DEV)
         pos = torch.arange(B, dtype=torch.int32, device=DEV)
         out = torch.empty(B, dtype=torch.int32, device=DEV)
         for name, t, k, p, mp in settings:
+            logits = flat_rows * (12 if "scale 12" in name else 3)
             T, K = torch.full((B,), t, device=DEV), torch.full((B,), k, dtype=torch.int32, device=DEV)
             P, MP = torch.full((B,), p, device=DEV), torch.full((B,), mp, device=DEV)
             cut = graph_time([lambda: ops.sample(logits, T, K, P, MP, lo, hi, pos, out, parts=True)])
