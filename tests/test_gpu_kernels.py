@@ -414,6 +414,8 @@ def test_sampler_with_a_small_top_k_over_a_large_vocabulary(ops):
             "peaked": torch.randn(len(configs), V) * 8,
             "flat": torch.randn(len(configs), V) * 0.01,                     # all within a hair of the maximum
             "ties": (torch.randn(len(configs), V) * 2).round(),              # many equal values: too many candidates
+            "zeros of both signs": torch.where(torch.rand(len(configs), V) < 0.5, (torch.randn(len(configs), V) * 0.3).round(),
+                                               torch.randn(len(configs), V) - 3.0),    # -0.0 and +0.0 are one value: the k-th largest is among them
             "far": torch.cat([torch.tensor([[50.0, 49.25, 48.5]]).expand(len(configs), 3),
                               torch.randn(len(configs), V - 3)], 1),           # the k-th largest far below the maximum
         }
@@ -423,28 +425,29 @@ def test_sampler_with_a_small_top_k_over_a_large_vocabulary(ops):
             pos = [3 * i for i in range(len(configs))]
             got = sampler.sample(logits.to(DEV), ps, seeds, pos)
             for i, c in enumerate(configs):
-                if name == "ties" and c[2] < 1.0:
+                if name in ("ties", "zeros of both signs") and c[2] < 1.0:
                     continue       # which of several equal values top-p drops follows the reference's sort; here all or none
                 assert got[i] in plain.sample_token_set(logits[i], *c, seeds[i], pos[i]), (V, name, c, got[i])
             again = sampler.sample(logits.flip(0).contiguous().to(DEV), ps[::-1], seeds[::-1], pos[::-1])
             assert again[::-1] == got
             whole = whole_rows.sample(logits.to(DEV), ps, seeds, pos)
             for i, c in enumerate(configs):
-                if name == "ties" and c[2] < 1.0:
+                if name in ("ties", "zeros of both signs") and c[2] < 1.0:
                     continue
                 assert whole[i] in plain.sample_token_set(logits[i], *c, seeds[i], pos[i]), (V, name, c, whole[i])
 
 
 def test_sampler_rows_cut_into_parts(ops):
-    """Temperature alone, top-k up to 64 and top-p without top-k take sums and candidates from parts of the row that
-    a first kernel makes (top-p where the nucleus lies within the 64 largest values of every part); the token is one the plain sampler may draw, whatever the row looks like and wherever in it the
+    """Every setting but greedy and a top-k above 64 takes sums and candidates from parts of the row that a first
+    kernel makes (top-p and min-p without top-k where what they keep lies within the 64 largest values of every part); the token is one the plain sampler may draw, whatever the row looks like and wherever in it the
     weight lies, and the same as in another batch position."""
     from ullm_amd.sampling import Sampler, SamplingParams
     torch.manual_seed(23)
     sampler = Sampler(torch.device(DEV))
     configs = [(0.7, -1, 1.0, 0.0), (1.0, 0, 1.0, 0.0), (1.5, -1, 1.0, 0.0), (0.6, 20, 0.95, 0.0), (1.0, 64, 1.0, 0.0),
                (0.8, 50, 0.9, 0.02), (1.0, 1, 1.0, 0.0), (0.3, 3, 1.0, 0.1), (1.0, 65, 1.0, 0.0),
-               (0.7, -1, 0.9, 0.0), (0.25, 0, 0.5, 0.02), (1.0, -1, 0.999, 0.0)]        # top-p without top-k
+               (0.7, -1, 0.9, 0.0), (0.25, 0, 0.5, 0.02), (1.0, -1, 0.999, 0.0),        # top-p without top-k
+               (0.8, -1, 1.0, 0.05), (1.0, 0, 1.0, 0.9), (0.5, -1, 1.0, 1e-6)]           # min-p alone
     for V in (10240, 10244, 40960, 151936, 327680, 327684):      # one part exactly, one value into the next, the most parts, too many
         rows = {
             "spread": torch.randn(len(configs), V) * 3,

@@ -180,8 +180,7 @@ def test_batch_buckets_of_the_captured_decode_graphs():
 
 def test_sampler_stages_one_word_for_the_host_beside_the_rows():
     """The staged parameters are seven words a row and one more that only the host reads: whether any row has
-    settings that the sampling kernels serve by cutting rows into parts (temperature alone, a small top-k, top-p
-    without top-k)."""
+    settings that the sampling kernels serve by cutting rows into parts (all but greedy and a large top-k)."""
     import torch
     from ullm_amd.sampling import Sampler, SamplingParams
     sampler = Sampler(torch.device("cpu"))
@@ -191,7 +190,7 @@ def test_sampler_stages_one_word_for_the_host_beside_the_rows():
              ([SamplingParams(temperature=0.7, top_p=0.9, min_p=0.1)], True),
              ([SamplingParams(temperature=0.7, top_k=20, top_p=0.9, min_p=0.05)], True),
              ([SamplingParams(temperature=0.7, top_k=100)], False),
-             ([SamplingParams(temperature=0.7, min_p=0.1)], False)]
+             ([SamplingParams(temperature=0.7, min_p=0.1)], True)]
     for params, cut in cases:
         n = len(params)
         staged = sampler.stage(params, list(range(n)), [5] * n)

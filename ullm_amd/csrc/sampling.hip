@@ -14,8 +14,10 @@
 
 #define SAMPLE_THREADS 1024
 
+// An unsigned integer that orders as the float does; -0.0 and +0.0, which compare equal, get one key.
 __device__ __forceinline__ uint32_t order_key(float f) {
-  const uint32_t u = __float_as_uint(f);
+  uint32_t u = __float_as_uint(f);
+  if (u == 0x80000000u) u = 0u;
   return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
 
@@ -480,17 +482,17 @@ __device__ int walk_range(const float* __restrict__ x, int rbeg, int rend, float
 
 // ------------------------------------------------------------------------------ parts of a row
 // One block per row reads 150 K values with one compute unit, pass after pass.  For the common settings
-// (temperature alone; top-k with a small k, with or without top-p and min-p; top-p without top-k) a first
+// (temperature alone; top-k with a small k, with or without top-p and min-p; top-p or min-p without top-k) a first
 // kernel cuts every row into parts of PART_VALUES values, one block each, which hold their values in
 // registers and leave per part: the maximum, the sum of exp(z - that maximum) and, unless temperature stands
 // alone, the candidates: every value of the part at or above a threshold that at least k of its values reach
-// (k = PART_K_MAX with top-p alone), in index order, and that threshold.  With top-k the k largest values of
+// (k = PART_K_MAX without top-k), in index order, and that threshold.  With top-k the k largest values of
 // the row, ties included, are then among the parts' candidates, and the row's k-th largest value is at or
-// above every part's threshold; with top-p alone every value of the row at or above the highest threshold is
+// above every part's threshold; without top-k every value of the row at or above the highest threshold is
 // a candidate.  The row's block then only scales and adds the parts' sums and walks the one part the draw
 // falls into, or runs the list phase over the candidates at or above a bound it raises from the highest
-// threshold.  A part with more candidates than it can pass on (many equal values) says so, a nucleus may
-// reach below the highest threshold: the row's block then takes the way over the whole vocabulary.
+// threshold.  A part with more candidates than it can pass on (many equal values) says so, and what top-p or
+// min-p keep may reach below the highest threshold: the row's block then takes the way over the whole vocabulary.
 #define PART_THREADS 256
 #define PART_HOLD 10                                         // 16-byte pieces a thread holds
 #define PART_WAVE_VALUES (4 * WAVE * PART_HOLD)              // a wave's consecutive values
@@ -501,16 +503,17 @@ __device__ int walk_range(const float* __restrict__ x, int rbeg, int rend, float
 #define MAX_PARTS 32
 #define TOP_K_PARTS 16                                       // with top-k: one wave holds all candidates, two per lane and part
 
-// What the parts leave for a row: nothing (greedy, a large top-k, min-p alone: the row's block does it all),
-// maxima and sums (temperature alone), or also candidates: the largest k values of every part with top-k, the
-// largest PART_K_MAX of every part with top-p and no top-k (a nucleus that lies within them is served from them).
+// What the parts leave for a row: nothing (greedy, a large top-k: the row's block does it all), maxima and
+// sums (temperature alone), or also candidates: the largest k values of every part with top-k, the largest
+// PART_K_MAX of every part with top-p or min-p and no top-k (what these keep is served from them if it lies
+// within them).
 enum { PARTS_NONE = 0, PARTS_SUMS = 1, PARTS_TOP_K = 2, PARTS_TOP_P = 3 };
 __device__ __forceinline__ int parts_mode(float t, int k, int V, float p, float mp) {
   if (t == 0.f) return PARTS_NONE;
   const bool lists_fit = V <= TOP_K_PARTS * PART_VALUES;
   if (k > 0 && k < V) return (k <= PART_K_MAX && lists_fit) ? PARTS_TOP_K : PARTS_NONE;
-  if (p > 0.f && p < 1.f) return lists_fit ? PARTS_TOP_P : PARTS_NONE;
-  return !(mp > 0.f) ? PARTS_SUMS : PARTS_NONE;
+  if ((p > 0.f && p < 1.f) || mp > 0.f) return lists_fit ? PARTS_TOP_P : PARTS_NONE;
+  return PARTS_SUMS;
 }
 
 // grid (parts, rows); V a multiple of 4 and rows 16-byte aligned
@@ -714,6 +717,9 @@ sample_kernel(const float* __restrict__ logits, int V, int ld, const float* __re
         bound = fmaxf(bound, part_w[p]);
         all_weight += part_s[p] * __builtin_amdgcn_exp2f((part_m[p] - m) * L2E);
       }
+      // min-p alone keeps the values within -log(min_p) of the maximum (logf: the hardware's log2)
+      const bool top_p_row = p_row > 0.f && p_row < 1.f;
+      const float min_p_reach = m + (__builtin_amdgcn_logf(mp_row) - 0.01f) / L2E;
       if (!bad) {
         // One wave does the rest.  It holds all candidates (two per lane and part).  With top-k the row's k-th
         // largest value is at or above every part's threshold; with top-p alone every value of the row at or
@@ -731,6 +737,11 @@ sample_kernel(const float* __restrict__ logits, int V, int ld, const float* __re
           }
           float lo = bound, hi = m;
           bool served = true;
+          const bool min_p_alone = mode == PARTS_TOP_P && !top_p_row;
+          if (min_p_alone && lo > -INFINITY) {
+            served = min_p_reach >= lo;     // all that min-p keeps are candidates, or the row is not served
+            lo = min_p_reach;
+          }
           if (mode == PARTS_TOP_K) {
             if (lo > -INFINITY) {
               for (int it = 0; it < 12; ++it) {
@@ -742,19 +753,19 @@ sample_kernel(const float* __restrict__ logits, int V, int ld, const float* __re
                 if (c >= k_row) lo = mid; else hi = mid;
               }
             }
-          } else if (lo > -INFINITY) {
-            auto weight_from = [&](float from) {
+          } else if (!min_p_alone && lo > -INFINITY) {
+            // first the weight at the bound itself (the nucleus must lie within the candidates), then the halvings
+            const float need = p_row * all_weight * 1.001f;
+            for (int it = 0; it <= 12 && served; ++it) {
+              const float mid = it == 0 ? lo : 0.5f * (lo + hi);
+              if (it > 0 && !(mid > lo && mid < hi)) break;
               float a = 0.f;
 #pragma unroll
-              for (int i = 0; i < HELD; ++i) a += held[i] >= from ? __builtin_amdgcn_exp2f((held[i] - m) * L2E) : 0.f;
-              return wave_sum(a);
-            };
-            const float need = p_row * all_weight * 1.001f;
-            served = weight_from(lo) >= need;
-            for (int it = 0; it < 12 && served; ++it) {
-              const float mid = 0.5f * (lo + hi);
-              if (!(mid > lo && mid < hi)) break;
-              if (weight_from(mid) >= need) lo = mid; else hi = mid;
+              for (int i = 0; i < HELD; ++i) a += held[i] >= mid ? __builtin_amdgcn_exp2f((held[i] - m) * L2E) : 0.f;
+              const bool enough = wave_sum(a) >= need;
+              if (it == 0) served = enough;
+              else if (enough) lo = mid;
+              else hi = mid;
             }
           }
           int n_all = 0;

@@ -46,11 +46,9 @@ class Sampler:
         host[5] = (s64 >> np.uint64(32)).astype(np.uint32).view(np.int32)
         host[6] = positions
         # one more word, for the host alone: whether any row has settings that the kernels serve by cutting rows
-        # into parts (temperature alone, top-k up to ops.SAMPLE_PARTS_TOP_K, top-p without top-k); without one,
-        # that kernel is not launched
-        flat[-1] = int(any(p.temperature != 0 and (0 < p.top_k <= ops.SAMPLE_PARTS_TOP_K or
-                                                   (p.top_k <= 0 and (0 < p.top_p < 1 or not p.min_p > 0)))
-                           for p in params))
+        # into parts (every setting but greedy and a top-k above ops.SAMPLE_PARTS_TOP_K); without one, that kernel
+        # is not launched
+        flat[-1] = int(any(p.temperature != 0 and p.top_k <= ops.SAMPLE_PARTS_TOP_K for p in params))
         return self._upload.stage(flat)
 
     def send(self, staged: torch.Tensor) -> SamplerInputs:
