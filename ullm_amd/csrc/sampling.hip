@@ -14,10 +14,10 @@
 
 #define SAMPLE_THREADS 1024
 
-// An unsigned integer that orders as the float does; -0.0 and +0.0, which compare equal, get one key.
+// An unsigned integer that orders as the float does; -0.0 and +0.0, which compare equal, get one key
+// (-0.0 + 0.0 is +0.0, and the sum of anything else with 0.0 is itself).
 __device__ __forceinline__ uint32_t order_key(float f) {
-  uint32_t u = __float_as_uint(f);
-  if (u == 0x80000000u) u = 0u;
+  const uint32_t u = __float_as_uint(f + 0.f);
   return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
 
