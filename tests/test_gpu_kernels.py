@@ -584,7 +584,10 @@ FUSED_CASES = [dict(nq=32, nkv=8, hd=128, P=16, lens=[1153, 31, 32, 33, 1], wind
                # kv head in one group of 16 columns over a long context, three heads per kv head cut in three
                dict(nq=48, nkv=8, hd=256, P=16, lens=[861, 906], window=0, norm=True, rope=True),
                dict(nq=96, nkv=8, hd=64, P=48, lens=[2492], window=0, norm=True, rope=True),
-               dict(nq=6, nkv=2, hd=128, P=48, lens=[1789], window=0, norm=True, rope=True)]
+               dict(nq=6, nkv=2, hd=128, P=48, lens=[1789], window=0, norm=True, rope=True),
+               # a request whose keys end with a tile's last key: the kernel of its own takes that tile without tests
+               # per score, the one that holds the newest key itself with them; both must round alike
+               dict(nq=24, nkv=2, hd=128, P=16, lens=[1643, 353, 1384, 25, 32], window=0, norm=True, rope=False)]
 
 
 @pytest.mark.parametrize("case", FUSED_CASES)

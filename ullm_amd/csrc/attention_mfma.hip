@@ -108,6 +108,9 @@ __device__ __forceinline__ void process_tile(const KVTile<NQK>& cur, int key0, c
                                              const int (&col_lo)[NG], const int (&col_hi)[NG], int max_hi,
                                              float scale_log2e, f32x4_t (&acc)[NG][2 * NQK], float (&m)[NG],
                                              float (&l)[NG], const bf16_t* own) {
+  // no product fused with a following sum here: the variant with tests keeps the scaled score in a select, the
+  // variant without would fuse it into the subtraction of the maximum, and the two would round differently
+#pragma clang fp contract(off)
   constexpr int HD = 32 * NQK;
   const int lane = threadIdx.x & 63, g = lane >> 4;
   const bool edge = !INNER && key0 + 32 > max_hi + 1;     // some keys of the tile hold no written data
