@@ -240,4 +240,8 @@ def test_limits_are_derived_from_times_by_the_time_saved_in_total():
     store = {"norm": {1: 2.5, 8: 2.5, 16: 2.5, 32: 2.5}, "library": {1: 14, 8: 14, 16: 14, 32: 15},
              "skinny": {1: 10, 8: 10.5, 16: 13, 32: 19}, "rows": {1: 10.5, 8: 10.6, 16: 10.7, 32: 12},
              "skinny+norm": {1: 11.5, 8: 12.5, 16: 16}}
-    assert derive_limits(store, {"store"}, 0, 0) == {"skinny": 8, "rows": 32, "fold_norm": 8}
+    assert derive_limits(store, {"store"}, 0, 0) == {"skinny": 8, "rows": 32, "fold_norm": 8, "sums_from": 0, "sums_to": 0}
+    # above the rows the weight-streaming kernels take, partial sums and the kernel that adds them as far as they save time
+    more = {"library": {32: 15, 64: 17, 65: 17, 128: 25, 256: 40, 512: 60}, "rows": {32: 12, 64: 16},
+            "partial sums>sum": {32: 14, 64: 16.5, 65: 16, 128: 21, 256: 31, 512: 70}, "norm": {}}
+    assert derive_limits(more, {"store"}, 0, 0) == {"skinny": 0, "rows": 64, "fold_norm": 0, "sums_from": 65, "sums_to": 256}

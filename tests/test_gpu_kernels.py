@@ -186,6 +186,39 @@ def test_qk_norm_rope_write(ops, dtype, cfg):
     assert int((k_pool.float().abs().sum(-1) > 0).sum()) == written * nkv       # nothing else was touched
 
 
+def test_stacks_of_partial_sums_added_to_one_result(ops, monkeypatch):
+    """A first projection above the rows of the weight-streaming kernels, where the table says so: the partial
+    sums of slices of the inner dimension, added in order by a kernel of its own, with the bias, rounded once."""
+    import dataclasses
+    from ullm_amd.kernels import dispatch
+    torch.manual_seed(12)
+    for S, M, N in ((5, 70, 36), (1, 3, 4), (8, 256, 1024)):
+        stacks = torch.randn(S, M, N, device=DEV)
+        bias = torch.randn(N, device=DEV)
+        want = stacks[0].clone()
+        for s in range(1, S):
+            want += stacks[s]
+        assert torch.equal(ops.sum_stacks(stacks, out_dtype=torch.float32), want)
+        assert torch.equal(ops.sum_stacks(stacks, bias), (want + bias).to(torch.bfloat16))
+    rules = dispatch.default_limits
+    monkeypatch.setattr(dispatch, "_table", {})
+    monkeypatch.setattr(dispatch, "default_limits", lambda c, k: dataclasses.replace(rules(c, k), sums_from=65, sums_to=256))
+    for M, N, K in ((96, 1536, 1024), (200, 520, 2048), (65, 6144, 4096)):
+        x, w = torch.randn(M, K, device=DEV).bfloat16(), (torch.randn(N, K, device=DEV) * 0.05).bfloat16()
+        bias = torch.randn(N, device=DEV)
+        calls = []
+        real = ops.sum_stacks
+        monkeypatch.setattr(ops, "sum_stacks", lambda *a, **k: (calls.append(1), real(*a, **k))[1])
+        got = ops.gemm_bf16(x, w, bias)
+        monkeypatch.setattr(ops, "sum_stacks", real)
+        assert calls, "the projection did not take the partial sums"
+        want = x.float() @ w.float().t() + bias
+        assert got.dtype == torch.bfloat16 and (got.float() - want).abs().max() <= tol(torch.bfloat16, want)
+        # a row's result does not depend on the other rows
+        assert torch.equal(ops.gemm_bf16(x[:70].contiguous(), w, bias)[:65], got[:65])
+    monkeypatch.setattr(dispatch, "_table", None)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("cfg", [dict(nq=32, nkv=8, hd=128, P=16, rot=128, style=1),    # 48 heads: three in turn per thread
                                  dict(nq=70, nkv=2, hd=32, P=8, rot=32, style=2),       # 74 heads of 4 lanes: two in turn

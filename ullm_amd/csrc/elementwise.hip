@@ -435,6 +435,45 @@ extern "C" int ullm_silu_mul(const void* gu, void* out, int T_, int I, int dtype
   ULLM_LAUNCH_CHECK();
 }
 
+// ------------------------------------------------------------------ stacks of partial sums to one result
+// out[m][n] = sum over s of stacks[s][m][n] (+ bias[n]), the stacks added in order, four columns a thread.
+// What a first projection needs from the partial-sums product (the last projections' stacks are added by
+// the norm that follows them).
+template <typename T>
+__global__ void __launch_bounds__(256)
+sum_stacks_kernel(const float* __restrict__ stacks, size_t stack_stride, int n_stacks, const float* __restrict__ bias,
+                  T* __restrict__ out, int N, size_t total4) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total4) return;
+  const size_t at = 4 * i;
+  float4 a = ld4_f32(stacks + at);
+  for (int s = 1; s < n_stacks; ++s) {
+    const float4 b = ld4_f32(stacks + (size_t)s * stack_stride + at);
+    a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
+  }
+  if (bias) {
+    const float4 b = ld4_f32(bias + at % N);
+    a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
+  }
+  st4_f32(out + at, a);
+}
+
+// stacks float32 [n_stacks, M, N] contiguous, N a multiple of 4; out [M, N] contiguous, float32 or bfloat16
+extern "C" int ullm_sum_stacks(const float* stacks, int n_stacks, const float* bias, void* out, int M, int N, int dtype,
+                               hipStream_t stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (n_stacks < 1 || N % 4 || (((uintptr_t)stacks | (uintptr_t)out | (uintptr_t)bias) & 15)) return ULLM_ERR_SHAPE;
+  const size_t total4 = (size_t)M * N / 4;
+  dim3 block(256), grid((unsigned)((total4 + 255) / 256));
+  if (dtype == ULLM_F32)
+    hipLaunchKernelGGL(sum_stacks_kernel<float>, grid, block, 0, stream, stacks, (size_t)M * N, n_stacks, bias, (float*)out, N, total4);
+  else if (dtype == ULLM_BF16)
+    hipLaunchKernelGGL(sum_stacks_kernel<bf16_t>, grid, block, 0, stream, stacks, (size_t)M * N, n_stacks, bias, (bf16_t*)out, N, total4);
+  else
+    return ULLM_ERR_DTYPE;
+  ULLM_LAUNCH_CHECK();
+}
+
 // ------------------------------------------------------------------ q/k norm + rotary + cache write
 // One wave per (token, head) of the fused projection row  [q heads | k heads | v heads].
 //   q heads: per-head RMS norm (gain shared by all heads, may be null), rotation, written to q_out

@@ -37,6 +37,10 @@ class Limits:
     # inner dimension from ``stacked_from`` to ``stacked_to`` rows (0, 0: never)
     stacked_from: int = 17
     stacked_to: int = 256
+    # y = x W^T in bfloat16 above ``skinny`` and ``rows``: partial sums over slices of the inner dimension and a
+    # kernel that adds them, from ``sums_from`` to ``sums_to`` rows (0, 0: never; only measured matrices have it)
+    sums_from: int = 0
+    sums_to: int = 0
     # 32-bit results (the logits head): the few-rows kernel up to here, then the library
     f32_skinny: int = 16
 

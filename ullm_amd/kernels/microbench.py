@@ -195,6 +195,10 @@ def derive_limits(times: dict, roles, columns: int, inner: int) -> dict:
         best = {r: min(t[r] for t in (get("skinny"), get("rows"), get("library")) if r in t) for r in rows}
         unfolded = {r: best[r] + get("norm")[r] for r in rows if r in get("norm")}
         changes["fold_norm"] = _ahead_up_to(rows, get("skinny+norm"), [unfolded])
+        # above the rows the weight-streaming kernels take: partial sums and the kernel that adds them, against the library
+        taken = max(changes["skinny"], changes["rows"])
+        upto = _ahead_up_to(rows, get("partial sums>sum"), [get("library")], start=taken)
+        changes["sums_from"], changes["sums_to"] = (taken + 1, upto) if upto > taken else (0, 0)
     if "silu" in roles:
         changes["silu_skinny"] = _ahead_up_to(rows, get("skinny+silu"), [get("rows+silu"), get("library+silu")])
         changes["silu_rows"] = _ahead_up_to(rows, get("rows+silu"), [get("library+silu")], start=changes["silu_skinny"])
@@ -245,6 +249,8 @@ def tune(args) -> None:
                 timed("skinny+norm", M, lambda v: (lambda: ops.gemm_skinny_normed(stream, gain, 1e-6, ws[v])))
             if M <= ops.ROWS_MAX_ROWS and ops.gemm_rows_supports(x, ws[0]):
                 timed("rows", M, lambda v: (lambda: ops.gemm_rows(x, ws[v])))
+            if M > 16 and N % 4 == 0 and ops.gemm_partial_sums_supports(x, ws[0]):
+                timed("partial sums>sum", M, lambda v: (lambda: ops.sum_stacks(ops.gemm_partial_sums(x, ws[v]))))
         if "silu" in roles:
             timed("library+silu", M, lambda v: (lambda: ops.silu_mul(torch.nn.functional.linear(x, ws[v]))))
             if skinny_ok:

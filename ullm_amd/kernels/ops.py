@@ -209,6 +209,22 @@ def silu_mul(gate_up: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch
     return out
 
 
+def sum_stacks(stacks: torch.Tensor, bias: Optional[torch.Tensor] = None,
+               out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    """The sum over the first dimension of float32 ``stacks`` [S, M, N] (what :func:`gemm_partial_sums` leaves), added
+    in order, plus ``bias`` [N], as [M, N] of ``out_dtype``."""
+    _need(stacks.dtype == torch.float32 and stacks.dim() == 3 and stacks.is_contiguous() and stacks.shape[2] % 4 == 0,
+          "stacks must be contiguous float32 [S, M, N] with N a multiple of 4")
+    S, M, N = stacks.shape
+    if bias is not None:
+        _need(bias.dtype == torch.float32 and bias.numel() == N and bias.is_contiguous(), "bias must be float32 [N]")
+    out = torch.empty((M, N), dtype=out_dtype, device=stacks.device)
+    lib = build.load("elementwise")
+    _check(lib.ullm_sum_stacks(_p(stacks), _c_int(S), _p(bias), _p(out), _c_int(M), _c_int(N), _c_int(_dt(out)), _stream()),
+           "sum_stacks")
+    return out
+
+
 def qk_norm_rope_write(qkv: torch.Tensor, q_out: torch.Tensor, q_gain: Optional[torch.Tensor],
                        k_gain: Optional[torch.Tensor], eps: float, cos_sin: Optional[torch.Tensor],
                        rotary_dim: int, style: int, positions: torch.Tensor, token_entry: torch.Tensor,
@@ -495,7 +511,8 @@ _MM_TAKES_OUT_DTYPE = "out_dtype" in (torch.mm.__doc__ or "")
 def gemm_bf16(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
               out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
     """bfloat16 operands, 32-bit accumulation.  Few rows go to the weight-streaming kernels (up to how many
-    for this matrix: :func:`dispatch.limits`); many rows go through the library product (as the reference's
+    for this matrix: :func:`dispatch.limits`), some more, where that was measured to be ahead, to the partial-sums
+    kernel and a kernel that adds its stacks; many rows go through the library product (as the reference's
     linears do, ullm/layers/linear.py:165), which for 32-bit output (logits) stores the accumulator unrounded."""
     out_dtype = out_dtype or a.dtype
     M = a.shape[0]
@@ -506,6 +523,9 @@ def gemm_bf16(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = N
         return gemm_skinny(a, w, bias, out_dtype=out_dtype)
     if out_dtype == torch.bfloat16 and M <= min(lim.rows, ROWS_MAX_ROWS) and gemm_rows_supports(a, w):
         return gemm_rows(a, w, bias)
+    if (out_dtype == torch.bfloat16 and 0 < lim.sums_from <= M <= lim.sums_to and w.shape[0] % 4 == 0
+            and gemm_partial_sums_supports(a, w)):
+        return sum_stacks(gemm_partial_sums(a, w), bias)
     if library and out_dtype == torch.float32 and a.is_contiguous() and w.is_contiguous() and _MM_TAKES_OUT_DTYPE:
         y = torch.mm(a, w.t(), out_dtype=torch.float32)
         return y if bias is None else add_bias(y, bias)
