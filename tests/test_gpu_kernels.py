@@ -480,19 +480,22 @@ def test_sampler_rows_cut_into_parts(ops):
     configs = [(0.7, -1, 1.0, 0.0), (1.0, 0, 1.0, 0.0), (1.5, -1, 1.0, 0.0), (0.6, 20, 0.95, 0.0), (1.0, 64, 1.0, 0.0),
                (0.8, 50, 0.9, 0.02), (1.0, 1, 1.0, 0.0), (0.3, 3, 1.0, 0.1), (1.0, 65, 1.0, 0.0),
                (0.7, -1, 0.9, 0.0), (0.25, 0, 0.5, 0.02), (1.0, -1, 0.999, 0.0),        # top-p without top-k
-               (0.8, -1, 1.0, 0.05), (1.0, 0, 1.0, 0.9), (0.5, -1, 1.0, 1e-6)]           # min-p alone
+               (0.8, -1, 1.0, 0.05), (1.0, 0, 1.0, 0.9), (0.5, -1, 1.0, 1e-6),           # min-p alone
+               (0.6, 0, 1.0, 1.0), (7.0, 20, 1.0, 1.0), (0.7, 2000, 1.0, 1.0)]           # a min-p of one: the ties for the maximum
     for V in (10240, 10244, 40960, 151936, 327680, 327684):      # one part exactly, one value into the next, the most parts, too many
         rows = {
             "spread": torch.randn(len(configs), V) * 3,
             "weight at the end": torch.cat([torch.randn(len(configs), V - 8) - 30.0, torch.randn(len(configs), 8) * 2], 1),
             "weight at a part's edge": torch.full((len(configs), V), -40.0),
-            "equal values": torch.zeros(len(configs), V),
+            "equal values": torch.full((len(configs), V), 7.3),             # 7.3 / temperature is no exact product
+            "several largest": torch.randn(len(configs), V) * 2,
             "the largest all in one part": torch.randn(len(configs), V),
             "peaked": torch.randn(len(configs), V) * 12,                     # a nucleus of few values
         }
         edge = min(10236, V - 8)
         rows["weight at a part's edge"][:, edge:edge + 8] = torch.randn(len(configs), 8)
         rows["the largest all in one part"][:, 3000:3100] += 20.0
+        rows["several largest"][:, [5, 4097, V // 2, V - 1]] = 12.7
         for name, logits in rows.items():
             ps = [SamplingParams(temperature=c[0], top_k=c[1], top_p=c[2], min_p=c[3]) for c in configs]
             seeds = [11 + i for i in range(len(configs))]
@@ -500,7 +503,7 @@ def test_sampler_rows_cut_into_parts(ops):
                 pos = [trial * 5 + i for i in range(len(configs))]
                 got = sampler.sample(logits.to(DEV), ps, seeds, pos)
                 for i, c in enumerate(configs):
-                    if name == "equal values" and c[2] < 1.0:
+                    if name in ("equal values", "several largest") and c[2] < 1.0:
                         continue   # which of several equal values top-p drops follows the reference's sort; here all or none
                     assert got[i] in plain.sample_token_set(logits[i], *c, seeds[i], pos[i]), (V, name, c, got[i])
                 again = sampler.sample(logits.flip(0).contiguous().to(DEV), ps[::-1], seeds[::-1], pos[::-1])

@@ -21,6 +21,14 @@ __device__ __forceinline__ uint32_t order_key(float f) {
   return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
 
+// A logit over the temperature, as a product of its own: never fused into the subtraction of the maximum that
+// follows, so that the largest value's distance from the maximum is exactly zero and its weight exactly one
+// in every pass (a min-p of one keeps the ties for the maximum, and the same ones in each pass).
+__device__ __forceinline__ float scaled(float v, float inv_t) {
+#pragma clang fp contract(off)
+  return v * inv_t;
+}
+
 __device__ __forceinline__ int block_sum_int(int v, int* scratch) {
   const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
   const int nwaves = (blockDim.x + WAVE - 1) / WAVE;
@@ -282,7 +290,7 @@ __device__ int sample_small_k(const float* __restrict__ x, int wbeg, int wend, f
     if (by_count) {
       int c1 = 0, c2 = 0, c3 = 0;
       for_range<VEC>(x, wbeg, wend, lane, [&](int, float v) {
-        const uint32_t key = order_key(v * inv_t);
+        const uint32_t key = order_key(scaled(v, inv_t));
         c1 += key >= k1; c2 += key >= k2; c3 += key >= k3;
       });
       c1 = block_sum_int(c1, iscratch); c2 = block_sum_int(c2, iscratch); c3 = block_sum_int(c3, iscratch);
@@ -290,7 +298,7 @@ __device__ int sample_small_k(const float* __restrict__ x, int wbeg, int wend, f
     } else {
       float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
       for_range<VEC>(x, wbeg, wend, lane, [&](int, float v) {
-        const float zz = v * inv_t;
+        const float zz = scaled(v, inv_t);
         const uint32_t key = order_key(zz);
         const float e = __builtin_amdgcn_exp2f((zz - m) * L2E);
         a0 += e;
@@ -329,7 +337,7 @@ __device__ int sample_small_k(const float* __restrict__ x, int wbeg, int wend, f
       int cnt = 0;
 #pragma unroll
       for (int c = 0; c < PER; ++c) {
-        z[c] = raw[u][c] * inv_t;
+        z[c] = scaled(raw[u][c], inv_t);
         keep[c] = ii + c < wend && order_key(z[c]) >= key_thr;
         cnt += keep[c];
       }
@@ -400,7 +408,7 @@ __device__ int walk_range(const float* __restrict__ x, int rbeg, int rend, float
 #pragma unroll
     for (int c = 0; c < PER; ++c) {
       const int i = i0 + PER * lane + c;
-      const float z = cur[c] * inv_t;
+      const float z = scaled(cur[c], inv_t);
       const float ev = __builtin_amdgcn_exp2f((z - m) * L2E);
       e[c] = (i < rend && order_key(z) >= kmin && ev >= mp) ? ev : 0.f;
       if (e[c] > 0.f) kept_hi = i;
@@ -547,7 +555,7 @@ sample_parts_kernel(const float* __restrict__ logits, int V, int ld, const float
     const int ii = wbeg + (j * WAVE + lane) * 4;
     in[j] = ii < pend;
     const float4 v = *reinterpret_cast<const float4*>(x + (in[j] ? ii : pend - 4));
-    z[j][0] = v.x * inv_t; z[j][1] = v.y * inv_t; z[j][2] = v.z * inv_t; z[j][3] = v.w * inv_t;
+    z[j][0] = scaled(v.x, inv_t); z[j][1] = scaled(v.y, inv_t); z[j][2] = scaled(v.z, inv_t); z[j][3] = scaled(v.w, inv_t);
   }
   float mloc = -INFINITY;
 #pragma unroll
@@ -848,7 +856,7 @@ sample_kernel(const float* __restrict__ logits, int V, int ld, const float* __re
   const float L2E = 1.4426950408889634f;
   float mloc = -INFINITY;
   for_range<VEC, 8>(x, wbeg, wend, lane, [&](int, float v) { mloc = fmaxf(mloc, v); });   // 1 / T is positive
-  const float m = block_max(mloc, fscratch) * inv_t;
+  const float m = scaled(block_max(mloc, fscratch), inv_t);
   const uint32_t key_max = order_key(m);
   uint32_t kmin = 0;
 #define E_OF(z) __builtin_amdgcn_exp2f(((z) - m) * L2E)
@@ -869,7 +877,7 @@ sample_kernel(const float* __restrict__ logits, int V, int ld, const float* __re
     while (lo < hi) {
       const uint32_t mid = lo + (hi - lo + 1) / 2;
       int c = 0;
-      for_range<VEC>(x, wbeg, wend, lane, [&](int, float v) { c += order_key(v * inv_t) >= mid; });
+      for_range<VEC>(x, wbeg, wend, lane, [&](int, float v) { c += order_key(scaled(v, inv_t)) >= mid; });
       if (block_sum_int(c, iscratch) >= k) lo = mid; else hi = mid - 1;
     }
     kmin = lo;
@@ -879,7 +887,7 @@ sample_kernel(const float* __restrict__ logits, int V, int ld, const float* __re
   if (p > 0.f && p < 1.f) {  // smallest key v with (mass of keys > v) < p * (mass kept so far)
     float s = 0.f;
     for_range<VEC>(x, wbeg, wend, lane, [&](int, float v) {
-      const float z = v * inv_t;
+      const float z = scaled(v, inv_t);
       if (order_key(z) >= kmin) s += E_OF(z);
     });
     const float bound = p * block_sum(s, fscratch);
@@ -888,7 +896,7 @@ sample_kernel(const float* __restrict__ logits, int V, int ld, const float* __re
       const uint32_t mid = lo + (hi - lo) / 2;
       float a = 0.f;
       for_range<VEC>(x, wbeg, wend, lane, [&](int, float v) {
-        const float z = v * inv_t;
+        const float z = scaled(v, inv_t);
         if (order_key(z) > mid) a += E_OF(z);
       });
       if (block_sum(a, fscratch) < bound) hi = mid; else lo = mid + 1;
@@ -899,10 +907,10 @@ sample_kernel(const float* __restrict__ logits, int V, int ld, const float* __re
   const float mp = mp_row;
   float s = 0.f;
   if (kmin == 0 && !(mp > 0.f)) {          // nothing filtered: every value counts (3 instructions a value)
-    for_range<VEC, 8>(x, wbeg, wend, lane, [&](int, float v) { s += E_OF(v * inv_t); });
+    for_range<VEC, 8>(x, wbeg, wend, lane, [&](int, float v) { s += E_OF(scaled(v, inv_t)); });
   } else {
     for_range<VEC>(x, wbeg, wend, lane, [&](int, float v) {
-      const float z = v * inv_t;
+      const float z = scaled(v, inv_t);
       const float e = E_OF(z);
       if (order_key(z) >= kmin && e >= mp) s += e;
     });
@@ -933,7 +941,7 @@ sample_kernel(const float* __restrict__ logits, int V, int ld, const float* __re
   if (chosen < 0) {  // rounding pushed the target past the total: take the last kept index
     int last = -1;
     for_range<VEC>(x, wbeg, wend, lane, [&](int i, float v) {
-      const float z = v * inv_t;
+      const float z = scaled(v, inv_t);
       if (order_key(z) >= kmin && E_OF(z) >= mp) last = i > last ? i : last;
     });
 #pragma unroll
