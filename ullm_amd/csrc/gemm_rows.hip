@@ -1,4 +1,4 @@
-// C[M, N] = X[M, K] * W[N, K]^T for 17 to 64 rows, bfloat16 in and out, 32-bit accumulation, with what
+// C[M, N] = X[M, K] * W[N, K]^T for 17 to 128 rows, bfloat16 in and out, 32-bit accumulation, with what
 // follows the product folded in:
 //   STORE : C = result (+ bias)
 //   SILU  : W is the stacked gate|up matrix [2 N, K]; C[M, N] = silu(gate) * up on the 32-bit sums
@@ -56,13 +56,20 @@ __device__ __forceinline__ void static_for(F&& f) {
 }
 
 #define ROWS_MAX_WAVES 8   // waves of a block (512 threads: two waves a SIMD, 256 registers each)
+#define ROWS_MAX_TILES 8   // 16-row tiles of X: 128 rows
 
 // Stages of W and of X a wave has in flight (of X as many as of W: loads complete in order, so waiting for a stage
 // of X waits for every load issued before it, and a stage of X fetched later than a stage of W would cut short
 // what W has in flight).  As many as about 150 registers hold: ntw tiles of W (two 16-byte pieces each) and xq
-// pieces of X per stage.
-__host__ __device__ constexpr int rows_depth(int ntw, int xq) {
-  const int d = 150 / ((2 * ntw + xq) * 4);
+// pieces of X per stage; from five tiles of rows on, as many as the sums (4 ntw mt registers), the operands of a
+// step (4 (ntw + mt)) and 64 more leave of the 256, and two stages at least.
+__host__ __device__ constexpr int rows_depth(int ntw, int xq, int mt) {
+  const int stage = (2 * ntw + xq) * 4;
+  if (mt > 4) {
+    const int d = (256 - 4 * ntw * mt - 4 * (ntw + mt) - 64) / stage;
+    return d < 2 ? 2 : (d > 8 ? 8 : d);
+  }
+  const int d = 150 / stage;
   return d < 3 ? 3 : (d > 8 ? 8 : d);
 }
 
@@ -74,7 +81,7 @@ gemm_rows_kernel(const bf16_t* __restrict__ X, int ldx, const bf16_t* __restrict
                  const float* __restrict__ bias, bf16_t* __restrict__ C, int ldc, int M, int N, int K,
                  int WN, int cols_per_wave, int cols_per_block, RowSquares before) {
   constexpr int NTW = EPI == ROWS_SILU ? 2 : 1;         // tiles of W per wave: gate and up rows of the same columns
-  constexpr int D = rows_depth(NTW, XQ);
+  constexpr int D = rows_depth(NTW, XQ, MT);
   constexpr int TILE = 16 * 128;                        // 16 rows x 64 values
   constexpr int XB = MT * TILE;                         // a stage of X
   __shared__ __attribute__((aligned(16))) unsigned char xs[2 * XB + 64 * 16];   // two stages, then a spare place per lane
@@ -243,6 +250,12 @@ static int rows_compute_units() {
   return units[dev];
 }
 
+// 16-row tiles of X that the kernel is compiled for: 1 to 6, then 8
+static int rows_tiles(int M) {
+  const int mt = (M + 15) / 16;
+  return mt <= 6 ? mt : ROWS_MAX_TILES;
+}
+
 struct RowsShape {
   int cols_per_block, cols_per_wave, wn, xq, blocks;
 };
@@ -250,7 +263,7 @@ struct RowsShape {
 // How a matrix of N result columns is cut: a whole number of rounds of one block per compute unit, and
 // the block's columns over its waves in steps of 4 (at most 16 per wave).  A function of the matrix, the
 // epilogue and the number of 16-row tiles of X alone.
-static bool rows_shape(int N, int mt, int units, RowsShape* s) {
+static bool rows_shape(int N, int mt, int epi, int units, RowsShape* s) {
   const int rounds = (N + units * 16 * ROWS_MAX_WAVES - 1) / (units * 16 * ROWS_MAX_WAVES);
   int cpb = (N + rounds * units - 1) / (rounds * units);
   cpb = (cpb + 3) / 4 * 4;
@@ -265,17 +278,58 @@ static bool rows_shape(int N, int mt, int units, RowsShape* s) {
   s->wn = wn;
   s->xq = (mt * 128 + 64 * wn - 1) / (64 * wn);
   s->blocks = (N + cpb - 1) / cpb;
+  // 128 rows of X over the 128 threads of two waves, with two tiles of W per wave: more registers than a lane has
+  if (epi == ROWS_SILU && mt == ROWS_MAX_TILES && s->xq > 6) return false;
   return true;
+}
+
+// What a launch takes, and the kernel picked step by step: only the combinations that rows_shape can give are
+// compiled (a thread never has more pieces of a stage of X than there are tiles of rows).
+struct RowsLaunch {
+  const bf16_t* X; int ldx;
+  const bf16_t* W; int ldw;
+  const float* bias;
+  bf16_t* C; int ldc;
+  int M, N, K;
+  RowsShape s;
+  RowSquares before;
+  hipStream_t stream;
+};
+
+template <int MT, int XQ, int EPI>
+static void rows_pick_pieces(const RowsLaunch& a) {
+  if constexpr (XQ >= MT) {
+    hipLaunchKernelGGL((gemm_rows_kernel<MT, XQ, EPI>), dim3(a.s.blocks), dim3(64 * a.s.wn), 0, a.stream, a.X, a.ldx, a.W,
+                       a.ldw, a.bias, a.C, a.ldc, a.M, a.N, a.K, a.s.wn, a.s.cols_per_wave, a.s.cols_per_block, a.before);
+  } else {
+    if (a.s.xq <= XQ)
+      hipLaunchKernelGGL((gemm_rows_kernel<MT, XQ, EPI>), dim3(a.s.blocks), dim3(64 * a.s.wn), 0, a.stream, a.X, a.ldx,
+                         a.W, a.ldw, a.bias, a.C, a.ldc, a.M, a.N, a.K, a.s.wn, a.s.cols_per_wave, a.s.cols_per_block,
+                         a.before);
+    else rows_pick_pieces<MT, XQ + 1, EPI>(a);
+  }
+}
+
+// tiles of rows: 1 to 6, then 8 (the row counts that steps are padded to: 16 .. 96, 128)
+template <int EPI>
+static void rows_pick_tiles(const RowsLaunch& a, int mt) {
+  if (mt == 1) rows_pick_pieces<1, 1, EPI>(a);
+  else if (mt == 2) rows_pick_pieces<2, 1, EPI>(a);
+  else if (mt == 3) rows_pick_pieces<3, 1, EPI>(a);
+  else if (mt == 4) rows_pick_pieces<4, 1, EPI>(a);
+  else if (mt == 5) rows_pick_pieces<5, 1, EPI>(a);
+  else if (mt == 6) rows_pick_pieces<6, 1, EPI>(a);
+  else rows_pick_pieces<8, 1, EPI>(a);
 }
 
 // N: columns of the result (with epi 1 the weights have 2 N rows)
 extern "C" int ullm_gemm_rows_supports(int M, int N, int K, int ldx, int ldw, int ldc, int epi) {
   RowsShape s;
-  return M >= 1 && M <= 64 && N >= 4 && K >= 64 && K % 64 == 0 && ldx % 8 == 0 && ldw % 8 == 0 && ldc % 4 == 0 &&
-         ldc >= N && (epi == ROWS_STORE || epi == ROWS_SILU) && rows_shape(N, (M + 15) / 16, rows_compute_units(), &s);
+  return M >= 1 && M <= 16 * ROWS_MAX_TILES && N >= 4 && K >= 64 && K % 64 == 0 && ldx % 8 == 0 && ldw % 8 == 0 && ldc % 4 == 0 &&
+         ldc >= N && (epi == ROWS_STORE || epi == ROWS_SILU) && rows_shape(N, rows_tiles(M), epi, rows_compute_units(), &s);
 }
 
-// X bfloat16 [M <= 64, K], K a multiple of 64; W bfloat16 [N, K] (epi 1: [2 N, K], gate rows then up rows);
+// X bfloat16 [M <= 128, K], K a multiple of 64; W bfloat16 [N, K] (epi 1: [2 N, K], gate rows then up rows);
 // C bfloat16 [M, N] with row stride ldc; bias float32 [N] or null (epi 0 only).
 // With row_sq (float32 [M <= 16, sq_parts], sq_parts a multiple of 4): the results of row m are scaled by
 // rsqrt(sum of row_sq[m][.] / K + eps) before the epilogue.
@@ -288,30 +342,11 @@ extern "C" int ullm_gemm_rows(const void* X, int ldx, const void* W, int ldw, co
   if (epi == ROWS_SILU && bias) return ULLM_ERR_UNSUPPORTED;
   if (row_sq && (M > 16 || sq_parts < 4 || sq_parts % 4 || ((uintptr_t)row_sq & 15))) return ULLM_ERR_UNSUPPORTED;
   const RowSquares before{row_sq, sq_parts / 4, eps};
-  const int mt = (M + 15) / 16;
+  const int mt = rows_tiles(M);
   RowsShape s;
-  rows_shape(N, mt, rows_compute_units(), &s);
-  dim3 grid(s.blocks), block(64 * s.wn);
-#define GO(MT, XQ, EPI) hipLaunchKernelGGL((gemm_rows_kernel<MT, XQ, EPI>), grid, block, 0, stream, (const bf16_t*)X, ldx, \
-    (const bf16_t*)W, ldw, bias, (bf16_t*)C, ldc, M, N, K, s.wn, s.cols_per_wave, s.cols_per_block, before)
-#define GO_XQ(MT, EPI)                                    \
-  do {                                                    \
-    if (s.xq <= 1) GO(MT, 1, EPI);                        \
-    else if (s.xq == 2) { if constexpr (MT >= 2) GO(MT, 2, EPI); } \
-    else if (s.xq == 3) { if constexpr (MT >= 3) GO(MT, 3, EPI); } \
-    else { if constexpr (MT >= 4) GO(MT, 4, EPI); }       \
-  } while (0)
-#define GO_MT(EPI)                         \
-  do {                                     \
-    if (mt == 1) GO_XQ(1, EPI);            \
-    else if (mt == 2) GO_XQ(2, EPI);       \
-    else if (mt == 3) GO_XQ(3, EPI);       \
-    else GO_XQ(4, EPI);                    \
-  } while (0)
-  if (epi == ROWS_SILU) GO_MT(ROWS_SILU);
-  else GO_MT(ROWS_STORE);
-#undef GO_MT
-#undef GO_XQ
-#undef GO
+  rows_shape(N, mt, epi, rows_compute_units(), &s);
+  const RowsLaunch go{(const bf16_t*)X, ldx, (const bf16_t*)W, ldw, bias, (bf16_t*)C, ldc, M, N, K, s, before, stream};
+  if (epi == ROWS_SILU) rows_pick_tiles<ROWS_SILU>(go, mt);
+  else rows_pick_tiles<ROWS_STORE>(go, mt);
   ULLM_LAUNCH_CHECK();
 }

@@ -50,7 +50,7 @@ def default_limits(columns: int, inner: int) -> Limits:
     measured matrices (2 M to 780 M elements) have in common: the rows kernel needs enough columns to give
     every compute unit a block; a small matrix has few blocks to pay for 32-bit rows of X, so the norm stays
     folded in for every row count the kernel takes; gate|up keeps the few-rows kernel to 32 rows unless the
-    matrix is very large; stacks of partial sums outweigh a matrix of a few M elements; the few-rows kernel
+    matrix is very large, and the rows kernel to 128 rows from 12 288 result columns on; stacks of partial sums outweigh a matrix of a few M elements; the few-rows kernel
     with four tiles a block is ahead of the library up to 32 rows on matrices with very many columns."""
     weight = columns * inner
     return Limits(
@@ -58,7 +58,7 @@ def default_limits(columns: int, inner: int) -> Limits:
         rows=64 if columns >= 2048 else 0,
         fold_norm=16 if weight <= (40 << 20) else 8,
         silu_skinny=32 if weight <= 200_000_000 else 16,
-        silu_rows=64 if columns // 2 >= 2048 else 0,
+        silu_rows=(128 if columns // 2 >= 12288 else 64) if columns // 2 >= 2048 else 0,
         stacked_from=17 if weight >= (8 << 20) else 0,
         stacked_to=256 if weight >= (8 << 20) else 0,
         f32_skinny=32 if columns >= 65536 else 16)

@@ -189,7 +189,7 @@ def derive_limits(times: dict, roles, columns: int, inner: int) -> dict:
     changes = {}
     if "store" in roles:
         changes["skinny"] = _ahead_up_to(rows, get("skinny"), [get("rows"), get("library")])
-        changes["rows"] = _ahead_up_to(rows, get("rows"), [get("library")], start=changes["skinny"])
+        changes["rows"] = _ahead_up_to(rows, get("rows"), [get("library"), get("partial sums>sum")], start=changes["skinny"])
         if changes["rows"] == changes["skinny"]:
             changes["rows"] = 0
         best = {r: min(t[r] for t in (get("skinny"), get("rows"), get("library")) if r in t) for r in rows}

@@ -467,7 +467,7 @@ def gemm_partial_sums(a: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     return out
 
 
-ROWS_MAX_ROWS = 64        # most rows the kernel takes (which matrices it is chosen for: dispatch.limits)
+ROWS_MAX_ROWS = 128       # most rows the kernel takes (which matrices it is chosen for: dispatch.limits)
 
 
 def gemm_rows_supports(a: torch.Tensor, w: torch.Tensor, silu: bool = False) -> bool:
@@ -483,13 +483,13 @@ def gemm_rows_supports(a: torch.Tensor, w: torch.Tensor, silu: bool = False) -> 
 
 def gemm_rows(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, silu: bool = False,
               squares: Optional[torch.Tensor] = None, eps: float = 0.0) -> torch.Tensor:
-    """a (bfloat16 [M <= 64, K]) times w (bfloat16 [N, K]) transposed (+ bias float32 [N]) as bfloat16 [M, N];
+    """a (bfloat16 [M <= 128, K]) times w (bfloat16 [N, K]) transposed (+ bias float32 [N]) as bfloat16 [M, N];
     with ``silu``, w is gate | up [2 I, K] and the result silu(gate) * up [M, I] on the 32-bit sums.  The
     matrix is cut into one block per compute unit and every wave keeps several stages of its rows of w in
     flight: for the row counts between the few-rows kernel and the library.  ``squares``, ``eps``: as in
     :func:`gemm_skinny`."""
     M, K = a.shape
-    _need(gemm_rows_supports(a, w, silu), "gemm_rows takes bfloat16, M <= 64, K a multiple of 8, N a multiple of 4")
+    _need(gemm_rows_supports(a, w, silu), "gemm_rows takes bfloat16, M <= 128, K a multiple of 64, N a multiple of 4")
     n_out = w.shape[0] // 2 if silu else w.shape[0]
     if bias is not None:
         _need(not silu and bias.dtype == torch.float32 and bias.numel() == n_out and bias.is_contiguous(),

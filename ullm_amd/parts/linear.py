@@ -82,7 +82,7 @@ def add_into_stream(x: torch.Tensor, weight: torch.Tensor, residual: torch.Tenso
 
 def gate_up(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     """silu(x g^T) * (x u^T) for the stacked weights g | u [2 I, K]: by the few-rows kernel or the kernel for up
-    to 64 rows with the activation on store, up to the row counts the matrix's limits name; else by the
+    to 128 rows with the activation on store, up to the row counts the matrix's limits name; else by the
     library product and the activation kernel (float32 always: the 32-bit product, then the kernel)."""
     rows = x.shape[0]
     if x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16:
