@@ -428,14 +428,17 @@ def test_sampler_kernel_against_the_plain_sampler(ops):
 
 def test_sampler_with_a_small_top_k_over_a_large_vocabulary(ops):
     """Top-k with a small k, and top-p alone on a peaked row, gather the few values that can matter and
-    filter those; rows where that cannot work (many equal values around the k-th largest, the k-th largest
-    far below the maximum, a flat row under top-p alone) take the passes over the whole vocabulary.  Either way the token is one the plain sampler may draw."""
+    filter those; rows where that cannot work (a large k, a flat row under top-p alone) find their thresholds by
+    bins of the distance from the maximum, and where that cannot work either (many equal values around the k-th
+    largest, the k-th largest far below the maximum) by halving over the whole vocabulary.  Either way the token
+    is one the plain sampler may draw."""
     from ullm_amd.sampling import Sampler, SamplingParams
     torch.manual_seed(17)
     sampler = Sampler(torch.device(DEV))
     configs = [(0.6, 20, 0.95, 0.0), (1.0, 5, 1.0, 0.0), (0.8, 50, 0.9, 0.02), (1.0, 1000, 1.0, 0.0), (1.2, 1, 1.0, 0.0),
                (0.7, 20, 0.5, 0.0), (1.0, 1024, 0.99, 0.0), (1.0, 1025, 1.0, 0.0),
-               (0.7, -1, 0.9, 0.0), (1.0, 0, 0.5, 0.02), (0.5, -1, 0.99, 0.0)]        # top-p alone
+               (0.7, -1, 0.9, 0.0), (1.0, 0, 0.5, 0.02), (0.5, -1, 0.99, 0.0),        # top-p alone
+               (1.0, 5000, 1.0, 0.0), (0.9, 3000, 0.8, 0.05), (1.3, 20000, 0.95, 0.0)]  # thresholds far down the row: by bins
     whole_rows = Sampler(torch.device(DEV), cut_rows=False)    # one block per row, no parts
     for V in (32000, 151936, 50257):       # 50257: rows not aligned for 16-byte loads
         masked = torch.randn(len(configs), V) * 3

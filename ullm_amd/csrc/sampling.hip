@@ -5,8 +5,10 @@
 // (keep values >= the k-th largest, ties kept, sampler.py:67-76), top-p on the softmax of what top-k
 // left (drop the low tail whose cumulative probability is <= 1 - p, sampler.py:78-92), min-p
 // (drop probabilities below min_p * max, sampler.py:95-107), softmax, draw.  How it is computed
-// differs: no sort of the vocabulary.  Every filter is a threshold on the value, found by bisection
-// over the order-preserving integer image of the floats with fixed-order block reductions, and the
+// differs: no sort of the vocabulary.  Every filter is a threshold on the value: among a few gathered
+// candidates where the setting and the row allow it, else by bins of the distance from the maximum (counts and
+// fixed-point weights, so that no sum depends on the order of its additions) and a search inside one bin, else by
+// bisection over the order-preserving integer image of the floats with fixed-order block reductions; and the
 // draw is an inverse-CDF walk in index order with a counter-based uniform from (seed, position), so
 // a row's token depends on nothing else in the batch.  T == 0 picks the first index of the maximum
 // (the reference has no greedy path that its runner reaches, sampler.py:28-36).
@@ -93,7 +95,7 @@ __device__ __forceinline__ void for_range(const float* __restrict__ x, int wbeg,
 // own range and its own segment); every filter and the draw then run over the candidates only, by
 // the same rules as over the whole vocabulary.  Where this does not work out (fewer than k values
 // within 32 of the maximum, or more candidates than a segment holds: many equal values, a flat row
-// under top-p alone) the caller takes the long way.
+// under top-p alone) the caller takes the long way (thresholds by bins, see below).
 #define SMALL_K_MAX 1024
 #define SEG 256                       // candidates a wave can hold
 #define DELTA_STEPS 16
@@ -488,6 +490,253 @@ __device__ int walk_range(const float* __restrict__ x, int rbeg, int rend, float
   return pick >= 0 ? pick : last_kept;
 }
 
+// ------------------------------------------------------------------------------ thresholds by bins
+// The long way's thresholds (the k-th largest key; the key at which the weight of the larger values falls below
+// the share p) without a pass per halving.  One pass puts every value that still counts into one of BIN_COUNT
+// bins by its distance from the maximum (1/64 wide; the last bin takes everything from BIN_RANGE on) and adds the
+// bins' counts and weights in shared memory.  Weights are 32.32 fixed-point integers (a weight is at most one),
+// so their sums do not depend on the order in which the atomic additions land, and neither does the token.  A scan
+// over the bins from the maximum down finds the bin in which the count reaches k or the weight reaches the
+// share; if that bin holds too many values for a list, a second pass cuts it into BIN_COUNT finer bins (the
+// difference of two distances inside one bin is exact), then a pass gathers the bin's values and the halvings
+// run over that list.  false: not decided here (the k-th largest or the nucleus's end lies further than
+// BIN_RANGE below the maximum, or too many values share one fine bin: equal values); the caller halves over the
+// whole vocabulary as before.  Every thread of the block returns the same.
+#define BIN_COUNT 2048
+#define BIN_PER_UNIT 64.f
+#define BIN_FINE (BIN_PER_UNIT * BIN_COUNT)
+#define BIN_LIST 2048                 // a bin with more values than this is cut again (a wave's segment holds SEG of them)
+
+__device__ __forceinline__ unsigned long long block_sum_u64(unsigned long long v, unsigned long long* scratch) {
+  const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE, nwaves = blockDim.x / WAVE;
+#pragma unroll
+  for (int d = WAVE / 2; d > 0; d >>= 1) v += __shfl_xor(v, d, WAVE);
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  unsigned long long r = 0;
+  for (int w = 0; w < nwaves; ++w) r += scratch[w];
+  return r;
+}
+
+// the sum of the threads before this one
+__device__ __forceinline__ unsigned long long block_sum_before_u64(unsigned long long v, unsigned long long* scratch) {
+  const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
+  unsigned long long incl = v;
+#pragma unroll
+  for (int d = 1; d < WAVE; d <<= 1) {
+    const unsigned long long o = __shfl_up(incl, d, WAVE);
+    if (lane >= d) incl += o;
+  }
+  __syncthreads();
+  if (lane == WAVE - 1) scratch[wave] = incl;
+  __syncthreads();
+  unsigned long long base = 0;
+  for (int w = 0; w < wave; ++w) base += scratch[w];
+  return base + incl - v;
+}
+
+struct BinPick {
+  int bin, count;
+  unsigned long long above;           // count or weight of everything in the bins before it
+};
+
+template <bool VEC, bool BY_COUNT>
+__device__ __noinline__ bool threshold_by_bins(const float* __restrict__ x, int wbeg, int wend, float inv_t, float m,
+                                  uint32_t kmin_in, int k, float p, Candidates& cand, unsigned long long* wide,
+                                  BinPick* pick, uint32_t* found) {
+  constexpr int PER = VEC ? 4 : 1;
+  constexpr int STEP = PER * WAVE;
+  const int tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE, nwaves = blockDim.x / WAVE;
+  const float L2E = 1.4426950408889634f;
+  unsigned long long* const bin_w = reinterpret_cast<unsigned long long*>(cand.lz);   // BIN_COUNT of them
+  unsigned* const bin_n = reinterpret_cast<unsigned*>(cand.le);
+  static_assert(sizeof(cand.lz) >= BIN_COUNT * sizeof(unsigned long long) && sizeof(cand.le) >= BIN_COUNT * sizeof(unsigned),
+                "the bins lie where the list of candidates lies otherwise");
+  // a value's bin: by its distance from the maximum; inside bin `coarse`, by the rest of that distance
+  auto bin_of = [&](float z, int coarse) {
+    const float dist = m - z;                                       // >= 0; +inf for a masked value
+    const int b1 = (int)fminf(dist * BIN_PER_UNIT, (float)(BIN_COUNT - 1));
+    if (coarse < 0) return b1;
+    if (b1 != coarse) return -1;
+    const float rest = dist - (float)b1 * (1.f / BIN_PER_UNIT);     // exact: both are multiples of the distance's last bit
+    const int b2 = (int)fminf(rest * BIN_FINE, (float)(BIN_COUNT - 1));
+    return b2 < 0 ? 0 : b2;
+  };
+  auto weight_of = [&](float z) {
+    return (unsigned long long)(__builtin_amdgcn_exp2f((z - m) * L2E) * 4294967296.f);
+  };
+  unsigned long long above = 0, bound = BY_COUNT ? (unsigned long long)k : 0;
+  int coarse = -1, fine = -1, count = 0;
+#pragma unroll 1
+  for (int level = 0; level < 2; ++level) {
+    for (int b = tid; b < BIN_COUNT; b += blockDim.x) { bin_w[b] = 0; bin_n[b] = 0; }
+    if (tid == 0) pick->bin = -1;
+    __syncthreads();
+    for_range<VEC>(x, wbeg, wend, lane, [&](int, float v) {
+      const float z = scaled(v, inv_t);
+      if (order_key(z) < kmin_in) return;
+      const int b = bin_of(z, coarse);
+      if (b < 0) return;
+      atomicAdd(&bin_n[b], 1u);
+      if (!BY_COUNT) atomicAdd(&bin_w[b], weight_of(z));
+    });
+    __syncthreads();
+    // this thread's bins, in order from the maximum down
+    const int per_thread = BIN_COUNT / SAMPLE_THREADS;
+    unsigned long long mine[per_thread], sum = 0;
+#pragma unroll
+    for (int i = 0; i < per_thread; ++i) {
+      mine[i] = BY_COUNT ? (unsigned long long)bin_n[per_thread * tid + i] : bin_w[per_thread * tid + i];
+      sum += mine[i];
+    }
+    if (!BY_COUNT && level == 0) {
+      const unsigned long long total = block_sum_u64(sum, wide);
+      bound = (unsigned long long)((double)p * (double)total);
+      if (bound == 0) bound = 1;
+    }
+    unsigned long long before = above + block_sum_before_u64(sum, wide);
+#pragma unroll
+    for (int i = 0; i < per_thread; ++i) {
+      if (before < bound && before + mine[i] >= bound) {             // one thread at most
+        pick->bin = per_thread * tid + i;
+        pick->count = (int)bin_n[per_thread * tid + i];
+        pick->above = before;
+      }
+      before += mine[i];
+    }
+    __syncthreads();
+    const int at = pick->bin;
+    count = pick->count;
+    above = pick->above;
+    __syncthreads();
+    if (at < 0) return false;                                        // fewer than k values, or no weight: not here
+    if (level == 0) {
+      if (at == BIN_COUNT - 1) return false;                         // further from the maximum than the bins reach
+      coarse = at;
+      if (count <= BIN_LIST) break;
+    } else {
+      fine = at;
+    }
+  }
+  if (count > 16 * SEG) return false;
+  // the bin's values, a wave's in its segment
+  int pos = 0;
+  bool overflow = false;
+  constexpr int AHEAD = 4;
+  for (int base = wbeg; base < wend && !overflow; base += AHEAD * STEP) {
+    float raw[AHEAD][PER];
+#pragma unroll
+    for (int u = 0; u < AHEAD; ++u) {
+      const int ii = base + u * STEP + PER * lane;
+      if (VEC) {
+        const float4 v = ii < wend ? *reinterpret_cast<const float4*>(x + ii) : make_float4(0.f, 0.f, 0.f, 0.f);
+        raw[u][0] = v.x;
+        if (PER > 1) { raw[u][1] = v.y; raw[u][2] = v.z; raw[u][3] = v.w; }
+      } else {
+        raw[u][0] = ii < wend ? x[ii] : 0.f;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < AHEAD; ++u) {
+      const int ii = base + u * STEP + PER * lane;
+      float z[PER];
+      bool keep[PER];
+      int cnt = 0;
+#pragma unroll
+      for (int c = 0; c < PER; ++c) {
+        z[c] = scaled(raw[u][c], inv_t);
+        keep[c] = ii + c < wend && order_key(z[c]) >= kmin_in &&
+                  (fine >= 0 ? bin_of(z[c], coarse) == fine : bin_of(z[c], -1) == coarse);
+        cnt += keep[c];
+      }
+      if (overflow || !__any(cnt)) continue;
+      int incl = cnt;
+#pragma unroll
+      for (int d = 1; d < WAVE; d <<= 1) {
+        const int o = __shfl_up(incl, d, WAVE);
+        if (lane >= d) incl += o;
+      }
+      const int total = __shfl(incl, WAVE - 1, WAVE);
+      if (pos + total > SEG) { overflow = true; continue; }
+      int o = wave * SEG + pos + incl - cnt;
+#pragma unroll
+      for (int c = 0; c < PER; ++c)
+        if (keep[c]) cand.z[o++] = z[c];
+      pos += total;
+    }
+  }
+  if (lane == 0) cand.n[wave] = overflow ? -1 : pos;
+  __syncthreads();
+  bool bad = false;
+  for (int w = 0; w < nwaves; ++w) bad = bad || cand.n[w] < 0;
+  if (bad) return false;
+  // The list's keys and weights side by side where the bins lay (the 64-bit weights of the first 8 SEG fill
+  // cand.lz, those of the others cand.lidx), the smallest and the largest key; then one wave halves between
+  // them with no barrier.
+  uint32_t* const slot_key = reinterpret_cast<uint32_t*>(cand.le);
+  unsigned long long* const slot_w = reinterpret_cast<unsigned long long*>(cand.lz);
+  unsigned long long* const slot_w_hi = reinterpret_cast<unsigned long long*>(cand.lidx);
+  static_assert(sizeof(cand.lz) == 8 * SEG * sizeof(unsigned long long) && sizeof(cand.lidx) == sizeof(cand.lz) &&
+                sizeof(cand.le) == 16 * SEG * sizeof(uint32_t), "the slots' keys and weights fill these arrays");
+  uint32_t lo = 0xffffffffu, hi = 0;
+  int n_all = 0;
+  for (int w = 0; w < nwaves; ++w) n_all += cand.n[w];
+  for (int e = tid; e < 16 * SEG; e += blockDim.x) {
+    const int seg = e / SEG, j = e & (SEG - 1);
+    if (j >= cand.n[seg]) continue;
+    int to = j;
+    for (int w = 0; w < seg; ++w) to += cand.n[w];
+    const float z = cand.z[e];
+    const uint32_t key = order_key(z);
+    slot_key[to] = key;
+    (to < 8 * SEG ? slot_w[to] : slot_w_hi[to - 8 * SEG]) = BY_COUNT ? 1ull : weight_of(z);
+    lo = key < lo ? key : lo;
+    hi = key > hi ? key : hi;
+  }
+#pragma unroll
+  for (int d = WAVE / 2; d > 0; d >>= 1) {
+    const uint32_t ol = __shfl_xor(lo, d, WAVE), oh = __shfl_xor(hi, d, WAVE);
+    lo = ol < lo ? ol : lo;
+    hi = oh > hi ? oh : hi;
+  }
+  __syncthreads();
+  if (lane == 0) { wide[wave] = lo; wide[16 + wave] = hi; }
+  __syncthreads();
+  for (int w = 0; w < nwaves; ++w) {
+    lo = (uint32_t)wide[w] < lo ? (uint32_t)wide[w] : lo;
+    hi = (uint32_t)wide[16 + w] > hi ? (uint32_t)wide[16 + w] : hi;
+  }
+  if (lo > hi) return false;                                         // an empty list: cannot be
+  if (wave == 0) {
+    auto weight_where = [&](auto pred) {
+      unsigned long long a = 0;
+#pragma unroll 4
+      for (int e = lane; e < n_all; e += WAVE)
+        a += pred(slot_key[e]) ? (e < 8 * SEG ? slot_w[e] : slot_w_hi[e - 8 * SEG]) : 0ull;
+#pragma unroll
+      for (int d = WAVE / 2; d > 0; d >>= 1) a += __shfl_xor(a, d, WAVE);
+      return a;
+    };
+    if (BY_COUNT) {                          // the largest key v with (values above the bin) + #{key >= v} >= k
+      while (lo < hi) {
+        const uint32_t mid = lo + (hi - lo + 1) / 2;
+        if (above + weight_where([&](uint32_t key) { return key >= mid; }) >= bound) lo = mid; else hi = mid - 1;
+      }
+    } else {                                 // the smallest key v with (weight above the bin) + (weight of keys > v) < bound
+      while (lo < hi) {
+        const uint32_t mid = lo + (hi - lo) / 2;
+        if (above + weight_where([&](uint32_t key) { return key > mid; }) < bound) hi = mid; else lo = mid + 1;
+      }
+    }
+    if (lane == 0) pick->bin = (int)lo;
+  }
+  __syncthreads();
+  lo = (uint32_t)pick->bin;
+  *found = lo;
+  return true;
+}
+
 // ------------------------------------------------------------------------------ parts of a row
 // One block per row reads 150 K values with one compute unit, pass after pass.  For the common settings
 // (temperature alone; top-k with a small k, with or without top-p and min-p; top-p or min-p without top-k) a first
@@ -682,6 +931,8 @@ sample_kernel(const float* __restrict__ logits, int V, int ld, const float* __re
   __shared__ float part_w[MAX_PARTS];
   __shared__ float step_sum[WAVE];
   __shared__ int step_kept[WAVE];
+  __shared__ unsigned long long wide[32];
+  __shared__ BinPick bin_pick;
   __shared__ Candidates cand;
   constexpr int STEP = VEC ? 4 * WAVE : WAVE;        // values a wave reads per access
   const int row = blockIdx.x, tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
@@ -863,7 +1114,8 @@ sample_kernel(const float* __restrict__ logits, int V, int ld, const float* __re
 
   const int k = k_row;
   const bool top_k_on = k > 0 && k < V, top_p_on = p_row > 0.f && p_row < 1.f;
-  if (((top_k_on && k <= SMALL_K_MAX) || (!top_k_on && top_p_on)) && blockDim.x == SAMPLE_THREADS) {
+  // (top-p alone on a row that the parts' candidates could not serve: its nucleus is long, the bins find its end)
+  if (((top_k_on && k <= SMALL_K_MAX) || (!top_k_on && top_p_on && mode != PARTS_TOP_P)) && blockDim.x == SAMPLE_THREADS) {
     const int token = sample_small_k<VEC>(x, wbeg, wend, inv_t, m, top_k_on ? k : 0, p_row, mp_row,
                                           uniform_from_seed(seed, position_row), cand, fscratch, iscratch);
     if (token >= 0) {
@@ -872,7 +1124,10 @@ sample_kernel(const float* __restrict__ logits, int V, int ld, const float* __re
     }
     __syncthreads();
   }
-  if (k > 0 && k < V) {  // largest key v with #{key >= v} >= k
+  bool by_bins = false;
+  if (k > 0 && k < V && blockDim.x == SAMPLE_THREADS)
+    by_bins = threshold_by_bins<VEC, true>(x, wbeg, wend, inv_t, m, 0u, k, 0.f, cand, wide, &bin_pick, &kmin);
+  if (k > 0 && k < V && !by_bins) {  // largest key v with #{key >= v} >= k
     uint32_t lo = 0, hi = key_max;
     while (lo < hi) {
       const uint32_t mid = lo + (hi - lo + 1) / 2;
@@ -884,7 +1139,13 @@ sample_kernel(const float* __restrict__ logits, int V, int ld, const float* __re
   }
 
   const float p = p_row;
-  if (p > 0.f && p < 1.f) {  // smallest key v with (mass of keys > v) < p * (mass kept so far)
+  by_bins = false;
+  if (p > 0.f && p < 1.f && blockDim.x == SAMPLE_THREADS) {
+    uint32_t at = 0;
+    by_bins = threshold_by_bins<VEC, false>(x, wbeg, wend, inv_t, m, kmin, 0, p, cand, wide, &bin_pick, &at);
+    if (by_bins) kmin = at;
+  }
+  if (p > 0.f && p < 1.f && !by_bins) {  // smallest key v with (mass of keys > v) < p * (mass kept so far)
     float s = 0.f;
     for_range<VEC>(x, wbeg, wend, lane, [&](int, float v) {
       const float z = scaled(v, inv_t);
