@@ -539,6 +539,7 @@ __device__ __forceinline__ unsigned long long block_sum_before_u64(unsigned long
 struct BinPick {
   int bin, count;
   unsigned long long above;           // count or weight of everything in the bins before it
+  uint32_t key;                       // the threshold, from the wave that found it to the block
 };
 
 template <bool VEC, bool BY_COUNT>
@@ -729,10 +730,10 @@ __device__ __noinline__ bool threshold_by_bins(const float* __restrict__ x, int 
         if (above + weight_where([&](uint32_t key) { return key > mid; }) < bound) hi = mid; else lo = mid + 1;
       }
     }
-    if (lane == 0) pick->bin = (int)lo;
+    if (lane == 0) pick->key = lo;
   }
   __syncthreads();
-  lo = (uint32_t)pick->bin;
+  lo = pick->key;
   *found = lo;
   return true;
 }
