@@ -498,10 +498,11 @@ __device__ int walk_range(const float* __restrict__ x, int rbeg, int rend, float
 // so their sums do not depend on the order in which the atomic additions land, and neither does the token.  A scan
 // over the bins from the maximum down finds the bin in which the count reaches k or the weight reaches the
 // share; if that bin holds too many values for a list, a second pass cuts it into BIN_COUNT finer bins (the
-// difference of two distances inside one bin is exact), then a pass gathers the bin's values and the halvings
-// run over that list.  false: not decided here (the k-th largest or the nucleus's end lies further than
-// BIN_RANGE below the maximum, or too many values share one fine bin: equal values); the caller halves over the
-// whole vocabulary as before.  Every thread of the block returns the same.
+// difference of two distances inside one bin is exact) and notes every fine bin's smallest and largest key: a
+// fine bin of equal values is its own answer.  Otherwise a pass gathers the bin's values and the halvings run
+// over that list.  false: not decided here (the k-th largest or the nucleus's end lies 32 or more below the
+// maximum, or thousands of different values share one fine bin); the caller halves over the whole vocabulary as
+// before.  Every thread of the block returns the same.
 #define BIN_COUNT 2048
 #define BIN_PER_UNIT 64.f
 #define BIN_FINE (BIN_PER_UNIT * BIN_COUNT)
@@ -552,6 +553,9 @@ __device__ __noinline__ bool threshold_by_bins(const float* __restrict__ x, int 
   const float L2E = 1.4426950408889634f;
   unsigned long long* const bin_w = reinterpret_cast<unsigned long long*>(cand.lz);   // BIN_COUNT of them
   unsigned* const bin_n = reinterpret_cast<unsigned*>(cand.le);
+  uint32_t* const bin_lo = reinterpret_cast<uint32_t*>(cand.lidx);                    // of the fine bins: smallest key,
+  uint32_t* const bin_hi = bin_lo + BIN_COUNT;                                        // largest key
+  static_assert(sizeof(cand.lidx) >= 2 * BIN_COUNT * sizeof(uint32_t), "the fine bins' keys lie in the list's indices");
   static_assert(sizeof(cand.lz) >= BIN_COUNT * sizeof(unsigned long long) && sizeof(cand.le) >= BIN_COUNT * sizeof(unsigned),
                 "the bins lie where the list of candidates lies otherwise");
   // a value's bin: by its distance from the maximum; inside bin `coarse`, by the rest of that distance
@@ -571,16 +575,19 @@ __device__ __noinline__ bool threshold_by_bins(const float* __restrict__ x, int 
   int coarse = -1, fine = -1, count = 0;
 #pragma unroll 1
   for (int level = 0; level < 2; ++level) {
-    for (int b = tid; b < BIN_COUNT; b += blockDim.x) { bin_w[b] = 0; bin_n[b] = 0; }
+    for (int b = tid; b < BIN_COUNT; b += blockDim.x) { bin_w[b] = 0; bin_n[b] = 0; bin_lo[b] = 0xffffffffu; bin_hi[b] = 0u; }
     if (tid == 0) pick->bin = -1;
     __syncthreads();
     for_range<VEC>(x, wbeg, wend, lane, [&](int, float v) {
       const float z = scaled(v, inv_t);
-      if (order_key(z) < kmin_in) return;
-      const int b = bin_of(z, coarse);
-      if (b < 0) return;
+      const uint32_t key = order_key(z);
+      const int b = key < kmin_in ? -1 : bin_of(z, coarse);
+      // the last coarse bin (32 or more below the maximum: masked values, the far tail) is not filled: its weights
+      // are below the fixed point's last bit, and a k-th largest value in it is not found here anyway
+      if (b < 0 || (level == 0 && b == BIN_COUNT - 1)) return;
       atomicAdd(&bin_n[b], 1u);
       if (!BY_COUNT) atomicAdd(&bin_w[b], weight_of(z));
+      if (level == 1) { atomicMin(&bin_lo[b], key); atomicMax(&bin_hi[b], key); }
     });
     __syncthreads();
     // this thread's bins, in order from the maximum down
@@ -611,13 +618,16 @@ __device__ __noinline__ bool threshold_by_bins(const float* __restrict__ x, int 
     count = pick->count;
     above = pick->above;
     __syncthreads();
-    if (at < 0) return false;                                        // fewer than k values, or no weight: not here
+    if (at < 0) return false;                 // the k-th largest lies further from the maximum than the bins reach
     if (level == 0) {
-      if (at == BIN_COUNT - 1) return false;                         // further from the maximum than the bins reach
       coarse = at;
       if (count <= BIN_LIST) break;
     } else {
       fine = at;
+      if (bin_lo[at] == bin_hi[at]) {                                // equal values: the k-th largest, the nucleus's end
+        *found = bin_lo[at];
+        return true;
+      }
     }
   }
   if (count > 16 * SEG) return false;
