@@ -87,7 +87,7 @@ def test_bfloat16_equals_the_32_bit_engine_at_real_widths(size):
     g = torch.Generator().manual_seed(1)
     lens = [LONG] * 4 + torch.randint(20, 61, (N_REQUESTS - 4,), generator=g).tolist()
     prompts = [torch.randint(0, config["vocab_size"], (n,), generator=g).tolist() for n in lens]
-    tails = [torch.randint(0, config["vocab_size"], (12,), generator=g).tolist() for _ in lens]   # tokens to decode with
+    tails = [torch.randint(0, config["vocab_size"], (14,), generator=g).tolist() for _ in lens]   # tokens to decode with
     graphs = Harness(config, "bfloat16", True)
     eager = Harness(config, "bfloat16", False, share=graphs)
     full = Harness(config, "float32", False)
@@ -119,7 +119,7 @@ def test_bfloat16_equals_the_32_bit_engine_at_real_widths(size):
     # one token per request: batches on both sides of the thresholds (8 | 9 folded norm, 16 | 17 folded adds,
     # 32 | 33 gate|up, 64 | 65 and 256 | 257 the stacked products, 256 | 257 also the largest graph)
     used = [0] * N_REQUESTS
-    for batch in (8, 9, 16, 17, 32, 33, 64, 65, 256, 257, 1, 128):
+    for batch in (8, 9, 16, 17, 32, 33, 64, 65, 80, 96, 256, 257, 1, 128):
         entries = []
         for r in range(batch):
             entries.append((r, [tails[r][used[r]]]))
